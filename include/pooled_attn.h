@@ -1,0 +1,163 @@
+/* pooled_attn.h -- C ABI of the MI355X (gfx950) attention library for pooled's engines.
+ *
+ * pooled has no FFI on this path: attention is dispatched inline by engine methods that record WebGPU
+ * compute passes.  Each entry point below replaces the group of WebGPU dispatches named in its comment
+ * (paths relative to the pooled repository).  All functions return PA_OK (0) or a PA_ERR_* code and never
+ * abort; pa_last_error() gives the message.  All calls for one context come from one host thread; kernels
+ * are enqueued in order on the context's HIP stream and only pa_sync / the host copies block.
+ *
+ * Pointers named d_* are device (HBM) addresses, h_* are host addresses.  Strides are in elements
+ * (floats for f32 buffers), like the FD / FA / MC uniforms of the reference kernels.
+ */
+#ifndef POOLED_ATTN_H
+#define POOLED_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PA_OK 0
+#define PA_ERR_INVALID 1      /* bad argument / shape */
+#define PA_ERR_UNSUPPORTED 2  /* shape outside the gfx950 table (caller may fall back) */
+#define PA_ERR_HIP 3          /* a HIP runtime call failed */
+#define PA_ERR_NOMEM 4
+
+/* pa_config.flags */
+#define PA_FLAG_QK_NORM 1u    /* per-head RMSNorm of q and k before RoPE (engine/wgsl/base.js:65-79) */
+#define PA_FLAG_GATE 2u       /* q input is interleaved [q(hd) | gate(hd)] per head and the output is
+                                 multiplied by sigmoid(gate) (engine/wgsl/qwen35.js:370-384, :406-416) */
+
+/* output element types */
+#define PA_OUT_F32 0          /* the engine's attnOut feeding wo (engine/qwen35.js:881) */
+#define PA_OUT_F16 1
+
+/* Model-shape constants: the fields of the reference's Config and DN uniforms that attention uses
+ * (engine/wgsl/base.js:4-9, engine/wgsl/qwen35.js:271-275) plus the engine's sizing inputs
+ * (engine/qwen35.js:354-368: maxSeq, batchCols). */
+typedef struct pa_config {
+  uint32_t n_heads;      /* nH */
+  uint32_t n_kv_heads;   /* nKV; nH % nKV == 0, G = nH / nKV */
+  uint32_t head_dim;     /* hd: 128 or 256 */
+  uint32_t n_rot;        /* rotated dims per head (== head_dim for full RoPE), even */
+  float rope_theta;
+  float eps;             /* RMSNorm epsilon */
+  uint32_t max_seq;      /* cache rows per layer */
+  uint32_t n_layers;     /* attention layers (one K and one V cache each) */
+  uint32_t max_cols;     /* widest pass (columns) the context must serve */
+  uint32_t flags;        /* PA_FLAG_* */
+} pa_config;
+
+typedef struct pa_ctx pa_ctx;
+
+/* What the gfx950 table chose for a pass (replaces the reference's load-time calibration and static
+ * formulas: engine/autotune.js:10-68, engine/wgsl/attn_dec.js:40-48, engine/wgsl/attn_tile.js:43-56). */
+typedef struct pa_plan {
+  uint32_t kernel;       /* 0 = split-K decode/verify kernel, 1 = MFMA prefill kernel */
+  uint32_t split_len;    /* cache rows per split */
+  uint32_t n_splits;     /* splits over the context (grid x) */
+  uint32_t col_groups;   /* column groups (grid z) */
+  uint32_t cols_per_group;
+  uint32_t waves;        /* wavefronts per workgroup */
+  uint32_t row_blocks;   /* 16-row (decode) or 32-row (prefill) query blocks per workgroup */
+  uint32_t slots;        /* partial slots per (column, head) the pass needs */
+} pa_plan;
+
+/* ---- life cycle (replaces Qwen35Engine / DenseEngine buffer creation, engine/qwen35.js:871-890,
+ *      :1102-1104; engine/dense.js:226-227; size check engine/qwen35.js:378-383) ---- */
+int pa_create(const pa_config* cfg, pa_ctx** out);
+int pa_destroy(pa_ctx* ctx);
+/* message of the last failing call on ctx (ctx == NULL: of the last failing pa_create) */
+const char* pa_last_error(const pa_ctx* ctx);
+/* allocate layer's K and V caches, f16 [max_seq][n_kv_heads][head_dim] row-major, zero-filled */
+int pa_layer_alloc(pa_ctx* ctx, uint32_t layer);
+/* use the caller's hipStream_t (NULL: the context's own stream) */
+int pa_set_stream(pa_ctx* ctx, void* hip_stream);
+int pa_sync(pa_ctx* ctx);
+
+/* ---- device memory helpers for hosts without their own HIP binding (the Node-API addon) ---- */
+int pa_malloc(pa_ctx* ctx, size_t bytes, void** d_ptr);
+int pa_free(pa_ctx* ctx, void* d_ptr);
+int pa_upload(pa_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);     /* blocking */
+int pa_download(pa_ctx* ctx, void* h_dst, const void* d_src, size_t bytes);   /* blocking, after queued work */
+
+/* ---- pre-step ----
+ * pa_glue_kv: q de-interleave + QK-RMSNorm + (partial) NeoX RoPE for n_cols columns at positions
+ * base_pos + c, and the f16 write of the k and v rows into layer's caches at those positions.
+ * Replaces attn_glue_kv (engine/wgsl/layer_fuse.js:87-146), i.e. attn_glue
+ * (engine/wgsl/qwen35.js:1082-1136) followed by kv_store (:889-906); for full RoPE shapes it replaces
+ * head_norm_dmc + rope_dmc + kv_store_d / attn_glue_d (engine/wgsl/dense.js:144-196, :233-352) with an
+ * f16 cache.  Call sites: engine/qwen35.js:1598-1617, :2473-2488; engine/dense.js:394-399.
+ *   d_q_in : f32 [n_cols][q_stride]; a column holds [nH][2*hd] (PA_FLAG_GATE) or [nH][hd]
+ *   d_k, d_v: f32 [n_cols][k_stride | v_stride], a column holds [nKV][hd]
+ *   d_qw, d_kw: f32 [hd] norm weights (ignored without PA_FLAG_QK_NORM)
+ * Results: roped q -> the context's q buffer (pa_q_buffer), gate -> pa_gate_buffer, cache rows written. */
+int pa_glue_kv(pa_ctx* ctx, uint32_t layer, const float* d_q_in, uint32_t q_stride, const float* d_k,
+               uint32_t k_stride, const float* d_v, uint32_t v_stride, const float* d_qw, const float* d_kw,
+               uint32_t base_pos, uint32_t n_cols);
+/* pa_glue: the same without the cache write; the normed + roped k is written back in place (d_k), as
+ * attn_glue does (engine/wgsl/qwen35.js:1082-1136; call site engine/qwen35.js:2473-2483). */
+int pa_glue(pa_ctx* ctx, const float* d_q_in, uint32_t q_stride, float* d_k, uint32_t k_stride,
+            const float* d_qw, const float* d_kw, uint32_t base_pos, uint32_t n_cols);
+/* pa_kv_store: f16 (round-to-nearest-even) write of already-roped k and raw v rows at base_pos + c.
+ * Replaces kv_store (engine/wgsl/qwen35.js:889-906; call site engine/qwen35.js:2488). */
+int pa_kv_store(pa_ctx* ctx, uint32_t layer, const float* d_k, uint32_t k_stride, const float* d_v,
+                uint32_t v_stride, uint32_t base_pos, uint32_t n_cols);
+/* the context's q / gate buffers written by pa_glue*: f32 [max_cols][nH*hd] (stride = nH*hd) */
+float* pa_q_buffer(pa_ctx* ctx);
+float* pa_gate_buffer(pa_ctx* ctx);
+
+/* ---- attention ----
+ * pa_attn_decode: split-K flash-decoding for one decode token (n_cols = 1) or a speculative-verify block
+ * (n_cols <= max_cols): column c at absolute position base_pos + c attends to cache rows [0, base_pos + c],
+ * followed by the log-sum-exp merge and, when d_gate != NULL, the sigmoid gate.
+ * Replaces attn_dec + attn_dec_combine(_g) + sigmoid_mul(_mc) (engine/wgsl/attn_dec.js:102-287,
+ * engine/wgsl/qwen35.js:406-416, :877-887) and the v1 pair attn_flash + attn_combine(_g)
+ * (engine/wgsl/qwen35.js:99-197, :1059-1080, engine/wgsl/layer_fuse.js:148-181).
+ * Call sites: engine/qwen35.js:1618-1640 (one token), :2494-2516 (verify columns).
+ *   d_q   : f32 [n_cols][q_stride], a column holds roped q [nH][hd]; NULL = pa_q_buffer
+ *   d_gate: f32 [n_cols][gate_stride] gate pre-activations [nH][hd]; NULL = no gate
+ *   d_out : [n_cols][out_stride] of out_dtype, a column holds [nH][hd]
+ * pa_attn_prefill: the same contract for a causal prefill chunk of any width on the f16 MFMA kernel.
+ * Replaces attn_flash_tile + attn_combine_tile + sigmoid_mul_mc (engine/wgsl/attn_tile.js:108-193;
+ * call site engine/qwen35.js:2489-2493, :2516); one call covers what the reference runs as
+ * ceil(n_cols / 16) consecutive 16-column passes (engine/qwen35.js:3843-3860). */
+int pa_attn_decode(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_stride, const float* d_gate,
+                   uint32_t gate_stride, uint32_t base_pos, uint32_t n_cols, void* d_out, uint32_t out_stride,
+                   int out_dtype);
+int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_stride, const float* d_gate,
+                    uint32_t gate_stride, uint32_t base_pos, uint32_t n_cols, void* d_out, uint32_t out_stride,
+                    int out_dtype);
+/* which kernel / split / tile shape the table picks (kind: 0 decode/verify, 1 prefill) */
+int pa_plan_query(const pa_ctx* ctx, int kind, uint32_t base_pos, uint32_t n_cols, pa_plan* out);
+/* override the table's split count for decode passes (0 = table); the reference's attnDecodeSplits
+ * option (engine/qwen35.js:266, engine/wgsl/attn_dec.js:42) */
+int pa_set_decode_splits(pa_ctx* ctx, uint32_t splits);
+
+/* ---- cache access for tests, checkpoints and slot copies (engine/dense.js:20-47 saveSlot/loadSlot
+ *      copy rows [0, pos) of each layer) ----  which: 0 = K, 1 = V; rows are f16 bits [n_rows][nKV*hd] */
+int pa_kv_read(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, void* h_dst);
+int pa_kv_write(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, const void* h_src);
+/* device address of a cache (read-only use; layout above) */
+const void* pa_kv_device_ptr(pa_ctx* ctx, uint32_t layer, int which);
+
+/* ---- timing on the context's stream (HIP events; replaces the reference's timestamp-query passes,
+ *      tests/prof/gpuprof.js:1-16) ----
+ * pa_timer_start / pa_timer_stop bracket a region; stop blocks and returns milliseconds.
+ * pa_profile_enable(1) additionally brackets every attention call's main kernel (the split-K or prefill
+ * kernel, not glue / merge) with its own event pair; pa_profile_read blocks, returns the sum of those
+ * durations and their count since the last read, and resets them. */
+int pa_timer_start(pa_ctx* ctx);
+int pa_timer_stop(pa_ctx* ctx, float* ms);
+int pa_profile_enable(pa_ctx* ctx, int on);
+int pa_profile_read(pa_ctx* ctx, float* ms_sum, uint32_t* count);
+
+/* library / device description, e.g. "pooled_attn 0.1 gfx950 256CU" (static storage) */
+const char* pa_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

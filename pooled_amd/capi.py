@@ -1,0 +1,259 @@
+"""ctypes binding of the C ABI in include/pooled_attn.h (used by the tests, smoke and bench).
+
+The product is libpooled_attn.so; this module only loads it and moves numpy arrays in and out of HBM through
+the library's own pa_malloc / pa_upload / pa_download.  There is no CPU fallback: if the shared library is
+missing, loading raises.
+"""
+import ctypes
+import os
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libpooled_attn.so")
+
+PA_OK, PA_ERR_INVALID, PA_ERR_UNSUPPORTED, PA_ERR_HIP, PA_ERR_NOMEM = 0, 1, 2, 3, 4
+PA_FLAG_QK_NORM, PA_FLAG_GATE = 1, 2
+PA_OUT_F32, PA_OUT_F16 = 0, 1
+
+u32, c_int, vp, f32p = ctypes.c_uint32, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p
+
+
+class PaConfig(ctypes.Structure):
+    _fields_ = [("n_heads", u32), ("n_kv_heads", u32), ("head_dim", u32), ("n_rot", u32),
+                ("rope_theta", ctypes.c_float), ("eps", ctypes.c_float), ("max_seq", u32), ("n_layers", u32),
+                ("max_cols", u32), ("flags", u32)]
+
+
+class PaPlan(ctypes.Structure):
+    _fields_ = [(n, u32) for n in ("kernel", "split_len", "n_splits", "col_groups", "cols_per_group", "waves",
+                                   "row_blocks", "slots")]
+
+
+# name -> (restype, argtypes); every symbol include/pooled_attn.h declares
+SYMBOLS = {
+    "pa_create": (c_int, [ctypes.POINTER(PaConfig), ctypes.POINTER(vp)]),
+    "pa_destroy": (c_int, [vp]),
+    "pa_last_error": (ctypes.c_char_p, [vp]),
+    "pa_layer_alloc": (c_int, [vp, u32]),
+    "pa_set_stream": (c_int, [vp, vp]),
+    "pa_sync": (c_int, [vp]),
+    "pa_malloc": (c_int, [vp, ctypes.c_size_t, ctypes.POINTER(vp)]),
+    "pa_free": (c_int, [vp, vp]),
+    "pa_upload": (c_int, [vp, vp, vp, ctypes.c_size_t]),
+    "pa_download": (c_int, [vp, vp, vp, ctypes.c_size_t]),
+    "pa_glue_kv": (c_int, [vp, u32, f32p, u32, f32p, u32, f32p, u32, f32p, f32p, u32, u32]),
+    "pa_glue": (c_int, [vp, f32p, u32, f32p, u32, f32p, f32p, u32, u32]),
+    "pa_kv_store": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32]),
+    "pa_q_buffer": (vp, [vp]),
+    "pa_gate_buffer": (vp, [vp]),
+    "pa_attn_decode": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32, vp, u32, c_int]),
+    "pa_attn_prefill": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32, vp, u32, c_int]),
+    "pa_plan_query": (c_int, [vp, c_int, u32, u32, ctypes.POINTER(PaPlan)]),
+    "pa_set_decode_splits": (c_int, [vp, u32]),
+    "pa_kv_read": (c_int, [vp, u32, c_int, u32, u32, vp]),
+    "pa_kv_write": (c_int, [vp, u32, c_int, u32, u32, vp]),
+    "pa_kv_device_ptr": (vp, [vp, u32, c_int]),
+    "pa_timer_start": (c_int, [vp]),
+    "pa_timer_stop": (c_int, [vp, ctypes.POINTER(ctypes.c_float)]),
+    "pa_profile_enable": (c_int, [vp, c_int]),
+    "pa_profile_read": (c_int, [vp, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(u32)]),
+    "pa_version": (ctypes.c_char_p, []),
+}
+
+_lib = None
+
+
+def load():
+    """Load libpooled_attn.so and type every exported function.  Raises if the library is not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libpooled_attn.so is not built (run `python -m pooled_amd.build`): %s" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+class PaError(RuntimeError):
+    def __init__(self, code, msg):
+        RuntimeError.__init__(self, "pooled_attn error %d: %s" % (code, msg))
+        self.code = code
+
+
+class DeviceBuffer:
+    """A block of HBM owned through pa_malloc / pa_free."""
+
+    def __init__(self, owner, nbytes):
+        self.owner, self.nbytes = owner, int(nbytes)
+        p = vp()
+        owner._chk(owner.L.pa_malloc(owner.ctx, self.nbytes, ctypes.byref(p)))
+        self.ptr = p.value
+
+    def upload(self, arr, offset=0):
+        a = np.ascontiguousarray(arr)
+        assert offset + a.nbytes <= self.nbytes
+        self.owner._chk(self.owner.L.pa_upload(self.owner.ctx, self.ptr + offset, a.ctypes.data, a.nbytes))
+        return self
+
+    def download(self, dtype, count, offset=0):
+        out = np.empty(count, dtype=dtype)
+        assert offset + out.nbytes <= self.nbytes
+        self.owner._chk(self.owner.L.pa_download(self.owner.ctx, out.ctypes.data, self.ptr + offset, out.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.owner.L.pa_free(self.owner.ctx, self.ptr)
+            self.ptr = None
+
+
+class PooledAttn:
+    """One pa_ctx.  cfg keys: n_heads, n_kv_heads, head_dim, n_rot, rope_theta, eps, qk_norm, gate."""
+
+    def __init__(self, cfg, max_seq, n_layers=1, max_cols=16):
+        self.L = load()
+        self.cfg = dict(cfg)
+        flags = (PA_FLAG_QK_NORM if cfg.get("qk_norm", True) else 0) | (PA_FLAG_GATE if cfg.get("gate", False) else 0)
+        c = PaConfig(cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["n_rot"], cfg["rope_theta"], cfg["eps"],
+                     max_seq, n_layers, max_cols, flags)
+        h = vp()
+        rc = self.L.pa_create(ctypes.byref(c), ctypes.byref(h))
+        if rc != PA_OK:
+            raise PaError(rc, (self.L.pa_last_error(None) or b"").decode())
+        self.ctx = h
+        self.max_seq, self.n_layers, self.max_cols = max_seq, n_layers, max_cols
+        self.q_dim = cfg["n_heads"] * cfg["head_dim"]
+        self.kv_dim = cfg["n_kv_heads"] * cfg["head_dim"]
+        self.q_in_dim = self.q_dim * (2 if cfg.get("gate", False) else 1)
+        self._bufs = []
+
+    def _chk(self, rc):
+        if rc != PA_OK:
+            raise PaError(rc, (self.L.pa_last_error(self.ctx) or b"").decode())
+
+    def close(self):
+        if self.ctx:
+            for b in self._bufs:
+                b.free()
+            self._bufs = []
+            self.L.pa_destroy(self.ctx)
+            self.ctx = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    # ---- memory ----
+    def alloc(self, nbytes):
+        b = DeviceBuffer(self, nbytes)
+        self._bufs.append(b)
+        return b
+
+    def to_device(self, arr):
+        a = np.ascontiguousarray(arr)
+        return self.alloc(max(a.nbytes, 16)).upload(a)
+
+    def layer_alloc(self, layer=0):
+        self._chk(self.L.pa_layer_alloc(self.ctx, layer))
+
+    def sync(self):
+        self._chk(self.L.pa_sync(self.ctx))
+
+    # ---- cache ----
+    def kv_write(self, layer, which, row0, rows16):
+        a = np.ascontiguousarray(rows16, dtype=np.uint16).reshape(-1, self.kv_dim)
+        self._chk(self.L.pa_kv_write(self.ctx, layer, which, row0, a.shape[0], a.ctypes.data))
+
+    def kv_read(self, layer, which, row0, n_rows):
+        out = np.empty((n_rows, self.cfg["n_kv_heads"], self.cfg["head_dim"]), dtype=np.uint16)
+        self._chk(self.L.pa_kv_read(self.ctx, layer, which, row0, n_rows, out.ctypes.data))
+        return out
+
+    # ---- launches (device buffers in, device buffers out) ----
+    def glue_kv(self, layer, d_q, q_stride, d_k, k_stride, d_v, v_stride, d_qw, d_kw, base_pos, n_cols):
+        self._chk(self.L.pa_glue_kv(self.ctx, layer, d_q.ptr, q_stride, d_k.ptr, k_stride, d_v.ptr, v_stride,
+                                    d_qw.ptr if d_qw else None, d_kw.ptr if d_kw else None, base_pos, n_cols))
+
+    def glue(self, d_q, q_stride, d_k, k_stride, d_qw, d_kw, base_pos, n_cols):
+        self._chk(self.L.pa_glue(self.ctx, d_q.ptr, q_stride, d_k.ptr, k_stride, d_qw.ptr if d_qw else None,
+                                 d_kw.ptr if d_kw else None, base_pos, n_cols))
+
+    def kv_store(self, layer, d_k, k_stride, d_v, v_stride, base_pos, n_cols):
+        self._chk(self.L.pa_kv_store(self.ctx, layer, d_k.ptr, k_stride, d_v.ptr, v_stride, base_pos, n_cols))
+
+    def attn(self, kind, layer, d_q, q_stride, d_gate, gate_stride, base_pos, n_cols, d_out, out_stride, out_dtype=PA_OUT_F32):
+        fn = self.L.pa_attn_decode if kind == "decode" else self.L.pa_attn_prefill
+        qp = d_q if isinstance(d_q, (int, type(None))) else d_q.ptr
+        gp = d_gate if isinstance(d_gate, (int, type(None))) else d_gate.ptr
+        self._chk(fn(self.ctx, layer, qp, q_stride, gp, gate_stride, base_pos, n_cols, d_out.ptr, out_stride, out_dtype))
+
+    def q_buffer_ptr(self):
+        return self.L.pa_q_buffer(self.ctx)
+
+    def gate_buffer_ptr(self):
+        return self.L.pa_gate_buffer(self.ctx)
+
+    def read_q_buffer(self, n_cols):
+        out = np.empty((n_cols, self.cfg["n_heads"], self.cfg["head_dim"]), dtype=np.float32)
+        self._chk(self.L.pa_download(self.ctx, out.ctypes.data, self.q_buffer_ptr(), out.nbytes))
+        return out
+
+    def read_gate_buffer(self, n_cols):
+        out = np.empty((n_cols, self.cfg["n_heads"], self.cfg["head_dim"]), dtype=np.float32)
+        self._chk(self.L.pa_download(self.ctx, out.ctypes.data, self.gate_buffer_ptr(), out.nbytes))
+        return out
+
+    def plan(self, kind, base_pos, n_cols):
+        pl = PaPlan()
+        self._chk(self.L.pa_plan_query(self.ctx, 0 if kind == "decode" else 1, base_pos, n_cols, ctypes.byref(pl)))
+        return {n: getattr(pl, n) for n, _ in PaPlan._fields_}
+
+    def set_decode_splits(self, n):
+        self._chk(self.L.pa_set_decode_splits(self.ctx, n))
+
+    # ---- timing ----
+    def timer_start(self):
+        self._chk(self.L.pa_timer_start(self.ctx))
+
+    def timer_stop(self):
+        ms = ctypes.c_float()
+        self._chk(self.L.pa_timer_stop(self.ctx, ctypes.byref(ms)))
+        return ms.value
+
+    def profile_enable(self, on=True):
+        self._chk(self.L.pa_profile_enable(self.ctx, 1 if on else 0))
+
+    def profile_read(self):
+        ms, n = ctypes.c_float(), u32()
+        self._chk(self.L.pa_profile_read(self.ctx, ctypes.byref(ms), ctypes.byref(n)))
+        return ms.value, n.value
+
+    # ---- numpy convenience used by tests / smoke: whole passes from host arrays ----
+    def run_glue_kv(self, layer, q_in, k_in, v_in, qw, kw, base_pos):
+        n = q_in.shape[0]
+        dq, dk, dv = self.to_device(q_in.astype(np.float32)), self.to_device(k_in.astype(np.float32)), self.to_device(v_in.astype(np.float32))
+        dqw, dkw = self.to_device(qw.astype(np.float32)), self.to_device(kw.astype(np.float32))
+        self.glue_kv(layer, dq, q_in.shape[1], dk, k_in.shape[1], dv, v_in.shape[1], dqw, dkw, base_pos, n)
+        self.sync()
+        for b in (dq, dk, dv, dqw, dkw):
+            b.free(); self._bufs.remove(b)
+
+    def run_attn(self, kind, layer, q, base_pos, gate=None, out_dtype=PA_OUT_F32):
+        """q [n, nH, hd] f32 (None: the context's q buffer, n from gate or 1) -> out [n, nH, hd]."""
+        n = q.shape[0]
+        dq = self.to_device(q.reshape(n, -1).astype(np.float32))
+        dg = self.to_device(gate.reshape(n, -1).astype(np.float32)) if gate is not None else None
+        esz = 4 if out_dtype == PA_OUT_F32 else 2
+        dout = self.alloc(n * self.q_dim * esz)
+        self.attn(kind, layer, dq, self.q_dim, dg, self.q_dim if dg else 0, base_pos, n, dout, self.q_dim, out_dtype)
+        self.sync()
+        out = dout.download(np.float32 if out_dtype == PA_OUT_F32 else np.float16, n * self.q_dim)
+        for b in (dq, dg, dout):
+            if b is not None:
+                b.free(); self._bufs.remove(b)
+        return out.reshape(n, self.cfg["n_heads"], self.cfg["head_dim"])

@@ -1,0 +1,356 @@
+// Split-K flash-decoding attention for decode and speculative-verify passes on gfx950 (MI355X).
+//
+// Replaces the reference's attn_dec + attn_dec_combine(_g) + sigmoid_mul
+// (engine/wgsl/attn_dec.js:102-287, engine/wgsl/qwen35.js:406-416).  Same outer shape -- one workgroup per
+// (split of the context, kv head, column group), per-split (m, l, O) partials, a second-pass log-sum-exp
+// merge -- with a CDNA4 inside:
+//
+//   * Every wavefront streams its own 32-position K/V tiles: 128-bit coalesced global loads (a 64-lane load
+//     covers whole 512-byte f16 rows) into registers, the next tile's loads issued as soon as the current
+//     tile's registers have been staged, so a wave always has ~32 KB in flight.
+//   * Tiles are staged in a wave-private LDS region (no workgroup barrier in the loop): K rows are read back
+//     as MFMA A-operands (ds_read_b128), V rows through the gfx950 LDS transpose read (ds_read_b64_tr_b16),
+//     which delivers 4 positions x 1 dim per lane -- the contraction-major layout PV needs.
+//   * S^T = K Q^T and O^T = V^T P^T run on v_mfma_f32_16x16x32_f16.  The S^T accumulator layout (lane =
+//     query row, 4+4 positions) is exactly the B-operand layout of the PV product, so probabilities never
+//     leave registers.  All G heads of a kv head and all columns of a verify block are rows of one tile, so
+//     K/V are read once for the whole block.
+//   * Softmax state (m, l) and O are f32; q and P are rounded to f16 for the MFMA operands.
+//   * Every reduction has a fixed order (lane-group shuffles, wave order, split order): run-to-run deterministic,
+//     no atomics.
+//
+// Row r of a workgroup's tile is (local column r / G, head r % G); column c (absolute position base_pos + c)
+// sees cache rows [0, base_pos + c].
+#include "pa_internal.h"
+#include <hip/hip_fp16.h>
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef __fp16 hh4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+
+#define TILE 32
+#define NEG_INF (-__builtin_inff())
+
+// Compiler-level ordering of LDS accesses inside one wavefront (hardware executes a wave's LDS operations
+// in order; lanes of one wave exchange data through the wave-private region without a workgroup barrier).
+static __device__ inline void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
+  hh4 t = __builtin_amdgcn_ds_read_tr16_b64_v4f16((hh4 __attribute__((address_space(3)))*)p);
+  h4 r; __builtin_memcpy(&r, &t, 8); return r;
+}
+
+template <int HD> struct DecShape {
+  static constexpr int LPR = HD / 8;            // lanes per f16 row at 16 bytes a lane
+  static constexpr int RPL = 64 / LPR;          // rows per wave-wide load
+  static constexpr int NLD = TILE / RPL;        // loads per tile and tensor
+  static constexpr int KROW = HD * 2 + 16;      // staged K row stride (bytes): 16 rows x 16 B hit distinct banks
+  static constexpr int VROW = HD * 2 + 32;      // staged V row stride (bytes)
+  static constexpr int STAGE = TILE * VROW;     // wave-private staging bytes (>= 16 x (HD + 4) floats for the merge)
+  static constexpr int QROW = HD * 2 + 16;      // staged q row stride (bytes)
+  static constexpr int OROW = (HD + 4) * 4;     // merge row stride (bytes)
+  static constexpr int KS = HD / 32;            // k-steps of the QK product
+  static constexpr int DB = HD / 16;            // 16-dim blocks of the output
+};
+
+template <int HD, int NB, int W>
+__global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
+  typedef DecShape<HD> S;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned char* q_lds = smem;                                       // [16*NB][QROW]
+  unsigned char* stage_all = smem + 16 * NB * S::QROW;               // [W][STAGE]
+  float* mex = (float*)(stage_all + W * S::STAGE);                   // [W][16*NB]
+  float* lex = mex + W * 16 * NB;                                    // [W][16*NB]
+
+  const uint32_t sp = blockIdx.x, g = blockIdx.y, cg = blockIdx.z;
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t ln = lane & 15, kg = lane >> 4;
+  const uint32_t G = p.group, nH = p.n_heads;
+  const uint32_t c0 = cg * p.cols_per_group;
+  const uint32_t ncl = min(p.cols_per_group, p.n_cols - c0);
+  const uint32_t R = ncl * G;                                        // live rows (<= 16*NB)
+  const uint32_t seq_max = p.base_pos + c0 + ncl;                    // rows visible to the group's last column
+  const uint32_t t_begin = sp * p.split_len;
+  if (t_begin >= seq_max) return;
+  const uint32_t t_end = min(t_begin + p.split_len, seq_max);
+  const uint32_t kvDim = p.n_kv_heads * HD;
+
+  // ---- q -> f16 rows in LDS (rows >= R are zero) ----
+  for (uint32_t e = tid; e < 16 * NB * (HD / 4); e += W * 64) {
+    const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (r < R) v = *(const float4*)(p.q + (size_t)(c0 + r / G) * p.q_stride + (size_t)(g * G + r % G) * HD + 4 * d4);
+    h4 hv = { (_Float16)v.x, (_Float16)v.y, (_Float16)v.z, (_Float16)v.w };
+    *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
+  }
+  // per-lane row bookkeeping: row nb*16 + ln ends (exclusive) at end_pos[nb]; 0 for padding rows
+  uint32_t end_pos[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    const uint32_t r = nb * 16 + ln;
+    end_pos[nb] = r < R ? p.base_pos + c0 + r / G + 1 : 0u;
+  }
+  __syncthreads();
+
+  unsigned char* stage = stage_all + wave * S::STAGE;
+  const size_t row_bytes = (size_t)kvDim * 2;
+  const uint32_t lrow = lane / S::LPR;
+  // per-lane byte offset inside a wave-wide load; the tile base below is wave-uniform (scalar registers)
+  const uint32_t voff = lrow * (uint32_t)row_bytes + (lane % S::LPR) * 16;
+  const unsigned char* kbase = (const unsigned char*)(p.k_cache + (size_t)g * HD);
+  const unsigned char* vbase = (const unsigned char*)(p.v_cache + (size_t)g * HD);
+
+  f4 acc[S::DB][NB];
+#pragma unroll
+  for (int db = 0; db < S::DB; db++)
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) acc[db][nb] = (f4){0.f, 0.f, 0.f, 0.f};
+  float m_run[NB], l_run[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) { m_run[nb] = NEG_INF; l_run[nb] = 0.f; }
+
+  const uint32_t n_tiles = (t_end - t_begin + TILE - 1) / TILE;
+  u4 kr[S::NLD], vr[S::NLD];
+  const u4 zero4 = {0u, 0u, 0u, 0u};
+
+  // Loads are unconditional: the caches carry TILE rows of padding past max_seq, so a tile that straddles the
+  // end of the context reads valid memory; rows at or past t_end are zeroed (V) or masked (scores) below.
+  uint32_t tile = __builtin_amdgcn_readfirstlane(wave);
+  if (tile < n_tiles) {
+    const size_t tb = (size_t)(t_begin + tile * TILE) * row_bytes;
+#pragma unroll
+    for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
+#pragma unroll
+    for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
+  }
+  for (; tile < n_tiles; tile += W) {
+    const uint32_t tp = t_begin + tile * TILE;
+    const size_t tnb = (size_t)(tp + W * TILE) * row_bytes;   // next tile of this wave
+    const bool more = tile + W < n_tiles;
+    // ---- K tile -> LDS, next K loads ----
+#pragma unroll
+    for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::KROW + (lane % S::LPR) * 16) = kr[i];
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
+    }
+    wave_lds_fence();
+    // ---- S^T = K Q^T ----
+    f4 s[2][NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) { s[0][nb] = (f4){0.f, 0.f, 0.f, 0.f}; s[1][nb] = (f4){0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+    for (int ks = 0; ks < S::KS; ks++) {
+      const h8 a0 = *(const h8*)(stage + ln * S::KROW + ks * 64 + kg * 16);
+      const h8 a1 = *(const h8*)(stage + (16 + ln) * S::KROW + ks * 64 + kg * 16);
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        const h8 b = *(const h8*)(q_lds + (nb * 16 + ln) * S::QROW + ks * 64 + kg * 16);
+        s[0][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b, s[0][nb], 0, 0, 0);
+        s[1][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b, s[1][nb], 0, 0, 0);
+      }
+    }
+    wave_lds_fence();
+    // ---- V tile -> LDS (rows at or past t_end as zeros: 0 x stale bits must not reach O), next V loads ----
+    if (tp + TILE > t_end) {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) if (tp + i * S::RPL + lrow >= t_end) vr[i] = zero4;
+    }
+#pragma unroll
+    for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
+    }
+    // ---- online softmax; lane holds row nb*16 + ln, positions tp + pb*16 + 4*kg + i ----
+    h8 pfrag[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+      float v[8];
+      float mx = NEG_INF;
+#pragma unroll
+      for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const uint32_t pos = tp + pb * 16 + 4 * kg + i;
+          const float x = pos < end_pos[nb] ? s[pb][nb][i] * p.scale : NEG_INF;
+          v[pb * 4 + i] = x;
+          mx = fmaxf(mx, x);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run[nb], mx);
+      const float m_safe = m_new == NEG_INF ? 0.f : m_new;
+      const float alpha = __expf(m_run[nb] - m_safe);
+      float ps = 0.f;
+      h8 pf;
+#pragma unroll
+      for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - m_safe); ps += e; pf[j] = (_Float16)e; }
+      pfrag[nb] = pf;
+      l_run[nb] = l_run[nb] * alpha + ps;
+      m_run[nb] = m_new;
+#pragma unroll
+      for (int db = 0; db < S::DB; db++) acc[db][nb] *= alpha;
+    }
+    wave_lds_fence();
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int db = 0; db < S::DB; db++) {
+      const unsigned char* vp = stage + (4 * kg + (ln >> 2)) * S::VROW + (db * 16 + 4 * (ln & 3)) * 2;
+      const h4 lo = lds_read_tr16(vp);
+      const h4 hi = lds_read_tr16(vp + 16 * S::VROW);
+      const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) acc[db][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pfrag[nb], acc[db][nb], 0, 0, 0);
+    }
+    wave_lds_fence();
+  }
+
+  // ---- merge the W waves of the workgroup ----
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    l_run[nb] += __shfl_xor(l_run[nb], 16, 64);
+    l_run[nb] += __shfl_xor(l_run[nb], 32, 64);
+    if (kg == 0) { mex[wave * 16 * NB + nb * 16 + ln] = m_run[nb]; lex[wave * 16 * NB + nb * 16 + ln] = l_run[nb]; }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    float M = NEG_INF;
+#pragma unroll
+    for (int w = 0; w < W; w++) M = fmaxf(M, mex[w * 16 * NB + nb * 16 + ln]);
+    const float m_safe = M == NEG_INF ? 0.f : M;
+    const float sc = __expf(m_run[nb] - m_safe);
+#pragma unroll
+    for (int db = 0; db < S::DB; db++) {
+      const f4 o = acc[db][nb] * sc;
+      *(f4*)(stage + ln * S::OROW + (db * 16 + 4 * kg) * 4) = o;
+    }
+    __syncthreads();
+    // rows nb*16 .. nb*16+15, HD/4 float4 each, summed over waves in wave order
+    for (uint32_t e = tid; e < 16 * (HD / 4); e += W * 64) {
+      const uint32_t rr = e / (HD / 4), d4 = e % (HD / 4);
+      const uint32_t r = nb * 16 + rr;
+      if (r < R) {
+        f4 o = *(const f4*)(stage_all + rr * S::OROW + d4 * 16);
+#pragma unroll
+        for (int w = 1; w < W; w++) o += *(const f4*)(stage_all + w * S::STAGE + rr * S::OROW + d4 * 16);
+        const uint32_t col = c0 + r / G, hq = g * G + r % G;
+        const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
+        *(f4*)(p.part_o + slot * HD + 4 * d4) = o;
+        if (d4 == 0) {
+          float Mr = NEG_INF;
+#pragma unroll
+          for (int w = 0; w < W; w++) Mr = fmaxf(Mr, mex[w * 16 * NB + r]);
+          const float ms = Mr == NEG_INF ? 0.f : Mr;
+          float L = 0.f;
+#pragma unroll
+          for (int w = 0; w < W; w++) L += lex[w * 16 * NB + r] * __expf(mex[w * 16 * NB + r] - ms);
+          p.part_ml[slot * 2] = Mr;
+          p.part_ml[slot * 2 + 1] = L;
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ---- second pass: log-sum-exp merge over a column's splits, sigmoid gate, output conversion ----
+// One workgroup per (head, column); 256 threads = NG split groups x HD/4 float4 lanes.
+template <int HD>
+__global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
+  constexpr int L4 = HD / 4, NG = 256 / L4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* wl = (float*)smem;                 // [slots] split weights
+  __shared__ float red[256];
+  __shared__ f4 ored[256];
+  const uint32_t h = blockIdx.x, col = blockIdx.y, tid = threadIdx.x;
+  const uint32_t col_end = p.base_pos + col + 1;
+  const uint32_t ns = (col_end + p.split_len - 1) / p.split_len;
+  const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
+  float lm = NEG_INF;
+  for (uint32_t s = tid; s < ns; s += 256) lm = fmaxf(lm, p.part_ml[(base + s) * 2]);
+  red[tid] = lm;
+  __syncthreads();
+  for (uint32_t k = 128; k > 0; k >>= 1) { if (tid < k) red[tid] = fmaxf(red[tid], red[tid + k]); __syncthreads(); }
+  const float M = red[0];
+  __syncthreads();
+  float ll = 0.f;
+  for (uint32_t s = tid; s < ns; s += 256) {
+    const float w = __expf(p.part_ml[(base + s) * 2] - M);
+    wl[s] = w;
+    ll += p.part_ml[(base + s) * 2 + 1] * w;
+  }
+  red[tid] = ll;
+  __syncthreads();
+  for (uint32_t k = 128; k > 0; k >>= 1) { if (tid < k) red[tid] += red[tid + k]; __syncthreads(); }
+  const float L = red[0];
+  const uint32_t grp = tid / L4, l4 = tid % L4;
+  f4 o = {0.f, 0.f, 0.f, 0.f};
+  for (uint32_t s = grp; s < ns; s += NG) o += *(const f4*)(p.part_o + (base + s) * HD + 4 * l4) * wl[s];
+  ored[tid] = o;
+  __syncthreads();
+  if (tid < L4) {
+    f4 t = ored[tid];
+#pragma unroll
+    for (int i = 1; i < NG; i++) t += ored[i * L4 + tid];
+    f4 r = t / L;
+    if (p.gate) {
+      const float4 gt = *(const float4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * HD + 4 * tid);
+      r[0] *= 1.f / (1.f + __expf(-gt.x)); r[1] *= 1.f / (1.f + __expf(-gt.y));
+      r[2] *= 1.f / (1.f + __expf(-gt.z)); r[3] *= 1.f / (1.f + __expf(-gt.w));
+    }
+    if (p.out_f16) {
+      h4 hv = { (_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3] };
+      *(h4*)((_Float16*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + 4 * tid) = hv;
+    } else {
+      *(f4*)((float*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + 4 * tid) = r;
+    }
+  }
+}
+
+template <int HD, int NB, int W>
+static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s) {
+  typedef DecShape<HD> S;
+  const size_t lds = 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((pa_decode_kernel<HD, NB, W>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, p);
+  return hipGetLastError();
+}
+
+template <int HD>
+static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t col_groups, hipStream_t s) {
+  switch (nb) {
+    case 1: return launch_decode_t<HD, 1, 4>(p, col_groups, s);
+    case 2: return launch_decode_t<HD, 2, 4>(p, col_groups, s);
+    case 3: return launch_decode_t<HD, 3, 4>(p, col_groups, s);
+    case 4: return launch_decode_t<HD, 4, 4>(p, col_groups, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s) {
+  if (waves != 4) return hipErrorInvalidValue;
+  if (hd == 256) return launch_decode_hd<256>(p, nb, col_groups, s);
+  if (hd == 128) return launch_decode_hd<128>(p, nb, col_groups, s);
+  return hipErrorInvalidValue;
+}
+
+hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s) {
+  const size_t lds = (size_t)p.slots * sizeof(float);
+  if (hd == 256) hipLaunchKernelGGL(pa_combine_kernel<256>, dim3(p.n_heads, p.n_cols), dim3(256), lds, s, p);
+  else if (hd == 128) hipLaunchKernelGGL(pa_combine_kernel<128>, dim3(p.n_heads, p.n_cols), dim3(256), lds, s, p);
+  else return hipErrorInvalidValue;
+  return hipGetLastError();
+}

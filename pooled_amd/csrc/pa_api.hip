@@ -1,0 +1,425 @@
+// Host side of the C ABI (include/pooled_attn.h): context, caches, the gfx950 plan table, launches.
+#include "pa_internal.h"
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+static thread_local std::string g_create_err;
+
+static int fail(pa_ctx* ctx, int code, const std::string& msg) {
+  if (ctx) ctx->err = msg; else g_create_err = msg;
+  return code;
+}
+static int fail_hip(pa_ctx* ctx, hipError_t e, const char* what) {
+  return fail(ctx, e == hipErrorOutOfMemory ? PA_ERR_NOMEM : PA_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+#define HIPCHK(ctx, call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return fail_hip(ctx, e_, #call); } while (0)
+
+static inline uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+extern "C" const char* pa_version(void) {
+  static char buf[128];
+  int dev = 0, cus = 0;
+  hipDeviceProp_t pr;
+  if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&pr, dev) == hipSuccess) {
+    cus = pr.multiProcessorCount;
+    snprintf(buf, sizeof buf, "pooled_attn 0.1 %s %dCU", pr.gcnArchName, cus);
+  } else {
+    snprintf(buf, sizeof buf, "pooled_attn 0.1 (no HIP device)");
+  }
+  return buf;
+}
+
+extern "C" const char* pa_last_error(const pa_ctx* ctx) { return ctx ? ctx->err.c_str() : g_create_err.c_str(); }
+
+extern "C" int pa_create(const pa_config* cfg, pa_ctx** out) {
+  if (!cfg || !out) return fail(nullptr, PA_ERR_INVALID, "pa_create: null argument");
+  *out = nullptr;
+  const pa_config& c = *cfg;
+  if (c.n_heads == 0 || c.n_kv_heads == 0 || c.n_heads % c.n_kv_heads != 0)
+    return fail(nullptr, PA_ERR_INVALID, "pa_create: n_heads must be a positive multiple of n_kv_heads");
+  if (c.head_dim != 128 && c.head_dim != 256)
+    return fail(nullptr, PA_ERR_UNSUPPORTED, "pa_create: head_dim must be 128 or 256 on the gfx950 table");
+  if (c.n_heads / c.n_kv_heads > (c.head_dim == 256 ? 32u : 64u))
+    return fail(nullptr, PA_ERR_UNSUPPORTED, "pa_create: too many query heads per kv head for the gfx950 table");
+  if (c.n_rot == 0 || (c.n_rot & 1) || c.n_rot > c.head_dim)
+    return fail(nullptr, PA_ERR_INVALID, "pa_create: n_rot must be even and in (0, head_dim]");
+  if (c.max_seq == 0 || c.n_layers == 0 || c.max_cols == 0 || c.max_cols > 65535)
+    return fail(nullptr, PA_ERR_INVALID, "pa_create: max_seq, n_layers, max_cols must be positive (max_cols <= 65535)");
+  if (!(c.rope_theta > 0.f) || !(c.eps >= 0.f))
+    return fail(nullptr, PA_ERR_INVALID, "pa_create: rope_theta must be > 0 and eps >= 0");
+  int ndev = 0;
+  hipError_t e = hipGetDeviceCount(&ndev);
+  if (e != hipSuccess || ndev == 0) return fail(nullptr, PA_ERR_HIP, "pa_create: no HIP device");
+  pa_ctx* ctx = new (std::nothrow) pa_ctx();
+  if (!ctx) return fail(nullptr, PA_ERR_NOMEM, "pa_create: out of host memory");
+  ctx->cfg = c;
+  ctx->layers.resize(c.n_layers);
+  hipDeviceProp_t pr;
+  if ((e = hipGetDevice(&ctx->device)) != hipSuccess || (e = hipGetDeviceProperties(&pr, ctx->device)) != hipSuccess) {
+    delete ctx; return fail_hip(nullptr, e, "pa_create: device query");
+  }
+  if (strncmp(pr.gcnArchName, "gfx950", 6) != 0) {
+    std::string m = std::string("pa_create: built for gfx950, device is ") + pr.gcnArchName;
+    delete ctx; return fail(nullptr, PA_ERR_UNSUPPORTED, m);
+  }
+  ctx->n_cu = pr.multiProcessorCount;
+  const size_t qbytes = (size_t)c.max_cols * c.n_heads * c.head_dim * sizeof(float);
+  std::vector<float> freq(c.n_rot / 2);
+  for (uint32_t i = 0; i < c.n_rot / 2; i++) freq[i] = (float)std::pow((double)c.rope_theta, -(2.0 * i) / (double)c.n_rot);
+  bool ok = (e = hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking)) == hipSuccess
+         && (e = hipMalloc((void**)&ctx->q_buf, qbytes)) == hipSuccess
+         && (e = hipMalloc((void**)&ctx->gate_buf, qbytes)) == hipSuccess
+         && (e = hipMalloc((void**)&ctx->inv_freq, freq.size() * sizeof(float))) == hipSuccess
+         && (e = hipMemcpy(ctx->inv_freq, freq.data(), freq.size() * sizeof(float), hipMemcpyHostToDevice)) == hipSuccess
+         && (e = hipEventCreate(&ctx->t0)) == hipSuccess && (e = hipEventCreate(&ctx->t1)) == hipSuccess;
+  if (!ok) { int rc = fail_hip(nullptr, e, "pa_create: allocation"); pa_destroy(ctx); return rc; }
+  ctx->stream = ctx->own_stream;
+  *out = ctx;
+  return PA_OK;
+}
+
+extern "C" int pa_destroy(pa_ctx* ctx) {
+  if (!ctx) return PA_OK;
+  if (ctx->own_stream) (void)hipStreamSynchronize(ctx->own_stream);
+  for (auto& L : ctx->layers) { if (L.k) (void)hipFree(L.k); if (L.v) (void)hipFree(L.v); }
+  if (ctx->q_buf) (void)hipFree(ctx->q_buf);
+  if (ctx->gate_buf) (void)hipFree(ctx->gate_buf);
+  if (ctx->inv_freq) (void)hipFree(ctx->inv_freq);
+  if (ctx->part_o) (void)hipFree(ctx->part_o);
+  if (ctx->part_ml) (void)hipFree(ctx->part_ml);
+  for (auto ev : ctx->prof_events) (void)hipEventDestroy(ev);
+  if (ctx->t0) (void)hipEventDestroy(ctx->t0);
+  if (ctx->t1) (void)hipEventDestroy(ctx->t1);
+  if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
+  delete ctx;
+  return PA_OK;
+}
+
+extern "C" int pa_layer_alloc(pa_ctx* ctx, uint32_t layer) {
+  if (!ctx) return PA_ERR_INVALID;
+  if (layer >= ctx->cfg.n_layers) return fail(ctx, PA_ERR_INVALID, "pa_layer_alloc: layer out of range");
+  pa_layer& L = ctx->layers[layer];
+  if (L.k) return PA_OK;
+  // 32 rows of zero padding past max_seq: the attention kernels load whole 32-row tiles unconditionally
+  const size_t bytes = ((size_t)ctx->cfg.max_seq + 32) * ctx->cfg.n_kv_heads * ctx->cfg.head_dim * 2;
+  HIPCHK(ctx, hipMalloc((void**)&L.k, bytes));
+  hipError_t e = hipMalloc((void**)&L.v, bytes);
+  if (e != hipSuccess) { (void)hipFree(L.k); L.k = nullptr; return fail_hip(ctx, e, "pa_layer_alloc: V cache"); }
+  HIPCHK(ctx, hipMemsetAsync(L.k, 0, bytes, ctx->stream));
+  HIPCHK(ctx, hipMemsetAsync(L.v, 0, bytes, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return PA_OK;
+}
+
+extern "C" int pa_set_stream(pa_ctx* ctx, void* hip_stream) {
+  if (!ctx) return PA_ERR_INVALID;
+  ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+  return PA_OK;
+}
+extern "C" int pa_sync(pa_ctx* ctx) {
+  if (!ctx) return PA_ERR_INVALID;
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return PA_OK;
+}
+
+extern "C" int pa_malloc(pa_ctx* ctx, size_t bytes, void** d_ptr) {
+  if (!ctx || !d_ptr) return PA_ERR_INVALID;
+  *d_ptr = nullptr;
+  HIPCHK(ctx, hipMalloc(d_ptr, bytes ? bytes : 16));
+  return PA_OK;
+}
+extern "C" int pa_free(pa_ctx* ctx, void* d_ptr) {
+  if (!ctx) return PA_ERR_INVALID;
+  if (d_ptr) { HIPCHK(ctx, hipStreamSynchronize(ctx->stream)); HIPCHK(ctx, hipFree(d_ptr)); }
+  return PA_OK;
+}
+extern "C" int pa_upload(pa_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {
+  if (!ctx || (!d_dst && bytes) || (!h_src && bytes)) return PA_ERR_INVALID;
+  if (!bytes) return PA_OK;
+  HIPCHK(ctx, hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return PA_OK;
+}
+extern "C" int pa_download(pa_ctx* ctx, void* h_dst, const void* d_src, size_t bytes) {
+  if (!ctx || (!h_dst && bytes) || (!d_src && bytes)) return PA_ERR_INVALID;
+  if (!bytes) return PA_OK;
+  HIPCHK(ctx, hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  return PA_OK;
+}
+
+extern "C" float* pa_q_buffer(pa_ctx* ctx) { return ctx ? ctx->q_buf : nullptr; }
+extern "C" float* pa_gate_buffer(pa_ctx* ctx) { return ctx ? ctx->gate_buf : nullptr; }
+
+// ---- pre-step ----------------------------------------------------------------------------------
+
+static int check_cols(pa_ctx* ctx, const char* who, uint32_t layer, bool need_layer, uint32_t base_pos, uint32_t n_cols) {
+  if (n_cols == 0 || n_cols > ctx->cfg.max_cols) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": n_cols must be in [1, max_cols]");
+  if ((uint64_t)base_pos + n_cols > ctx->cfg.max_seq) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": base_pos + n_cols exceeds max_seq");
+  if (need_layer) {
+    if (layer >= ctx->cfg.n_layers) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": layer out of range");
+    if (!ctx->layers[layer].k) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": layer has no cache (call pa_layer_alloc)");
+  }
+  return PA_OK;
+}
+
+static void fill_glue(const pa_ctx* ctx, GlueParams& p) {
+  const pa_config& c = ctx->cfg;
+  memset(&p, 0, sizeof p);
+  p.inv_freq = ctx->inv_freq;
+  p.q_out = ctx->q_buf; p.gate_out = ctx->gate_buf;
+  p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.head_dim = c.head_dim; p.n_rot = c.n_rot;
+  p.flags = c.flags | 0x100u;
+  p.eps = c.eps;
+}
+
+extern "C" int pa_glue_kv(pa_ctx* ctx, uint32_t layer, const float* d_q_in, uint32_t q_stride, const float* d_k,
+                          uint32_t k_stride, const float* d_v, uint32_t v_stride, const float* d_qw, const float* d_kw,
+                          uint32_t base_pos, uint32_t n_cols) {
+  if (!ctx) return PA_ERR_INVALID;
+  int rc = check_cols(ctx, "pa_glue_kv", layer, true, base_pos, n_cols);
+  if (rc) return rc;
+  const pa_config& c = ctx->cfg;
+  const uint32_t qcol = c.n_heads * c.head_dim * ((c.flags & PA_FLAG_GATE) ? 2 : 1), kvd = c.n_kv_heads * c.head_dim;
+  if (!d_q_in || !d_k || !d_v) return fail(ctx, PA_ERR_INVALID, "pa_glue_kv: null input");
+  if ((c.flags & PA_FLAG_QK_NORM) && (!d_qw || !d_kw)) return fail(ctx, PA_ERR_INVALID, "pa_glue_kv: norm weights required");
+  if (q_stride < qcol || k_stride < kvd || v_stride < kvd) return fail(ctx, PA_ERR_INVALID, "pa_glue_kv: column stride shorter than a column");
+  GlueParams p; fill_glue(ctx, p);
+  p.q_in = d_q_in; p.k_in = d_k; p.v_in = d_v; p.qw = d_qw; p.kw = d_kw;
+  p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+  p.q_stride = q_stride; p.k_stride = k_stride; p.v_stride = v_stride;
+  p.base_pos = base_pos; p.n_cols = n_cols;
+  HIPCHK(ctx, pa_launch_glue(p, ctx->stream));
+  return PA_OK;
+}
+
+extern "C" int pa_glue(pa_ctx* ctx, const float* d_q_in, uint32_t q_stride, float* d_k, uint32_t k_stride,
+                       const float* d_qw, const float* d_kw, uint32_t base_pos, uint32_t n_cols) {
+  if (!ctx) return PA_ERR_INVALID;
+  int rc = check_cols(ctx, "pa_glue", 0, false, base_pos, n_cols);
+  if (rc) return rc;
+  const pa_config& c = ctx->cfg;
+  const uint32_t qcol = c.n_heads * c.head_dim * ((c.flags & PA_FLAG_GATE) ? 2 : 1), kvd = c.n_kv_heads * c.head_dim;
+  if (!d_q_in || !d_k) return fail(ctx, PA_ERR_INVALID, "pa_glue: null input");
+  if ((c.flags & PA_FLAG_QK_NORM) && (!d_qw || !d_kw)) return fail(ctx, PA_ERR_INVALID, "pa_glue: norm weights required");
+  if (q_stride < qcol || k_stride < kvd) return fail(ctx, PA_ERR_INVALID, "pa_glue: column stride shorter than a column");
+  GlueParams p; fill_glue(ctx, p);
+  p.q_in = d_q_in; p.k_in = d_k; p.k_out = d_k; p.qw = d_qw; p.kw = d_kw;
+  p.q_stride = q_stride; p.k_stride = k_stride;
+  p.base_pos = base_pos; p.n_cols = n_cols;
+  HIPCHK(ctx, pa_launch_glue(p, ctx->stream));
+  return PA_OK;
+}
+
+extern "C" int pa_kv_store(pa_ctx* ctx, uint32_t layer, const float* d_k, uint32_t k_stride, const float* d_v,
+                           uint32_t v_stride, uint32_t base_pos, uint32_t n_cols) {
+  if (!ctx) return PA_ERR_INVALID;
+  int rc = check_cols(ctx, "pa_kv_store", layer, true, base_pos, n_cols);
+  if (rc) return rc;
+  const pa_config& c = ctx->cfg;
+  const uint32_t kvd = c.n_kv_heads * c.head_dim;
+  if (!d_k || !d_v) return fail(ctx, PA_ERR_INVALID, "pa_kv_store: null input");
+  if (k_stride < kvd || v_stride < kvd) return fail(ctx, PA_ERR_INVALID, "pa_kv_store: column stride shorter than a column");
+  GlueParams p; fill_glue(ctx, p);
+  p.n_heads = 0;            // key heads only
+  p.flags = 0;              // pack only: no norm, no rope
+  p.k_in = d_k; p.v_in = d_v;
+  p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+  p.k_stride = k_stride; p.v_stride = v_stride;
+  p.base_pos = base_pos; p.n_cols = n_cols;
+  HIPCHK(ctx, pa_launch_glue(p, ctx->stream));
+  return PA_OK;
+}
+
+// ---- the gfx950 plan table ----------------------------------------------------------------------
+// Decode / verify (split-K kernel): a workgroup is 4 wavefronts, each streaming 32-position tiles of one
+// kv head; rows = columns x G stacked into 16-row MFMA blocks (at most 4 per workgroup, more columns go to
+// further column groups).  Splits are sized so that about two workgroups (one when the row blocks need the
+// whole register file) land on each CU, but never shorter than the tiles-per-wave floor that keeps the
+// partial (m, l, O) traffic a few percent of the K/V bytes.
+static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl) {
+  const pa_config& c = ctx->cfg;
+  const uint32_t G = c.n_heads / c.n_kv_heads;
+  // rows per workgroup: 16-row blocks whose O^T accumulators still fit the register file next to the
+  // in-flight K/V tile (hd 256: 2 blocks, hd 128: 4 blocks)
+  const uint32_t max_rows = c.head_dim == 256 ? 32 : 64;
+  uint32_t cw = n_cols, groups = 1;
+  if (n_cols * G > max_rows) { cw = max_rows / G; if (cw == 0) return PA_ERR_UNSUPPORTED; groups = ceil_div(n_cols, cw); }
+  const uint32_t nb = ceil_div(cw * G, 16);
+  const uint32_t W = 4;
+  const uint32_t seq_max = base_pos + n_cols;
+  const uint32_t tiles = ceil_div(seq_max, 32);
+  const uint32_t occ = nb == 1 ? 2 : 1;
+  uint32_t target = ctx->decode_splits_override ? ctx->decode_splits_override
+                                                : std::max(1u, (occ * (uint32_t)ctx->n_cu) / (c.n_kv_heads * groups));
+  static const uint32_t floor_tiles[5] = {1, 1, 4, 6, 8};     // tiles per wave, by row blocks
+  uint32_t tpw = std::max(ceil_div(tiles, target * W), ctx->decode_splits_override ? 1u : floor_tiles[nb]);
+  uint32_t sl = 32 * W * tpw;
+  pl->kernel = 0; pl->split_len = sl; pl->n_splits = ceil_div(seq_max, sl);
+  pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = W; pl->row_blocks = nb; pl->slots = pl->n_splits;
+  return PA_OK;
+}
+
+static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl) {
+  // until the MFMA prefill kernel covers a shape, chunks run on the split-K kernel in column groups
+  return plan_decode(ctx, base_pos, n_cols, pl);
+}
+
+extern "C" int pa_plan_query(const pa_ctx* ctx, int kind, uint32_t base_pos, uint32_t n_cols, pa_plan* out) {
+  if (!ctx || !out || n_cols == 0) return PA_ERR_INVALID;
+  return kind == 0 ? plan_decode(ctx, base_pos, n_cols, out) : plan_prefill(ctx, base_pos, n_cols, out);
+}
+extern "C" int pa_set_decode_splits(pa_ctx* ctx, uint32_t splits) {
+  if (!ctx) return PA_ERR_INVALID;
+  ctx->decode_splits_override = splits;
+  return PA_OK;
+}
+
+// ---- attention ----------------------------------------------------------------------------------
+
+static int ensure_partials(pa_ctx* ctx, uint32_t n_cols, uint32_t slots) {
+  const pa_config& c = ctx->cfg;
+  const size_t need_o = (size_t)n_cols * c.n_heads * slots * c.head_dim * sizeof(float);
+  const size_t need_ml = (size_t)n_cols * c.n_heads * slots * 2 * sizeof(float);
+  if (need_o > ctx->part_o_bytes) {
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->part_o) { HIPCHK(ctx, hipFree(ctx->part_o)); ctx->part_o = nullptr; ctx->part_o_bytes = 0; }
+    HIPCHK(ctx, hipMalloc((void**)&ctx->part_o, need_o));
+    ctx->part_o_bytes = need_o;
+  }
+  if (need_ml > ctx->part_ml_bytes) {
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->part_ml) { HIPCHK(ctx, hipFree(ctx->part_ml)); ctx->part_ml = nullptr; ctx->part_ml_bytes = 0; }
+    HIPCHK(ctx, hipMalloc((void**)&ctx->part_ml, need_ml));
+    ctx->part_ml_bytes = need_ml;
+  }
+  return PA_OK;
+}
+
+static int prof_begin(pa_ctx* ctx) {
+  if (!ctx->profiling) return PA_OK;
+  if (ctx->prof_used + 2 > ctx->prof_events.size()) {
+    for (int i = 0; i < 2; i++) { hipEvent_t ev; HIPCHK(ctx, hipEventCreate(&ev)); ctx->prof_events.push_back(ev); }
+  }
+  HIPCHK(ctx, hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream));
+  return PA_OK;
+}
+static int prof_end(pa_ctx* ctx) {
+  if (!ctx->profiling) return PA_OK;
+  HIPCHK(ctx, hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream));
+  ctx->prof_used += 2;
+  return PA_OK;
+}
+
+static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, const float* d_q, uint32_t q_stride,
+                       const float* d_gate, uint32_t gate_stride, uint32_t base_pos, uint32_t n_cols, void* d_out,
+                       uint32_t out_stride, int out_dtype) {
+  if (!ctx) return PA_ERR_INVALID;
+  int rc = check_cols(ctx, who, layer, true, base_pos, n_cols);
+  if (rc) return rc;
+  const pa_config& c = ctx->cfg;
+  const uint32_t qd = c.n_heads * c.head_dim;
+  if (!d_out) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null output");
+  if (out_dtype != PA_OUT_F32 && out_dtype != PA_OUT_F16) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": bad out_dtype");
+  if (!d_q) { d_q = ctx->q_buf; q_stride = qd; }
+  if (q_stride < qd || out_stride < qd || (d_gate && gate_stride < qd))
+    return fail(ctx, PA_ERR_INVALID, std::string(who) + ": column stride shorter than a column");
+  if ((q_stride & 3) || (out_stride & 3) || (d_gate && (gate_stride & 3)) || ((uintptr_t)d_q & 15) || ((uintptr_t)d_out & 15) || ((uintptr_t)d_gate & 15))
+    return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned with strides a multiple of 4 elements");
+  pa_plan pl;
+  rc = kind == 0 ? plan_decode(ctx, base_pos, n_cols, &pl) : plan_prefill(ctx, base_pos, n_cols, &pl);
+  if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
+  if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
+  rc = ensure_partials(ctx, n_cols, pl.slots);
+  if (rc) return rc;
+  AttnParams p; memset(&p, 0, sizeof p);
+  p.q = d_q; p.gate = d_gate; p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+  p.part_o = ctx->part_o; p.part_ml = ctx->part_ml; p.out = d_out;
+  p.q_stride = q_stride; p.gate_stride = gate_stride; p.out_stride = out_stride;
+  p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
+  p.base_pos = base_pos; p.n_cols = n_cols;
+  p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
+  p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
+  p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
+  if ((rc = prof_begin(ctx))) return rc;
+  if (pl.kernel == 0) HIPCHK(ctx, pa_launch_decode(p, c.head_dim, pl.row_blocks, pl.waves, pl.col_groups, ctx->stream));
+  else HIPCHK(ctx, pa_launch_prefill(p, c.head_dim, pl.row_blocks, pl.col_groups, ctx->stream));
+  if ((rc = prof_end(ctx))) return rc;
+  HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
+  return PA_OK;
+}
+
+extern "C" int pa_attn_decode(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_stride, const float* d_gate,
+                              uint32_t gate_stride, uint32_t base_pos, uint32_t n_cols, void* d_out, uint32_t out_stride,
+                              int out_dtype) {
+  return attn_common(ctx, "pa_attn_decode", 0, layer, d_q, q_stride, d_gate, gate_stride, base_pos, n_cols, d_out, out_stride, out_dtype);
+}
+extern "C" int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_stride, const float* d_gate,
+                               uint32_t gate_stride, uint32_t base_pos, uint32_t n_cols, void* d_out, uint32_t out_stride,
+                               int out_dtype) {
+  return attn_common(ctx, "pa_attn_prefill", 1, layer, d_q, q_stride, d_gate, gate_stride, base_pos, n_cols, d_out, out_stride, out_dtype);
+}
+
+// ---- cache access ---------------------------------------------------------------------------------
+
+static int kv_rows(pa_ctx* ctx, const char* who, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, uint16_t** base, size_t* bytes) {
+  if (layer >= ctx->cfg.n_layers || !ctx->layers[layer].k) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": layer not allocated");
+  if (which != 0 && which != 1) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": which must be 0 (K) or 1 (V)");
+  if ((uint64_t)row0 + n_rows > ctx->cfg.max_seq) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": rows exceed max_seq");
+  const size_t kvd = (size_t)ctx->cfg.n_kv_heads * ctx->cfg.head_dim;
+  *base = (which ? ctx->layers[layer].v : ctx->layers[layer].k) + (size_t)row0 * kvd;
+  *bytes = (size_t)n_rows * kvd * 2;
+  return PA_OK;
+}
+extern "C" int pa_kv_read(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, void* h_dst) {
+  if (!ctx) return PA_ERR_INVALID;
+  uint16_t* b; size_t n;
+  int rc = kv_rows(ctx, "pa_kv_read", layer, which, row0, n_rows, &b, &n);
+  return rc ? rc : pa_download(ctx, h_dst, b, n);
+}
+extern "C" int pa_kv_write(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, const void* h_src) {
+  if (!ctx) return PA_ERR_INVALID;
+  uint16_t* b; size_t n;
+  int rc = kv_rows(ctx, "pa_kv_write", layer, which, row0, n_rows, &b, &n);
+  return rc ? rc : pa_upload(ctx, b, h_src, n);
+}
+extern "C" const void* pa_kv_device_ptr(pa_ctx* ctx, uint32_t layer, int which) {
+  if (!ctx || layer >= ctx->cfg.n_layers) return nullptr;
+  return which ? (const void*)ctx->layers[layer].v : (const void*)ctx->layers[layer].k;
+}
+
+// ---- timing -----------------------------------------------------------------------------------------
+
+extern "C" int pa_timer_start(pa_ctx* ctx) {
+  if (!ctx) return PA_ERR_INVALID;
+  HIPCHK(ctx, hipEventRecord(ctx->t0, ctx->stream));
+  return PA_OK;
+}
+extern "C" int pa_timer_stop(pa_ctx* ctx, float* ms) {
+  if (!ctx || !ms) return PA_ERR_INVALID;
+  HIPCHK(ctx, hipEventRecord(ctx->t1, ctx->stream));
+  HIPCHK(ctx, hipEventSynchronize(ctx->t1));
+  HIPCHK(ctx, hipEventElapsedTime(ms, ctx->t0, ctx->t1));
+  return PA_OK;
+}
+extern "C" int pa_profile_enable(pa_ctx* ctx, int on) {
+  if (!ctx) return PA_ERR_INVALID;
+  ctx->profiling = on != 0;
+  ctx->prof_used = 0;
+  return PA_OK;
+}
+extern "C" int pa_profile_read(pa_ctx* ctx, float* ms_sum, uint32_t* count) {
+  if (!ctx || !ms_sum || !count) return PA_ERR_INVALID;
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  float sum = 0.f;
+  for (size_t i = 0; i + 1 < ctx->prof_used; i += 2) {
+    float ms = 0.f;
+    HIPCHK(ctx, hipEventElapsedTime(&ms, ctx->prof_events[i], ctx->prof_events[i + 1]));
+    sum += ms;
+  }
+  *ms_sum = sum; *count = (uint32_t)(ctx->prof_used / 2);
+  ctx->prof_used = 0;
+  return PA_OK;
+}

@@ -1,0 +1,72 @@
+// Internal declarations shared by the host C ABI and the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string>
+#include <vector>
+#include "../../include/pooled_attn.h"
+
+// ---- kernel-side parameter blocks -------------------------------------------------------------
+
+struct GlueParams {
+  const float* q_in; const float* k_in; const float* v_in;   // column-batched f32 inputs
+  float* k_out;                                              // in-place k write-back (pa_glue) or nullptr
+  const float* qw; const float* kw;                          // norm weights [hd]
+  const float* inv_freq;                                     // [n_rot/2] f32, theta^(-2i/n_rot)
+  float* q_out; float* gate_out;                             // [n_cols][nH*hd]
+  uint16_t* k_cache; uint16_t* v_cache;                      // f16 [max_seq][nKV*hd] or nullptr
+  uint32_t q_stride, k_stride, v_stride;
+  uint32_t n_heads, n_kv_heads, head_dim, n_rot;
+  uint32_t base_pos, n_cols;
+  uint32_t flags;                                            // PA_FLAG_*; bit 8: rope/norm enabled (0 = pack only)
+  float eps;
+};
+
+struct AttnParams {
+  const float* q; const float* gate;          // f32 [n_cols][stride]
+  const uint16_t* k_cache; const uint16_t* v_cache;
+  float* part_o; float* part_ml;              // split partials: [(col*nH + h)*slots + sp][hd], [..][2]
+  void* out;                                  // [n_cols][out_stride]
+  uint32_t q_stride, gate_stride, out_stride;
+  uint32_t n_heads, n_kv_heads, group;        // group = nH / nKV
+  uint32_t base_pos, n_cols;                  // column c sees rows [0, base_pos + c]
+  uint32_t split_len, n_splits, slots;
+  uint32_t cols_per_group;                    // columns per workgroup (grid z = column groups)
+  uint32_t max_seq;
+  int out_f16;
+  float scale;                                // 1 / sqrt(hd)
+};
+
+// ---- kernel launchers (defined next to their kernels) ------------------------------------------
+
+hipError_t pa_launch_glue(const GlueParams& p, hipStream_t s);
+// waves per workgroup W in {4, 8}; NB = 16-row query blocks per workgroup (1..4); hd in {128, 256}
+hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s);
+hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);
+// MFMA prefill; returns hipErrorNotSupported for shapes it does not cover
+hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s);
+
+// ---- context -----------------------------------------------------------------------------------
+
+struct pa_layer { uint16_t* k = nullptr; uint16_t* v = nullptr; };
+
+struct pa_ctx {
+  pa_config cfg{};
+  int device = 0;
+  int n_cu = 0;
+  hipStream_t own_stream = nullptr;
+  hipStream_t stream = nullptr;
+  std::vector<pa_layer> layers;
+  float* q_buf = nullptr;       // [max_cols][nH*hd]
+  float* gate_buf = nullptr;    // [max_cols][nH*hd]
+  float* inv_freq = nullptr;    // [n_rot/2]
+  float* part_o = nullptr; float* part_ml = nullptr;
+  size_t part_o_bytes = 0, part_ml_bytes = 0;
+  uint32_t decode_splits_override = 0;
+  // timing
+  hipEvent_t t0 = nullptr, t1 = nullptr;
+  bool profiling = false;
+  std::vector<hipEvent_t> prof_events;   // pairs
+  size_t prof_used = 0;
+  std::string err;
+};

@@ -1,0 +1,192 @@
+"""GPU parity of decode / speculative-verify attention through the C ABI against the CPU oracle.
+Tolerance (floating point): max-abs <= 2e-3 and max|d|/max|ref| <= 1e-2 of the f32/f64 reference."""
+import numpy as np
+import pytest
+from oracle import attn_oracle as O
+from oracle import c_oracle as C
+from pooled_amd.capi import PooledAttn, PA_OUT_F16
+from helpers import SHAPES, assert_parity, random_cache, oracle_cache
+
+pytestmark = pytest.mark.gpu
+
+NAN16 = 0x7E00
+
+
+def _ctx_with_cache(cfg, k16, v16, max_seq, max_cols=16, poison_from=None):
+    pa = PooledAttn(cfg, max_seq, n_layers=1, max_cols=max_cols)
+    pa.layer_alloc(0)
+    K, V = k16.copy(), v16.copy()
+    if poison_from is not None:
+        K[poison_from:] = NAN16; V[poison_from:] = NAN16
+    pa.kv_write(0, 0, 0, K); pa.kv_write(0, 1, 0, V)
+    return pa
+
+
+SEQ_LENS = [1, 2, 5, 31, 32, 33, 63, 64, 65, 127, 128, 129, 300, 1000, 2049, 4097]
+
+
+@pytest.mark.parametrize("shape", ["qwen36_moe", "qwen38_27b", "qwen3_1p7b"])
+def test_decode_seq_lens(shape):
+    """The context lengths of tests/test_attn_dec.js:106-107 (split-length steps), K in +-0.3-like spread."""
+    cfg = SHAPES[shape]
+    rng = np.random.default_rng(7)
+    max_seq = max(SEQ_LENS) + 40
+    k16, v16 = random_cache(cfg, max_seq, seed=8)
+    q = rng.standard_normal((1, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32) * 2
+    with _ctx_with_cache(cfg, k16, v16, max_seq) as pa:
+        for L in SEQ_LENS:
+            # rows at or past L are NaN: any causal leak poisons the output (tests/unit/attn_tile_test.js:43-50)
+            pa.kv_write(0, 0, 0, np.where(np.arange(max_seq)[:, None, None] < L, k16, NAN16).astype(np.uint16))
+            pa.kv_write(0, 1, 0, np.where(np.arange(max_seq)[:, None, None] < L, v16, NAN16).astype(np.uint16))
+            got = pa.run_attn("decode", 0, q, L - 1)
+            ref = C.attention(q, k16, v16, L - 1)
+            assert_parity(got, ref, "%s seqLen %d" % (shape, L))
+
+
+def test_decode_closed_forms():
+    cfg = SHAPES["qwen36_moe"]
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    rng = np.random.default_rng(9)
+    L = 1500
+    k16, v16 = random_cache(cfg, L, seed=10)
+    q = rng.standard_normal((1, nH, hd), dtype=np.float32)
+    v = v16.view(np.float16)
+    with _ctx_with_cache(cfg, k16, v16, L) as pa:
+        o = pa.run_attn("decode", 0, q, 0)                                 # one row -> that V row
+        for h in range(nH):
+            assert np.allclose(o[0, h], v[0, h // (nH // nKV)].astype(np.float32), atol=1e-6)
+        o = pa.run_attn("decode", 0, np.zeros_like(q), L - 1)               # q = 0 -> mean of V rows
+        assert np.abs(o[0, 3] - v[:, 0].astype(np.float64).mean(0)).max() < 2e-4
+        pa.kv_write(0, 1, 0, np.full((L, nKV, hd), 0x3A00, np.uint16))      # constant V = 0.75
+        assert np.abs(pa.run_attn("decode", 0, q, L - 1) - 0.75).max() < 1e-3
+
+
+def test_decode_split_invariance_and_plan():
+    cfg = SHAPES["qwen36_moe"]
+    rng = np.random.default_rng(11)
+    L = 5000
+    k16, v16 = random_cache(cfg, L, seed=12)
+    q = rng.standard_normal((1, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32) * 1.5
+    ref = C.attention(q, k16, v16, L - 1)
+    with _ctx_with_cache(cfg, k16, v16, L) as pa:
+        outs = []
+        for s in (0, 1, 3, 16, 40):
+            pa.set_decode_splits(s)
+            pl = pa.plan("decode", L - 1, 1)
+            assert pl["n_splits"] * pl["split_len"] >= L and pl["split_len"] % 32 == 0
+            if s:
+                assert pl["n_splits"] <= s
+            outs.append(pa.run_attn("decode", 0, q, L - 1))
+            assert_parity(outs[-1], ref, "splits %d" % s)
+        assert max(np.abs(o - outs[0]).max() for o in outs) < 2e-4
+        # deterministic run to run
+        pa.set_decode_splits(0)
+        assert np.array_equal(pa.run_attn("decode", 0, q, L - 1), pa.run_attn("decode", 0, q, L - 1))
+
+
+@pytest.mark.parametrize("shape,n_cols,base", [("qwen36_moe", 4, 996), ("qwen36_moe", 16, 3000), ("qwen38_27b", 8, 2040),
+                                               ("qwen3_1p7b", 4, 510), ("qwen38_27b", 16, 17), ("qwen36_moe", 7, 0)])
+def test_verify_equals_sequential_decodes(shape, n_cols, base):
+    """A verify block must equal n sequential single-token decodes (engine/wgsl/attn_dec.js:12-16;
+    tests/test_attn_dec.js:89-97) -- here within tolerance -- and the oracle."""
+    cfg = SHAPES[shape]
+    rng = np.random.default_rng(base + n_cols)
+    L = base + n_cols
+    k16, v16 = random_cache(cfg, L + 5, seed=13)
+    q = rng.standard_normal((n_cols, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    gate = rng.standard_normal((n_cols, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32) if cfg["gate"] else None
+    ref = C.attention(q, k16, v16, base, gate=gate)
+    with _ctx_with_cache(cfg, k16, v16, L + 5, poison_from=L) as pa:
+        multi = pa.run_attn("decode", 0, q, base, gate=gate)
+        assert_parity(multi, ref, "verify block")
+        for c in range(n_cols):
+            single = pa.run_attn("decode", 0, q[c:c + 1], base + c, gate=None if gate is None else gate[c:c + 1])
+            assert_parity(single, ref[c:c + 1], "single decode col %d" % c)
+            assert np.abs(single[0] - multi[c]).max() <= 1e-3
+
+
+def test_decode_f16_output_and_strides():
+    cfg = SHAPES["qwen36_moe"]
+    rng = np.random.default_rng(14)
+    L, n = 700, 3
+    k16, v16 = random_cache(cfg, L + n, seed=15)
+    q = rng.standard_normal((n, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    gate = rng.standard_normal(q.shape, dtype=np.float32)
+    ref = C.attention(q, k16, v16, L, gate=gate)
+    with _ctx_with_cache(cfg, k16, v16, L + n) as pa:
+        got = pa.run_attn("decode", 0, q, L, gate=gate, out_dtype=PA_OUT_F16)
+        assert got.dtype == np.float16
+        assert_parity(got.astype(np.float32), ref, "f16 out")
+        # padded column strides (the engine aligns columns to 256 bytes, engine/qwen35.js:2054-2055)
+        qd, pad = pa.q_dim, 64
+        qp = np.full((n, qd + pad), np.nan, np.float32); qp[:, :qd] = q.reshape(n, -1)
+        gp = np.full((n, qd + pad), np.nan, np.float32); gp[:, :qd] = gate.reshape(n, -1)
+        dq, dg = pa.to_device(qp), pa.to_device(gp)
+        dout = pa.to_device(np.full((n, qd + pad), -7.0, np.float32))
+        pa.attn("decode", 0, dq, qd + pad, dg, qd + pad, L, n, dout, qd + pad)
+        pa.sync()
+        o = dout.download(np.float32, n * (qd + pad)).reshape(n, qd + pad)
+        assert_parity(o[:, :qd].reshape(ref.shape), ref, "padded strides")
+        assert np.all(o[:, qd:] == -7.0), "wrote into the padding between columns"
+
+
+def test_c1_decode_full_pipeline():
+    """Config 1: Qwen3-1.7B shape, ctx 2048, pre-step (QK-RMSNorm + full RoPE theta 1e6) on the GPU for the
+    query column, cache rows built by the oracle's pre-step; f32 softmax; f16 output."""
+    cfg = SHAPES["qwen3_1p7b"]
+    ctx = 2048
+    d = O.make_inputs(cfg, ctx, 1, seed=0x5EED0001)
+    k16, v16 = oracle_cache(cfg, d["kraw"][:ctx], d["vraw"][:ctx], d["kw"])
+    g = O.glue_kv(d["qraw"], d["kraw"][ctx:], d["vraw"][ctx:], d["qw"], d["kw"], ctx, cfg)
+    kall = np.concatenate([k16, g["k16"]]); vall = np.concatenate([v16, g["v16"]])
+    ref = C.attention(g["q"], kall, vall, ctx)
+    with PooledAttn(cfg, ctx + 1, n_layers=1, max_cols=1) as pa:
+        pa.layer_alloc(0)
+        pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
+        pa.run_glue_kv(0, d["qraw"], d["kraw"][ctx:], d["vraw"][ctx:], d["qw"], d["kw"], ctx)
+        assert np.array_equal(pa.kv_read(0, 0, ctx, 1), g["k16"])
+        dout = pa.alloc(pa.q_dim * 2)
+        pa.attn("decode", 0, None, 0, None, 0, ctx, 1, dout, pa.q_dim, PA_OUT_F16)    # q from the context's buffer
+        pa.sync()
+        got = dout.download(np.float16, pa.q_dim).reshape(ref.shape).astype(np.float32)
+    assert_parity(got, ref, "C1")
+
+
+def test_c3_gated_decode_32k():
+    """Config 3: Qwen3.6-35B-MoE attention shape, ctx 32768, partial RoPE (64 dims, theta 1e7), sigmoid gate."""
+    cfg = SHAPES["qwen36_moe"]
+    ctx = 32768
+    d = O.make_inputs(cfg, ctx, 1, seed=0x5EED0003)
+    k16, v16 = oracle_cache(cfg, d["kraw"][:ctx], d["vraw"][:ctx], d["kw"])
+    g = O.glue_kv(d["qraw"], d["kraw"][ctx:], d["vraw"][ctx:], d["qw"], d["kw"], ctx, cfg)
+    kall = np.concatenate([k16, g["k16"]]); vall = np.concatenate([v16, g["v16"]])
+    ref = C.attention(g["q"], kall, vall, ctx, gate=g["gate"])
+    with PooledAttn(cfg, ctx + 1, n_layers=1, max_cols=1) as pa:
+        pa.layer_alloc(0)
+        pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
+        pa.run_glue_kv(0, d["qraw"], d["kraw"][ctx:], d["vraw"][ctx:], d["qw"], d["kw"], ctx)
+        dout = pa.alloc(pa.q_dim * 4)
+        pa.attn("decode", 0, None, 0, pa.gate_buffer_ptr(), pa.q_dim, ctx, 1, dout, pa.q_dim)
+        pa.sync()
+        got = dout.download(np.float32, pa.q_dim).reshape(ref.shape)
+    assert_parity(got, ref, "C3")
+
+
+def test_c4_verify_64k():
+    """Config 4: 8-token draft block over a 65536-token cache, Qwen3.8-27B attention shape, gate; equals 8
+    sequential decodes (checked on columns 0 and 7) and the oracle."""
+    cfg = SHAPES["qwen38_27b"]
+    ctx, n = 65536, 8
+    rng = np.random.default_rng(0x5EED0004)
+    k16, v16 = random_cache(cfg, ctx + n, seed=0x5EED0004)
+    q = O.rope_neox(O.head_rmsnorm(rng.standard_normal((n, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32),
+                                   np.ones(cfg["head_dim"], np.float32), cfg["eps"]), ctx + np.arange(n), cfg["n_rot"], cfg["rope_theta"])
+    gate = rng.standard_normal(q.shape, dtype=np.float32)
+    ref = C.attention(q, k16, v16, ctx, gate=gate)
+    with _ctx_with_cache(cfg, k16, v16, ctx + n, max_cols=n) as pa:
+        multi = pa.run_attn("decode", 0, q, ctx, gate=gate)
+        assert_parity(multi, ref, "C4 block")
+        for c in (0, 7):
+            single = pa.run_attn("decode", 0, q[c:c + 1], ctx + c, gate=gate[c:c + 1])
+            assert_parity(single, ref[c:c + 1], "C4 decode col %d" % c)
+            assert np.abs(single[0] - multi[c]).max() <= 1e-3
