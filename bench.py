@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Headline workload (BASELINE.json's metric, "decode attn KV-read GB/s @32K ctx"): configuration 3 --
+single-token gated decode attention, Qwen3.6-35B-MoE attention shape (16 q heads, 2 kv heads, head_dim 256),
+context 32768.  A step is one pass of the hot path for one token on one attention layer: pre-step (q
+de-interleave + QK-RMSNorm + partial RoPE + f16 KV write at position 32768), split-K decode kernel, log-sum-exp
+merge with the sigmoid gate.  Consecutive steps walk over N_LAYERS distinct layers' caches (as a model does),
+so the 64 MiB of K/V a step reads is never resident in the 256 MB last-level cache from the previous step.
+value = algorithmic KV bytes per step / wall time per step, all inputs resident in HBM.
+
+One JSON line on stdout; progress on stderr.
+"""
+import argparse
+import json
+import os
+import shutil
+import struct
+import subprocess
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+C3 = dict(n_heads=16, n_kv_heads=2, head_dim=256, n_rot=64, rope_theta=1e7, eps=1e-6, qk_norm=True, gate=True)
+C3_CTX = 32768
+N_LAYERS = 6          # 6 x 64 MiB of K/V > 256 MB last-level cache
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def fill_cache(pa, cfg, layer, ctx, seed, chunk):
+    """Write cache rows [0, ctx) of one layer by running the library's own pre-step on seeded N(0,1) k / v."""
+    rng = np.random.default_rng(seed)
+    kvd = cfg["n_kv_heads"] * cfg["head_dim"]
+    qin = cfg["n_heads"] * cfg["head_dim"] * (2 if cfg.get("gate") else 1)
+    qw = pa.to_device(np.ones(cfg["head_dim"], np.float32)); kw = pa.to_device(np.ones(cfg["head_dim"], np.float32))
+    dq = pa.to_device(np.zeros((chunk, qin), np.float32) + 0.5)
+    dk = pa.alloc(chunk * kvd * 4); dv = pa.alloc(chunk * kvd * 4)
+    for t0 in range(0, ctx, chunk):
+        n = min(chunk, ctx - t0)
+        dk.upload(rng.standard_normal((n, kvd), dtype=np.float32)); dv.upload(rng.standard_normal((n, kvd), dtype=np.float32))
+        pa.glue_kv(layer, dq, qin, dk, kvd, dv, kvd, qw, kw, t0, n)
+    pa.sync()
+    for b in (qw, kw, dq, dk, dv):
+        b.free(); pa._bufs.remove(b)
+
+
+def cpu_baseline_c3(pa, cfg, ctx, q, gate, gpu_out, budget_s=25.0):
+    """The reference's CPU attention loops (JavaScript restatement, one thread) on the same column: reads the
+    layer-0 cache back from HBM, times node oracle/attn_ref.js, and compares its output with the GPU's."""
+    node = shutil.which("node")
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    rows = ctx + 1
+    k16 = pa.kv_read(0, 0, 0, rows); v16 = pa.kv_read(0, 1, 0, rows)
+    kv_bytes = 2 * rows * nKV * hd * 2
+    if node is None:
+        from oracle import c_oracle
+        K = k16.view(np.float16).astype(np.float32).reshape(rows, -1); V = v16.view(np.float16).astype(np.float32).reshape(rows, -1)
+        out = np.zeros(nH * hd, np.float32)
+        qf = np.ascontiguousarray(q.reshape(-1)); gf = np.ascontiguousarray(gate.reshape(-1))
+        t0 = time.perf_counter()
+        c_oracle.lib().pa_oracle_attention_ref_loops(qf.ctypes.data, K.ctypes.data, V.ctypes.data, rows, nH, nKV, hd, gf.ctypes.data, out.ctypes.data)
+        dt = time.perf_counter() - t0
+        diff = float(np.abs(out - gpu_out.reshape(-1)).max())
+        return dict(value=kv_bytes / dt / 1e9, unit="GB/s", cores=1, kind="port",
+                    sample="full C3 column, 1 rep, C restatement of the reference loops (node not found)", ms=dt * 1e3, max_abs_diff_vs_gpu=diff)
+    with tempfile.TemporaryDirectory() as td:
+        inp, outp = os.path.join(td, "in.bin"), os.path.join(td, "out.bin")
+        with open(inp, "wb") as f:
+            f.write(struct.pack("8i", 1, nH, nKV, hd, ctx, rows, 1, 1))
+            f.write(np.array([0], np.int32).tobytes()); f.write(q.astype(np.float32).tobytes())
+            f.write(k16.tobytes()); f.write(v16.tobytes()); f.write(gate.astype(np.float32).tobytes())
+        reps = 4
+        r = subprocess.run([node, os.path.join(ROOT, "oracle", "attn_ref.js"), inp, outp, str(reps)], capture_output=True, text=True, timeout=300)
+        if r.returncode != 0:
+            raise RuntimeError("attn_ref.js failed: " + r.stderr[-500:])
+        info = json.loads(r.stdout.strip().splitlines()[-1])
+        out = np.fromfile(outp, dtype=np.float32)
+    diff = float(np.abs(out - gpu_out.reshape(-1)).max())
+    return dict(value=kv_bytes / (info["ms"] / 1e3) / 1e9, unit="GB/s", cores=1, kind="port",
+                sample="full C3 column (1 token over 32769 rows), best of %d reps, node %s, 1 thread" % (reps, info["node"]),
+                ms=info["ms"], max_abs_diff_vs_gpu=diff)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=600)
+    ap.add_argument("--warmup", type=int, default=60)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no sharding, no collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    from pooled_amd.capi import PooledAttn, PA_OUT_F16, load
+    L = load()
+    log("library:", L.pa_version().decode())
+    cfg, ctx = C3, C3_CTX
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    qd, kvd = nH * hd, nKV * hd
+    pa = PooledAttn(cfg, ctx + 1, n_layers=N_LAYERS, max_cols=4096)
+    t_fill = time.time()
+    for layer in range(N_LAYERS):
+        pa.layer_alloc(layer)
+        fill_cache(pa, cfg, layer, ctx, seed=0x5EED0003 + layer, chunk=4096)
+    log("caches filled: %d layers x %.1f MiB in %.1fs" % (N_LAYERS, 2 * ctx * kvd * 2 / 2**20, time.time() - t_fill))
+
+    rng = np.random.default_rng(0x5EED0003)
+    qfull = rng.standard_normal((1, 2 * qd), dtype=np.float32)
+    knew = rng.standard_normal((1, kvd), dtype=np.float32); vnew = rng.standard_normal((1, kvd), dtype=np.float32)
+    qw = (1 + 0.1 * rng.standard_normal(hd)).astype(np.float32); kw = (1 + 0.1 * rng.standard_normal(hd)).astype(np.float32)
+    d_qfull, d_k, d_v, d_qw, d_kw = (pa.to_device(a) for a in (qfull, knew, vnew, qw, kw))
+    d_out = pa.alloc(qd * 2)
+    gate_ptr = pa.gate_buffer_ptr()
+
+    def step(i):
+        layer = i % N_LAYERS
+        pa.glue_kv(layer, d_qfull, 2 * qd, d_k, kvd, d_v, kvd, d_qw, d_kw, ctx, 1)
+        pa.attn("decode", layer, None, 0, gate_ptr, qd, ctx, 1, d_out, qd, PA_OUT_F16)
+
+    kv_bytes = 2 * (ctx + 1) * kvd * 2            # K and V rows [0, 32768], f16
+    for i in range(args.warmup):
+        step(i)
+    pa.sync()
+    t0 = time.perf_counter()
+    pa.timer_start()
+    for i in range(args.steps):
+        step(i)
+    gpu_ms = pa.timer_stop()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = max(gpu_ms, wall_ms) / args.steps
+    value = kv_bytes / (ms_per_step * 1e-3) / 1e9
+    log("timed %d steps: %.2f us/step (events %.2f ms, wall %.2f ms) -> %.0f GB/s" % (args.steps, ms_per_step * 1e3, gpu_ms, wall_ms, value))
+
+    # the dominant kernel alone: one HIP event pair around every split-K launch, on the launch stream
+    pa.profile_enable(True)
+    for i in range(args.steps):
+        step(i)
+    ksum, kcount = pa.profile_read()
+    pa.profile_enable(False)
+    k_ms = ksum / max(kcount, 1)
+    achieved = kv_bytes / (k_ms * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "decode_c3_traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+    roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
+                    traffic=traffic, kernel="pa_decode_kernel<256,1,4>", kernel_us=round(k_ms * 1e3, 3),
+                    algorithmic_bytes_per_launch=kv_bytes, launches=kcount)
+    log("split-K kernel: %.2f us/launch -> %.0f GB/s (%.1f%% of 8 TB/s)" % (k_ms * 1e3, achieved, 100 * achieved / HBM_PEAK_GBS))
+    plan = pa.plan("decode", ctx, 1)
+
+    cpu = None
+    if not args.no_cpu:
+        # GPU output of layer 0 for this token (f32), then the reference CPU loops on the same inputs
+        d_o32 = pa.alloc(qd * 4)
+        pa.glue_kv(0, d_qfull, 2 * qd, d_k, kvd, d_v, kvd, d_qw, d_kw, ctx, 1)
+        pa.attn("decode", 0, None, 0, gate_ptr, qd, ctx, 1, d_o32, qd)
+        pa.sync()
+        gpu_out = d_o32.download(np.float32, qd)
+        q = pa.read_q_buffer(1); gate = pa.read_gate_buffer(1)
+        try:
+            cpu = cpu_baseline_c3(pa, cfg, ctx, q, gate, gpu_out)
+            log("cpu baseline: %.1f ms -> %.3f GB/s; max |gpu - cpu| = %.2e" % (cpu["ms"], cpu["value"], cpu["max_abs_diff_vs_gpu"]))
+        except Exception as e:                     # the baseline is a reported figure; never let it sink the GPU line
+            log("cpu baseline failed:", e)
+            cpu = dict(value=None, unit="GB/s", cores=1, kind="port", sample="failed: %s" % e)
+
+    line = dict(
+        metric="decode attn KV-read GB/s (% HBM peak) @32K ctx; prefill attn TFLOP/s (% MFMA)",
+        value=round(value, 1), unit="GB/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
+        ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None,
+        dtype="f16", data="synthetic",
+        config=dict(workload="C3 gated decode: 16q/2kv heads, head_dim 256, ctx 32768, 1 token, f16 KV, partial RoPE 64 dims theta 1e7, sigmoid gate, f16 out",
+                    step="glue_kv + split-K decode + LSE merge/gate on one layer; %d layers' caches in rotation (cold HBM)" % N_LAYERS,
+                    kv_bytes_per_step=kv_bytes, plan=plan, pct_hbm_peak=round(100 * value / HBM_PEAK_GBS, 2)),
+        roofline=roofline, cpu_baseline=cpu)
+    pa.close()
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

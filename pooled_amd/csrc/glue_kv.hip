@@ -17,6 +17,7 @@
 #include <hip/hip_fp16.h>
 
 // every product and sum below is rounded on its own: no fused multiply-add may be formed in this file
+// (plain operators are used instead of the __fmul_rn family, whose header bodies are compiled with contraction on)
 #pragma clang fp contract(off)
 
 #define GLUE_DO_MATH 0x100u
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const uint32_t i = lane + 64 * j;
-      if (i < hd) x[j] = __fmul_rn(x[j], __fmul_rn(inv, w[i]));
+      if (i < hd) { const float sw = inv * w[i]; x[j] = x[j] * sw; }
     }
   }
 #pragma unroll
@@ -75,13 +76,14 @@ __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
     for (int j = 0; j < 2; j++) {
       const uint32_t i = lane + 64 * j;
       if (i < half) {
-        const float ang = __fmul_rn((float)pos, p.inv_freq[i]);
+        const float ang = (float)pos * p.inv_freq[i];
         double sd, cd;
         sincos((double)ang, &sd, &cd);
         const float c = (float)cd, s = (float)sd;
         const float a = xs[i], b = xs[i + half];
-        ra[j] = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s));
-        rb[j] = __fadd_rn(__fmul_rn(b, c), __fmul_rn(a, s));
+        const float ac = a * c, bs = b * s, bc = b * c, as = a * s;   // rounded one by one (contract off above)
+        ra[j] = ac - bs;
+        rb[j] = bc + as;
       }
     }
     __syncthreads();
