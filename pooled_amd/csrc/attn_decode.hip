@@ -33,6 +33,14 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 #define TILE 32
 #define NEG_INF (-__builtin_inff())
 
+// Optional per-wave timeline (development builds only): lane 0 of every wave stores the 100 MHz wall clock at
+// up to 12 points into p.trace.  Compiled out unless PA_TRACE is defined.
+#ifdef PA_TRACE
+#define PA_TP(k) do { if (p.trace && lane == 0) p.trace[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * W * 12 + wave * 12 + (k)] = wall_clock64(); } while (0)
+#else
+#define PA_TP(k) do { } while (0)
+#endif
+
 // Compiler-level ordering of LDS accesses inside one wavefront (hardware executes a wave's LDS operations
 // in order; lanes of one wave exchange data through the wave-private region without a workgroup barrier).
 static __device__ inline void wave_lds_fence() {
@@ -80,23 +88,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
   if (t_begin >= seq_max) return;
   const uint32_t t_end = min(t_begin + p.split_len, seq_max);
   const uint32_t kvDim = p.n_kv_heads * HD;
-
-  // ---- q -> f16 rows in LDS (rows >= R are zero) ----
-  for (uint32_t e = tid; e < 16 * NB * (HD / 4); e += W * 64) {
-    const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (r < R) v = *(const float4*)(p.q + (size_t)(c0 + r / G) * p.q_stride + (size_t)(g * G + r % G) * HD + 4 * d4);
-    h4 hv = { (_Float16)v.x, (_Float16)v.y, (_Float16)v.z, (_Float16)v.w };
-    *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
-  }
-  // per-lane row bookkeeping: row nb*16 + ln ends (exclusive) at end_pos[nb]; 0 for padding rows
-  uint32_t end_pos[NB];
-#pragma unroll
-  for (int nb = 0; nb < NB; nb++) {
-    const uint32_t r = nb * 16 + ln;
-    end_pos[nb] = r < R ? p.base_pos + c0 + r / G + 1 : 0u;
-  }
-  __syncthreads();
+  PA_TP(0);
 
   unsigned char* stage = stage_all + wave * S::STAGE;
   const size_t row_bytes = (size_t)kvDim * 2;
@@ -119,16 +111,48 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
   u4 kr[S::NLD], vr[S::NLD];
   const u4 zero4 = {0u, 0u, 0u, 0u};
 
+  // q loads first (they return first), then the first tile's K/V loads; staging q below overlaps the K/V latency.
+  constexpr int QPT = 16 * NB * (HD / 4) / (W * 64);               // float4 of q per thread
+  f4 qv[QPT];
+#pragma unroll
+  for (int j = 0; j < QPT; j++) {
+    const uint32_t e = tid + j * W * 64;
+    const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
+    const uint32_t rc = min(r, R - 1);                             // padding rows copy the last live row (masked out later)
+    qv[j] = *(const f4*)(p.q + (size_t)(c0 + rc / G) * p.q_stride + (size_t)(g * G + rc % G) * HD + 4 * d4);
+  }
   // Loads are unconditional: the caches carry TILE rows of padding past max_seq, so a tile that straddles the
   // end of the context reads valid memory; rows at or past t_end are zeroed (V) or masked (scores) below.
+  // A wave with no tile of its own (short splits) loads the split's last tile and discards it: the prologue
+  // stays branch-free, so the q staging below waits for the q loads only.
   uint32_t tile = __builtin_amdgcn_readfirstlane(wave);
-  if (tile < n_tiles) {
-    const size_t tb = (size_t)(t_begin + tile * TILE) * row_bytes;
+  {
+    const size_t tb = (size_t)(t_begin + min(tile, n_tiles - 1) * TILE) * row_bytes;
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
   }
+  PA_TP(1);
+  __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the K/V load issue
+  // ---- q -> f16 rows in LDS; waits only for the q loads, which were issued first ----
+#pragma unroll
+  for (int j = 0; j < QPT; j++) {
+    const uint32_t e = tid + j * W * 64;
+    const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
+    const h4 hv = { (_Float16)qv[j][0], (_Float16)qv[j][1], (_Float16)qv[j][2], (_Float16)qv[j][3] };
+    *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
+  }
+  // per-lane row bookkeeping: row nb*16 + ln ends (exclusive) at end_pos[nb]; 0 for padding rows
+  uint32_t end_pos[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
+    const uint32_t r = nb * 16 + ln;
+    end_pos[nb] = r < R ? p.base_pos + c0 + r / G + 1 : 0u;
+  }
+  __syncthreads();
+  PA_TP(2);
+
   for (; tile < n_tiles; tile += W) {
     const uint32_t tp = t_begin + tile * TILE;
     const size_t tnb = (size_t)(tp + W * TILE) * row_bytes;   // next tile of this wave
@@ -141,6 +165,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
       for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
     }
     wave_lds_fence();
+    PA_TP(3);
     // ---- S^T = K Q^T ----
     f4 s[2][NB];
 #pragma unroll
@@ -157,6 +182,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
       }
     }
     wave_lds_fence();
+    PA_TP(4);
     // ---- V tile -> LDS (rows at or past t_end as zeros: 0 x stale bits must not reach O), next V loads ----
     if (tp + TILE > t_end) {
 #pragma unroll
@@ -168,6 +194,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
 #pragma unroll
       for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
     }
+    PA_TP(5);
     // ---- online softmax; lane holds row nb*16 + ln, positions tp + pb*16 + 4*kg + i ----
     h8 pfrag[NB];
 #pragma unroll
@@ -199,6 +226,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
       for (int db = 0; db < S::DB; db++) acc[db][nb] *= alpha;
     }
     wave_lds_fence();
+    PA_TP(6);
     // ---- O^T += V^T P^T ----
 #pragma unroll
     for (int db = 0; db < S::DB; db++) {
@@ -210,6 +238,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
       for (int nb = 0; nb < NB; nb++) acc[db][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pfrag[nb], acc[db][nb], 0, 0, 0);
     }
     wave_lds_fence();
+    PA_TP(7);
   }
 
   // ---- merge the W waves of the workgroup ----
@@ -220,6 +249,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
     if (kg == 0) { mex[wave * 16 * NB + nb * 16 + ln] = m_run[nb]; lex[wave * 16 * NB + nb * 16 + ln] = l_run[nb]; }
   }
   __syncthreads();
+  PA_TP(8);
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     float M = NEG_INF;
@@ -227,10 +257,12 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
     for (int w = 0; w < W; w++) M = fmaxf(M, mex[w * 16 * NB + nb * 16 + ln]);
     const float m_safe = M == NEG_INF ? 0.f : M;
     const float sc = __expf(m_run[nb] - m_safe);
+    if (nb * 16 + ln < R) {                                            // padding rows are never read back
 #pragma unroll
-    for (int db = 0; db < S::DB; db++) {
-      const f4 o = acc[db][nb] * sc;
-      *(f4*)(stage + ln * S::OROW + (db * 16 + 4 * kg) * 4) = o;
+      for (int db = 0; db < S::DB; db++) {
+        const f4 o = acc[db][nb] * sc;
+        *(f4*)(stage + ln * S::OROW + (db * 16 + 4 * kg) * 4) = o;
+      }
     }
     __syncthreads();
     // rows nb*16 .. nb*16+15, HD/4 float4 each, summed over waves in wave order
@@ -257,23 +289,34 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
         }
       }
     }
-    __syncthreads();
+    if (nb + 1 < NB) __syncthreads();                                  // the regions are rewritten by the next row block
   }
+  PA_TP(9);
 }
 
 // ---- second pass: log-sum-exp merge over a column's splits, sigmoid gate, output conversion ----
-// One workgroup per (head, column); 256 threads = NG split groups x HD/4 float4 lanes.
+// One workgroup per (head, 64-dim slice, column) -- the reference's layout (engine/wgsl/attn_dec.js:215-287,
+// DEC_CQ slices per head) -- so the merge of a decode token runs on nH * HD/64 workgroups instead of nH.
+// 256 threads = 16 split groups x 16 float4 lanes; every split is read in parallel, the maximum and the
+// weighted sum of l by fixed-order tree reductions, the 16 groups' partial outputs summed in group order.
 template <int HD>
 __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
-  constexpr int L4 = HD / 4, NG = 256 / L4;
+  constexpr int CQ = HD / 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  float* wl = (float*)smem;                 // [slots] split weights
+  float* wl = (float*)smem;                 // [slots] split weights exp(m_s - M)
   __shared__ float red[256];
   __shared__ f4 ored[256];
-  const uint32_t h = blockIdx.x, col = blockIdx.y, tid = threadIdx.x;
+  const uint32_t h = blockIdx.x / CQ, dq = blockIdx.x % CQ, col = blockIdx.y, tid = threadIdx.x;
   const uint32_t col_end = p.base_pos + col + 1;
   const uint32_t ns = (col_end + p.split_len - 1) / p.split_len;
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
+  const uint32_t grp = tid >> 4, l4 = tid & 15;
+  const float* po = p.part_o + base * HD + dq * 64 + 4 * l4;
+  // the first output partials go out before the (m, l) reductions: their latency overlaps the barriers below
+  f4 o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
+  const bool h0 = grp < ns, h1 = grp + 16 < ns;
+  if (h0) o0 = *(const f4*)(po + (size_t)grp * HD);
+  if (h1) o1 = *(const f4*)(po + (size_t)(grp + 16) * HD);
   float lm = NEG_INF;
   for (uint32_t s = tid; s < ns; s += 256) lm = fmaxf(lm, p.part_ml[(base + s) * 2]);
   red[tid] = lm;
@@ -291,26 +334,35 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   __syncthreads();
   for (uint32_t k = 128; k > 0; k >>= 1) { if (tid < k) red[tid] += red[tid + k]; __syncthreads(); }
   const float L = red[0];
-  const uint32_t grp = tid / L4, l4 = tid % L4;
   f4 o = {0.f, 0.f, 0.f, 0.f};
-  for (uint32_t s = grp; s < ns; s += NG) o += *(const f4*)(p.part_o + (base + s) * HD + 4 * l4) * wl[s];
+  if (h0) o = o0 * wl[grp];
+  if (h1) o += o1 * wl[grp + 16];
+  for (uint32_t s = grp + 32; s < ns; s += 32) {
+    const f4 a = *(const f4*)(po + (size_t)s * HD);
+    f4 b = {0.f, 0.f, 0.f, 0.f};
+    const bool hb = s + 16 < ns;
+    if (hb) b = *(const f4*)(po + (size_t)(s + 16) * HD);
+    o += a * wl[s];
+    if (hb) o += b * wl[s + 16];
+  }
   ored[tid] = o;
   __syncthreads();
-  if (tid < L4) {
+  if (tid < 16) {
     f4 t = ored[tid];
 #pragma unroll
-    for (int i = 1; i < NG; i++) t += ored[i * L4 + tid];
+    for (int i = 1; i < 16; i++) t += ored[i * 16 + tid];
     f4 r = t / L;
+    const uint32_t d = dq * 64 + 4 * tid;
     if (p.gate) {
-      const float4 gt = *(const float4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * HD + 4 * tid);
-      r[0] *= 1.f / (1.f + __expf(-gt.x)); r[1] *= 1.f / (1.f + __expf(-gt.y));
-      r[2] *= 1.f / (1.f + __expf(-gt.z)); r[3] *= 1.f / (1.f + __expf(-gt.w));
+      const f4 gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * HD + d);
+#pragma unroll
+      for (int i = 0; i < 4; i++) r[i] *= 1.f / (1.f + __expf(-gt[i]));
     }
     if (p.out_f16) {
-      h4 hv = { (_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3] };
-      *(h4*)((_Float16*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + 4 * tid) = hv;
+      const h4 hv = { (_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3] };
+      *(h4*)((_Float16*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + d) = hv;
     } else {
-      *(f4*)((float*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + 4 * tid) = r;
+      *(f4*)((float*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + d) = r;
     }
   }
 }
@@ -349,8 +401,8 @@ hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint3
 
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s) {
   const size_t lds = (size_t)p.slots * sizeof(float);
-  if (hd == 256) hipLaunchKernelGGL(pa_combine_kernel<256>, dim3(p.n_heads, p.n_cols), dim3(256), lds, s, p);
-  else if (hd == 128) hipLaunchKernelGGL(pa_combine_kernel<128>, dim3(p.n_heads, p.n_cols), dim3(256), lds, s, p);
+  if (hd == 256) hipLaunchKernelGGL(pa_combine_kernel<256>, dim3(p.n_heads * 4, p.n_cols), dim3(256), lds, s, p);
+  else if (hd == 128) hipLaunchKernelGGL(pa_combine_kernel<128>, dim3(p.n_heads * 2, p.n_cols), dim3(256), lds, s, p);
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }

@@ -32,6 +32,29 @@ static __device__ inline uint32_t pack_f16x2(float lo, float hi) {
   return (uint32_t)__half_as_ushort(__float2half_rn(lo)) | ((uint32_t)__half_as_ushort(__float2half_rn(hi)) << 16);
 }
 
+// c, s of the f32 angle f32(pos) * inv_freq, evaluated in f64 and rounded once
+static __device__ inline void rope_cos_sin(uint32_t pos, float inv_freq, float& c, float& s) {
+  const float ang = (float)pos * inv_freq;
+  double sd, cd;
+  sincos((double)ang, &sd, &cd);
+  c = (float)cd; s = (float)sd;
+}
+
+// The same values for every (position, pair), computed once per context: rope_tab[pos * half + i] = (cos, sin).
+__global__ __launch_bounds__(256) void pa_rope_table_kernel(float2* tab, const float* inv_freq, uint32_t half, uint32_t n_pos) {
+  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (size_t)n_pos * half) return;
+  float c, s;
+  rope_cos_sin((uint32_t)(e / half), inv_freq[e % half], c, s);
+  tab[e] = make_float2(c, s);
+}
+
+hipError_t pa_launch_rope_table(float2* tab, const float* inv_freq, uint32_t half, uint32_t n_pos, hipStream_t st) {
+  const size_t n = (size_t)n_pos * half;
+  hipLaunchKernelGGL(pa_rope_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, tab, inv_freq, half, n_pos);
+  return hipGetLastError();
+}
+
 __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
   __shared__ float xs[256];
   const uint32_t hh = blockIdx.x, col = blockIdx.y, lane = threadIdx.x;
@@ -76,10 +99,9 @@ __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
     for (int j = 0; j < 2; j++) {
       const uint32_t i = lane + 64 * j;
       if (i < half) {
-        const float ang = (float)pos * p.inv_freq[i];
-        double sd, cd;
-        sincos((double)ang, &sd, &cd);
-        const float c = (float)cd, s = (float)sd;
+        float c, s;
+        if (p.rope_tab) { const float2 cs = p.rope_tab[(size_t)pos * half + i]; c = cs.x; s = cs.y; }
+        else rope_cos_sin(pos, p.inv_freq[i], c, s);
         const float a = xs[i], b = xs[i + half];
         const float ac = a * c, bs = b * s, bc = b * c, as = a * s;   // rounded one by one (contract off above)
         ra[j] = ac - bs;

@@ -76,6 +76,15 @@ extern "C" int pa_create(const pa_config* cfg, pa_ctx** out) {
          && (e = hipEventCreate(&ctx->t0)) == hipSuccess && (e = hipEventCreate(&ctx->t1)) == hipSuccess;
   if (!ok) { int rc = fail_hip(nullptr, e, "pa_create: allocation"); pa_destroy(ctx); return rc; }
   ctx->stream = ctx->own_stream;
+  // (cos, sin) of every (position, rotated pair), built once: the pre-step then loads 8 bytes instead of
+  // evaluating an f64 sincos per pair.  Contexts whose table would pass 1 GiB evaluate in the kernel.
+  const size_t tab_bytes = (size_t)c.max_seq * (c.n_rot / 2) * sizeof(float2);
+  if (tab_bytes <= ((size_t)1 << 30)) {
+    ok = (e = hipMalloc((void**)&ctx->rope_tab, tab_bytes)) == hipSuccess
+      && (e = pa_launch_rope_table(ctx->rope_tab, ctx->inv_freq, c.n_rot / 2, c.max_seq, ctx->stream)) == hipSuccess
+      && (e = hipStreamSynchronize(ctx->stream)) == hipSuccess;
+    if (!ok) { int rc = fail_hip(nullptr, e, "pa_create: rope table"); pa_destroy(ctx); return rc; }
+  }
   *out = ctx;
   return PA_OK;
 }
@@ -87,6 +96,7 @@ extern "C" int pa_destroy(pa_ctx* ctx) {
   if (ctx->q_buf) (void)hipFree(ctx->q_buf);
   if (ctx->gate_buf) (void)hipFree(ctx->gate_buf);
   if (ctx->inv_freq) (void)hipFree(ctx->inv_freq);
+  if (ctx->rope_tab) (void)hipFree(ctx->rope_tab);
   if (ctx->part_o) (void)hipFree(ctx->part_o);
   if (ctx->part_ml) (void)hipFree(ctx->part_ml);
   for (auto ev : ctx->prof_events) (void)hipEventDestroy(ev);
@@ -168,7 +178,7 @@ static int check_cols(pa_ctx* ctx, const char* who, uint32_t layer, bool need_la
 static void fill_glue(const pa_ctx* ctx, GlueParams& p) {
   const pa_config& c = ctx->cfg;
   memset(&p, 0, sizeof p);
-  p.inv_freq = ctx->inv_freq;
+  p.inv_freq = ctx->inv_freq; p.rope_tab = ctx->rope_tab;
   p.q_out = ctx->q_buf; p.gate_out = ctx->gate_buf;
   p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.head_dim = c.head_dim; p.n_rot = c.n_rot;
   p.flags = c.flags | 0x100u;

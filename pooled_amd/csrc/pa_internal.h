@@ -13,6 +13,7 @@ struct GlueParams {
   float* k_out;                                              // in-place k write-back (pa_glue) or nullptr
   const float* qw; const float* kw;                          // norm weights [hd]
   const float* inv_freq;                                     // [n_rot/2] f32, theta^(-2i/n_rot)
+  const float2* rope_tab;                                    // [max_seq][n_rot/2] (cos, sin) or nullptr
   float* q_out; float* gate_out;                             // [n_cols][nH*hd]
   uint16_t* k_cache; uint16_t* v_cache;                      // f16 [max_seq][nKV*hd] or nullptr
   uint32_t q_stride, k_stride, v_stride;
@@ -35,11 +36,13 @@ struct AttnParams {
   uint32_t max_seq;
   int out_f16;
   float scale;                                // 1 / sqrt(hd)
+  unsigned long long* trace;                  // per-wave timestamps when built with PA_TRACE (else unused, nullptr)
 };
 
 // ---- kernel launchers (defined next to their kernels) ------------------------------------------
 
 hipError_t pa_launch_glue(const GlueParams& p, hipStream_t s);
+hipError_t pa_launch_rope_table(float2* tab, const float* inv_freq, uint32_t half, uint32_t n_pos, hipStream_t s);
 // waves per workgroup W in {4, 8}; NB = 16-row query blocks per workgroup (1..4); hd in {128, 256}
 hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s);
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);
@@ -60,6 +63,7 @@ struct pa_ctx {
   float* q_buf = nullptr;       // [max_cols][nH*hd]
   float* gate_buf = nullptr;    // [max_cols][nH*hd]
   float* inv_freq = nullptr;    // [n_rot/2]
+  float2* rope_tab = nullptr;   // [max_seq][n_rot/2] (cos, sin); nullptr when it would exceed 1 GiB
   float* part_o = nullptr; float* part_ml = nullptr;
   size_t part_o_bytes = 0, part_ml_bytes = 0;
   uint32_t decode_splits_override = 0;
