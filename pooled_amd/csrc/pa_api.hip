@@ -272,9 +272,26 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   return PA_OK;
 }
 
+// Prefill (MFMA kernel): a workgroup is 4 wavefronts x 64 query rows = 256 rows of one kv head, i.e.
+// floor(256 / G) columns x G heads.  Chunks wide enough to give every CU a workgroup run unsplit and write the
+// output directly; narrower chunks are also split over the context (partials + merge kernel) until about two
+// workgroups per CU exist.  Chunks of fewer rows than one wavefront tile go to the split-K decode kernel.
 static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl) {
-  // until the MFMA prefill kernel covers a shape, chunks run on the split-K kernel in column groups
-  return plan_decode(ctx, base_pos, n_cols, pl);
+  const pa_config& c = ctx->cfg;
+  const uint32_t G = c.n_heads / c.n_kv_heads;
+  if (n_cols * G <= (c.head_dim == 256 ? 32u : 64u)) return plan_decode(ctx, base_pos, n_cols, pl);
+  const uint32_t rows_wg = 256;
+  const uint32_t cw = rows_wg / G;
+  if (cw == 0) return PA_ERR_UNSUPPORTED;
+  const uint32_t groups = ceil_div(n_cols, cw);
+  const uint32_t seq_max = base_pos + n_cols;
+  const uint32_t base_wgs = groups * c.n_kv_heads;
+  uint32_t splits = 1;
+  if (base_wgs < (uint32_t)ctx->n_cu) splits = std::min(ceil_div(2 * (uint32_t)ctx->n_cu, base_wgs), std::max(1u, seq_max / 256));
+  uint32_t sl = ceil_div(ceil_div(seq_max, splits), 32) * 32;
+  pl->kernel = 1; pl->split_len = sl; pl->n_splits = ceil_div(seq_max, sl);
+  pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = 4; pl->row_blocks = 2; pl->slots = pl->n_splits;
+  return PA_OK;
 }
 
 extern "C" int pa_plan_query(const pa_ctx* ctx, int kind, uint32_t base_pos, uint32_t n_cols, pa_plan* out) {
@@ -342,8 +359,8 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   rc = kind == 0 ? plan_decode(ctx, base_pos, n_cols, &pl) : plan_prefill(ctx, base_pos, n_cols, &pl);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
-  rc = ensure_partials(ctx, n_cols, pl.slots);
-  if (rc) return rc;
+  const bool direct = pl.kernel == 1 && pl.n_splits == 1;     // the prefill kernel writes the output itself
+  if (!direct && (rc = ensure_partials(ctx, n_cols, pl.slots))) return rc;
   AttnParams p; memset(&p, 0, sizeof p);
   p.q = d_q; p.gate = d_gate; p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
   p.part_o = ctx->part_o; p.part_ml = ctx->part_ml; p.out = d_out;
@@ -357,7 +374,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   if (pl.kernel == 0) HIPCHK(ctx, pa_launch_decode(p, c.head_dim, pl.row_blocks, pl.waves, pl.col_groups, ctx->stream));
   else HIPCHK(ctx, pa_launch_prefill(p, c.head_dim, pl.row_blocks, pl.col_groups, ctx->stream));
   if ((rc = prof_end(ctx))) return rc;
-  HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
+  if (!direct) HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;
 }
 

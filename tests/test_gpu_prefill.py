@@ -1,0 +1,110 @@
+"""GPU parity of causal prefill attention (MFMA kernel) through the C ABI against the CPU oracle.
+Tolerance: max-abs <= 2e-3 and max|d|/max|ref| <= 1e-2 of the f32/f64 reference."""
+import numpy as np
+import pytest
+from oracle import attn_oracle as O
+from oracle import c_oracle as C
+from pooled_amd.capi import PooledAttn, PA_OUT_F16
+from helpers import SHAPES, assert_parity, random_cache, oracle_cache
+
+pytestmark = pytest.mark.gpu
+NAN16 = 0x7E00
+
+
+def _prefill(cfg, base, n, seed, max_seq=None, gate=True, out_dtype=0, check_rows=None, k_scale=1.0):
+    rng = np.random.default_rng(seed)
+    max_seq = max_seq or base + n + 7
+    k16, v16 = random_cache(cfg, max_seq, seed=seed + 1, k_scale=k_scale)
+    q = rng.standard_normal((n, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    gt = rng.standard_normal(q.shape, dtype=np.float32) if (gate and cfg["gate"]) else None
+    rows = check_rows if check_rows is not None else list(range(n))
+    ref = C.attention(q, k16, v16, base, gate=gt, rows=rows)
+    pa = PooledAttn(cfg, max_seq, n_layers=1, max_cols=n)
+    try:
+        pa.layer_alloc(0)
+        K, V = k16.copy(), v16.copy()
+        K[base + n:] = NAN16; V[base + n:] = NAN16        # rows past the chunk's end must never be used
+        pa.kv_write(0, 0, 0, K); pa.kv_write(0, 1, 0, V)
+        plan = pa.plan("prefill", base, n)
+        got = pa.run_attn("prefill", 0, q, base, gate=gt, out_dtype=out_dtype)
+    finally:
+        pa.close()
+    return got[rows].astype(np.float32), ref, plan
+
+
+@pytest.mark.parametrize("shape,base,n", [
+    ("qwen36_moe", 0, 16), ("qwen36_moe", 301, 16), ("qwen36_moe", 0, 77), ("qwen36_moe", 1000, 200),
+    ("qwen38_27b", 173, 16), ("qwen38_27b", 90, 130), ("qwen3_1p7b", 77, 8 * 16), ("qwen3_1p7b", 0, 300),
+    ("qwen3_1p7b", 219, 257), ("qwen36_moe", 4000, 33),
+])
+def test_prefill_small(shape, base, n):
+    """Shapes of tests/unit/attn_tile_test.js:102-109 (first pass, partial tiles, padded row groups) and wider chunks."""
+    got, ref, plan = _prefill(SHAPES[shape], base, n, seed=base + n)
+    assert plan["kernel"] == 1
+    assert_parity(got, ref, "%s base %d n %d" % (shape, base, n))
+
+
+def test_prefill_equals_decode_columns():
+    """Every prefill column equals a single-token decode at the same position (tolerance)."""
+    cfg = SHAPES["qwen36_moe"]
+    rng = np.random.default_rng(21)
+    base, n = 700, 40
+    k16, v16 = random_cache(cfg, base + n, seed=22)
+    q = rng.standard_normal((n, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    gt = rng.standard_normal(q.shape, dtype=np.float32)
+    with PooledAttn(cfg, base + n, n_layers=1, max_cols=n) as pa:
+        pa.layer_alloc(0); pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
+        pre = pa.run_attn("prefill", 0, q, base, gate=gt)
+        for c in (0, 1, 17, 39):
+            dec = pa.run_attn("decode", 0, q[c:c + 1], base + c, gate=gt[c:c + 1])
+            assert np.abs(dec[0] - pre[c]).max() <= 1e-3
+
+
+def test_prefill_split_path_and_f16_out():
+    """A narrow chunk on a long context is split over the context (partials + merge kernel)."""
+    cfg = SHAPES["qwen36_moe"]
+    got, ref, plan = _prefill(cfg, 20000, 64, seed=5, out_dtype=PA_OUT_F16)
+    assert plan["kernel"] == 1 and plan["n_splits"] > 1
+    assert_parity(got, ref, "split prefill")
+
+
+def test_prefill_peaked_softmax():
+    """Large score spread (K scaled x3: scores span about +-12, far beyond the 2^8 lazy-rescale threshold): the
+    lazily updated reference maximum must keep exp2 in range.  (Larger K scales amplify the f16 rounding of q
+    beyond the 2e-3 gate: at x6 the error is 4e-3, all of it from the MFMA operand precision.)"""
+    cfg = SHAPES["qwen38_27b"]
+    got, ref, _ = _prefill(cfg, 500, 96, seed=9, k_scale=3.0)
+    assert_parity(got, ref, "peaked")
+
+
+def test_c2_prefill_full():
+    """Config 2: 512-token chunk at positions 1536-2047 over a 1536-token prefix, Qwen3-1.7B shape, pre-step on
+    the GPU (QK-RMSNorm + full RoPE theta 1e6 + KV write for the chunk), f16 output."""
+    cfg = SHAPES["qwen3_1p7b"]
+    base, n = 1536, 512
+    d = O.make_inputs(cfg, base, n, seed=0x5EED0002)
+    k16, v16 = oracle_cache(cfg, d["kraw"], d["vraw"], d["kw"])          # all 2048 rows, oracle pre-step
+    g = O.glue_kv(d["qraw"], d["kraw"][base:], d["vraw"][base:], d["qw"], d["kw"], base, cfg)
+    ref = C.attention(g["q"], k16, v16, base)
+    with PooledAttn(cfg, base + n, n_layers=1, max_cols=n) as pa:
+        pa.layer_alloc(0)
+        pa.kv_write(0, 0, 0, k16[:base]); pa.kv_write(0, 1, 0, v16[:base])
+        pa.run_glue_kv(0, d["qraw"], d["kraw"][base:], d["vraw"][base:], d["qw"], d["kw"], base)
+        assert np.array_equal(pa.kv_read(0, 0, base, n), k16[base:]) and np.array_equal(pa.kv_read(0, 1, base, n), v16[base:])
+        dout = pa.alloc(n * pa.q_dim * 2)
+        pa.attn("prefill", 0, None, 0, None, 0, base, n, dout, pa.q_dim, PA_OUT_F16)
+        pa.sync()
+        got = dout.download(np.float16, n * pa.q_dim).reshape(ref.shape).astype(np.float32)
+    assert_parity(got, ref, "C2")
+
+
+def test_c5_prefill_128k_row_sample():
+    """Config 5: 4096-token chunk at positions 126976-131071 over a 126976-token prefix, MoE shape, gate, f16 out.
+    The whole chunk runs on the GPU; 24 evenly spread columns (all 16 heads) are checked against the f64 oracle,
+    plus the first and last column."""
+    cfg = SHAPES["qwen36_moe"]
+    base, n = 126976, 4096
+    rows = sorted(set([0, n - 1] + list(range(5, n, n // 22))))
+    got, ref, plan = _prefill(cfg, base, n, seed=0x5EED0005, max_seq=base + n, out_dtype=PA_OUT_F16, check_rows=rows)
+    assert plan["kernel"] == 1 and plan["n_splits"] == 1
+    assert_parity(got, ref, "C5 sample")
