@@ -94,12 +94,94 @@ def cpu_baseline_c3(pa, cfg, ctx, q, gate, gpu_out, budget_s=25.0):
                 ms=info["ms"], max_abs_diff_vs_gpu=diff)
 
 
+C5 = dict(n_heads=16, n_kv_heads=2, head_dim=256, n_rot=64, rope_theta=1e7, eps=1e-6, qk_norm=True, gate=True)
+C5_BASE, C5_COLS = 126976, 4096
+
+
+def causal_flops(cfg, base, n):
+    """QK^T and PV multiply-adds of the causal chunk, masked-out work not counted: 4 nH hd sum_c (base + c + 1)."""
+    return 4.0 * cfg["n_heads"] * cfg["head_dim"] * (n * base + n * (n + 1) // 2)
+
+
+def prefill_leg(steps, with_cpu):
+    """Configuration 5: a 4096-token causal chunk at positions 126976-131071 over a 126976-token f16 prefix,
+    Qwen3.6-35B-MoE attention shape, sigmoid gate, f16 output.  A step = pre-step for the 4096 columns
+    (QK-RMSNorm + partial RoPE + KV write) + the MFMA prefill kernel."""
+    from pooled_amd.capi import PooledAttn, PA_OUT_F16
+    cfg, base, n = C5, C5_BASE, C5_COLS
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    qd, kvd = nH * hd, nKV * hd
+    pa = PooledAttn(cfg, base + n, n_layers=1, max_cols=n)
+    pa.layer_alloc(0)
+    fill_cache(pa, cfg, 0, base, seed=0x5EED0005, chunk=4096)
+    rng = np.random.default_rng(0x5EED0005)
+    d_qfull = pa.to_device(rng.standard_normal((n, 2 * qd), dtype=np.float32))
+    d_k = pa.to_device(rng.standard_normal((n, kvd), dtype=np.float32)); d_v = pa.to_device(rng.standard_normal((n, kvd), dtype=np.float32))
+    d_qw = pa.to_device((1 + 0.1 * rng.standard_normal(hd)).astype(np.float32)); d_kw = pa.to_device((1 + 0.1 * rng.standard_normal(hd)).astype(np.float32))
+    d_out = pa.alloc(n * qd * 2)
+    gate_ptr = pa.gate_buffer_ptr()
+
+    def step():
+        pa.glue_kv(0, d_qfull, 2 * qd, d_k, kvd, d_v, kvd, d_qw, d_kw, base, n)
+        pa.attn("prefill", 0, None, 0, gate_ptr, qd, base, n, d_out, qd, PA_OUT_F16)
+
+    step(); pa.sync()
+    pa.profile_enable(True)
+    pa.timer_start()
+    for _ in range(steps):
+        step()
+    ms_step = pa.timer_stop() / steps
+    ksum, kcount = pa.profile_read()
+    pa.profile_enable(False)
+    k_ms = ksum / max(kcount, 1)
+    flops = causal_flops(cfg, base, n)
+    tf_step, tf_kernel = flops / (ms_step * 1e-3) / 1e12, flops / (k_ms * 1e-3) / 1e12
+    log("prefill C5: %.3f ms/step -> %.1f TFLOP/s; kernel %.3f ms -> %.1f TFLOP/s (%.1f%% of f16 MFMA peak)" % (ms_step, tf_step, k_ms, tf_kernel, 100 * tf_kernel / MFMA_F16_PEAK_TFLOPS))
+    res = dict(workload="C5 causal chunked prefill: 4096 columns at positions 126976-131071 over a 126976-token f16 prefix, 16q/2kv heads, head_dim 256, partial RoPE, sigmoid gate, f16 out",
+               value=round(tf_step, 1), unit="TFLOP/s", ms_per_step=round(ms_step, 4), steps=steps, flops_per_step=flops, plan=pa.plan("prefill", base, n),
+               roofline=dict(bound="mfma", achieved=round(tf_kernel, 1), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s", frac=round(tf_kernel / MFMA_F16_PEAK_TFLOPS, 4),
+                             traffic=None, kernel="pa_prefill_kernel<256, 1, 8>", kernel_ms=round(k_ms, 4), algorithmic_flops_per_launch=flops, launches=kcount))
+    if with_cpu:
+        # CPU leg: the reference loops on a fixed subsample (head group of kv head 0 is irrelevant to the loops: all
+        # 16 heads of 4 evenly spaced columns), scaled by columns; labelled extrapolated
+        try:
+            sel = np.array([0, n // 3, 2 * n // 3, n - 1], np.int32)
+            node = shutil.which("node")
+            rows = base + n
+            q = pa.read_q_buffer(n); gate = pa.read_gate_buffer(n)
+            gpu = d_out.download(np.float16, n * qd).reshape(n, qd)[sel].astype(np.float32)
+            k16 = pa.kv_read(0, 0, 0, rows); v16 = pa.kv_read(0, 1, 0, rows)
+            if node is None:
+                raise RuntimeError("node not found")
+            with tempfile.TemporaryDirectory() as td:
+                inp, outp = os.path.join(td, "in.bin"), os.path.join(td, "out.bin")
+                with open(inp, "wb") as f:
+                    f.write(struct.pack("8i", n, nH, nKV, hd, base, rows, 1, len(sel)))
+                    f.write(sel.tobytes()); f.write(q.astype(np.float32).tobytes()); f.write(k16.tobytes()); f.write(v16.tobytes()); f.write(gate.astype(np.float32).tobytes())
+                r = subprocess.run([node, os.path.join(ROOT, "oracle", "attn_ref.js"), inp, outp, "1"], capture_output=True, text=True, timeout=600)
+                if r.returncode != 0:
+                    raise RuntimeError("attn_ref.js failed: " + r.stderr[-300:])
+                info = json.loads(r.stdout.strip().splitlines()[-1])
+                out = np.fromfile(outp, dtype=np.float32).reshape(len(sel), qd)
+            sub_flops = 4.0 * nH * hd * sum(base + int(c) + 1 for c in sel)
+            res["cpu_baseline"] = dict(value=sub_flops / (info["ms"] * 1e-3) / 1e12, unit="TFLOP/s", cores=1, kind="port",
+                                       sample="4 of 4096 columns x 16 heads (%.2f GFLOP), 1 rep, node %s, 1 thread; whole chunk extrapolates to %.0f s" % (sub_flops / 1e9, info["node"], info["ms"] * 1e-3 * flops / sub_flops),
+                                       ms=info["ms"], max_abs_diff_vs_gpu=float(np.abs(out - gpu).max()))
+            log("prefill cpu baseline: %.0f ms for %.2f GFLOP -> %.5f TFLOP/s; max |gpu - cpu| = %.2e" % (info["ms"], sub_flops / 1e9, res["cpu_baseline"]["value"], res["cpu_baseline"]["max_abs_diff_vs_gpu"]))
+        except Exception as e:
+            res["cpu_baseline"] = dict(value=None, unit="TFLOP/s", cores=1, kind="port", sample="failed: %s" % e)
+    pa.close()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=600)
     ap.add_argument("--warmup", type=int, default=60)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (configuration 5) leg")
+    ap.add_argument("--prefill-steps", type=int, default=5)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
@@ -189,6 +271,8 @@ def main():
                     kv_bytes_per_step=kv_bytes, plan=plan, pct_hbm_peak=round(100 * value / HBM_PEAK_GBS, 2)),
         roofline=roofline, cpu_baseline=cpu)
     pa.close()
+    if not args.no_prefill:
+        line["prefill"] = prefill_leg(args.prefill_steps, not args.no_cpu)
     print(json.dumps(line), flush=True)
 
 
