@@ -1,0 +1,181 @@
+// Host-side mirror of pooled's attention dispatch for the MI355X library (CommonJS, runs on Node >= 12).
+//
+// pooled's engines record attention as WebGPU compute passes from these methods:
+//   Qwen35Engine._encAttnGlue(p, M, nCols)                      engine/qwen35.js:2473-2483
+//   Qwen35Engine._encAttnCore(p, LB, M, basePos, nCols)         engine/qwen35.js:2485-2517
+//   Qwen35Engine._encodeLayerR (attention part, one token)      engine/qwen35.js:1598-1640
+//   DenseEngine._encodeAttn(pass, BG, seqLen)                   engine/dense.js:463-469
+//   DenseEngine._encodeAttnBatch(pass, LB, basePos, n)          engine/dense.js:796-805
+// HipAttention keeps those names, argument meanings and buffer conventions (column-batched f32 q / k / v with
+// 256-byte aligned column strides, engine/qwen35.js:2054-2055; f16 KV cache [maxSeq][nKV][hd]; attnOut f32
+// [nCols][stride]) and forwards each to the C ABI through the Node-API addon.  `p` (the compute pass in the
+// reference) is accepted and ignored: work is enqueued in order on the context's HIP stream, which is the
+// ordering the engine relies on ("the queue is ordered", engine/dense.js:899-901).
+//
+// There is no CPU path here: if the addon is missing, require() throws.
+"use strict";
+const path = require("path");
+const addon = require(path.join(__dirname, "..", "lib", "pooled_attn.node"));
+
+const PA_FLAG_QK_NORM = 1, PA_FLAG_GATE = 2, PA_OUT_F32 = 0, PA_OUT_F16 = 1;
+
+// ---- the reference's sizing formulas, kept for callers that still size grids or slot buffers with them.
+//      The HIP kernels take their splits from the gfx950 table instead (HipAttention.plan). ----
+// engine/wgsl/attn_dec.js:40-51
+function attnDecConfig(o) {
+  const hd = o.hd, G = o.G, nKV = o.nKV, splits = o.splits || 0, R = o.R || 1;
+  if (o.kvQ8 || hd !== 256 || !(G >= 1 && G <= 8) || !(R >= 1)) return null;
+  const S = splits > 0 ? splits | 0 : Math.max(16, Math.floor(256 / nKV));
+  return { HD: hd, G: G, S: S, R: R };
+}
+const decSplitLen = (s, S) => Math.max(64, Math.ceil(Math.ceil(s / S) / 64) * 64);
+const decSplits = (s, S) => Math.ceil(s / decSplitLen(s, S));
+const DEC_CQ = 4;
+// engine/wgsl/attn_tile.js:43-56
+function attnTileConfig(o) {
+  const hd = o.hd, G = o.G, wgMem = o.wgMem || 16384;
+  if (!(hd % 16 === 0 && hd >= 16 && hd <= 256 && G >= 1 && G <= 64)) return null;
+  if (o.faSplit % 64 !== 0 || o.faSplits < 1) return null;
+  const bytes = (TK) => TK * hd * 4 + TK * 256 * 4;
+  const TK = o.tk || [16, 8, 4].find((t) => bytes(t) <= wgMem);
+  if (!TK || bytes(TK) > wgMem) return null;
+  return { HD: hd, G: G, CW: Math.floor(64 / G), TK: TK, FASPLIT: o.faSplit, FASPLITS: o.faSplits, TARGET: Math.max(1, (o.target === undefined ? 32 : o.target) | 0) };
+}
+function tileSplitLen(seqEnd, c) {
+  const up64 = (x) => Math.ceil(x / 64) * 64;
+  return Math.min(c.FASPLIT, Math.max(64, up64(Math.ceil(seqEnd / c.TARGET)), up64(Math.ceil(seqEnd / c.FASPLITS))));
+}
+// engine/qwen35.js:367-368
+function faSizing(maxSeq) {
+  const faSplit = Math.max(256, Math.ceil(maxSeq / 128 / 64) * 64);
+  return { faSplit: faSplit, faSplits: Math.ceil(maxSeq / faSplit) };
+}
+
+class HipAttention {
+  // opts: { nH, nKV, hd, nRot, ropeTheta, eps, maxSeq, nLayers, batchCols, qkNorm = true, gate = false, outF16 = false }
+  constructor(opts) {
+    const nH = opts.nH, nKV = opts.nKV, hd = opts.hd;
+    if (!(nH > 0 && nKV > 0 && nH % nKV === 0)) throw new Error("HipAttention: nH must be a positive multiple of nKV");
+    this.dims = { nH: nH, nKV: nKV, hd: hd, nRot: opts.nRot || hd, qDim: nH * hd, kvDim: nKV * hd };
+    this.maxSeq = opts.maxSeq;
+    this.NC = Math.max(1, opts.batchCols || 16);                 // full pass width (engine/qwen35.js batchCols)
+    this.gate = !!opts.gate;
+    this.qkNorm = opts.qkNorm !== false;
+    this.outDtype = opts.outF16 ? PA_OUT_F16 : PA_OUT_F32;
+    // engine fields the attention dispatch reads (engine/qwen35.js:366, :416-419): always the f16-KV split-K path here
+    this.flash = true; this.kvQ8 = false; this.attnDecode = "v2"; this.attnPrefillTile = true;
+    this._snapNow = null;                                          // set by a verify pass (engine/qwen35.js:2960-2965)
+    this.pos = 0;
+    const flags = (this.qkNorm ? PA_FLAG_QK_NORM : 0) | (this.gate ? PA_FLAG_GATE : 0);
+    // a readable throw at create, like the engine's KV binding check (engine/qwen35.js:378-383)
+    this.ctx = addon.create({ nH: nH, nKV: nKV, hd: hd, nRot: this.dims.nRot, ropeTheta: opts.ropeTheta, eps: opts.eps,
+      maxSeq: opts.maxSeq, nLayers: opts.nLayers || 1, maxCols: this.NC, flags: flags });
+    this.kvBufBytes = opts.maxSeq * this.dims.kvDim * 2;
+    this.layers = [];
+    for (let i = 0; i < (opts.nLayers || 1); i++) { addon.layerAlloc(this.ctx, i); this.layers.push({ index: i, qNorm: null, kNorm: null }); }
+    // column-batched activations, 256-byte aligned column strides (engine/qwen35.js:2054-2055 mkB)
+    const al = (n) => Math.ceil(n * 4 / 256) * 256;
+    const mkB = (n) => ({ ptr: addon.malloc(this.ctx, this.NC * al(n)), stride: al(n), n: n });
+    const qIn = this.gate ? nH * hd * 2 : nH * hd;
+    this.B = { qFull: mkB(qIn), k: mkB(this.dims.kvDim), v: mkB(this.dims.kvDim), attnOut: mkB(this.dims.qDim) };
+    this._ones = addon.malloc(this.ctx, hd * 4);
+    addon.upload(this.ctx, this._ones, new Float32Array(hd).fill(1));
+  }
+
+  destroy() {
+    if (!this.ctx) return;
+    for (const k of Object.keys(this.B)) addon.free(this.ctx, this.B[k].ptr);
+    for (const L of this.layers) { if (L.qNorm) addon.free(this.ctx, L.qNorm); if (L.kNorm) addon.free(this.ctx, L.kNorm); }
+    addon.free(this.ctx, this._ones);
+    addon.destroy(this.ctx);
+    this.ctx = null;
+  }
+
+  // ---- uploads the engine does with queue.writeBuffer ----
+  setLayerNorms(i, qNorm, kNorm) {
+    const L = this.layers[i], hd = this.dims.hd;
+    if (qNorm.length !== hd || kNorm.length !== hd) throw new Error("setLayerNorms: weights must have headDim elements");
+    if (!L.qNorm) { L.qNorm = addon.malloc(this.ctx, hd * 4); L.kNorm = addon.malloc(this.ctx, hd * 4); }
+    addon.upload(this.ctx, L.qNorm, Float32Array.from(qNorm));
+    addon.upload(this.ctx, L.kNorm, Float32Array.from(kNorm));
+  }
+  // column c of buffer b <- Float32Array (b.n floats)
+  writeColumn(b, c, data) {
+    if (data.length !== b.n) throw new Error("writeColumn: expected " + b.n + " floats");
+    if (c >= this.NC) throw new Error("writeColumn: column " + c + " >= batchCols " + this.NC);
+    addon.upload(this.ctx, b.ptr, data, c * b.stride);
+  }
+  readColumn(b, c) {
+    const out = new Float32Array(b.n);
+    addon.download(this.ctx, out, b.ptr, c * b.stride);
+    return out;
+  }
+  // attnOut as the engine reads it back (f32 columns; f16 when constructed with outF16)
+  readAttnOut(nCols) {
+    const D = this.dims, out = [];
+    for (let c = 0; c < nCols; c++) {
+      if (this.outDtype === PA_OUT_F32) out.push(this.readColumn(this.B.attnOut, c));
+      else { const h = new Uint16Array(D.qDim); addon.download(this.ctx, h, this.B.attnOut.ptr, c * this.B.attnOut.stride); out.push(h); }
+    }
+    return out;
+  }
+  kvRead(layer, which, row0, nRows) { const a = new Uint16Array(nRows * this.dims.kvDim); addon.kvRead(this.ctx, layer, which, row0, nRows, a); return a; }
+  kvWrite(layer, which, row0, rows) { addon.kvWrite(this.ctx, layer, which, row0, rows.length / this.dims.kvDim, rows); }
+  sync() { addon.sync(this.ctx); }
+  plan(kind, basePos, nCols) { return addon.planQuery(this.ctx, kind === "prefill" ? 1 : 0, basePos, nCols); }
+
+  _norms(L) { return [L.qNorm || this._ones, L.kNorm || this._ones]; }
+  _strideF(b) { return b.stride / 4; }
+  _outStride() { return this.outDtype === PA_OUT_F32 ? this.B.attnOut.stride / 4 : this.B.attnOut.stride / 2; }
+
+  // ---- Qwen35Engine: batched pass ----
+  // qsplit + q/k head-norm + (partial) rope for nCols columns; k is rewritten in place, like attn_glue.
+  // M = { layer, basePos } stands where the reference passes the layer's bind-group table (LB.mc); the columns'
+  // positions come from the frame uniform there (engine/qwen35.js:3846), from M.basePos here.
+  _encAttnGlue(p, M, nCols) {
+    const L = this.layers[M.layer], n = this._norms(L);
+    addon.glue(this.ctx, this.B.qFull.ptr, this._strideF(this.B.qFull), this.B.k.ptr, this._strideF(this.B.k), n[0], n[1], M.basePos, nCols);
+  }
+  // kv_store + attention + sigmoid gate: B.q / B.k / B.v / gate -> B.attnOut.  Kernel selection as the reference's:
+  // a full-width pass that is not a verify runs the tiled prefill kernel, everything else the split-K decode kernel
+  // (so a verify column is a decode at the same position).
+  _encAttnCore(p, LB, M, basePos, nCols) {
+    const B = this.B, layer = LB.layer;
+    addon.kvStore(this.ctx, layer, B.k.ptr, this._strideF(B.k), B.v.ptr, this._strideF(B.v), basePos, nCols);
+    const gate = this.gate ? addon.gateBuffer(this.ctx) : null;
+    const kind = (this.attnPrefillTile && nCols === this.NC && nCols > 1 && !this._snapNow) ? 1 : 0;
+    addon.attn(this.ctx, kind, layer, null, 0, gate, this.dims.qDim, basePos, nCols, B.attnOut.ptr, this._outStride(), this.outDtype);
+  }
+  // a whole batched attention block, as _encodeLayerBatch strings the two together (engine/qwen35.js:2416, :2425)
+  encodeLayerBatchAttn(p, i, basePos, nCols, snapshot) {
+    this._snapNow = snapshot ? 1 : null;
+    this._encAttnGlue(p, { layer: i, basePos: basePos }, nCols);
+    this._encAttnCore(p, { layer: i }, { layer: i, basePos: basePos }, basePos, nCols);
+    this._snapNow = null;
+  }
+  // ---- Qwen35Engine: one token (fused glue + KV write, split-K decode, merge + gate in one go) ----
+  encodeLayerAttn(p, i, pos) {
+    const B = this.B, L = this.layers[i], n = this._norms(L);
+    addon.glueKv(this.ctx, i, B.qFull.ptr, this._strideF(B.qFull), B.k.ptr, this._strideF(B.k), B.v.ptr, this._strideF(B.v), n[0], n[1], pos, 1);
+    const gate = this.gate ? addon.gateBuffer(this.ctx) : null;
+    addon.attn(this.ctx, 0, i, null, 0, gate, this.dims.qDim, pos, 1, B.attnOut.ptr, this._outStride(), this.outDtype);
+  }
+
+  // ---- DenseEngine shapes (full RoPE, no gate): the glue writes the cache, then attention ----
+  // _encodeAttn(pass, BG, seqLen): BG = { layer }; attention of the token at position seqLen - 1
+  _encodeAttn(pass, BG, seqLen) {
+    addon.attn(this.ctx, 0, BG.layer, null, 0, null, 0, seqLen - 1, 1, this.B.attnOut.ptr, this._outStride(), this.outDtype);
+  }
+  // _encodeAttnBatch(pass, LB, basePos, n): n columns at basePos .. basePos + n - 1 (the reference runs 4)
+  _encodeAttnBatch(pass, LB, basePos, n) {
+    addon.attn(this.ctx, 0, LB.layer, null, 0, null, 0, basePos, n === undefined ? 4 : n, this.B.attnOut.ptr, this._outStride(), this.outDtype);
+  }
+  // the dense layer's glue (head_norm_dmc + rope_dmc + kv_store_d, engine/dense.js:394-399) for n columns
+  encodeGlueDense(pass, i, basePos, n) {
+    const B = this.B, L = this.layers[i], w = this._norms(L);
+    addon.glueKv(this.ctx, i, B.qFull.ptr, this._strideF(B.qFull), B.k.ptr, this._strideF(B.k), B.v.ptr, this._strideF(B.v), w[0], w[1], basePos, n);
+  }
+}
+
+module.exports = { HipAttention, addon, attnDecConfig, decSplitLen, decSplits, DEC_CQ, attnTileConfig, tileSplitLen, faSizing,
+  PA_FLAG_QK_NORM, PA_FLAG_GATE, PA_OUT_F32, PA_OUT_F16 };

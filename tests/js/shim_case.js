@@ -1,0 +1,61 @@
+// Runs the JavaScript host shim (pooled_amd/js/hip_attention.js) on a case written by tests/test_gpu_js_shim.py:
+// a cache prefix, per-column raw q / k / v, norm weights and the oracle's expected attention outputs, and checks
+//   1. a full-width pass (prefill kernel)            _encAttnGlue + _encAttnCore
+//   2. the same columns as a verify pass (decode kernel, snapshot set)
+//   3. one token at a time                            encodeLayerAttn
+// against the expected values (max-abs 2e-3, rel 1e-2) and the written KV rows bit for bit.
+"use strict";
+const fs = require("fs"), path = require("path");
+const { HipAttention, decSplits, decSplitLen, faSizing } = require(path.join(__dirname, "..", "..", "pooled_amd", "js", "hip_attention.js"));
+const dir = process.argv[2];
+const C = JSON.parse(fs.readFileSync(path.join(dir, "case.json"), "utf8"));
+const f32 = (n) => { const b = fs.readFileSync(path.join(dir, n)); return new Float32Array(b.buffer.slice(b.byteOffset, b.byteOffset + b.byteLength)); };
+const u16 = (n) => { const b = fs.readFileSync(path.join(dir, n)); return new Uint16Array(b.buffer.slice(b.byteOffset, b.byteOffset + b.byteLength)); };
+let fails = 0;
+const check = (what, got, ref) => {
+  let md = 0, mr = 0;
+  for (let i = 0; i < ref.length; i++) { md = Math.max(md, Math.abs(got[i] - ref[i])); mr = Math.max(mr, Math.abs(ref[i])); }
+  const ok = md <= 2e-3 && md / mr <= 1e-2 && Number.isFinite(md);
+  console.log(what + ": max-abs " + md.toExponential(2) + " rel " + (md / mr).toExponential(2) + (ok ? " ok" : " FAIL"));
+  if (!ok) fails++;
+};
+// the reference's sizing mirrors (engine/wgsl/attn_dec.js:47-48, engine/qwen35.js:367-368)
+if (decSplitLen(32769, 128) !== 320 || decSplits(32769, 128) !== 103 || faSizing(131072).faSplit !== 1024) { console.log("sizing mirrors FAIL"); fails++; }
+
+const cfg = C.cfg, n = C.nCols, base = C.basePos;
+const A = new HipAttention({ nH: cfg.n_heads, nKV: cfg.n_kv_heads, hd: cfg.head_dim, nRot: cfg.n_rot, ropeTheta: cfg.rope_theta, eps: cfg.eps,
+  maxSeq: base + n, nLayers: 1, batchCols: n, qkNorm: true, gate: !!cfg.gate });
+const D = A.dims, qIn = cfg.gate ? 2 * D.qDim : D.qDim;
+A.setLayerNorms(0, f32("qw.bin"), f32("kw.bin"));
+const K0 = u16("k16.bin"), V0 = u16("v16.bin"), qraw = f32("qraw.bin"), kraw = f32("kraw.bin"), vraw = f32("vraw.bin"), expect = f32("expect.bin");
+const kNew = u16("knew16.bin"), vNew = u16("vnew16.bin");
+const loadCols = (c0, cnt) => { for (let c = 0; c < cnt; c++) {
+  A.writeColumn(A.B.qFull, c, qraw.subarray((c0 + c) * qIn, (c0 + c + 1) * qIn));
+  A.writeColumn(A.B.k, c, kraw.subarray((c0 + c) * D.kvDim, (c0 + c + 1) * D.kvDim));
+  A.writeColumn(A.B.v, c, vraw.subarray((c0 + c) * D.kvDim, (c0 + c + 1) * D.kvDim)); } };
+const flat = (cols) => { const o = new Float32Array(cols.length * D.qDim); cols.forEach((c, i) => o.set(c, i * D.qDim)); return o; };
+const eqBits = (a, b) => { if (a.length !== b.length) return false; for (let i = 0; i < a.length; i++) if (a[i] !== b[i]) return false; return true; };
+
+A.kvWrite(0, 0, 0, K0); A.kvWrite(0, 1, 0, V0);
+// 1. full-width pass
+loadCols(0, n);
+A.encodeLayerBatchAttn(null, 0, base, n, false);
+A.sync();
+if (A.plan("prefill", base, n).kernel !== 1) { console.log("full-width pass did not take the prefill kernel FAIL"); fails++; }
+check("full-width pass (prefill kernel)", flat(A.readAttnOut(n)), expect);
+if (!eqBits(A.kvRead(0, 0, base, n), kNew) || !eqBits(A.kvRead(0, 1, base, n), vNew)) { console.log("KV rows written by the pass differ FAIL"); fails++; }
+// 2. verify pass (snapshot): decode kernel, same expected values
+loadCols(0, n);
+A.encodeLayerBatchAttn(null, 0, base, n, true);
+A.sync();
+check("verify pass (decode kernel)", flat(A.readAttnOut(n)), expect);
+// 3. token by token
+const outs = [];
+for (let c = 0; c < n; c++) { loadCols(c, 1); A.encodeLayerAttn(null, 0, base + c); A.sync(); outs.push(A.readAttnOut(1)[0]); }
+check("token by token (fused glue + decode)", flat(outs), expect);
+if (!eqBits(A.kvRead(0, 0, base, n), kNew)) { console.log("KV rows written token by token differ FAIL"); fails++; }
+// error path: a readable throw, not an abort
+try { A.encodeLayerAttn(null, 0, base + n); console.log("out-of-range position did not throw FAIL"); fails++; } catch (e) { if (!/max_seq/.test(e.message)) { console.log("unexpected error text: " + e.message + " FAIL"); fails++; } }
+A.destroy();
+console.log(fails ? "SHIM FAIL" : "SHIM PASS");
+process.exit(fails ? 1 : 0);

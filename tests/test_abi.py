@@ -31,3 +31,14 @@ def test_struct_layouts_match_header():
 def test_version_string_without_gpu():
     L = capi.load()
     assert L.pa_version().decode().startswith("pooled_attn")
+
+
+def test_addon_exports_when_built():
+    import shutil, subprocess
+    addon = os.path.join(ROOT, "pooled_amd", "lib", "pooled_attn.node")
+    if not (os.path.exists(addon) and shutil.which("node")):
+        import pytest
+        pytest.skip("addon or node missing")
+    js = "const a=require(%r); const want=['create','destroy','layerAlloc','sync','malloc','free','upload','download','glueKv','glue','kvStore','attn','planQuery','kvRead','kvWrite','timerStart','timerStop','version']; for (const w of want) if (typeof a[w] !== 'function') { console.log('missing', w); process.exit(1); } console.log('ok', a.version());" % addon
+    r = subprocess.run(["node", "-e", js], capture_output=True, text=True)
+    assert r.returncode == 0 and r.stdout.startswith("ok"), r.stdout + r.stderr
