@@ -182,6 +182,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (configuration 5) leg")
     ap.add_argument("--prefill-steps", type=int, default=5)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run 10 device-to-device copies of 256 MiB (the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
@@ -190,6 +192,17 @@ def main():
     from pooled_amd.capi import PooledAttn, PA_OUT_F16, load
     L = load()
     log("library:", L.pa_version().decode())
+    if args.copy_calibration:
+        pa = PooledAttn(C3, 64, n_layers=1, max_cols=1)
+        nbytes = 256 << 20
+        src, dst = pa.alloc(nbytes), pa.alloc(nbytes)
+        src.upload(np.zeros(nbytes // 4, np.float32))
+        for _ in range(10):
+            pa.copy_d2d(dst, src, nbytes)
+        pa.sync()
+        pa.close()
+        print(json.dumps({"copy_calibration": {"bytes_per_copy": nbytes, "copies": 10}}))
+        return
     cfg, ctx = C3, C3_CTX
     nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
     qd, kvd = nH * hd, nKV * hd

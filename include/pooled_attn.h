@@ -83,6 +83,10 @@ int pa_free(pa_ctx* ctx, void* d_ptr);
 int pa_upload(pa_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);     /* blocking */
 int pa_download(pa_ctx* ctx, void* h_dst, const void* d_src, size_t bytes);   /* blocking, after queued work */
 
+/* device-to-device copy on the context's stream (not blocking): the engine's slot copies of KV rows are
+ * copyBufferToBuffer calls (engine/dense.js:20-47 saveSlot / loadSlot) */
+int pa_copy_d2d(pa_ctx* ctx, void* d_dst, const void* d_src, size_t bytes);
+
 /* ---- pre-step ----
  * pa_glue_kv: q de-interleave + QK-RMSNorm + (partial) NeoX RoPE for n_cols columns at positions
  * base_pos + c, and the f16 write of the k and v rows into layer's caches at those positions.

@@ -41,6 +41,7 @@ SYMBOLS = {
     "pa_free": (c_int, [vp, vp]),
     "pa_upload": (c_int, [vp, vp, vp, ctypes.c_size_t]),
     "pa_download": (c_int, [vp, vp, vp, ctypes.c_size_t]),
+    "pa_copy_d2d": (c_int, [vp, vp, vp, ctypes.c_size_t]),
     "pa_glue_kv": (c_int, [vp, u32, f32p, u32, f32p, u32, f32p, u32, f32p, f32p, u32, u32]),
     "pa_glue": (c_int, [vp, f32p, u32, f32p, u32, f32p, f32p, u32, u32]),
     "pa_kv_store": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32]),
@@ -157,6 +158,9 @@ class PooledAttn:
     def to_device(self, arr):
         a = np.ascontiguousarray(arr)
         return self.alloc(max(a.nbytes, 16)).upload(a)
+
+    def copy_d2d(self, dst, src, nbytes):
+        self._chk(self.L.pa_copy_d2d(self.ctx, dst.ptr, src.ptr, nbytes))
 
     def layer_alloc(self, layer=0):
         self._chk(self.L.pa_layer_alloc(self.ctx, layer))

@@ -160,6 +160,13 @@ extern "C" int pa_download(pa_ctx* ctx, void* h_dst, const void* d_src, size_t b
   return PA_OK;
 }
 
+extern "C" int pa_copy_d2d(pa_ctx* ctx, void* d_dst, const void* d_src, size_t bytes) {
+  if (!ctx || (!d_dst && bytes) || (!d_src && bytes)) return PA_ERR_INVALID;
+  if (!bytes) return PA_OK;
+  HIPCHK(ctx, hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+  return PA_OK;
+}
+
 extern "C" float* pa_q_buffer(pa_ctx* ctx) { return ctx ? ctx->q_buf : nullptr; }
 extern "C" float* pa_gate_buffer(pa_ctx* ctx) { return ctx ? ctx->gate_buf : nullptr; }
 
