@@ -9,8 +9,13 @@
 //   * A workgroup (4 wavefronts, one per SIMD) owns one kv head and a block of columns; its 4 x 64 = 256 query
 //     rows are (column, head-in-group) pairs, so every K/V tile it stages serves all G heads of the group
 //     (the reference's "up to 64 rows share a tile", scaled to the MFMA shape).
-//   * K/V tiles of 32 positions go global -> registers -> LDS (double buffered, one barrier a step); the next
-//     tile's loads are in flight while the current one is consumed.
+//   * K/V tiles of 32 positions go global -> LDS directly (global_load_lds_dwordx4: no staging registers),
+//     double buffered, one barrier a step; the next tile's loads are in flight while the current one is consumed.
+//     An LDS-direct load writes 64 lanes x 16 B contiguously, so rows cannot be padded; bank conflicts are
+//     avoided by an XOR swizzle applied on the *global* side (lane i fetches the chunk that belongs at its LDS
+//     slot): K chunk c of row r sits at slot c ^ (r & 15) (conflict-free ds_read_b128 fragments), V chunk c at
+//     c ^ 4 (r & 3) (2-way = optimal ds_read_b64_tr_b16).  Rows at or past the end of the context are fetched
+//     from the cache's zero padding row instead, so 0 x stale bits never reaches O.
 //   * S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_f16.  Q fragments stay in registers for the whole
 //     kernel; K fragments are ds_read_b128, V^T fragments come from the gfx950 LDS transpose read
 //     (ds_read_b64_tr_b16).  The S^T accumulator layout (lane = query row, 16 positions) is the B-operand
@@ -27,6 +32,7 @@
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef __fp16 hh4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
@@ -42,23 +48,28 @@ static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
 }
 
 template <int HD, int W> struct PfShape {
-  static constexpr int KROW = HD * 2 + 16;        // staged K row stride (bytes): conflict-free b128 fragment reads
-  static constexpr int VROW = HD * 2 + 32;        // staged V row stride (bytes): 2-way (optimal) transpose reads
-  static constexpr int KBUF = PF_TN * KROW;
-  static constexpr int VBUF = PF_TN * VROW;
+  static constexpr int ROWB = HD * 2;             // bytes of one kv head's row
+  static constexpr int TILE = PF_TN * ROWB;       // bytes of one staged tile (K or V)
   static constexpr int KS = HD / 16;              // k-steps of QK^T
   static constexpr int DB = HD / 32;              // 32-dim blocks of the output
   static constexpr int CPR = HD / 8;              // 16-byte chunks per row
-  static constexpr int LD = PF_TN * CPR / (W * 64);   // 16-byte loads per thread, tensor and step
+  static constexpr int RPB = 64 / CPR;            // rows per 1 KB LDS-direct load
+  static constexpr int NLD = PF_TN / RPB / W;     // LDS-direct loads per wave, tensor and step
+  static_assert(NLD >= 1 && NLD * W * RPB == PF_TN, "tile must divide evenly over the waves");
 };
+
+#define PF_GLL(gptr, lptr) __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(gptr), (void __attribute__((address_space(3)))*)(lptr), 16, 0, 0)
 
 template <int HD, int QB, int W>
 __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p, uint32_t n_col_blocks) {
   typedef PfShape<HD, W> S;
   constexpr int RW = W * QB * 32;                  // query rows per workgroup
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  unsigned char* kbuf = smem;                      // [2][KBUF]
-  unsigned char* vbuf = smem + 2 * S::KBUF;        // [2][VBUF]
+  // four separate LDS objects (two K, two V buffers): the compiler then orders an LDS read only after the
+  // LDS-direct loads into the *same* buffer, and the prefetch into the other buffer stays in flight
+  __shared__ __attribute__((aligned(1024))) unsigned char kbuf0[S::TILE];
+  __shared__ __attribute__((aligned(1024))) unsigned char kbuf1[S::TILE];
+  __shared__ __attribute__((aligned(1024))) unsigned char vbuf0[S::TILE];
+  __shared__ __attribute__((aligned(1024))) unsigned char vbuf1[S::TILE];
 
   // ---- XCD-aware id -> (kv head, column block) ----
   const uint32_t total = n_col_blocks * p.n_kv_heads;
@@ -67,7 +78,8 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   if (lid >= total) return;
   const uint32_t g = lid / n_col_blocks, cb = lid % n_col_blocks, sp = blockIdx.y;
 
-  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t tid = threadIdx.x, lane = tid & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform (scalar) so per-wave branches are scalar branches
   const uint32_t ln = lane & 31, hb = lane >> 5;   // MFMA row / column index, k half
   const uint32_t G = p.group, nH = p.n_heads;
   const uint32_t c0 = cb * p.cols_per_group;
@@ -82,17 +94,37 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   const unsigned char* kg_base = (const unsigned char*)(p.k_cache + (size_t)g * HD);
   const unsigned char* vg_base = (const unsigned char*)(p.v_cache + (size_t)g * HD);
 
-  // ---- first K/V tile: global -> registers ----
-  u4 kr[S::LD], vr[S::LD];
-  uint32_t ld_row[S::LD], ld_chunk[S::LD];
+  // ---- LDS-direct tile loads: wave w fills 1 KB blocks w*NLD .. of each buffer; lane i of a block lands at
+  //      (row i / CPR, slot i % CPR) and therefore fetches chunk slot ^ swizzle(row) of that row ----
+  uint32_t k_src[S::NLD], v_src[S::NLD], ld_row[S::NLD];
 #pragma unroll
-  for (int i = 0; i < S::LD; i++) {
-    const uint32_t e = tid + i * W * 64;
-    ld_row[i] = e / S::CPR; ld_chunk[i] = e % S::CPR;
-    const size_t off = (size_t)(t_begin + ld_row[i]) * row_bytes + ld_chunk[i] * 16;
-    kr[i] = *(const u4*)(kg_base + off);
-    vr[i] = *(const u4*)(vg_base + off);
+  for (int i = 0; i < S::NLD; i++) {
+    const uint32_t row = (wave * S::NLD + i) * S::RPB + lane / S::CPR, slot = lane % S::CPR;
+    ld_row[i] = row;
+    k_src[i] = row * (uint32_t)row_bytes + (slot ^ (row & 15)) * 16;
+    v_src[i] = row * (uint32_t)row_bytes + (slot ^ (4 * (row & 3))) * 16;
   }
+  auto issue_tile = [&](unsigned char* kdst, unsigned char* vdst, uint32_t tpos) {
+    const unsigned char* kt = kg_base + (size_t)tpos * row_bytes;
+    const unsigned char* vt = vg_base + (size_t)tpos * row_bytes;
+    if (tpos + PF_TN <= t_end) {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) {
+        PF_GLL(kt + k_src[i], kdst + (wave * S::NLD + i) * 1024);
+        PF_GLL(vt + v_src[i], vdst + (wave * S::NLD + i) * 1024);
+      }
+    } else {
+      // last tile of the context: rows at or past t_end come from the zero padding row max_seq
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) {
+        const bool live = tpos + ld_row[i] < t_end;
+        const size_t pad = (size_t)p.max_seq * row_bytes - (size_t)ld_row[i] * row_bytes;
+        PF_GLL(live ? kt + k_src[i] : kg_base + pad + k_src[i], kdst + (wave * S::NLD + i) * 1024);
+        PF_GLL(live ? vt + v_src[i] : vg_base + pad + v_src[i], vdst + (wave * S::NLD + i) * 1024);
+      }
+    }
+  };
+  issue_tile(kbuf0, vbuf0, t_begin);
 
   // ---- per-lane rows: query row of block qb is wave*QB*32 + qb*32 + ln = (column r / G, head r % G) ----
   uint32_t end_pos[QB], row_id[QB];
@@ -133,29 +165,15 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   for (int qb = 0; qb < QB; qb++) { m_ref[qb] = NEG_INF; l_run[qb] = 0.f; }
   const float c1 = p.scale * 1.4426950408889634f;   // scores -> log2 domain
 
-  // ---- stage tile 0 ----
-#pragma unroll
-  for (int i = 0; i < S::LD; i++) {
-    *(u4*)(kbuf + ld_row[i] * S::KROW + ld_chunk[i] * 16) = kr[i];
-    const u4 z = {0u, 0u, 0u, 0u};
-    *(u4*)(vbuf + ld_row[i] * S::VROW + ld_chunk[i] * 16) = (t_begin + ld_row[i] < t_end) ? vr[i] : z;
-  }
+  // per-lane LDS read offsets with the swizzles folded in (buffer bases are 1 KB aligned, so XOR == add on the
+  // swizzled bits): K fragment of k-step ks is at k_rd ^ (ks * 32); V fragment of dim block db at v_rd ^ (db * 64)
+  const uint32_t k_rd = ln * S::ROWB + ((hb ^ (ln & 1)) * 16) + ((ln & 15) >> 1) * 32;
+  const uint32_t b4 = lane >> 4, sl = lane & 15;
+  const uint32_t v_rd = (4 * (b4 >> 1) + (sl >> 2)) * S::ROWB + (2 * (b4 & 1) + ((sl & 3) >> 1)) * 16 + (sl & 1) * 8 + ((sl >> 2) & 3) * 64;
   __syncthreads();
 
-  for (uint32_t step = 0; step < n_steps; step++) {
-    const uint32_t tp = t_begin + step * PF_TN;
-    const bool more = step + 1 < n_steps;
-    const unsigned char* kb = kbuf + (step & 1) * S::KBUF;
-    const unsigned char* vb = vbuf + (step & 1) * S::VBUF;
-    // next tile's loads (the caches carry 32 rows of padding, so a straddling tile reads valid memory)
-    if (more) {
-#pragma unroll
-      for (int i = 0; i < S::LD; i++) {
-        const size_t off = (size_t)(tp + PF_TN + ld_row[i]) * row_bytes + ld_chunk[i] * 16;
-        kr[i] = *(const u4*)(kg_base + off);
-        vr[i] = *(const u4*)(vg_base + off);
-      }
-    }
+  // one step on a staged tile: kb / vb are the buffers holding positions tp .. tp + 31
+  auto compute = [&](const unsigned char* kb, const unsigned char* vb, const uint32_t tp) {
     if (tp < w_max_end) {
       // ---- S^T = K Q^T : rows = 32 positions, columns = 32 query rows per block ----
       f16v s[QB];
@@ -163,26 +181,50 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
       for (int qb = 0; qb < QB; qb++)
 #pragma unroll
         for (int i = 0; i < 16; i++) s[qb][i] = 0.f;
+      {
+        // K fragments are fetched KD k-steps ahead of the MFMA that consumes them (LDS latency off the MFMA chain)
+        constexpr int KD = 4;
+        h8 ka[KD];
 #pragma unroll
-      for (int ks = 0; ks < S::KS; ks++) {
-        const h8 a = *(const h8*)(kb + ln * S::KROW + ks * 32 + hb * 16);
+        for (int i = 0; i < KD; i++) ka[i] = *(const h8*)(kb + (k_rd ^ (i * 32)));
 #pragma unroll
-        for (int qb = 0; qb < QB; qb++) s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[qb][ks], s[qb], 0, 0, 0);
+        for (int ks = 0; ks < S::KS; ks++) {
+          const h8 a = ka[ks % KD];
+          if (ks + KD < S::KS) ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
+#pragma unroll
+          for (int qb = 0; qb < QB; qb++) s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[qb][ks], s[qb], 0, 0, 0);
+        }
+        // pin the issue order the source states: KD reads up front, then one read per k-step behind its MFMAs
+#pragma unroll
+        for (int i = 0; i < KD; i++) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+#pragma unroll
+        for (int ks = 0; ks < S::KS; ks++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
+          if (ks + KD < S::KS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
       }
       // ---- online softmax; lane holds query row ln of each block, positions tp + 8 (i / 4) + 4 hb + i % 4 ----
-      const bool diag = tp + PF_TN > w_min_end;      // some row of this wave ends inside the tile
+      // Raw scores stay unscaled: the scale rides in the exp2 argument (one fma per element), the row sum is a
+      // v_dot2 over the f16-rounded probabilities (the values PV really uses), and the mask is a separate pass
+      // that only tiles straddling a row end execute.
+      if (tp + PF_TN > w_min_end) {
+        asm volatile("; causal tile" ::: "memory");   // keeps this a branch: most tiles skip the 3 ops per element
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            const uint32_t pos = tp + 8 * (i >> 2) + 4 * hb + (i & 3);
+            s[qb][i] = pos < end_pos[qb] ? s[qb][i] : NEG_INF;
+          }
+      }
       float mt[QB];
 #pragma unroll
       for (int qb = 0; qb < QB; qb++) {
-        float mx = NEG_INF;
+        float mx = fmaxf(s[qb][0], s[qb][1]);
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          float x = s[qb][i] * c1;
-          if (diag) { const uint32_t pos = tp + 8 * (i >> 2) + 4 * hb + (i & 3); x = pos < end_pos[qb] ? x : NEG_INF; }
-          s[qb][i] = x;
-          mx = fmaxf(mx, x);
-        }
-        mt[qb] = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[qb][i]), s[qb][i + 1]);
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+        mt[qb] = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * c1;      // both k halves of the row, log2 domain
       }
       bool grow = false;
 #pragma unroll
@@ -199,44 +241,64 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
         }
       }
       h8 pf[QB][2];
+      const h2 ones = { (_Float16)1.f, (_Float16)1.f };
 #pragma unroll
       for (int qb = 0; qb < QB; qb++) {
-        const float mr = m_ref[qb] == NEG_INF ? 0.f : m_ref[qb];
-        float ps = 0.f;
+        const float nmr = m_ref[qb] == NEG_INF ? 0.f : -m_ref[qb];
+        float ps = l_run[qb];
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const float e = __builtin_amdgcn_exp2f(s[qb][i] - mr);
-          ps += e;
-          pf[qb][i >> 3][i & 7] = (_Float16)e;
+        for (int i = 0; i < 16; i += 2) {
+          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], c1, nmr));
+          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], c1, nmr));
+          const h2 pp = { (_Float16)e0, (_Float16)e1 };
+          ps = __builtin_amdgcn_fdot2(pp, ones, ps, false);
+          pf[qb][i >> 3][i & 7] = pp[0]; pf[qb][i >> 3][(i & 7) + 1] = pp[1];
         }
-        l_run[qb] += ps;
+        l_run[qb] = ps;
       }
       // ---- O^T += V^T P^T : rows = 32 dims, contraction over 2 x 16 positions ----
-      const uint32_t b4 = lane >> 4, sl = lane & 15;
+      {
+        // fragment f = 2 db + j: dims 32 db .., positions 16 j ..; fetched VD fragments ahead
+        constexpr int VD = 3, NF = 2 * S::DB;
+        h4 vlo[VD], vhi[VD];
 #pragma unroll
-      for (int db = 0; db < S::DB; db++) {
+        for (int f = 0; f < VD; f++) {
+          const unsigned char* vp = vb + (v_rd ^ ((f >> 1) * 64)) + (f & 1) * 16 * S::ROWB;
+          vlo[f] = lds_read_tr16(vp);
+          vhi[f] = lds_read_tr16(vp + 8 * S::ROWB);
+        }
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-          const unsigned char* vp = vb + (16 * j + 4 * (b4 >> 1) + (sl >> 2)) * S::VROW + (32 * db + 16 * (b4 & 1) + 4 * (sl & 3)) * 2;
-          const h4 lo = lds_read_tr16(vp);
-          const h4 hi = lds_read_tr16(vp + 8 * S::VROW);
+        for (int f = 0; f < NF; f++) {
+          const h4 lo = vlo[f % VD], hi = vhi[f % VD];
+          if (f + VD < NF) {
+            const int fn = f + VD;
+            const unsigned char* vp = vb + (v_rd ^ ((fn >> 1) * 64)) + (fn & 1) * 16 * S::ROWB;
+            vlo[f % VD] = lds_read_tr16(vp);
+            vhi[f % VD] = lds_read_tr16(vp + 8 * S::ROWB);
+          }
           const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
 #pragma unroll
-          for (int qb = 0; qb < QB; qb++) acc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[qb][j], acc[db][qb], 0, 0, 0);
+          for (int qb = 0; qb < QB; qb++) acc[f >> 1][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[qb][f & 1], acc[f >> 1][qb], 0, 0, 0);
+        }
+#pragma unroll
+        for (int f = 0; f < VD; f++) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, QB, 1);
+          if (f + VD < NF) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
         }
       }
     }
-    // ---- stage the next tile into the other buffer ----
-    if (more) {
-      unsigned char* kn = kbuf + ((step + 1) & 1) * S::KBUF;
-      unsigned char* vn = vbuf + ((step + 1) & 1) * S::VBUF;
-#pragma unroll
-      for (int i = 0; i < S::LD; i++) {
-        *(u4*)(kn + ld_row[i] * S::KROW + ld_chunk[i] * 16) = kr[i];
-        const u4 z = {0u, 0u, 0u, 0u};
-        *(u4*)(vn + ld_row[i] * S::VROW + ld_chunk[i] * 16) = (tp + PF_TN + ld_row[i] < t_end) ? vr[i] : z;
-      }
-    }
+  };
+
+  for (uint32_t step = 0; step < n_steps; step += 2) {
+    const uint32_t tp = t_begin + step * PF_TN;
+    if (step + 1 < n_steps) issue_tile(kbuf1, vbuf1, tp + PF_TN);
+    compute(kbuf0, vbuf0, tp);
+    __syncthreads();                       // buffer 1 has landed (the barrier waits for this wave's own loads first)
+    if (step + 1 >= n_steps) break;
+    if (step + 2 < n_steps) issue_tile(kbuf0, vbuf0, tp + 2 * PF_TN);
+    compute(kbuf1, vbuf1, tp + PF_TN);
     __syncthreads();
   }
 
@@ -291,17 +353,9 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 
 template <int HD, int QB, int W>
 static hipError_t launch_prefill_t(const AttnParams& p, uint32_t col_groups, hipStream_t s) {
-  typedef PfShape<HD, W> S;
-  const size_t lds = 2 * (S::KBUF + S::VBUF);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)pa_prefill_kernel<HD, QB, W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
   const uint32_t total = col_groups * p.n_kv_heads;
   const uint32_t gx = ((total + 7) / 8) * 8;       // whole rounds of the 8 XCDs
-  hipLaunchKernelGGL((pa_prefill_kernel<HD, QB, W>), dim3(gx, p.n_splits), dim3(W * 64), lds, s, p, col_groups);
+  hipLaunchKernelGGL((pa_prefill_kernel<HD, QB, W>), dim3(gx, p.n_splits), dim3(W * 64), 0, s, p, col_groups);
   return hipGetLastError();
 }
 
