@@ -29,6 +29,8 @@
 //     (m, l, O) go to the same buffers the decode kernel uses and the same merge kernel finishes them.
 #include "pa_internal.h"
 #include <hip/hip_fp16.h>
+#include <type_traits>
+#include <cstdlib>
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
@@ -52,15 +54,34 @@ template <int HD, int W> struct PfShape {
   static constexpr int TILE = PF_TN * ROWB;       // bytes of one staged tile (K or V)
   static constexpr int KS = HD / 16;              // k-steps of QK^T
   static constexpr int DB = HD / 32;              // 32-dim blocks of the output
+  static constexpr int QR = HD == 256 ? 8 : KS;   // k-steps whose Q fragments stay in registers
   static constexpr int CPR = HD / 8;              // 16-byte chunks per row
   static constexpr int RPB = 64 / CPR;            // rows per 1 KB LDS-direct load
   static constexpr int NLD = PF_TN / RPB / W;     // LDS-direct loads per wave, tensor and step
   static_assert(NLD >= 1 && NLD * W * RPB == PF_TN, "tile must divide evenly over the waves");
 };
 
-#define PF_GLL(gptr, lptr) __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(gptr), (void __attribute__((address_space(3)))*)(lptr), 16, 0, 0)
+// Optional per-wave timeline (development builds only, -DPA_TRACE): lane 0 stores the 100 MHz wall clock at 6
+// points of 8 consecutive steps starting at step 1000 into p.trace.
+#ifdef PA_TRACE
+#define PF_TP(k) do { if (p.trace && lane == 0 && blockIdx.y == 0) { const uint32_t st_ = (tp - t_begin) / PF_TN; if (st_ >= 1000 && st_ < 1008) p.trace[(((size_t)blockIdx.x * W + wave) * 8 + (st_ - 1000)) * 6 + (k)] = wall_clock64(); } } while (0)
+#else
+#define PF_TP(k) do { } while (0)
+#endif
 
-template <int HD, int QB, int W>
+// LDS-direct load of 64 x 16 bytes: lane i's 16 bytes land at LDS byte address lds_addr + 16 i (lds_addr is
+// wave-uniform and goes through M0).  Issued as inline assembly on purpose: the compiler then keeps ordinary
+// partial lgkmcnt waits for the LDS fragment reads around it (with its own LDS-DMA bookkeeping every LDS wait
+// becomes lgkmcnt(0)), and the only wait for these loads is the explicit vmcnt(0) before the end-of-step barrier.
+static __device__ inline void pf_gll(const unsigned char* gptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(lds_addr), "v"(gptr) : "memory");
+}
+static __device__ inline uint32_t lds_addr_of(const unsigned char* p) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)p;
+}
+#define PF_GLL(gptr, lptr) pf_gll((gptr), __builtin_amdgcn_readfirstlane(lds_addr_of(lptr)))
+
+template <int HD, int QB, int W, bool PP>
 __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p, uint32_t n_col_blocks) {
   typedef PfShape<HD, W> S;
   constexpr int RW = W * QB * 32;                  // query rows per workgroup
@@ -104,27 +125,35 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     k_src[i] = row * (uint32_t)row_bytes + (slot ^ (row & 15)) * 16;
     v_src[i] = row * (uint32_t)row_bytes + (slot ^ (4 * (row & 3))) * 16;
   }
-  auto issue_tile = [&](unsigned char* kdst, unsigned char* vdst, uint32_t tpos) {
+  // rows at or past t_end (only in the last tile of the context) come from the zero padding row max_seq
+  auto issue_k = [&](unsigned char* kdst, uint32_t tpos) {
     const unsigned char* kt = kg_base + (size_t)tpos * row_bytes;
-    const unsigned char* vt = vg_base + (size_t)tpos * row_bytes;
     if (tpos + PF_TN <= t_end) {
 #pragma unroll
-      for (int i = 0; i < S::NLD; i++) {
-        PF_GLL(kt + k_src[i], kdst + (wave * S::NLD + i) * 1024);
-        PF_GLL(vt + v_src[i], vdst + (wave * S::NLD + i) * 1024);
-      }
+      for (int i = 0; i < S::NLD; i++) PF_GLL(kt + k_src[i], kdst + (wave * S::NLD + i) * 1024);
     } else {
-      // last tile of the context: rows at or past t_end come from the zero padding row max_seq
 #pragma unroll
       for (int i = 0; i < S::NLD; i++) {
-        const bool live = tpos + ld_row[i] < t_end;
         const size_t pad = (size_t)p.max_seq * row_bytes - (size_t)ld_row[i] * row_bytes;
-        PF_GLL(live ? kt + k_src[i] : kg_base + pad + k_src[i], kdst + (wave * S::NLD + i) * 1024);
-        PF_GLL(live ? vt + v_src[i] : vg_base + pad + v_src[i], vdst + (wave * S::NLD + i) * 1024);
+        PF_GLL(tpos + ld_row[i] < t_end ? kt + k_src[i] : kg_base + pad + k_src[i], kdst + (wave * S::NLD + i) * 1024);
       }
     }
   };
-  issue_tile(kbuf0, vbuf0, t_begin);
+  auto issue_v = [&](unsigned char* vdst, uint32_t tpos) {
+    const unsigned char* vt = vg_base + (size_t)tpos * row_bytes;
+    if (tpos + PF_TN <= t_end) {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) PF_GLL(vt + v_src[i], vdst + (wave * S::NLD + i) * 1024);
+    } else {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) {
+        const size_t pad = (size_t)p.max_seq * row_bytes - (size_t)ld_row[i] * row_bytes;
+        PF_GLL(tpos + ld_row[i] < t_end ? vt + v_src[i] : vg_base + pad + v_src[i], vdst + (wave * S::NLD + i) * 1024);
+      }
+    }
+  };
+  issue_k(kbuf0, t_begin);
+  if (!PP) issue_v(vbuf0, t_begin);
 
   // ---- per-lane rows: query row of block qb is wave*QB*32 + qb*32 + ln = (column r / G, head r % G) ----
   uint32_t end_pos[QB], row_id[QB];
@@ -141,15 +170,24 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   }
 
   // ---- Q fragments (B operand of S^T = K Q^T): row ln of block qb, dims 16 ks + 8 hb .. + 7, as f16 ----
-  h8 qf[QB][S::KS];
+  // The first QR k-steps stay in registers for the whole kernel; the others are parked in LDS in fragment order
+  // ([wave][qb][ks - QR][lane] x 16 B: conflict-free b128 reads of a wave's own region) and re-read every step.
+  // At hd 256 all 16 in registers (64 VGPRs) leave too little room beside the 128 accumulators; a single spill
+  // reload inside the loop would also force the in-order vmcnt to drain the LDS-direct loads in flight.
+  constexpr int QR = S::QR;
+  extern __shared__ __attribute__((aligned(16))) unsigned char q_lds_all[];
+  unsigned char* q_lds = q_lds_all + (size_t)wave * QB * (S::KS - QR) * 1024 + lane * 16;
+  h8 qf[QB][QR];
 #pragma unroll
   for (int qb = 0; qb < QB; qb++) {
     const float* qrow = p.q + (size_t)(c0 + row_id[qb] / G) * p.q_stride + (size_t)(g * G + row_id[qb] % G) * HD + 8 * hb;
 #pragma unroll
     for (int ks = 0; ks < S::KS; ks++) {
       const f4 a = *(const f4*)(qrow + 16 * ks), b = *(const f4*)(qrow + 16 * ks + 4);
-      qf[qb][ks] = (h8){ (_Float16)a[0], (_Float16)a[1], (_Float16)a[2], (_Float16)a[3],
-                         (_Float16)b[0], (_Float16)b[1], (_Float16)b[2], (_Float16)b[3] };
+      const h8 f = { (_Float16)a[0], (_Float16)a[1], (_Float16)a[2], (_Float16)a[3],
+                     (_Float16)b[0], (_Float16)b[1], (_Float16)b[2], (_Float16)b[3] };
+      if (ks < QR) qf[qb][ks] = f;
+      else *(h8*)(q_lds + (qb * (S::KS - QR) + (ks - QR)) * 1024) = f;
     }
   }
 
@@ -170,136 +208,217 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   const uint32_t k_rd = ln * S::ROWB + ((hb ^ (ln & 1)) * 16) + ((ln & 15) >> 1) * 32;
   const uint32_t b4 = lane >> 4, sl = lane & 15;
   const uint32_t v_rd = (4 * (b4 >> 1) + (sl >> 2)) * S::ROWB + (2 * (b4 & 1) + ((sl & 3) >> 1)) * 16 + (sl & 1) * 8 + ((sl >> 2) & 3) * 64;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  // one step on a staged tile: kb / vb are the buffers holding positions tp .. tp + 31
-  auto compute = [&](const unsigned char* kb, const unsigned char* vb, const uint32_t tp) {
-    if (tp < w_max_end) {
-      // ---- S^T = K Q^T : rows = 32 positions, columns = 32 query rows per block ----
-      f16v s[QB];
+  // The three phases of a tile.  s (raw scores) lives from qk to sm, pf (f16 probabilities) from sm to pv.
+  f16v s[QB];
+  h8 pf[QB][2];
+  // ---- S^T = K Q^T : rows = 32 positions, columns = 32 query rows per block ----
+  auto qk = [&](const unsigned char* kb, const uint32_t tp) {
+    PF_TP(0);
+#pragma unroll
+    for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) s[qb][i] = 0.f;
+    // K fragments (and the Q fragments parked in LDS) are fetched KD k-steps ahead of the MFMA that consumes them
+    constexpr int KD = 4;
+    h8 ka[KD], qa[QB][KD];
+#pragma unroll
+    for (int i = 0; i < KD; i++) {
+      ka[i] = *(const h8*)(kb + (k_rd ^ (i * 32)));
+      if (i >= QR) {
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++) qa[qb][i] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (i - QR)) * 1024);
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < S::KS; ks++) {
+      const h8 a = ka[ks % KD];
+      h8 b[QB];
+#pragma unroll
+      for (int qb = 0; qb < QB; qb++) b[qb] = ks < QR ? qf[qb][ks < QR ? ks : 0] : qa[qb][ks % KD];
+      if (ks + KD < S::KS) {
+        ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
+        if (ks + KD >= QR) {
+#pragma unroll
+          for (int qb = 0; qb < QB; qb++) qa[qb][ks % KD] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (ks + KD - QR)) * 1024);
+        }
+      }
+#pragma unroll
+      for (int qb = 0; qb < QB; qb++) s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b[qb], s[qb], 0, 0, 0);
+    }
+    // pin the issue order the source states: the first KD fetches up front, then each k-step's fetches behind its MFMAs
+#pragma unroll
+    for (int i = 0; i < KD; i++) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); if (i >= QR) __builtin_amdgcn_sched_group_barrier(0x100, QB, 0); }
+#pragma unroll
+    for (int ks = 0; ks < S::KS; ks++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
+      if (ks + KD < S::KS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); if (ks + KD >= QR) __builtin_amdgcn_sched_group_barrier(0x100, QB, 0); }
+    }
+    PF_TP(1);
+  };
+  // ---- online softmax; lane holds query row ln of each block, positions tp + 8 (i / 4) + 4 hb + i % 4 ----
+  // Raw scores stay unscaled: the scale rides in the exp2 argument (one fma per element), the row sum is a
+  // v_dot2 over the f16-rounded probabilities (the values PV really uses), and the mask is a separate pass
+  // that only tiles straddling a row end execute.
+  auto sm = [&](const uint32_t tp) {
+    PF_TP(2);
+    if (tp + PF_TN > w_min_end) {
+      asm volatile("; causal tile" ::: "memory");   // keeps this a branch: most tiles skip the 3 ops per element
 #pragma unroll
       for (int qb = 0; qb < QB; qb++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) s[qb][i] = 0.f;
-      {
-        // K fragments are fetched KD k-steps ahead of the MFMA that consumes them (LDS latency off the MFMA chain)
-        constexpr int KD = 4;
-        h8 ka[KD];
-#pragma unroll
-        for (int i = 0; i < KD; i++) ka[i] = *(const h8*)(kb + (k_rd ^ (i * 32)));
-#pragma unroll
-        for (int ks = 0; ks < S::KS; ks++) {
-          const h8 a = ka[ks % KD];
-          if (ks + KD < S::KS) ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
-#pragma unroll
-          for (int qb = 0; qb < QB; qb++) s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[qb][ks], s[qb], 0, 0, 0);
+        for (int i = 0; i < 16; i++) {
+          const uint32_t pos = tp + 8 * (i >> 2) + 4 * hb + (i & 3);
+          s[qb][i] = pos < end_pos[qb] ? s[qb][i] : NEG_INF;
         }
-        // pin the issue order the source states: KD reads up front, then one read per k-step behind its MFMAs
+    }
+    float mt[QB];
 #pragma unroll
-        for (int i = 0; i < KD; i++) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    for (int qb = 0; qb < QB; qb++) {
+      float mx = fmaxf(s[qb][0], s[qb][1]);
 #pragma unroll
-        for (int ks = 0; ks < S::KS; ks++) {
-          __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
-          if (ks + KD < S::KS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-      }
-      // ---- online softmax; lane holds query row ln of each block, positions tp + 8 (i / 4) + 4 hb + i % 4 ----
-      // Raw scores stay unscaled: the scale rides in the exp2 argument (one fma per element), the row sum is a
-      // v_dot2 over the f16-rounded probabilities (the values PV really uses), and the mask is a separate pass
-      // that only tiles straddling a row end execute.
-      if (tp + PF_TN > w_min_end) {
-        asm volatile("; causal tile" ::: "memory");   // keeps this a branch: most tiles skip the 3 ops per element
+      for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[qb][i]), s[qb][i + 1]);
+      const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+      mt[qb] = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * c1;      // both k halves of the row, log2 domain
+    }
+    bool grow = false;
 #pragma unroll
-        for (int qb = 0; qb < QB; qb++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const uint32_t pos = tp + 8 * (i >> 2) + 4 * hb + (i & 3);
-            s[qb][i] = pos < end_pos[qb] ? s[qb][i] : NEG_INF;
-          }
-      }
-      float mt[QB];
+    for (int qb = 0; qb < QB; qb++) grow |= mt[qb] > m_ref[qb] + PF_RESCALE_TH;
+    if (__any(grow)) {
 #pragma unroll
       for (int qb = 0; qb < QB; qb++) {
-        float mx = fmaxf(s[qb][0], s[qb][1]);
+        const float m_new = fmaxf(m_ref[qb], mt[qb]);
+        const float alpha = m_new == NEG_INF ? 1.f : __builtin_amdgcn_exp2f(m_ref[qb] - m_new);
+        m_ref[qb] = m_new;
+        l_run[qb] *= alpha;
 #pragma unroll
-        for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[qb][i]), s[qb][i + 1]);
-        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
-        mt[qb] = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * c1;      // both k halves of the row, log2 domain
-      }
-      bool grow = false;
-#pragma unroll
-      for (int qb = 0; qb < QB; qb++) grow |= mt[qb] > m_ref[qb] + PF_RESCALE_TH;
-      if (__any(grow)) {
-#pragma unroll
-        for (int qb = 0; qb < QB; qb++) {
-          const float m_new = fmaxf(m_ref[qb], mt[qb]);
-          const float alpha = m_new == NEG_INF ? 1.f : __builtin_amdgcn_exp2f(m_ref[qb] - m_new);
-          m_ref[qb] = m_new;
-          l_run[qb] *= alpha;
-#pragma unroll
-          for (int db = 0; db < S::DB; db++) acc[db][qb] *= alpha;
-        }
-      }
-      h8 pf[QB][2];
-      const h2 ones = { (_Float16)1.f, (_Float16)1.f };
-#pragma unroll
-      for (int qb = 0; qb < QB; qb++) {
-        const float nmr = m_ref[qb] == NEG_INF ? 0.f : -m_ref[qb];
-        float ps = l_run[qb];
-#pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], c1, nmr));
-          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], c1, nmr));
-          const h2 pp = { (_Float16)e0, (_Float16)e1 };
-          ps = __builtin_amdgcn_fdot2(pp, ones, ps, false);
-          pf[qb][i >> 3][i & 7] = pp[0]; pf[qb][i >> 3][(i & 7) + 1] = pp[1];
-        }
-        l_run[qb] = ps;
-      }
-      // ---- O^T += V^T P^T : rows = 32 dims, contraction over 2 x 16 positions ----
-      {
-        // fragment f = 2 db + j: dims 32 db .., positions 16 j ..; fetched VD fragments ahead
-        constexpr int VD = 3, NF = 2 * S::DB;
-        h4 vlo[VD], vhi[VD];
-#pragma unroll
-        for (int f = 0; f < VD; f++) {
-          const unsigned char* vp = vb + (v_rd ^ ((f >> 1) * 64)) + (f & 1) * 16 * S::ROWB;
-          vlo[f] = lds_read_tr16(vp);
-          vhi[f] = lds_read_tr16(vp + 8 * S::ROWB);
-        }
-#pragma unroll
-        for (int f = 0; f < NF; f++) {
-          const h4 lo = vlo[f % VD], hi = vhi[f % VD];
-          if (f + VD < NF) {
-            const int fn = f + VD;
-            const unsigned char* vp = vb + (v_rd ^ ((fn >> 1) * 64)) + (fn & 1) * 16 * S::ROWB;
-            vlo[f % VD] = lds_read_tr16(vp);
-            vhi[f % VD] = lds_read_tr16(vp + 8 * S::ROWB);
-          }
-          const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
-#pragma unroll
-          for (int qb = 0; qb < QB; qb++) acc[f >> 1][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[qb][f & 1], acc[f >> 1][qb], 0, 0, 0);
-        }
-#pragma unroll
-        for (int f = 0; f < VD; f++) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
-#pragma unroll
-        for (int f = 0; f < NF; f++) {
-          __builtin_amdgcn_sched_group_barrier(0x008, QB, 1);
-          if (f + VD < NF) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
-        }
+        for (int db = 0; db < S::DB; db++) acc[db][qb] *= alpha;
       }
     }
+    const h2 ones = { (_Float16)1.f, (_Float16)1.f };
+#pragma unroll
+    for (int qb = 0; qb < QB; qb++) {
+      const float nmr = m_ref[qb] == NEG_INF ? 0.f : -m_ref[qb];
+      float ps = l_run[qb];
+#pragma unroll
+      for (int i = 0; i < 16; i += 2) {
+        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], c1, nmr));
+        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], c1, nmr));
+        const h2 pp = { (_Float16)e0, (_Float16)e1 };
+        ps = __builtin_amdgcn_fdot2(pp, ones, ps, false);
+        pf[qb][i >> 3][i & 7] = pp[0]; pf[qb][i >> 3][(i & 7) + 1] = pp[1];
+      }
+      l_run[qb] = ps;
+    }
+    PF_TP(3);
+  };
+  // ---- O^T += V^T P^T : rows = 32 dims, contraction over 2 x 16 positions ----
+  auto pv = [&](const unsigned char* vb, const uint32_t tp) {
+    // fragment f = j DB + db: positions 16 j .., dims 32 db .. (consecutive MFMAs hit different accumulators);
+    // fetched VD fragments ahead
+    constexpr int VD = 3, NF = 2 * S::DB;
+    h4 vlo[VD], vhi[VD];
+#pragma unroll
+    for (int f = 0; f < VD; f++) {
+      const unsigned char* vp = vb + (v_rd ^ ((f % S::DB) * 64)) + (f / S::DB) * 16 * S::ROWB;
+      vlo[f] = lds_read_tr16(vp);
+      vhi[f] = lds_read_tr16(vp + 8 * S::ROWB);
+    }
+#pragma unroll
+    for (int f = 0; f < NF; f++) {
+      const h4 lo = vlo[f % VD], hi = vhi[f % VD];
+      if (f + VD < NF) {
+        const int fn = f + VD;
+        const unsigned char* vp = vb + (v_rd ^ ((fn % S::DB) * 64)) + (fn / S::DB) * 16 * S::ROWB;
+        vlo[f % VD] = lds_read_tr16(vp);
+        vhi[f % VD] = lds_read_tr16(vp + 8 * S::ROWB);
+      }
+      const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+#pragma unroll
+      for (int qb = 0; qb < QB; qb++) acc[f % S::DB][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[qb][f / S::DB], acc[f % S::DB][qb], 0, 0, 0);
+    }
+#pragma unroll
+    for (int f = 0; f < VD; f++) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+#pragma unroll
+    for (int f = 0; f < NF; f++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, QB, 1);
+      if (f + VD < NF) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+    }
+    PF_TP(4);
   };
 
-  for (uint32_t step = 0; step < n_steps; step += 2) {
-    const uint32_t tp = t_begin + step * PF_TN;
-    if (step + 1 < n_steps) issue_tile(kbuf1, vbuf1, tp + PF_TN);
-    compute(kbuf0, vbuf0, tp);
-    __syncthreads();                       // buffer 1 has landed (the barrier waits for this wave's own loads first)
-    if (step + 1 >= n_steps) break;
-    if (step + 2 < n_steps) issue_tile(kbuf0, vbuf0, tp + 2 * PF_TN);
-    compute(kbuf1, vbuf1, tp + PF_TN);
+  // ---- main loop: two wave groups in anti-phase ----
+  // Waves w and w + W/2 share a SIMD.  Group 0 runs [PV(i-1) QK(i)] | SM(i) in the two halves of step i, group 1
+  // runs SM(i-1) | [PV(i-1) QK(i)], so in each half one wave of a SIMD owns the MFMA pipe while the other does its
+  // softmax on the VALU.  The mid-step barrier only keeps the phases aligned (no memory is exchanged across it, so
+  // it is a bare s_barrier that does not wait for the loads in flight); the end-of-step barrier publishes the tiles
+  // the LDS-direct loads of this step brought in: K(i+1) into the K buffer not in use, V(i) into the V buffer
+  // that tile i-2 has left.  V(i) is consumed during step i + 1 by both groups.
+  const bool grp1 = W >= 8 && wave >= W / 2;
+  auto issue_next = [&](auto PAR, const uint32_t i, const uint32_t tp) {
+    constexpr int par = decltype(PAR)::value;
+    if (i + 1 < n_steps) issue_k(par ? kbuf0 : kbuf1, tp + PF_TN);
+    issue_v(par ? vbuf1 : vbuf0, tp);
+  };
+  auto step_a = [&](auto PAR, const uint32_t i) {          // group 0
+    constexpr int par = decltype(PAR)::value;
+    const uint32_t tp = t_begin + i * PF_TN;
+    issue_next(PAR, i, tp);
+    if (i > 0) pv(par ? vbuf0 : vbuf1, tp - PF_TN);
+    qk(par ? kbuf1 : kbuf0, tp);
+    __builtin_amdgcn_s_barrier();
+    sm(tp);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wave's LDS-direct loads have landed
     __syncthreads();
+  };
+  auto step_b = [&](auto PAR, const uint32_t i) {          // group 1
+    constexpr int par = decltype(PAR)::value;
+    const uint32_t tp = t_begin + i * PF_TN;
+    issue_next(PAR, i, tp);
+    if (i > 0) sm(tp - PF_TN);
+    __builtin_amdgcn_s_barrier();
+    if (i > 0) pv(par ? vbuf0 : vbuf1, tp - PF_TN);
+    qk(par ? kbuf1 : kbuf0, tp);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+  const uint32_t tl = t_begin + (n_steps - 1) * PF_TN;
+  const unsigned char* v_last = ((n_steps - 1) & 1) ? vbuf1 : vbuf0;
+  const uint32_t n_even = n_steps & ~1u;
+  if (!PP) {
+    // all waves in phase: QK, softmax, PV of a tile between two barriers (tile i + 1 of both K and V in flight)
+    auto step_s = [&](auto PAR, const uint32_t i) {
+      constexpr int par = decltype(PAR)::value;
+      const uint32_t tp = t_begin + i * PF_TN;
+      if (i + 1 < n_steps) { issue_k(par ? kbuf0 : kbuf1, tp + PF_TN); issue_v(par ? vbuf0 : vbuf1, tp + PF_TN); }
+      qk(par ? kbuf1 : kbuf0, tp);
+      sm(tp);
+      pv(par ? vbuf1 : vbuf0, tp);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    };
+    for (uint32_t i = 0; i < n_even; i += 2) {
+      step_s(std::integral_constant<int, 0>{}, i);
+      step_s(std::integral_constant<int, 1>{}, i + 1);
+    }
+    if (n_steps & 1) step_s(std::integral_constant<int, 0>{}, n_even);
+  } else if (!grp1) {
+    for (uint32_t i = 0; i < n_even; i += 2) {
+      step_a(std::integral_constant<int, 0>{}, i);
+      step_a(std::integral_constant<int, 1>{}, i + 1);
+    }
+    if (n_steps & 1) step_a(std::integral_constant<int, 0>{}, n_even);
+    pv(v_last, tl);                                         // drain: the last tile's V landed before the last barrier
+  } else {
+    for (uint32_t i = 0; i < n_even; i += 2) {
+      step_b(std::integral_constant<int, 0>{}, i);
+      step_b(std::integral_constant<int, 1>{}, i + 1);
+    }
+    if (n_steps & 1) step_b(std::integral_constant<int, 0>{}, n_even);
+    sm(tl);
+    pv(v_last, tl);
   }
 
   // ---- epilogue ----
@@ -351,18 +470,30 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   }
 }
 
-template <int HD, int QB, int W>
+template <int HD, int QB, int W, bool PP>
 static hipError_t launch_prefill_t(const AttnParams& p, uint32_t col_groups, hipStream_t s) {
+  typedef PfShape<HD, W> S;
+  const size_t lds = (size_t)W * QB * (S::KS - S::QR) * 1024;     // Q fragments parked in LDS (dynamic part)
+  static bool attr_set = false;
+  if (!attr_set && lds > 0) {
+    hipError_t e = hipFuncSetAttribute((const void*)pa_prefill_kernel<HD, QB, W, PP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
   const uint32_t total = col_groups * p.n_kv_heads;
   const uint32_t gx = ((total + 7) / 8) * 8;       // whole rounds of the 8 XCDs
-  hipLaunchKernelGGL((pa_prefill_kernel<HD, QB, W>), dim3(gx, p.n_splits), dim3(W * 64), 0, s, p, col_groups);
+  hipLaunchKernelGGL((pa_prefill_kernel<HD, QB, W, PP>), dim3(gx, p.n_splits), dim3(W * 64), lds, s, p, col_groups);
   return hipGetLastError();
 }
 
 // row_blocks = 32-row query blocks per wavefront (2); the workgroup covers 4 * row_blocks * 32 rows
 hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s) {
   if (row_blocks != 2) return hipErrorNotSupported;
-  if (hd == 256) return launch_prefill_t<256, 1, 8>(p, col_groups, s);
-  if (hd == 128) return launch_prefill_t<128, 2, 4>(p, col_groups, s);
+  // In-phase waves measure faster than the anti-phase schedule on MI355X (C5: 7.27 ms vs 7.77 ms): with one wave
+  // of a SIMD alone on the MFMA pipe, every LDS fragment wait is exposed.  The anti-phase variant stays selectable
+  // for measurements.
+  static const bool anti_phase = getenv("POOLED_ATTN_PREFILL_ANTI_PHASE") != nullptr;
+  if (hd == 256) return anti_phase ? launch_prefill_t<256, 1, 8, true>(p, col_groups, s) : launch_prefill_t<256, 1, 8, false>(p, col_groups, s);
+  if (hd == 128) return anti_phase ? launch_prefill_t<128, 1, 8, true>(p, col_groups, s) : launch_prefill_t<128, 1, 8, false>(p, col_groups, s);
   return hipErrorNotSupported;
 }
