@@ -2,6 +2,7 @@
 #include "pa_internal.h"
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -379,6 +380,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   if ((rc = prof_begin(ctx))) return rc;
   if (pl.kernel == 0) HIPCHK(ctx, pa_launch_decode(p, c.head_dim, pl.row_blocks, pl.waves, pl.col_groups, ctx->stream));
+  else if (getenv("POOLED_ATTN_PREFILL_WIDE")) HIPCHK(ctx, pa_launch_prefill_wide(p, c.head_dim, pl.col_groups, ctx->stream));
   else HIPCHK(ctx, pa_launch_prefill(p, c.head_dim, pl.row_blocks, pl.col_groups, ctx->stream));
   if ((rc = prof_end(ctx))) return rc;
   if (!direct) HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));

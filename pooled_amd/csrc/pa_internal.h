@@ -48,6 +48,8 @@ hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint3
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);
 // MFMA prefill; returns hipErrorNotSupported for shapes it does not cover
 hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s);
+// the 4-wave, 64-rows-per-wave software-pipelined variant (same contract)
+hipError_t pa_launch_prefill_wide(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s);
 
 // ---- context -----------------------------------------------------------------------------------
 
