@@ -134,6 +134,17 @@ int pa_attn_decode(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_str
 int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_stride, const float* d_gate,
                     uint32_t gate_stride, uint32_t base_pos, uint32_t n_cols, void* d_out, uint32_t out_stride,
                     int out_dtype);
+/* pa_attn_decode_step: the whole attention block of one decode token in one call -- pre-step, cache write,
+ * split-K attention, merge and gate -- with the pre-step fused into the attention kernel (no separate launch, the
+ * roped q never leaves the chip).  Replaces the one-token sequence attn_glue_kv + attn_dec + attn_dec_combine_g
+ * (call site engine/qwen35.js:1598-1640; dense: engine/dense.js:394-399 + :463-469) and gives the same cache row
+ * bits and the same output as pa_glue_kv followed by pa_attn_decode.
+ *   d_q_in: f32 one column [nH][2*hd] (PA_FLAG_GATE: [q | gate] per head) or [nH][hd]
+ *   d_k, d_v: f32 [nKV][hd];  d_qw, d_kw: f32 [hd] (ignored without PA_FLAG_QK_NORM)
+ *   d_out : [nH][hd] of out_dtype
+ * pa_q_buffer / pa_gate_buffer are not written by this call. */
+int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
+                        const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype);
 /* which kernel / split / tile shape the table picks (kind: 0 decode/verify, 1 prefill) */
 int pa_plan_query(const pa_ctx* ctx, int kind, uint32_t base_pos, uint32_t n_cols, pa_plan* out);
 /* override the table's split count for decode passes (0 = table); the reference's attnDecodeSplits

@@ -49,6 +49,7 @@ SYMBOLS = {
     "pa_gate_buffer": (vp, [vp]),
     "pa_attn_decode": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32, vp, u32, c_int]),
     "pa_attn_prefill": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32, vp, u32, c_int]),
+    "pa_attn_decode_step": (c_int, [vp, u32, f32p, f32p, f32p, f32p, f32p, u32, vp, c_int]),
     "pa_plan_query": (c_int, [vp, c_int, u32, u32, ctypes.POINTER(PaPlan)]),
     "pa_set_decode_splits": (c_int, [vp, u32]),
     "pa_kv_read": (c_int, [vp, u32, c_int, u32, u32, vp]),
@@ -196,6 +197,10 @@ class PooledAttn:
         gp = d_gate if isinstance(d_gate, (int, type(None))) else d_gate.ptr
         self._chk(fn(self.ctx, layer, qp, q_stride, gp, gate_stride, base_pos, n_cols, d_out.ptr, out_stride, out_dtype))
 
+    def attn_decode_step(self, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype=PA_OUT_F32):
+        self._chk(self.L.pa_attn_decode_step(self.ctx, layer, d_q_in.ptr, d_k.ptr, d_v.ptr, d_qw.ptr if d_qw else None,
+                                             d_kw.ptr if d_kw else None, pos, d_out.ptr, out_dtype))
+
     def q_buffer_ptr(self):
         return self.L.pa_q_buffer(self.ctx)
 
@@ -246,6 +251,18 @@ class PooledAttn:
         self.sync()
         for b in (dq, dk, dv, dqw, dkw):
             b.free(); self._bufs.remove(b)
+
+    def run_decode_step(self, layer, q_in, k_in, v_in, qw, kw, pos, out_dtype=PA_OUT_F32):
+        """One decode token through the fused entry point: q_in [qcol], k_in / v_in [nKV*hd] f32 -> out [nH, hd]."""
+        bufs = [self.to_device(np.ascontiguousarray(a, dtype=np.float32)) for a in (q_in, k_in, v_in, qw, kw)]
+        esz = 4 if out_dtype == PA_OUT_F32 else 2
+        dout = self.alloc(self.q_dim * esz)
+        self.attn_decode_step(layer, bufs[0], bufs[1], bufs[2], bufs[3], bufs[4], pos, dout, out_dtype)
+        self.sync()
+        out = dout.download(np.float32 if out_dtype == PA_OUT_F32 else np.float16, self.q_dim)
+        for b in bufs + [dout]:
+            b.free(); self._bufs.remove(b)
+        return out.reshape(self.cfg["n_heads"], self.cfg["head_dim"])
 
     def run_attn(self, kind, layer, q, base_pos, gate=None, out_dtype=PA_OUT_F32):
         """q [n, nH, hd] f32 (None: the context's q buffer, n from gate or 1) -> out [n, nH, hd]."""

@@ -22,7 +22,7 @@
 // Row r of a workgroup's tile is (local column r / G, head r % G); column c (absolute position base_pos + c)
 // sees cache rows [0, base_pos + c].
 #include "pa_internal.h"
-#include <hip/hip_fp16.h>
+#include "glue_math.h"
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
@@ -40,14 +40,6 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 #else
 #define PA_TP(k) do { } while (0)
 #endif
-
-// Compiler-level ordering of LDS accesses inside one wavefront (hardware executes a wave's LDS operations
-// in order; lanes of one wave exchange data through the wave-private region without a workgroup barrier).
-static __device__ inline void wave_lds_fence() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 
 static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
   hh4 t = __builtin_amdgcn_ds_read_tr16_b64_v4f16((hh4 __attribute__((address_space(3)))*)p);
@@ -67,8 +59,13 @@ template <int HD> struct DecShape {
   static constexpr int DB = HD / 16;            // 16-dim blocks of the output
 };
 
-template <int HD, int NB, int W>
+// FUSED: the workgroup also runs the pre-step of its kv head for the one column at base_pos (n_cols == 1, NB == 1):
+// its G query heads are normed and roped from the raw projection on the way into LDS, and the wave whose tile
+// holds position base_pos norms / ropes the new key row, writes it and the value row to the cache and patches them
+// into its staged tile (the tile's own load of that row raced the write and is discarded).
+template <int HD, int NB, int W, bool FUSED>
 __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
+  static_assert(!FUSED || NB == 1, "the fused pre-step serves one column");
   typedef DecShape<HD> S;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]
@@ -113,13 +110,47 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
 
   // q loads first (they return first), then the first tile's K/V loads; staging q below overlaps the K/V latency.
   constexpr int QPT = 16 * NB * (HD / 4) / (W * 64);               // float4 of q per thread
-  f4 qv[QPT];
+  constexpr int HPW = 16 / W;                                      // fused: query heads per wave (G <= 16)
+  f4 qv[FUSED ? 1 : QPT];
+  float xq[FUSED ? HPW : 1][4], xk[4], wq[4], wk[4];
+  f4 xv4 = {0.f, 0.f, 0.f, 0.f};
+  float2 cs[2] = { make_float2(1.f, 0.f), make_float2(1.f, 0.f) };
+  const uint32_t half = FUSED ? p.n_rot / 2 : 0;
+  if constexpr (FUSED) {
+    // every load is unconditional (indices clamped) so that the waits below stay exact
 #pragma unroll
-  for (int j = 0; j < QPT; j++) {
-    const uint32_t e = tid + j * W * 64;
-    const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
-    const uint32_t rc = min(r, R - 1);                             // padding rows copy the last live row (masked out later)
-    qv[j] = *(const f4*)(p.q + (size_t)(c0 + rc / G) * p.q_stride + (size_t)(g * G + rc % G) * HD + 4 * d4);
+    for (int t = 0; t < HPW; t++) {
+      const uint32_t h = g * G + min(wave + W * t, G - 1);
+#pragma unroll
+      for (int j = 0; j < 4; j++) xq[t][j] = p.f_q_in[(size_t)h * p.f_q_head_stride + min(lane + 64 * j, (uint32_t)HD - 1)];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const uint32_t i = min(lane + 64 * j, (uint32_t)HD - 1);
+      xk[j] = p.f_k_in[(size_t)g * HD + i];
+      wq[j] = p.f_qw ? p.f_qw[i] : 1.f;
+      wk[j] = p.f_kw ? p.f_kw[i] : 1.f;
+    }
+    xv4 = *(const f4*)(p.f_v_in + (size_t)g * HD + 4 * min(lane, (uint32_t)HD / 4 - 1));
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const uint32_t i = lane + 64 * j;
+      if (half) cs[j] = rope_pair(p.rope_tab, p.inv_freq, p.base_pos, half, min(i, half - 1));
+    }
+#pragma unroll
+    for (int t = 0; t < HPW; t++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) if (lane + 64 * j >= HD) xq[t][j] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) if (lane + 64 * j >= HD) xk[j] = 0.f;
+  } else {
+#pragma unroll
+    for (int j = 0; j < QPT; j++) {
+      const uint32_t e = tid + j * W * 64;
+      const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
+      const uint32_t rc = min(r, R - 1);                             // padding rows copy the last live row (masked out later)
+      qv[j] = *(const f4*)(p.q + (size_t)(c0 + rc / G) * p.q_stride + (size_t)(g * G + rc % G) * HD + 4 * d4);
+    }
   }
   // Loads are unconditional: the caches carry TILE rows of padding past max_seq, so a tile that straddles the
   // end of the context reads valid memory; rows at or past t_end are zeroed (V) or masked (scores) below.
@@ -136,12 +167,50 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
   PA_TP(1);
   __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the K/V load issue
   // ---- q -> f16 rows in LDS; waits only for the q loads, which were issued first ----
+  h4 kpatch = {0, 0, 0, 0}, vpatch = {0, 0, 0, 0};
+  bool own_pos = false;              // this wave's tile sequence holds position base_pos
+  uint32_t pos_tile = 0;
+  if constexpr (FUSED) {
+    float* xs = (float*)stage;       // wave-private scratch (the staging region is not in use yet)
 #pragma unroll
-  for (int j = 0; j < QPT; j++) {
-    const uint32_t e = tid + j * W * 64;
-    const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
-    const h4 hv = { (_Float16)qv[j][0], (_Float16)qv[j][1], (_Float16)qv[j][2], (_Float16)qv[j][3] };
-    *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
+    for (int t = 0; t < HPW; t++) {
+      const uint32_t r = wave + W * t;
+      if (r < G) {
+        glue_head_wave(xq[t], wq, p.f_qw != nullptr, p.eps, HD, half, cs, xs, lane);
+        if (lane < HD / 4) {
+          const f4 v = *(const f4*)(xs + 4 * lane);
+          const h4 hv = { (_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3] };
+          *(h4*)(q_lds + r * S::QROW + lane * 8) = hv;
+        }
+        wave_lds_fence();
+      }
+    }
+    for (uint32_t e = tid; e < (16 - G) * (HD / 4); e += W * 64)     // padding rows (masked out later)
+      *(h4*)(q_lds + (G + e / (HD / 4)) * S::QROW + (e % (HD / 4)) * 8) = (h4){0, 0, 0, 0};
+    if (p.base_pos >= t_begin && p.base_pos < t_end) {
+      pos_tile = (p.base_pos - t_begin) / TILE;
+      own_pos = pos_tile % W == wave;
+    }
+    if (own_pos) {
+      glue_head_wave(xk, wk, p.f_kw != nullptr, p.eps, HD, half, cs, xs, lane);
+      if (lane < HD / 4) {
+        const f4 v = *(const f4*)(xs + 4 * lane);
+        kpatch = (h4){ (_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3] };
+        vpatch = (h4){ (_Float16)xv4[0], (_Float16)xv4[1], (_Float16)xv4[2], (_Float16)xv4[3] };
+        const size_t ro = (size_t)p.base_pos * kvDim + (size_t)g * HD + 4 * lane;
+        *(h4*)((_Float16*)const_cast<uint16_t*>(p.k_cache) + ro) = kpatch;
+        *(h4*)((_Float16*)const_cast<uint16_t*>(p.v_cache) + ro) = vpatch;
+      }
+      wave_lds_fence();
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < QPT; j++) {
+      const uint32_t e = tid + j * W * 64;
+      const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
+      const h4 hv = { (_Float16)qv[j][0], (_Float16)qv[j][1], (_Float16)qv[j][2], (_Float16)qv[j][3] };
+      *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
+    }
   }
   // per-lane row bookkeeping: row nb*16 + ln ends (exclusive) at end_pos[nb]; 0 for padding rows
   uint32_t end_pos[NB];
@@ -164,6 +233,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
 #pragma unroll
       for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
     }
+    if (FUSED && own_pos && tile == pos_tile && lane < HD / 4)      // the new key row (in-order LDS: lands after the staged copy)
+      *(h4*)(stage + (p.base_pos - tp) * S::KROW + lane * 8) = kpatch;
     wave_lds_fence();
     PA_TP(3);
     // ---- S^T = K Q^T ----
@@ -194,6 +265,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
 #pragma unroll
       for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
     }
+    if (FUSED && own_pos && tile == pos_tile && lane < HD / 4)      // the new value row
+      *(h4*)(stage + (p.base_pos - tp) * S::VROW + lane * 8) = vpatch;
     PA_TP(5);
     // ---- online softmax; lane holds row nb*16 + ln, positions tp + pb*16 + 4*kg + i ----
     h8 pfrag[NB];
@@ -354,7 +427,7 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
     f4 r = t / L;
     const uint32_t d = dq * 64 + 4 * tid;
     if (p.gate) {
-      const f4 gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * HD + d);
+      const f4 gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d);
 #pragma unroll
       for (int i = 0; i < 4; i++) r[i] *= 1.f / (1.f + __expf(-gt[i]));
     }
@@ -367,27 +440,27 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   }
 }
 
-template <int HD, int NB, int W>
+template <int HD, int NB, int W, bool FUSED>
 static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s) {
   typedef DecShape<HD> S;
   const size_t lds = 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W, FUSED>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL((pa_decode_kernel<HD, NB, W>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, p);
+  hipLaunchKernelGGL((pa_decode_kernel<HD, NB, W, FUSED>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, p);
   return hipGetLastError();
 }
 
 template <int HD>
 static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t col_groups, hipStream_t s) {
   switch (nb) {
-    case 1: return launch_decode_t<HD, 1, 4>(p, col_groups, s);
-    case 2: return launch_decode_t<HD, 2, 4>(p, col_groups, s);
-    case 3: return launch_decode_t<HD, 3, 4>(p, col_groups, s);
-    case 4: return launch_decode_t<HD, 4, 4>(p, col_groups, s);
+    case 1: return launch_decode_t<HD, 1, 4, false>(p, col_groups, s);
+    case 2: return launch_decode_t<HD, 2, 4, false>(p, col_groups, s);
+    case 3: return launch_decode_t<HD, 3, 4, false>(p, col_groups, s);
+    case 4: return launch_decode_t<HD, 4, 4, false>(p, col_groups, s);
     default: return hipErrorInvalidValue;
   }
 }
@@ -396,6 +469,13 @@ hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint3
   if (waves != 4) return hipErrorInvalidValue;
   if (hd == 256) return launch_decode_hd<256>(p, nb, col_groups, s);
   if (hd == 128) return launch_decode_hd<128>(p, nb, col_groups, s);
+  return hipErrorInvalidValue;
+}
+
+hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s) {
+  if (!p.f_q_in || p.n_cols != 1 || p.group > 16) return hipErrorInvalidValue;
+  if (hd == 256) return launch_decode_t<256, 1, 4, true>(p, 1, s);
+  if (hd == 128) return launch_decode_t<128, 1, 4, true>(p, 1, s);
   return hipErrorInvalidValue;
 }
 

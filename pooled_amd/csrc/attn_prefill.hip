@@ -71,6 +71,9 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform (scalar) so per-wave branches are scalar branches
   const uint32_t ln = lane & 31, hb = lane >> 5;   // MFMA row / column index, k half
+#ifdef PF_CLK   // development builds: shader clock vs 100 MHz wall clock over the kernel
+  long long clk0 = clock64(), wc0 = wall_clock64();
+#endif
   const uint32_t G = p.group, nH = p.n_heads;
   const uint32_t c0 = cb * p.cols_per_group;
   const uint32_t ncl = min(p.cols_per_group, p.n_cols - c0);
@@ -390,6 +393,9 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     pv(v_last, tl);
   }
 
+#ifdef PF_CLK
+  if (p.trace && tid == 0) { p.trace[blockIdx.x * 2] = clock64() - clk0; p.trace[blockIdx.x * 2 + 1] = wall_clock64() - wc0; }
+#endif
   // ---- epilogue ----
 #pragma unroll
   for (int qb = 0; qb < QB; qb++) {

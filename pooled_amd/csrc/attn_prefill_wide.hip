@@ -100,6 +100,9 @@ __global__ __launch_bounds__(256, 1) void pa_prefill_wide_kernel(AttnParams p, u
   const uint32_t ln = lane & 31, hb = lane >> 5;
   const uint32_t G = p.group, nH = p.n_heads;
   const uint32_t c0 = cb * p.cols_per_group;
+#ifdef PW_CLK   // development builds: shader clock vs 100 MHz wall clock over the kernel
+  long long clk0 = clock64(), wc0 = wall_clock64();
+#endif
   const uint32_t ncl = min(p.cols_per_group, p.n_cols - c0);
   const uint32_t R = ncl * G;
   const uint32_t seq_max = p.base_pos + c0 + ncl;
@@ -134,7 +137,9 @@ __global__ __launch_bounds__(256, 1) void pa_prefill_wide_kernel(AttnParams p, u
     }
   };
   issue(kg_base, k_src, kbuf0, t_begin);
-  issue(vg_base, v_src, vbuf0, t_begin);
+  if (n_steps > 1) issue(kg_base, k_src, kbuf1, t_begin + PF_TN);
+  // iteration 0 runs the PV product of a tile "-1": P = 0 times this zeroed buffer
+  for (uint32_t o = tid * 16; o < (uint32_t)S::TILE; o += 256 * 16) *(u4*)(vbuf1 + o) = u4{0, 0, 0, 0};
 
   // ---- per-lane rows: query row of block qb is wave*64 + qb*32 + ln = (column r / G, head r % G) ----
   uint32_t end_pos[QB], row_id[QB];
@@ -172,15 +177,26 @@ __global__ __launch_bounds__(256, 1) void pa_prefill_wide_kernel(AttnParams p, u
   const uint32_t k_rd = ln * S::ROWB + ((hb ^ (ln & 1)) * 16) + ((ln & 15) >> 1) * 32;
   const uint32_t b4 = lane >> 4, sl = lane & 15;
   const uint32_t v_rd = (4 * (b4 >> 1) + (sl >> 2)) * S::ROWB + (2 * (b4 & 1) + ((sl & 3) >> 1)) * 16 + (sl & 1) * 8 + ((sl >> 2) & 3) * 64;
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
 
-  f16v s[QB];
+  // ---- software-pipelined main loop ----
+  // A single wave per SIMD has nobody to fill the MFMA pipe during its softmax, so the loop is pipelined across
+  // tiles.  Iteration i issues, in this order:
+  //   phase A: the PV MFMAs of tile i-1, with the row maxima of tile i (VALU) slotted between them,
+  //   the (rare) rescale of O, which in program order follows PV(i-1) and so scales it too,
+  //   phase C: the QK MFMAs of tile i+1, with exp2 / f16 conversion / row sums of tile i slotted between them.
+  // S^T is double buffered in registers (s[i & 1]); LDS holds K(i+1) and V(i-1) while the LDS-direct loads of
+  // K(i+2) and V(i) are in flight; one barrier per iteration.  A scheduling barrier after every pair of MFMAs with
+  // its fragment reads and softmax slice keeps the compiler from regrouping the two instruction streams.
+  constexpr int KD = 4, QD = 2, VD = 4;
+  f16v s[2][QB];
   h8 pf[QB][2];
-  // ---- S^T = K Q^T : a K fragment is fetched KD k-steps ahead and feeds both query blocks ----
-  auto qk = [&](const unsigned char* kb) __attribute__((always_inline)) {
-    constexpr int KD = 4, QD = 2;
-    h8 ka[KD], qa[QB][QD];
+#pragma unroll
+  for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) pf[qb][j] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+  h8 ka[KD], qa[QB][QD];
+  h4 vlo[VD], vhi[VD];
+  auto k_preload = [&](const unsigned char* kb) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < KD; i++) ka[i] = *(const h8*)(kb + (k_rd ^ (i * 32)));
 #pragma unroll
@@ -189,45 +205,94 @@ __global__ __launch_bounds__(256, 1) void pa_prefill_wide_kernel(AttnParams p, u
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) qa[qb][i] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (i - QR)) * 1024);
       }
-    pw_for<S::KS>([&](auto KSI) {
-      constexpr int ks = decltype(KSI)::value;
-      const h8 a = ka[ks % KD];
-#pragma unroll
-      for (int qb = 0; qb < QB; qb++) {
-        const h8 b = ks < QR ? qf[qb][ks < QR ? ks : 0] : qa[qb][ks % QD];
-        pw_s_mfma<ks == 0, (ks == S::KS - 1)>(s[qb], a, b);
-      }
-      if (ks + KD < S::KS) ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
-      if (ks + QD < S::KS && ks + QD >= QR) {
-#pragma unroll
-        for (int qb = 0; qb < QB; qb++) qa[qb][ks % QD] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (ks + QD - QR)) * 1024);
-      }
-    });
   };
-  // ---- online softmax (as in pa_prefill_kernel); lane holds query row ln of each block ----
-  auto sm = [&](const uint32_t tp) __attribute__((always_inline)) {
+  auto v_preload = [&](const unsigned char* vb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int f = 0; f < VD; f++) {
+      const unsigned char* vp = vb + (v_rd ^ ((f % S::DB) * 64)) + (f / S::DB) * 16 * S::ROWB;
+      vlo[f] = lds_read_tr16(vp);
+      vhi[f] = lds_read_tr16(vp + 8 * S::ROWB);
+    }
+  };
+  // k-step ks of S^T = K Q^T into sd (both query blocks share the K fragment), then the fetches KD / QD steps ahead
+  auto qk_step = [&](auto KSI, f16v (&sd)[QB], const unsigned char* kb) __attribute__((always_inline)) {
+    constexpr int ks = decltype(KSI)::value;
+    const h8 a = ka[ks % KD];
+#pragma unroll
+    for (int qb = 0; qb < QB; qb++) {
+      const h8 b = ks < QR ? qf[qb][ks < QR ? ks : 0] : qa[qb][ks % QD];
+      pw_s_mfma<ks == 0, (ks == S::KS - 1)>(sd[qb], a, b);
+    }
+    if (ks + KD < S::KS) ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
+    if (ks + QD < S::KS && ks + QD >= QR) {
+#pragma unroll
+      for (int qb = 0; qb < QB; qb++) qa[qb][ks % QD] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (ks + QD - QR)) * 1024);
+    }
+  };
+  // fragment f = j DB + db of O^T += V^T P^T (positions 16 j .., dims 32 db ..; both query blocks share it)
+  auto pv_step = [&](auto FI, const unsigned char* vb) __attribute__((always_inline)) {
+    constexpr int f = decltype(FI)::value;
+    const h4 lo = vlo[f % VD], hi = vhi[f % VD];
+    const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+    pw_acc_mfma<(f % S::DB) * QB + 0>(a, pf[0][f / S::DB]);
+    pw_acc_mfma<(f % S::DB) * QB + 1>(a, pf[1][f / S::DB]);
+    if (f + VD < S::NF) {
+      constexpr int fn = f + VD;
+      const unsigned char* vp = vb + (v_rd ^ ((fn % S::DB) * 64)) + (fn / S::DB) * 16 * S::ROWB;
+      vlo[f % VD] = lds_read_tr16(vp);
+      vhi[f % VD] = lds_read_tr16(vp + 8 * S::ROWB);
+    }
+  };
+
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  k_preload(kbuf0);
+  pw_for<S::KS>([&](auto KSI) { qk_step(KSI, s[0], kbuf0); });
+
+  const h2 ones = { (_Float16)1.f, (_Float16)1.f };
+  auto iter = [&](auto PAR, const uint32_t i) __attribute__((always_inline)) {
+    constexpr int par = decltype(PAR)::value;         // tile i lives in s[par], K(i+1) in kbuf[1-par], V(i-1) in vbuf[1-par]
+    const uint32_t tp = t_begin + i * PF_TN;
+    f16v (&sc)[QB] = s[par];
+    const unsigned char* vb = par ? vbuf0 : vbuf1;
+    const unsigned char* kb = par ? kbuf0 : kbuf1;
+    v_preload(vb);
+    if (i + 2 < n_steps) issue(kg_base, k_src, par ? kbuf1 : kbuf0, tp + 2 * PF_TN);
+    issue(vg_base, v_src, par ? vbuf1 : vbuf0, tp);
     if (tp + PF_TN > w_min_end) {
       asm volatile("; causal tile" ::: "memory");
 #pragma unroll
       for (int qb = 0; qb < QB; qb++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const uint32_t pos = tp + 8 * (i >> 2) + 4 * hb + (i & 3);
-          s[qb][i] = pos < end_pos[qb] ? s[qb][i] : NEG_INF;
+        for (int e = 0; e < 16; e++) {
+          const uint32_t pos = tp + 8 * (e >> 2) + 4 * hb + (e & 3);
+          sc[qb][e] = pos < end_pos[qb] ? sc[qb][e] : NEG_INF;
         }
     }
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase A: PV(i-1) || row maxima of tile i ----
+    float mx[QB];
+    constexpr int MPG = 16 / S::NF;                   // max slices per fragment
+    pw_for<S::NF>([&](auto FI) {
+      constexpr int f = decltype(FI)::value;
+      pv_step(FI, vb);
+      if (f == S::NF - 2) k_preload(kb);
+#pragma unroll
+      for (int t = 0; t < MPG; t++) {
+        const int c = f * MPG + t, qb = c / 8, j = c % 8;
+        if (j == 0) mx[qb] = fmaxf(sc[qb][0], sc[qb][1]);
+        else mx[qb] = fmaxf(fmaxf(mx[qb], sc[qb][2 * j]), sc[qb][2 * j + 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
     float mt[QB];
-#pragma unroll
-    for (int qb = 0; qb < QB; qb++) {
-      float mx = fmaxf(s[qb][0], s[qb][1]);
-#pragma unroll
-      for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[qb][i]), s[qb][i + 1]);
-      const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
-      mt[qb] = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * c1;
-    }
     bool grow = false;
 #pragma unroll
-    for (int qb = 0; qb < QB; qb++) grow |= mt[qb] > m_ref[qb] + PF_RESCALE_TH;
+    for (int qb = 0; qb < QB; qb++) {
+      const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx[qb]), __float_as_uint(mx[qb]), false, false);
+      mt[qb] = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * c1;
+      grow |= mt[qb] > m_ref[qb] + PF_RESCALE_TH;
+    }
     if (__any(grow)) {
       float alpha[QB];
 #pragma unroll
@@ -244,68 +309,45 @@ __global__ __launch_bounds__(256, 1) void pa_prefill_wide_kernel(AttnParams p, u
       });
       asm volatile("s_nop 3" ::: "memory");           // v_accvgpr_write -> next MFMA
     }
-    const h2 ones = { (_Float16)1.f, (_Float16)1.f };
+    float nmr[QB];
 #pragma unroll
-    for (int qb = 0; qb < QB; qb++) {
-      const float nmr = m_ref[qb] == NEG_INF ? 0.f : -m_ref[qb];
-      float ps = l_run[qb];
+    for (int qb = 0; qb < QB; qb++) nmr[qb] = m_ref[qb] == NEG_INF ? 0.f : -m_ref[qb];
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase C: QK(i+1) || exp2, f16 conversion and row sums of tile i ----
+    constexpr int EPG = 16 / S::KS;                   // exp pairs per k-step
+    pw_for<S::KS>([&](auto KSI) {
+      constexpr int ks = decltype(KSI)::value;
+      qk_step(KSI, s[1 - par], kb);
 #pragma unroll
-      for (int i = 0; i < 16; i += 2) {
-        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], c1, nmr));
-        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], c1, nmr));
+      for (int t = 0; t < EPG; t++) {
+        const int c = ks * EPG + t, qb = c / 8, e = 2 * (c % 8);
+        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[qb][e], c1, nmr[qb]));
+        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[qb][e + 1], c1, nmr[qb]));
         const h2 pp = { (_Float16)e0, (_Float16)e1 };
-        ps = __builtin_amdgcn_fdot2(pp, ones, ps, false);
-        pf[qb][i >> 3][i & 7] = pp[0]; pf[qb][i >> 3][(i & 7) + 1] = pp[1];
+        l_run[qb] = __builtin_amdgcn_fdot2(pp, ones, l_run[qb], false);
+        pf[qb][e >> 3][e & 7] = pp[0]; pf[qb][e >> 3][(e & 7) + 1] = pp[1];
       }
-      l_run[qb] = ps;
-    }
-  };
-  // ---- O^T += V^T P^T : fragment f = j DB + db (positions 16 j .., dims 32 db ..) feeds both query blocks ----
-  auto pv = [&](const unsigned char* vb) __attribute__((always_inline)) {
-    constexpr int VD = 4;
-    h4 vlo[VD], vhi[VD];
-#pragma unroll
-    for (int f = 0; f < VD; f++) {
-      const unsigned char* vp = vb + (v_rd ^ ((f % S::DB) * 64)) + (f / S::DB) * 16 * S::ROWB;
-      vlo[f] = lds_read_tr16(vp);
-      vhi[f] = lds_read_tr16(vp + 8 * S::ROWB);
-    }
-    pw_for<S::NF>([&](auto FI) {
-      constexpr int f = decltype(FI)::value;
-      const h4 lo = vlo[f % VD], hi = vhi[f % VD];
-      const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
-      pw_acc_mfma<(f % S::DB) * QB + 0>(a, pf[0][f / S::DB]);
-      pw_acc_mfma<(f % S::DB) * QB + 1>(a, pf[1][f / S::DB]);
-      if (f + VD < S::NF) {
-        constexpr int fn = f + VD;
-        const unsigned char* vp = vb + (v_rd ^ ((fn % S::DB) * 64)) + (fn / S::DB) * 16 * S::ROWB;
-        vlo[f % VD] = lds_read_tr16(vp);
-        vhi[f % VD] = lds_read_tr16(vp + 8 * S::ROWB);
-      }
+      __builtin_amdgcn_sched_barrier(0);
     });
-  };
-
-  // ---- main loop: QK, softmax, PV of tile i between two barriers while tile i + 1 of K and V is in flight ----
-  auto step = [&](auto PAR, const uint32_t i) __attribute__((always_inline)) {
-    constexpr int par = decltype(PAR)::value;
-    const uint32_t tp = t_begin + i * PF_TN;
-    if (i + 1 < n_steps) {
-      issue(kg_base, k_src, par ? kbuf0 : kbuf1, tp + PF_TN);
-      issue(vg_base, v_src, par ? vbuf0 : vbuf1, tp + PF_TN);
-    }
-    qk(par ? kbuf1 : kbuf0);
-    sm(tp);
-    pv(par ? vbuf1 : vbuf0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   };
   const uint32_t n_even = n_steps & ~1u;
   for (uint32_t i = 0; i < n_even; i += 2) {
-    step(std::integral_constant<int, 0>{}, i);
-    step(std::integral_constant<int, 1>{}, i + 1);
+    iter(std::integral_constant<int, 0>{}, i);
+    iter(std::integral_constant<int, 1>{}, i + 1);
   }
-  if (n_steps & 1) step(std::integral_constant<int, 0>{}, n_even);
+  if (n_steps & 1) iter(std::integral_constant<int, 0>{}, n_even);
+  // drain: PV of the last tile (its V landed before the last barrier)
+  {
+    const unsigned char* vb = ((n_steps - 1) & 1) ? vbuf1 : vbuf0;
+    v_preload(vb);
+    pw_for<S::NF>([&](auto FI) { pv_step(FI, vb); });
+  }
 
+#ifdef PW_CLK
+  if (p.trace && tid == 0) { p.trace[blockIdx.x * 2] = clock64() - clk0; p.trace[blockIdx.x * 2 + 1] = wall_clock64() - wc0; }
+#endif
   // ---- epilogue (same outputs as pa_prefill_kernel) ----
   asm volatile("s_nop 15" ::: "memory");              // last PV MFMA -> v_accvgpr_read
   pw_for<QB>([&](auto QBI) {
@@ -347,7 +389,7 @@ __global__ __launch_bounds__(256, 1) void pa_prefill_wide_kernel(AttnParams p, u
 }
 
 #ifndef PW_QR
-#define PW_QR 12
+#define PW_QR 10
 #endif
 
 template <int HD>

@@ -5,39 +5,15 @@
 // reference's fused glue kernels (engine/wgsl/qwen35.js:1082-1136 attn_glue, engine/wgsl/layer_fuse.js:87-146
 // attn_glue_kv, engine/wgsl/dense.js:144-196 attn_glue_d), which it replaces.
 //
-// Arithmetic (chosen so a CPU restatement can reproduce the bits):
-//   ss   = sum v_i^2 in f64 (exact products), inv = f32(1 / sqrt(ss / hd + eps)) evaluated in f64
-//   v_i  = v_i * (inv * w_i)                 two f32 multiplies (engine/wgsl/base.js:65-79)
-//   ang  = f32(pos) * inv_freq[i]            f32 product; inv_freq is a host-built f32 table of
-//                                            theta^(-2i/n_rot) (engine/wgsl/qwen35.js:397)
-//   c, s = f32(cos(f64(ang))), f32(sin(f64(ang)))
-//   a'   = a*c - b*s,  b' = b*c + a*s        separately rounded f32 products and sums (no FMA)
-//   cache element = f16 round-to-nearest-even of the f32 value (engine/wgsl/qwen35.js:889-906)
+// The per-head arithmetic lives in glue_math.h (shared with the fused decode-step kernel); cache elements are the
+// f16 round-to-nearest-even of the f32 values (engine/wgsl/qwen35.js:889-906).
 #include "pa_internal.h"
-#include <hip/hip_fp16.h>
-
-// every product and sum below is rounded on its own: no fused multiply-add may be formed in this file
-// (plain operators are used instead of the __fmul_rn family, whose header bodies are compiled with contraction on)
-#pragma clang fp contract(off)
+#include "glue_math.h"
 
 #define GLUE_DO_MATH 0x100u
 
-static __device__ inline double wave_sum_f64(double v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
-
 static __device__ inline uint32_t pack_f16x2(float lo, float hi) {
   return (uint32_t)__half_as_ushort(__float2half_rn(lo)) | ((uint32_t)__half_as_ushort(__float2half_rn(hi)) << 16);
-}
-
-// c, s of the f32 angle f32(pos) * inv_freq, evaluated in f64 and rounded once
-static __device__ inline void rope_cos_sin(uint32_t pos, float inv_freq, float& c, float& s) {
-  const float ang = (float)pos * inv_freq;
-  double sd, cd;
-  sincos((double)ang, &sd, &cd);
-  c = (float)cd; s = (float)sd;
 }
 
 // The same values for every (position, pair), computed once per context: rope_tab[pos * half + i] = (cos, sin).
@@ -68,54 +44,30 @@ __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
   const float* src = isQ ? p.q_in + (size_t)col * p.q_stride + (size_t)h * (gated ? 2 * hd : hd)
                          : p.k_in + (size_t)col * p.k_stride + (size_t)h * hd;
   float x[4];
-  double ss = 0.0;
 #pragma unroll
   for (int j = 0; j < 4; j++) {
     const uint32_t i = lane + 64 * j;
     x[j] = 0.f;
     if (i < hd) {
       x[j] = src[i];
-      ss += (double)x[j] * (double)x[j];
       if (isQ && gated) p.gate_out[(size_t)col * qDim + h * hd + i] = src[hd + i];
     }
   }
-  if (math && (p.flags & PA_FLAG_QK_NORM)) {
-    ss = wave_sum_f64(ss);
-    const float inv = (float)(1.0 / sqrt(ss / (double)hd + (double)p.eps));
-    const float* w = isQ ? p.qw : p.kw;
+  const uint32_t half = math ? p.n_rot / 2 : 0;
+  float2 cs[2] = { make_float2(1.f, 0.f), make_float2(1.f, 0.f) };
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const uint32_t i = lane + 64 * j;
-      if (i < hd) { const float sw = inv * w[i]; x[j] = x[j] * sw; }
-    }
+  for (int j = 0; j < 2; j++) {
+    const uint32_t i = lane + 64 * j;
+    if (i < half) cs[j] = rope_pair(p.rope_tab, p.inv_freq, pos, half, i);
   }
+  const bool norm = math && (p.flags & PA_FLAG_QK_NORM);
+  float w[4] = {0.f, 0.f, 0.f, 0.f};
+  if (norm) {
+    const float* wp = isQ ? p.qw : p.kw;
 #pragma unroll
-  for (int j = 0; j < 4; j++) { const uint32_t i = lane + 64 * j; if (i < hd) xs[i] = x[j]; }
-  __syncthreads();
-  if (math) {
-    const uint32_t half = p.n_rot / 2;
-    float ra[2], rb[2];
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const uint32_t i = lane + 64 * j;
-      if (i < half) {
-        float c, s;
-        if (p.rope_tab) { const float2 cs = p.rope_tab[(size_t)pos * half + i]; c = cs.x; s = cs.y; }
-        else rope_cos_sin(pos, p.inv_freq[i], c, s);
-        const float a = xs[i], b = xs[i + half];
-        const float ac = a * c, bs = b * s, bc = b * c, as = a * s;   // rounded one by one (contract off above)
-        ra[j] = ac - bs;
-        rb[j] = bc + as;
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const uint32_t i = lane + 64 * j;
-      if (i < half) { xs[i] = ra[j]; xs[i + half] = rb[j]; }
-    }
-    __syncthreads();
+    for (int j = 0; j < 4; j++) { const uint32_t i = lane + 64 * j; if (i < hd) w[j] = wp[i]; }
   }
+  glue_head_wave(x, w, norm, p.eps, hd, half, cs, xs, lane);
   if (isQ) {
     for (uint32_t i = lane; i < hd; i += 64) p.q_out[(size_t)col * qDim + h * hd + i] = xs[i];
     return;

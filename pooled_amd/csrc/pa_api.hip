@@ -378,6 +378,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
+  p.gate_head_stride = c.head_dim;
   if ((rc = prof_begin(ctx))) return rc;
   if (pl.kernel == 0) HIPCHK(ctx, pa_launch_decode(p, c.head_dim, pl.row_blocks, pl.waves, pl.col_groups, ctx->stream));
   else if (getenv("POOLED_ATTN_PREFILL_WIDE")) HIPCHK(ctx, pa_launch_prefill_wide(p, c.head_dim, pl.col_groups, ctx->stream));
@@ -396,6 +397,48 @@ extern "C" int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, ui
                                uint32_t gate_stride, uint32_t base_pos, uint32_t n_cols, void* d_out, uint32_t out_stride,
                                int out_dtype) {
   return attn_common(ctx, "pa_attn_prefill", 1, layer, d_q, q_stride, d_gate, gate_stride, base_pos, n_cols, d_out, out_stride, out_dtype);
+}
+
+extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
+                                   const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
+  const char* who = "pa_attn_decode_step";
+  if (!ctx) return PA_ERR_INVALID;
+  int rc = check_cols(ctx, who, layer, true, pos, 1);
+  if (rc) return rc;
+  const pa_config& c = ctx->cfg;
+  const bool gated = (c.flags & PA_FLAG_GATE) != 0, norm = (c.flags & PA_FLAG_QK_NORM) != 0;
+  if (!d_q_in || !d_k || !d_v || !d_out) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null buffer");
+  if (norm && (!d_qw || !d_kw)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": norm weights required");
+  if (out_dtype != PA_OUT_F32 && out_dtype != PA_OUT_F16) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": bad out_dtype");
+  if (((uintptr_t)d_q_in & 15) || ((uintptr_t)d_k & 15) || ((uintptr_t)d_v & 15) || ((uintptr_t)d_out & 15))
+    return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned");
+  if (c.n_heads / c.n_kv_heads > 16) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": more than 16 query heads per kv head");
+  pa_plan pl;
+  rc = plan_decode(ctx, pos, 1, &pl);
+  if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
+  if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
+  if (pl.row_blocks != 1 || pl.waves != 4 || pl.col_groups != 1) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": plan is not a one-block decode");
+  if ((rc = ensure_partials(ctx, 1, pl.slots))) return rc;
+  AttnParams p; memset(&p, 0, sizeof p);
+  p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+  p.part_o = ctx->part_o; p.part_ml = ctx->part_ml; p.out = d_out;
+  p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
+  p.base_pos = pos; p.n_cols = 1;
+  p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
+  p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
+  p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
+  // the pre-step inputs; the gate is read in place from the interleaved [q | gate] heads
+  p.f_q_in = d_q_in; p.f_k_in = d_k; p.f_v_in = d_v;
+  p.f_qw = norm ? d_qw : nullptr; p.f_kw = norm ? d_kw : nullptr;
+  p.rope_tab = ctx->rope_tab; p.inv_freq = ctx->inv_freq;
+  p.f_q_head_stride = c.head_dim * (gated ? 2 : 1); p.n_rot = c.n_rot; p.eps = c.eps;
+  p.gate = gated ? d_q_in + c.head_dim : nullptr;
+  p.gate_head_stride = p.f_q_head_stride;
+  if ((rc = prof_begin(ctx))) return rc;
+  HIPCHK(ctx, pa_launch_decode_step(p, c.head_dim, ctx->stream));
+  if ((rc = prof_end(ctx))) return rc;
+  HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
+  return PA_OK;
 }
 
 // ---- cache access ---------------------------------------------------------------------------------

@@ -37,6 +37,14 @@ struct AttnParams {
   int out_f16;
   float scale;                                // 1 / sqrt(hd)
   unsigned long long* trace;                  // per-wave timestamps when built with PA_TRACE (else unused, nullptr)
+  uint32_t gate_head_stride;                  // floats between consecutive heads in gate (head_dim, or 2*head_dim
+                                              // when gate is read in place from an interleaved [q | gate] column)
+  // fused pre-step of pa_attn_decode_step (one column at base_pos; f_q_in == nullptr otherwise): raw projections
+  const float* f_q_in; const float* f_k_in; const float* f_v_in;   // [nH][q_head_stride], [nKV][hd], [nKV][hd]
+  const float* f_qw; const float* f_kw;       // norm weights [hd] or nullptr
+  const float2* rope_tab; const float* inv_freq;
+  uint32_t f_q_head_stride, n_rot;
+  float eps;
 };
 
 // ---- kernel launchers (defined next to their kernels) ------------------------------------------
@@ -45,6 +53,8 @@ hipError_t pa_launch_glue(const GlueParams& p, hipStream_t s);
 hipError_t pa_launch_rope_table(float2* tab, const float* inv_freq, uint32_t half, uint32_t n_pos, hipStream_t s);
 // waves per workgroup W in {4, 8}; NB = 16-row query blocks per workgroup (1..4); hd in {128, 256}
 hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s);
+// the same with the pre-step of the one column fused in (p.f_* set; one 16-row block, n_cols == 1)
+hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s);
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);
 // MFMA prefill; returns hipErrorNotSupported for shapes it does not cover
 hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s);

@@ -137,6 +137,21 @@ static napi_value Attn(napi_env env, napi_callback_info info) {
   if (rc) return throw_pa(env, c, rc, kind == 0 ? "pa_attn_decode" : "pa_attn_prefill");
   return undefined(env);
 }
+// attnDecodeStep(ctx, layer, qIn, k, v, qw|null, kw|null, pos, out, outDtype): the fused one-token block
+static napi_value AttnDecodeStep(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0);
+  uint32_t layer = a.u32(1); const float* q = (const float*)a.ptr(2); const float* k = (const float*)a.ptr(3); const float* v = (const float*)a.ptr(4);
+  const float* qw = (const float*)a.ptr(5); const float* kw = (const float*)a.ptr(6); uint32_t pos = a.u32(7);
+  void* out = a.ptr(8); int dt = (int)a.u32(9); CHECK_ARGS("attnDecodeStep");
+  int rc = pa_attn_decode_step(c, layer, q, k, v, qw, kw, pos, out, dt);
+  if (rc) return throw_pa(env, c, rc, "pa_attn_decode_step");
+  return undefined(env);
+}
+// copyD2d(ctx, dst, src, bytes): device-to-device copy on the context's stream
+static napi_value CopyD2d(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); void* dst = a.ptr(1); const void* src = a.ptr(2); size_t n = (size_t)a.num(3); CHECK_ARGS("copyD2d");
+  int rc = pa_copy_d2d(c, dst, src, n); if (rc) return throw_pa(env, c, rc, "pa_copy_d2d"); return undefined(env);
+}
 // planQuery(ctx, kind, basePos, nCols) -> {kernel, splitLen, nSplits, colGroups, colsPerGroup, waves, rowBlocks, slots}
 static napi_value PlanQuery(napi_env env, napi_callback_info info) {
   ARGS; pa_ctx* c = a.ctx(0); int kind = (int)a.u32(1); uint32_t base = a.u32(2), n = a.u32(3); CHECK_ARGS("planQuery");
@@ -172,7 +187,8 @@ static napi_value Init(napi_env env, napi_value exports) {
     {"setStream", SetStream}, {"malloc", Malloc}, {"free", Free}, {"upload", Upload}, {"download", Download}, {"glueKv", GlueKv}, {"glue", Glue},
     {"kvStore", KvStore}, {"qBuffer", QBuffer}, {"gateBuffer", GateBuffer}, {"attn", Attn}, {"planQuery", PlanQuery},
     {"setDecodeSplits", SetDecodeSplits}, {"kvRead", KvRead}, {"kvWrite", KvWrite}, {"kvDevicePtr", KvDevicePtr}, {"timerStart", TimerStart},
-    {"timerStop", TimerStop}, {"profileEnable", ProfileEnable}, {"profileRead", ProfileRead},
+    {"timerStop", TimerStop}, {"profileEnable", ProfileEnable}, {"profileRead", ProfileRead}, {"attnDecodeStep", AttnDecodeStep},
+    {"copyD2d", CopyD2d},
   };
   for (auto& t : table) {
     napi_value fn;

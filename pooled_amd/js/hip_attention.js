@@ -62,6 +62,7 @@ class HipAttention {
     this.gate = !!opts.gate;
     this.qkNorm = opts.qkNorm !== false;
     this.outDtype = opts.outF16 ? PA_OUT_F16 : PA_OUT_F32;
+    this.fusedStep = opts.fusedStep !== false;
     // engine fields the attention dispatch reads (engine/qwen35.js:366, :416-419): always the f16-KV split-K path here
     this.flash = true; this.kvQ8 = false; this.attnDecode = "v2"; this.attnPrefillTile = true;
     this._snapNow = null;                                          // set by a verify pass (engine/qwen35.js:2960-2965)
@@ -154,8 +155,14 @@ class HipAttention {
     this._snapNow = null;
   }
   // ---- Qwen35Engine: one token (fused glue + KV write, split-K decode, merge + gate in one go) ----
+  // By default this is the single fused call; { fusedStep: false } in the constructor options keeps the three
+  // dispatches of the reference (glue + KV write, split-K decode, merge + gate) as separate launches.
   encodeLayerAttn(p, i, pos) {
     const B = this.B, L = this.layers[i], n = this._norms(L);
+    if (this.fusedStep) {
+      addon.attnDecodeStep(this.ctx, i, B.qFull.ptr, B.k.ptr, B.v.ptr, n[0], n[1], pos, B.attnOut.ptr, this.outDtype);
+      return;
+    }
     addon.glueKv(this.ctx, i, B.qFull.ptr, this._strideF(B.qFull), B.k.ptr, this._strideF(B.k), B.v.ptr, this._strideF(B.v), n[0], n[1], pos, 1);
     const gate = this.gate ? addon.gateBuffer(this.ctx) : null;
     addon.attn(this.ctx, 0, i, null, 0, gate, this.dims.qDim, pos, 1, B.attnOut.ptr, this._outStride(), this.outDtype);

@@ -1,0 +1,91 @@
+"""GPU parity of the fused one-token entry point (pre-step + cache write + split-K attention + merge + gate in one
+call) through the C ABI.  The written cache row equals the oracle's bits, the rows around it stay untouched, and
+the output equals pa_glue_kv followed by pa_attn_decode bit for bit (same kernels' arithmetic) and the oracle
+within the floating-point bar: max-abs <= 2e-3 and max|d|/max|ref| <= 1e-2."""
+import numpy as np
+import pytest
+from oracle import attn_oracle as O
+from oracle import c_oracle as C
+from pooled_amd.capi import PooledAttn, PaError, PA_OUT_F16, PA_ERR_INVALID
+from helpers import SHAPES, assert_parity, random_cache
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(cfg, pos, seed):
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    max_seq = pos + 5
+    k16, v16 = random_cache(cfg, max_seq, seed=seed)
+    d = O.make_inputs(cfg, 0, 1, seed + 1)
+    ref_g = O.glue_kv(d["qraw"], d["kraw"], d["vraw"], d["qw"], d["kw"], pos, cfg)
+    K = k16.copy(); V = v16.copy()
+    K[pos] = ref_g["k16"].reshape(nKV, hd); V[pos] = ref_g["v16"].reshape(nKV, hd)
+    gate = ref_g["gate"].reshape(1, nH, hd) if cfg.get("gate") else None
+    ref = C.attention(ref_g["q"].reshape(1, nH, hd), K, V, pos, gate=gate)
+    return d, k16, v16, K, V, ref, max_seq
+
+
+@pytest.mark.parametrize("shape,pos", [
+    ("qwen36_moe", 0), ("qwen36_moe", 1), ("qwen36_moe", 31), ("qwen36_moe", 32), ("qwen36_moe", 95), ("qwen36_moe", 777),
+    ("qwen36_moe", 4096), ("qwen36_moe", 20001), ("qwen38_27b", 300), ("qwen38_27b", 5000), ("qwen3_1p7b", 129),
+    ("qwen3_1p7b", 2500),
+])
+def test_decode_step_matches_oracle_and_unfused(shape, pos):
+    cfg = SHAPES[shape]
+    d, k16, v16, K, V, ref, max_seq = _case(cfg, pos, seed=pos + 3)
+    poison = np.uint16(0x7E00)
+    with PooledAttn(cfg, max_seq, n_layers=1, max_cols=1) as pa:
+        pa.layer_alloc(0)
+        for which, a in ((0, k16), (1, v16)):
+            a = a.copy(); a[pos] = poison                        # the row the call must write is NaN before it
+            pa.kv_write(0, which, 0, a)
+        got = pa.run_decode_step(0, d["qraw"][0], d["kraw"][0], d["vraw"][0], d["qw"], d["kw"], pos)
+        Kg = pa.kv_read(0, 0, 0, max_seq); Vg = pa.kv_read(0, 1, 0, max_seq)
+        # the unfused pair on a fresh copy of the same cache
+        for which, a in ((0, k16), (1, v16)):
+            pa.kv_write(0, which, 0, a)
+        pa.run_glue_kv(0, d["qraw"], d["kraw"], d["vraw"], d["qw"], d["kw"], pos)
+        gate = pa.read_gate_buffer(1) if cfg.get("gate") else None
+        unf = pa.run_attn("decode", 0, pa.read_q_buffer(1), pos, gate=gate)
+    assert np.array_equal(Kg.reshape(K.shape), K) and np.array_equal(Vg.reshape(V.shape), V), "cache differs from the oracle's bits"
+    assert_parity(got[None], ref, "%s pos %d" % (shape, pos))
+    assert np.array_equal(got.view(np.uint32), unf[0].view(np.uint32)), "fused output differs from pa_glue_kv + pa_attn_decode"
+
+
+def test_decode_step_f16_out_and_no_norm():
+    cfg = dict(SHAPES["qwen3_1p7b"], qk_norm=False)
+    pos = 600
+    d, k16, v16, K, V, ref, max_seq = _case(cfg, pos, seed=5)
+    with PooledAttn(cfg, max_seq, n_layers=1, max_cols=1) as pa:
+        pa.layer_alloc(0); pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
+        got = pa.run_decode_step(0, d["qraw"][0], d["kraw"][0], d["vraw"][0], d["qw"], d["kw"], pos, out_dtype=PA_OUT_F16)
+        Kg = pa.kv_read(0, 0, 0, max_seq)
+    assert np.array_equal(Kg.reshape(K.shape), K)
+    assert_parity(got[None].astype(np.float32), ref, "f16 out, no norm")
+
+
+def test_decode_step_sequence():
+    """Twelve consecutive tokens through the fused call: every step sees the rows the earlier steps wrote."""
+    cfg = SHAPES["qwen36_moe"]
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    base, n = 250, 12
+    k16, v16 = random_cache(cfg, base + n, seed=31)
+    d = O.make_inputs(cfg, 0, n, 32)
+    ref_g = O.glue_kv(d["qraw"], d["kraw"], d["vraw"], d["qw"], d["kw"], base, cfg)
+    K = k16.copy(); V = v16.copy()
+    K[base:base + n] = ref_g["k16"].reshape(n, nKV, hd); V[base:base + n] = ref_g["v16"].reshape(n, nKV, hd)
+    ref = C.attention(ref_g["q"].reshape(n, nH, hd), K, V, base, gate=ref_g["gate"].reshape(n, nH, hd))
+    with PooledAttn(cfg, base + n, n_layers=1, max_cols=1) as pa:
+        pa.layer_alloc(0); pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
+        outs = [pa.run_decode_step(0, d["qraw"][c], d["kraw"][c], d["vraw"][c], d["qw"], d["kw"], base + c) for c in range(n)]
+    assert_parity(np.stack(outs), ref, "sequence")
+
+
+def test_decode_step_rejects_bad_arguments():
+    cfg = SHAPES["qwen36_moe"]
+    with PooledAttn(cfg, 64, n_layers=1, max_cols=1) as pa:
+        pa.layer_alloc(0)
+        d = O.make_inputs(cfg, 0, 1, 1)
+        with pytest.raises(PaError) as e:
+            pa.run_decode_step(0, d["qraw"][0], d["kraw"][0], d["vraw"][0], d["qw"], d["kw"], 64)   # pos == max_seq
+        assert e.value.code == PA_ERR_INVALID

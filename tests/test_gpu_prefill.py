@@ -77,6 +77,19 @@ def test_prefill_peaked_softmax():
     assert_parity(got, ref, "peaked")
 
 
+@pytest.mark.parametrize("shape,base,n,k_scale", [
+    ("qwen36_moe", 301, 16, 1.0), ("qwen36_moe", 1000, 200, 1.0), ("qwen3_1p7b", 219, 257, 1.0),
+    ("qwen38_27b", 500, 96, 3.0), ("qwen36_moe", 20000, 64, 1.0),
+])
+def test_prefill_wide_variant(shape, base, n, k_scale, monkeypatch):
+    """The 4-wave, 64-rows-per-wave variant of the prefill kernel (selected by an environment variable read at
+    each call): same parity bar, including the rescale path (peaked scores) and the split path."""
+    monkeypatch.setenv("POOLED_ATTN_PREFILL_WIDE", "1")
+    got, ref, plan = _prefill(SHAPES[shape], base, n, seed=base + n + 1, k_scale=k_scale)
+    assert plan["kernel"] == 1
+    assert_parity(got, ref, "wide %s base %d n %d" % (shape, base, n))
+
+
 def test_c2_prefill_full():
     """Config 2: 512-token chunk at positions 1536-2047 over a 1536-token prefix, Qwen3-1.7B shape, pre-step on
     the GPU (QK-RMSNorm + full RoPE theta 1e6 + KV write for the chunk), f16 output."""
