@@ -7,7 +7,8 @@ Headline workload (BASELINE.json's metric, "decode attn KV-read GB/s @32K ctx"):
 single-token gated decode attention, Qwen3.6-35B-MoE attention shape (16 q heads, 2 kv heads, head_dim 256),
 context 32768.  A step is one pass of the hot path for one token on one attention layer: pre-step (q
 de-interleave + QK-RMSNorm + partial RoPE + f16 KV write at position 32768), split-K decode kernel, log-sum-exp
-merge with the sigmoid gate.  Consecutive steps walk over N_LAYERS distinct layers' caches (as a model does),
+merge with the sigmoid gate -- by default through the fused entry point pa_attn_decode_step (--unfused: the three
+separate launches).  Consecutive steps walk over N_LAYERS distinct layers' caches (as a model does),
 so the 64 MiB of K/V a step reads is never resident in the 256 MB last-level cache from the previous step.
 value = algorithmic KV bytes per step / wall time per step, all inputs resident in HBM.
 
@@ -181,6 +182,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=60)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (configuration 5) leg")
+    ap.add_argument("--unfused", action="store_true", help="decode step as three launches (pa_glue_kv + pa_attn_decode) instead of the fused pa_attn_decode_step")
     ap.add_argument("--prefill-steps", type=int, default=5)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 10 device-to-device copies of 256 MiB (the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
@@ -223,8 +225,11 @@ def main():
 
     def step(i):
         layer = i % N_LAYERS
-        pa.glue_kv(layer, d_qfull, 2 * qd, d_k, kvd, d_v, kvd, d_qw, d_kw, ctx, 1)
-        pa.attn("decode", layer, None, 0, gate_ptr, qd, ctx, 1, d_out, qd, PA_OUT_F16)
+        if args.unfused:
+            pa.glue_kv(layer, d_qfull, 2 * qd, d_k, kvd, d_v, kvd, d_qw, d_kw, ctx, 1)
+            pa.attn("decode", layer, None, 0, gate_ptr, qd, ctx, 1, d_out, qd, PA_OUT_F16)
+        else:
+            pa.attn_decode_step(layer, d_qfull, d_k, d_v, d_qw, d_kw, ctx, d_out, PA_OUT_F16)
 
     kv_bytes = 2 * (ctx + 1) * kvd * 2            # K and V rows [0, 32768], f16
     for i in range(args.warmup):
@@ -253,7 +258,7 @@ def main():
     if os.path.exists(tpath):
         traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
-                    traffic=traffic, kernel="pa_decode_kernel<256, 1, 4>", kernel_us=round(k_ms * 1e3, 3),
+                    traffic=traffic, kernel="pa_decode_kernel<256, 1, 4, %s>" % ("false" if args.unfused else "true"), kernel_us=round(k_ms * 1e3, 3),
                     algorithmic_bytes_per_launch=kv_bytes, launches=kcount)
     log("split-K kernel: %.2f us/launch -> %.0f GB/s (%.1f%% of 8 TB/s)" % (k_ms * 1e3, achieved, 100 * achieved / HBM_PEAK_GBS))
     plan = pa.plan("decode", ctx, 1)
@@ -280,7 +285,7 @@ def main():
         ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None,
         dtype="f16", data="synthetic",
         config=dict(workload="C3 gated decode: 16q/2kv heads, head_dim 256, ctx 32768, 1 token, f16 KV, partial RoPE 64 dims theta 1e7, sigmoid gate, f16 out",
-                    step="glue_kv + split-K decode + LSE merge/gate on one layer; %d layers' caches in rotation (cold HBM)" % N_LAYERS,
+                    step="%s on one layer; %d layers' caches in rotation (cold HBM)" % ("pa_glue_kv + pa_attn_decode (pre-step, split-K decode, LSE merge/gate: 3 launches)" if args.unfused else "pa_attn_decode_step (pre-step fused into the split-K decode kernel + LSE merge/gate: 2 launches)", N_LAYERS),
                     kv_bytes_per_step=kv_bytes, plan=plan, pct_hbm_peak=round(100 * value / HBM_PEAK_GBS, 2)),
         roofline=roofline, cpu_baseline=cpu)
     pa.close()

@@ -370,11 +370,13 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
 // ---- second pass: log-sum-exp merge over a column's splits, sigmoid gate, output conversion ----
 // One workgroup per (head, 64-dim slice, column) -- the reference's layout (engine/wgsl/attn_dec.js:215-287,
 // DEC_CQ slices per head) -- so the merge of a decode token runs on nH * HD/64 workgroups instead of nH.
-// 256 threads = 16 split groups x 16 float4 lanes; every split is read in parallel, the maximum and the
-// weighted sum of l by fixed-order tree reductions, the 16 groups' partial outputs summed in group order.
+// 256 threads = 16 split groups x 16 float4 lanes.  The kernel is latency-bound (a few KB per workgroup, read
+// once, from the memory side), so it is written as one round trip: a thread issues all 16 output-partial loads of
+// its first 256-split chunk and its (m, l) loads before anything waits; the maximum and the weighted sum of l are
+// fixed-order tree reductions, a group's splits are accumulated in split order and the 16 groups in group order.
 template <int HD>
 __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
-  constexpr int CQ = HD / 64;
+  constexpr int CQ = HD / 64, CH = 16;      // CH loads in flight per thread = 256 splits per chunk
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* wl = (float*)smem;                 // [slots] split weights exp(m_s - M)
   __shared__ float red[256];
@@ -385,11 +387,13 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
   const uint32_t grp = tid >> 4, l4 = tid & 15;
   const float* po = p.part_o + base * HD + dq * 64 + 4 * l4;
-  // the first output partials go out before the (m, l) reductions: their latency overlaps the barriers below
-  f4 o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
-  const bool h0 = grp < ns, h1 = grp + 16 < ns;
-  if (h0) o0 = *(const f4*)(po + (size_t)grp * HD);
-  if (h1) o1 = *(const f4*)(po + (size_t)(grp + 16) * HD);
+  const f4 zero = {0.f, 0.f, 0.f, 0.f};
+  f4 ov[CH];
+#pragma unroll
+  for (int k = 0; k < CH; k++) {
+    const uint32_t s = grp + 16 * k;
+    ov[k] = s < ns ? *(const f4*)(po + (size_t)s * HD) : zero;
+  }
   float lm = NEG_INF;
   for (uint32_t s = tid; s < ns; s += 256) lm = fmaxf(lm, p.part_ml[(base + s) * 2]);
   red[tid] = lm;
@@ -407,16 +411,23 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   __syncthreads();
   for (uint32_t k = 128; k > 0; k >>= 1) { if (tid < k) red[tid] += red[tid + k]; __syncthreads(); }
   const float L = red[0];
-  f4 o = {0.f, 0.f, 0.f, 0.f};
-  if (h0) o = o0 * wl[grp];
-  if (h1) o += o1 * wl[grp + 16];
-  for (uint32_t s = grp + 32; s < ns; s += 32) {
-    const f4 a = *(const f4*)(po + (size_t)s * HD);
-    f4 b = {0.f, 0.f, 0.f, 0.f};
-    const bool hb = s + 16 < ns;
-    if (hb) b = *(const f4*)(po + (size_t)(s + 16) * HD);
-    o += a * wl[s];
-    if (hb) o += b * wl[s + 16];
+  f4 o = zero;
+#pragma unroll
+  for (int k = 0; k < CH; k++) {
+    const uint32_t s = grp + 16 * k;
+    if (s < ns) o += ov[k] * wl[s];
+  }
+  for (uint32_t s0 = 16 * CH; s0 < ns; s0 += 16 * CH) {          // contexts with more than 256 splits
+#pragma unroll
+    for (int k = 0; k < CH; k++) {
+      const uint32_t s = s0 + grp + 16 * k;
+      ov[k] = s < ns ? *(const f4*)(po + (size_t)s * HD) : zero;
+    }
+#pragma unroll
+    for (int k = 0; k < CH; k++) {
+      const uint32_t s = s0 + grp + 16 * k;
+      if (s < ns) o += ov[k] * wl[s];
+    }
   }
   ored[tid] = o;
   __syncthreads();
