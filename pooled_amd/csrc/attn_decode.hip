@@ -34,11 +34,13 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 #define NEG_INF (-__builtin_inff())
 
 // Optional per-wave timeline (development builds only): lane 0 of every wave stores the 100 MHz wall clock at
-// up to 12 points into p.trace.  Compiled out unless PA_TRACE is defined.
+// up to 10 points (and the shader clock counter at entry and exit, slots 10 and 11) into p.trace.  Compiled out unless PA_TRACE is defined.
 #ifdef PA_TRACE
 #define PA_TP(k) do { if (p.trace && lane == 0) p.trace[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * W * 12 + wave * 12 + (k)] = wall_clock64(); } while (0)
+#define PA_TC(k) do { if (p.trace && lane == 0) p.trace[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * W * 12 + wave * 12 + (k)] = clock64(); } while (0)
 #else
 #define PA_TP(k) do { } while (0)
+#define PA_TC(k) do { } while (0)
 #endif
 
 static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
@@ -83,9 +85,10 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
   const uint32_t seq_max = p.base_pos + c0 + ncl;                    // rows visible to the group's last column
   const uint32_t t_begin = sp * p.split_len;
   if (t_begin >= seq_max) return;
-  const uint32_t t_end = min(t_begin + p.split_len, seq_max);
+  // the last split is open-ended: the plan may hand it up to one split length of remainder
+  const uint32_t t_end = sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
   const uint32_t kvDim = p.n_kv_heads * HD;
-  PA_TP(0);
+  PA_TP(0); PA_TC(10);
 
   unsigned char* stage = stage_all + wave * S::STAGE;
   const size_t row_bytes = (size_t)kvDim * 2;
@@ -254,20 +257,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
     }
     wave_lds_fence();
     PA_TP(4);
-    // ---- V tile -> LDS (rows at or past t_end as zeros: 0 x stale bits must not reach O), next V loads ----
-    if (tp + TILE > t_end) {
-#pragma unroll
-      for (int i = 0; i < S::NLD; i++) if (tp + i * S::RPL + lrow >= t_end) vr[i] = zero4;
-    }
-#pragma unroll
-    for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
-    if (more) {
-#pragma unroll
-      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
-    }
-    if (FUSED && own_pos && tile == pos_tile && lane < HD / 4)      // the new value row
-      *(h4*)(stage + (p.base_pos - tp) * S::VROW + lane * 8) = vpatch;
-    PA_TP(5);
     // ---- online softmax; lane holds row nb*16 + ln, positions tp + pb*16 + 4*kg + i ----
     h8 pfrag[NB];
 #pragma unroll
@@ -298,6 +287,20 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
 #pragma unroll
       for (int db = 0; db < S::DB; db++) acc[db][nb] *= alpha;
     }
+    // ---- V tile -> LDS, after the softmax so that the wait for the V loads comes as late as possible (rows at or past t_end as zeros: 0 x stale bits must not reach O), next V loads ----
+    if (tp + TILE > t_end) {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) if (tp + i * S::RPL + lrow >= t_end) vr[i] = zero4;
+    }
+#pragma unroll
+    for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
+    }
+    if (FUSED && own_pos && tile == pos_tile && lane < HD / 4)      // the new value row
+      *(h4*)(stage + (p.base_pos - tp) * S::VROW + lane * 8) = vpatch;
+    PA_TP(5);
     wave_lds_fence();
     PA_TP(6);
     // ---- O^T += V^T P^T ----
@@ -364,7 +367,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
     }
     if (nb + 1 < NB) __syncthreads();                                  // the regions are rewritten by the next row block
   }
-  PA_TP(9);
+  PA_TP(9); PA_TC(11);
 }
 
 // ---- second pass: log-sum-exp merge over a column's splits, sigmoid gate, output conversion ----
@@ -383,7 +386,7 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   __shared__ f4 ored[256];
   const uint32_t h = blockIdx.x / CQ, dq = blockIdx.x % CQ, col = blockIdx.y, tid = threadIdx.x;
   const uint32_t col_end = p.base_pos + col + 1;
-  const uint32_t ns = (col_end + p.split_len - 1) / p.split_len;
+  const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits);   // the last split is open-ended
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
   const uint32_t grp = tid >> 4, l4 = tid & 15;
   const float* po = p.part_o + base * HD + dq * 64 + 4 * l4;

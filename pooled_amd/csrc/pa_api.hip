@@ -274,8 +274,16 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
                                                 : std::max(1u, (occ * (uint32_t)ctx->n_cu) / (c.n_kv_heads * groups));
   static const uint32_t floor_tiles[5] = {1, 1, 4, 6, 8};     // tiles per wave, by row blocks
   uint32_t tpw = std::max(ceil_div(tiles, target * W), ctx->decode_splits_override ? 1u : floor_tiles[nb]);
-  uint32_t sl = 32 * W * tpw;
-  pl->kernel = 0; pl->split_len = sl; pl->n_splits = ceil_div(seq_max, sl);
+  uint32_t sl = 32 * W * tpw, ns = ceil_div(seq_max, sl);
+  // A context a little past target x split_len (a 32K context plus the token being decoded) would double the
+  // split length and leave half the workgroup slots empty, or spill a near-empty split into a second round of
+  // workgroups.  The last split takes the remainder instead (the kernels treat split n_splits - 1 as open-ended),
+  // as long as that is less than one more split.
+  if (!ctx->decode_splits_override && tpw > floor_tiles[nb]) {
+    const uint32_t tpw_lo = std::max(tiles / (target * W), floor_tiles[nb]), sl_lo = 32 * W * tpw_lo;
+    if ((uint64_t)seq_max < (uint64_t)(target + 1) * sl_lo) { sl = sl_lo; ns = std::max(1u, std::min(target, seq_max / sl_lo)); }
+  }
+  pl->kernel = 0; pl->split_len = sl; pl->n_splits = ns;
   pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = W; pl->row_blocks = nb; pl->slots = pl->n_splits;
   return PA_OK;
 }

@@ -169,7 +169,27 @@ def test_c3_gated_decode_32k():
         pa.attn("decode", 0, None, 0, pa.gate_buffer_ptr(), pa.q_dim, ctx, 1, dout, pa.q_dim)
         pa.sync()
         got = dout.download(np.float32, pa.q_dim).reshape(ref.shape)
+        # 32769 rows over 256 workgroup slots per kv head: the last split takes the one row past 256 x 128
+        pl = pa.plan("decode", ctx, 1)
+        assert (pl["n_splits"] + 1) * pl["split_len"] > ctx + 1 >= pl["n_splits"] * pl["split_len"] and pl["split_len"] % 32 == 0
     assert_parity(got, ref, "C3")
+
+
+@pytest.mark.parametrize("extra", [1, 2, 31, 32, 33, 127])
+def test_decode_open_ended_last_split(extra):
+    """Contexts a little past a whole number of splits: the last split also serves the remainder, which may add
+    tiles to some of its waves (the new row included: poisoned rows past the context must stay unused)."""
+    cfg = SHAPES["qwen36_moe"]
+    L = 32768 + extra
+    rng = np.random.default_rng(40 + extra)
+    k16, v16 = random_cache(cfg, L + 40, seed=41)
+    q = rng.standard_normal((1, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    ref = C.attention(q, k16, v16, L - 1)
+    with _ctx_with_cache(cfg, k16, v16, L + 40, poison_from=L) as pa:
+        pl = pa.plan("decode", L - 1, 1)
+        assert pl["n_splits"] * pl["split_len"] < L, "this case is meant to exercise the open-ended last split"
+        got = pa.run_attn("decode", 0, q, L - 1)
+    assert_parity(got, ref, "open-ended last split, +%d rows" % extra)
 
 
 def test_c4_verify_64k():
