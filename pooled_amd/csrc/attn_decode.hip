@@ -397,23 +397,32 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
     const uint32_t s = grp + 16 * k;
     ov[k] = s < ns ? *(const f4*)(po + (size_t)s * HD) : zero;
   }
-  float lm = NEG_INF;
-  for (uint32_t s = tid; s < ns; s += 256) lm = fmaxf(lm, p.part_ml[(base + s) * 2]);
-  red[tid] = lm;
+  // the gate of this thread's output dims (only the 16 writer threads need it) goes out with the first loads
+  const uint32_t d_out = dq * 64 + 4 * (tid & 15);
+  f4 gt = zero;
+  if (p.gate && tid < 16) gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d_out);
+  // (m, l) of this thread's first split; further ones (more than 256 splits) in the loops below
+  const float2 ml0 = tid < ns ? *(const float2*)(p.part_ml + (base + tid) * 2) : make_float2(NEG_INF, 0.f);
+  float lm = ml0.x;
+  for (uint32_t s = tid + 256; s < ns; s += 256) lm = fmaxf(lm, p.part_ml[(base + s) * 2]);
+  // maximum: xor-shuffle tree inside each wave, then the 4 waves' values in wave order
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) lm = fmaxf(lm, __shfl_xor(lm, o, 64));
+  if ((tid & 63) == 0) red[tid >> 6] = lm;
   __syncthreads();
-  for (uint32_t k = 128; k > 0; k >>= 1) { if (tid < k) red[tid] = fmaxf(red[tid], red[tid + k]); __syncthreads(); }
-  const float M = red[0];
-  __syncthreads();
+  const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   float ll = 0.f;
-  for (uint32_t s = tid; s < ns; s += 256) {
+  if (tid < ns) { const float w = __expf(ml0.x - M); wl[tid] = w; ll = ml0.y * w; }
+  for (uint32_t s = tid + 256; s < ns; s += 256) {
     const float w = __expf(p.part_ml[(base + s) * 2] - M);
     wl[s] = w;
     ll += p.part_ml[(base + s) * 2 + 1] * w;
   }
-  red[tid] = ll;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ll += __shfl_xor(ll, o, 64);
+  if ((tid & 63) == 0) red[4 + (tid >> 6)] = ll;
   __syncthreads();
-  for (uint32_t k = 128; k > 0; k >>= 1) { if (tid < k) red[tid] += red[tid + k]; __syncthreads(); }
-  const float L = red[0];
+  const float L = (red[4] + red[5]) + (red[6] + red[7]);
   f4 o = zero;
 #pragma unroll
   for (int k = 0; k < CH; k++) {
@@ -439,9 +448,8 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
 #pragma unroll
     for (int i = 1; i < 16; i++) t += ored[i * 16 + tid];
     f4 r = t / L;
-    const uint32_t d = dq * 64 + 4 * tid;
+    const uint32_t d = d_out;
     if (p.gate) {
-      const f4 gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d);
 #pragma unroll
       for (int i = 0; i < 4; i++) r[i] *= 1.f / (1.f + __expf(-gt[i]));
     }
