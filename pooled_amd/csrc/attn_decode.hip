@@ -34,13 +34,11 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 #define NEG_INF (-__builtin_inff())
 
 // Optional per-wave timeline (development builds only): lane 0 of every wave stores the 100 MHz wall clock at
-// up to 10 points (and the shader clock counter at entry and exit, slots 10 and 11) into p.trace.  Compiled out unless PA_TRACE is defined.
+// up to 12 points into p.trace.  Compiled out unless PA_TRACE is defined.
 #ifdef PA_TRACE
 #define PA_TP(k) do { if (p.trace && lane == 0) p.trace[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * W * 12 + wave * 12 + (k)] = wall_clock64(); } while (0)
-#define PA_TC(k) do { if (p.trace && lane == 0) p.trace[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * W * 12 + wave * 12 + (k)] = clock64(); } while (0)
 #else
 #define PA_TP(k) do { } while (0)
-#define PA_TC(k) do { } while (0)
 #endif
 
 static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
@@ -88,7 +86,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
   // the last split is open-ended: the plan may hand it up to one split length of remainder
   const uint32_t t_end = sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
   const uint32_t kvDim = p.n_kv_heads * HD;
-  PA_TP(0); PA_TC(10);
+  PA_TP(0);
 
   unsigned char* stage = stage_all + wave * S::STAGE;
   const size_t row_bytes = (size_t)kvDim * 2;
@@ -341,6 +339,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
       }
     }
     __syncthreads();
+    PA_TP(10);
     // rows nb*16 .. nb*16+15, HD/4 float4 each, summed over waves in wave order
     for (uint32_t e = tid; e < 16 * (HD / 4); e += W * 64) {
       const uint32_t rr = e / (HD / 4), d4 = e % (HD / 4);
@@ -367,7 +366,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
     }
     if (nb + 1 < NB) __syncthreads();                                  // the regions are rewritten by the next row block
   }
-  PA_TP(9); PA_TC(11);
+  PA_TP(9);
 }
 
 // ---- second pass: log-sum-exp merge over a column's splits, sigmoid gate, output conversion ----
