@@ -71,7 +71,8 @@ int pa_create(const pa_config* cfg, pa_ctx** out);
 int pa_destroy(pa_ctx* ctx);
 /* message of the last failing call on ctx (ctx == NULL: of the last failing pa_create) */
 const char* pa_last_error(const pa_ctx* ctx);
-/* allocate layer's K and V caches, f16 [max_seq][n_kv_heads][head_dim] row-major, zero-filled */
+/* allocate layer's K and V caches, zero-filled f16.  Device layout (head-major, chosen for the HBM stream of the
+ * attention kernels): [n_kv_heads][max_seq + 32][head_dim]; the 32 extra rows per head stay zero. */
 int pa_layer_alloc(pa_ctx* ctx, uint32_t layer);
 /* use the caller's hipStream_t (NULL: the context's own stream) */
 int pa_set_stream(pa_ctx* ctx, void* hip_stream);
@@ -152,10 +153,11 @@ int pa_plan_query(const pa_ctx* ctx, int kind, uint32_t base_pos, uint32_t n_col
 int pa_set_decode_splits(pa_ctx* ctx, uint32_t splits);
 
 /* ---- cache access for tests, checkpoints and slot copies (engine/dense.js:20-47 saveSlot/loadSlot
- *      copy rows [0, pos) of each layer) ----  which: 0 = K, 1 = V; rows are f16 bits [n_rows][nKV*hd] */
+ *      copy rows [0, pos) of each layer) ----  which: 0 = K, 1 = V; the host side is the engine's position-major
+ *      view, f16 bits [n_rows][nKV*hd]; the calls translate to and from the device layout and block */
 int pa_kv_read(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, void* h_dst);
 int pa_kv_write(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, const void* h_src);
-/* device address of a cache (read-only use; layout above) */
+/* device address of a cache (read-only use; the head-major device layout described at pa_layer_alloc) */
 const void* pa_kv_device_ptr(pa_ctx* ctx, uint32_t layer, int which);
 
 /* ---- timing on the context's stream (HIP events; replaces the reference's timestamp-query passes,

@@ -6,7 +6,7 @@
 // merge -- with a CDNA4 inside:
 //
 //   * Every wavefront streams its own 32-position K/V tiles: 128-bit coalesced global loads (a 64-lane load
-//     covers whole 512-byte f16 rows) into registers, the next tile's loads issued as soon as the current
+//     covers two whole 512-byte f16 rows; the caches are head-major, so a tile is one contiguous 16 KB block) into registers, the next tile's loads issued as soon as the current
 //     tile's registers have been staged, so a wave always has ~32 KB in flight.
 //   * Tiles are staged in a wave-private LDS region (no workgroup barrier in the loop): K rows are read back
 //     as MFMA A-operands (ds_read_b128), V rows through the gfx950 LDS transpose read (ds_read_b64_tr_b16),
@@ -85,16 +85,16 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
   if (t_begin >= seq_max) return;
   // the last split is open-ended: the plan may hand it up to one split length of remainder
   const uint32_t t_end = sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
-  const uint32_t kvDim = p.n_kv_heads * HD;
+  const size_t head_rows = (size_t)p.max_seq + TILE;              // rows of one kv head's plane, padding included
   PA_TP(0);
 
   unsigned char* stage = stage_all + wave * S::STAGE;
-  const size_t row_bytes = (size_t)kvDim * 2;
+  const size_t row_bytes = (size_t)HD * 2;                         // head-major caches: a kv head's rows are contiguous
   const uint32_t lrow = lane / S::LPR;
   // per-lane byte offset inside a wave-wide load; the tile base below is wave-uniform (scalar registers)
   const uint32_t voff = lrow * (uint32_t)row_bytes + (lane % S::LPR) * 16;
-  const unsigned char* kbase = (const unsigned char*)(p.k_cache + (size_t)g * HD);
-  const unsigned char* vbase = (const unsigned char*)(p.v_cache + (size_t)g * HD);
+  const unsigned char* kbase = (const unsigned char*)(p.k_cache + (size_t)g * head_rows * HD);
+  const unsigned char* vbase = (const unsigned char*)(p.v_cache + (size_t)g * head_rows * HD);
 
   f4 acc[S::DB][NB];
 #pragma unroll
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
         const f4 v = *(const f4*)(xs + 4 * lane);
         kpatch = (h4){ (_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3] };
         vpatch = (h4){ (_Float16)xv4[0], (_Float16)xv4[1], (_Float16)xv4[2], (_Float16)xv4[3] };
-        const size_t ro = (size_t)p.base_pos * kvDim + (size_t)g * HD + 4 * lane;
+        const size_t ro = ((size_t)g * head_rows + p.base_pos) * HD + 4 * lane;
         *(h4*)((_Float16*)const_cast<uint16_t*>(p.k_cache) + ro) = kpatch;
         *(h4*)((_Float16*)const_cast<uint16_t*>(p.v_cache) + ro) = vpatch;
       }

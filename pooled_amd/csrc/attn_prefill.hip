@@ -83,9 +83,10 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   if (t_begin >= seq_max) return;
   const uint32_t t_end = min(t_begin + p.split_len, seq_max);
   const uint32_t n_steps = (t_end - t_begin + PF_TN - 1) / PF_TN;
-  const size_t row_bytes = (size_t)p.n_kv_heads * HD * 2;
-  const unsigned char* kg_base = (const unsigned char*)(p.k_cache + (size_t)g * HD);
-  const unsigned char* vg_base = (const unsigned char*)(p.v_cache + (size_t)g * HD);
+  const size_t row_bytes = (size_t)HD * 2;                       // head-major caches: a kv head's rows are contiguous
+  const size_t head_rows = (size_t)p.max_seq + PF_TN;            // rows of one kv head's plane, padding included
+  const unsigned char* kg_base = (const unsigned char*)(p.k_cache + (size_t)g * head_rows * HD);
+  const unsigned char* vg_base = (const unsigned char*)(p.v_cache + (size_t)g * head_rows * HD);
 
   // ---- LDS-direct tile loads: wave w fills 1 KB blocks w*NLD .. of each buffer; lane i of a block lands at
   //      (row i / CPR, slot i % CPR) and therefore fetches chunk slot ^ swizzle(row) of that row ----

@@ -40,7 +40,7 @@ __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
   const bool gated = (p.flags & PA_FLAG_GATE) != 0;
   const bool math = (p.flags & GLUE_DO_MATH) != 0;
   const uint32_t pos = p.base_pos + col;
-  const uint32_t qDim = nH * hd, kvDim = p.n_kv_heads * hd;
+  const uint32_t qDim = nH * hd;
   const float* src = isQ ? p.q_in + (size_t)col * p.q_stride + (size_t)h * (gated ? 2 * hd : hd)
                          : p.k_in + (size_t)col * p.k_stride + (size_t)h * hd;
   float x[4];
@@ -74,8 +74,9 @@ __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
   }
   if (p.k_out) for (uint32_t i = lane; i < hd; i += 64) p.k_out[(size_t)col * p.k_stride + h * hd + i] = xs[i];
   if (p.k_cache) {
-    uint32_t* kc = (uint32_t*)(p.k_cache + (size_t)pos * kvDim + h * hd);
-    uint32_t* vc = (uint32_t*)(p.v_cache + (size_t)pos * kvDim + h * hd);
+    const size_t ro = ((size_t)h * p.head_rows + pos) * hd;           // head-major caches
+    uint32_t* kc = (uint32_t*)(p.k_cache + ro);
+    uint32_t* vc = (uint32_t*)(p.v_cache + ro);
     const float* vs = p.v_in + (size_t)col * p.v_stride + (size_t)h * hd;
     for (uint32_t w = lane; w < hd / 2; w += 64) {
       kc[w] = pack_f16x2(xs[2 * w], xs[2 * w + 1]);

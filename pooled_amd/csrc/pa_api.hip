@@ -113,7 +113,8 @@ extern "C" int pa_layer_alloc(pa_ctx* ctx, uint32_t layer) {
   if (layer >= ctx->cfg.n_layers) return fail(ctx, PA_ERR_INVALID, "pa_layer_alloc: layer out of range");
   pa_layer& L = ctx->layers[layer];
   if (L.k) return PA_OK;
-  // 32 rows of zero padding past max_seq: the attention kernels load whole 32-row tiles unconditionally
+  // head-major, 32 rows of zero padding after each kv head's max_seq rows: the attention kernels load whole
+  // 32-row tiles unconditionally
   const size_t bytes = ((size_t)ctx->cfg.max_seq + 32) * ctx->cfg.n_kv_heads * ctx->cfg.head_dim * 2;
   HIPCHK(ctx, hipMalloc((void**)&L.k, bytes));
   hipError_t e = hipMalloc((void**)&L.v, bytes);
@@ -191,6 +192,7 @@ static void fill_glue(const pa_ctx* ctx, GlueParams& p) {
   p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.head_dim = c.head_dim; p.n_rot = c.n_rot;
   p.flags = c.flags | 0x100u;
   p.eps = c.eps;
+  p.head_rows = c.max_seq + 32;
 }
 
 extern "C" int pa_glue_kv(pa_ctx* ctx, uint32_t layer, const float* d_q_in, uint32_t q_stride, const float* d_k,
@@ -451,26 +453,41 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
 
 // ---- cache access ---------------------------------------------------------------------------------
 
-static int kv_rows(pa_ctx* ctx, const char* who, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, uint16_t** base, size_t* bytes) {
+// The caches are head-major on the device ([nKV][max_seq + 32][hd]: every kv head's rows are one contiguous
+// stream for the attention kernels); the host view of pa_kv_read / pa_kv_write stays the engine's position-major
+// [rows][nKV * hd], so each call is one strided copy per kv head.
+static int kv_copy(pa_ctx* ctx, const char* who, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, void* host, bool to_host) {
   if (layer >= ctx->cfg.n_layers || !ctx->layers[layer].k) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": layer not allocated");
   if (which != 0 && which != 1) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": which must be 0 (K) or 1 (V)");
   if ((uint64_t)row0 + n_rows > ctx->cfg.max_seq) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": rows exceed max_seq");
-  const size_t kvd = (size_t)ctx->cfg.n_kv_heads * ctx->cfg.head_dim;
-  *base = (which ? ctx->layers[layer].v : ctx->layers[layer].k) + (size_t)row0 * kvd;
-  *bytes = (size_t)n_rows * kvd * 2;
+  if (!host) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null host buffer");
+  if (n_rows == 0) return PA_OK;
+  const pa_config& c = ctx->cfg;
+  const size_t hd_bytes = (size_t)c.head_dim * 2, host_pitch = hd_bytes * c.n_kv_heads, head_rows = (size_t)c.max_seq + 32;
+  unsigned char* dev = (unsigned char*)(which ? ctx->layers[layer].v : ctx->layers[layer].k);
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  // one contiguous transfer per kv head through a host staging plane (a pitched copy of 512-byte rows is far slower)
+  std::vector<unsigned char> plane((size_t)n_rows * hd_bytes);
+  for (uint32_t g = 0; g < c.n_kv_heads; g++) {
+    unsigned char* d = dev + ((size_t)g * head_rows + row0) * hd_bytes;
+    unsigned char* h = (unsigned char*)host + (size_t)g * hd_bytes;
+    if (to_host) {
+      HIPCHK(ctx, hipMemcpy(plane.data(), d, plane.size(), hipMemcpyDeviceToHost));
+      for (uint32_t r = 0; r < n_rows; r++) memcpy(h + (size_t)r * host_pitch, plane.data() + (size_t)r * hd_bytes, hd_bytes);
+    } else {
+      for (uint32_t r = 0; r < n_rows; r++) memcpy(plane.data() + (size_t)r * hd_bytes, h + (size_t)r * host_pitch, hd_bytes);
+      HIPCHK(ctx, hipMemcpy(d, plane.data(), plane.size(), hipMemcpyHostToDevice));
+    }
+  }
   return PA_OK;
 }
 extern "C" int pa_kv_read(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, void* h_dst) {
   if (!ctx) return PA_ERR_INVALID;
-  uint16_t* b; size_t n;
-  int rc = kv_rows(ctx, "pa_kv_read", layer, which, row0, n_rows, &b, &n);
-  return rc ? rc : pa_download(ctx, h_dst, b, n);
+  return kv_copy(ctx, "pa_kv_read", layer, which, row0, n_rows, h_dst, true);
 }
 extern "C" int pa_kv_write(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, const void* h_src) {
   if (!ctx) return PA_ERR_INVALID;
-  uint16_t* b; size_t n;
-  int rc = kv_rows(ctx, "pa_kv_write", layer, which, row0, n_rows, &b, &n);
-  return rc ? rc : pa_upload(ctx, b, h_src, n);
+  return kv_copy(ctx, "pa_kv_write", layer, which, row0, n_rows, const_cast<void*>(h_src), false);
 }
 extern "C" const void* pa_kv_device_ptr(pa_ctx* ctx, uint32_t layer, int which) {
   if (!ctx || layer >= ctx->cfg.n_layers) return nullptr;

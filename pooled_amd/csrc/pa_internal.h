@@ -15,7 +15,8 @@ struct GlueParams {
   const float* inv_freq;                                     // [n_rot/2] f32, theta^(-2i/n_rot)
   const float2* rope_tab;                                    // [max_seq][n_rot/2] (cos, sin) or nullptr
   float* q_out; float* gate_out;                             // [n_cols][nH*hd]
-  uint16_t* k_cache; uint16_t* v_cache;                      // f16 [max_seq][nKV*hd] or nullptr
+  uint16_t* k_cache; uint16_t* v_cache;                      // f16 [nKV][head_rows][hd] or nullptr
+  uint32_t head_rows;                                        // rows of one kv head's plane (max_seq + padding)
   uint32_t q_stride, k_stride, v_stride;
   uint32_t n_heads, n_kv_heads, head_dim, n_rot;
   uint32_t base_pos, n_cols;
