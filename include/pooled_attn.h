@@ -163,9 +163,10 @@ const void* pa_kv_device_ptr(pa_ctx* ctx, uint32_t layer, int which);
 /* ---- timing on the context's stream (HIP events; replaces the reference's timestamp-query passes,
  *      tests/prof/gpuprof.js:1-16) ----
  * pa_timer_start / pa_timer_stop bracket a region; stop blocks and returns milliseconds.
- * pa_profile_enable(1) additionally brackets every attention call's main kernel (the split-K or prefill
- * kernel, not glue / merge) with its own event pair; pa_profile_read blocks, returns the sum of those
- * durations and their count since the last read, and resets them. */
+ * pa_profile_enable(1) additionally times every attention call's main kernel (the split-K or prefill kernel, not
+ * glue / merge) with an event pair stamped by the dispatch itself (the kernel's own begin / end timestamps, the
+ * figure a kernel trace reports); pa_profile_read blocks, returns the sum of those durations and their count
+ * since the last read, and resets them. */
 int pa_timer_start(pa_ctx* ctx);
 int pa_timer_stop(pa_ctx* ctx, float* ms);
 int pa_profile_enable(pa_ctx* ctx, int on);

@@ -462,7 +462,7 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
 }
 
 template <int HD, int NB, int W, bool FUSED>
-static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s) {
+static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   typedef DecShape<HD> S;
   const size_t lds = 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float);
   static bool attr_set = false;
@@ -471,32 +471,32 @@ static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipS
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL((pa_decode_kernel<HD, NB, W, FUSED>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, p);
+  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
   return hipGetLastError();
 }
 
 template <int HD>
-static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t col_groups, hipStream_t s) {
+static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   switch (nb) {
-    case 1: return launch_decode_t<HD, 1, 4, false>(p, col_groups, s);
-    case 2: return launch_decode_t<HD, 2, 4, false>(p, col_groups, s);
-    case 3: return launch_decode_t<HD, 3, 4, false>(p, col_groups, s);
-    case 4: return launch_decode_t<HD, 4, 4, false>(p, col_groups, s);
+    case 1: return launch_decode_t<HD, 1, 4, false>(p, col_groups, s, t);
+    case 2: return launch_decode_t<HD, 2, 4, false>(p, col_groups, s, t);
+    case 3: return launch_decode_t<HD, 3, 4, false>(p, col_groups, s, t);
+    case 4: return launch_decode_t<HD, 4, 4, false>(p, col_groups, s, t);
     default: return hipErrorInvalidValue;
   }
 }
 
-hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s) {
+hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   if (waves != 4) return hipErrorInvalidValue;
-  if (hd == 256) return launch_decode_hd<256>(p, nb, col_groups, s);
-  if (hd == 128) return launch_decode_hd<128>(p, nb, col_groups, s);
+  if (hd == 256) return launch_decode_hd<256>(p, nb, col_groups, s, t);
+  if (hd == 128) return launch_decode_hd<128>(p, nb, col_groups, s, t);
   return hipErrorInvalidValue;
 }
 
-hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s) {
+hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t) {
   if (!p.f_q_in || p.n_cols != 1 || p.group > 16) return hipErrorInvalidValue;
-  if (hd == 256) return launch_decode_t<256, 1, 4, true>(p, 1, s);
-  if (hd == 128) return launch_decode_t<128, 1, 4, true>(p, 1, s);
+  if (hd == 256) return launch_decode_t<256, 1, 4, true>(p, 1, s, t);
+  if (hd == 128) return launch_decode_t<128, 1, 4, true>(p, 1, s, t);
   return hipErrorInvalidValue;
 }
 

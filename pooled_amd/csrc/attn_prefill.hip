@@ -447,7 +447,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 }
 
 template <int HD, int QB, int W, bool PP>
-static hipError_t launch_prefill_t(const AttnParams& p, uint32_t col_groups, hipStream_t s) {
+static hipError_t launch_prefill_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   typedef PfShape<HD, W> S;
   const size_t lds = (size_t)W * QB * (S::KS - S::QR) * 1024;     // Q fragments parked in LDS (dynamic part)
   static bool attr_set = false;
@@ -458,18 +458,18 @@ static hipError_t launch_prefill_t(const AttnParams& p, uint32_t col_groups, hip
   }
   const uint32_t total = col_groups * p.n_kv_heads;
   const uint32_t gx = ((total + 7) / 8) * 8;       // whole rounds of the 8 XCDs
-  hipLaunchKernelGGL((pa_prefill_kernel<HD, QB, W, PP>), dim3(gx, p.n_splits), dim3(W * 64), lds, s, p, col_groups);
+  PA_LAUNCH((pa_prefill_kernel<HD, QB, W, PP>), dim3(gx, p.n_splits), dim3(W * 64), lds, s, t, p, col_groups);
   return hipGetLastError();
 }
 
 // row_blocks = 32-row query blocks per wavefront (2); the workgroup covers 4 * row_blocks * 32 rows
-hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s) {
+hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   if (row_blocks != 2) return hipErrorNotSupported;
   // In-phase waves measure faster than the anti-phase schedule on MI355X (C5: 7.27 ms vs 7.77 ms): with one wave
   // of a SIMD alone on the MFMA pipe, every LDS fragment wait is exposed.  The anti-phase variant stays selectable
   // for measurements.
   static const bool anti_phase = getenv("POOLED_ATTN_PREFILL_ANTI_PHASE") != nullptr;
-  if (hd == 256) return anti_phase ? launch_prefill_t<256, 1, 8, true>(p, col_groups, s) : launch_prefill_t<256, 1, 8, false>(p, col_groups, s);
-  if (hd == 128) return anti_phase ? launch_prefill_t<128, 1, 8, true>(p, col_groups, s) : launch_prefill_t<128, 1, 8, false>(p, col_groups, s);
+  if (hd == 256) return anti_phase ? launch_prefill_t<256, 1, 8, true>(p, col_groups, s, t) : launch_prefill_t<256, 1, 8, false>(p, col_groups, s, t);
+  if (hd == 128) return anti_phase ? launch_prefill_t<128, 1, 8, true>(p, col_groups, s, t) : launch_prefill_t<128, 1, 8, false>(p, col_groups, s, t);
   return hipErrorNotSupported;
 }

@@ -394,7 +394,7 @@ __global__ __launch_bounds__(256, 1) void pa_prefill_wide_kernel(AttnParams p, u
 #endif
 
 template <int HD>
-static hipError_t launch_wide_t(const AttnParams& p, uint32_t col_groups, hipStream_t s) {
+static hipError_t launch_wide_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   typedef PwShape<HD, PW_QR> S;
   const size_t lds = (size_t)S::W * S::QB * (S::KS - S::QR) * 1024;     // Q fragments parked in LDS (dynamic part)
   static bool attr_set = false;
@@ -405,12 +405,12 @@ static hipError_t launch_wide_t(const AttnParams& p, uint32_t col_groups, hipStr
   }
   const uint32_t total = col_groups * p.n_kv_heads;
   const uint32_t gx = ((total + 7) / 8) * 8;
-  hipLaunchKernelGGL((pa_prefill_wide_kernel<HD, PW_QR>), dim3(gx, p.n_splits), dim3(256), lds, s, p, col_groups);
+  PA_LAUNCH((pa_prefill_wide_kernel<HD, PW_QR>), dim3(gx, p.n_splits), dim3(256), lds, s, t, p, col_groups);
   return hipGetLastError();
 }
 
-hipError_t pa_launch_prefill_wide(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s) {
-  if (hd == 256) return launch_wide_t<256>(p, col_groups, s);
-  if (hd == 128) return launch_wide_t<128>(p, col_groups, s);
+hipError_t pa_launch_prefill_wide(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
+  if (hd == 256) return launch_wide_t<256>(p, col_groups, s, t);
+  if (hd == 128) return launch_wide_t<128>(p, col_groups, s, t);
   return hipErrorNotSupported;
 }

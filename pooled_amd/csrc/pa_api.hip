@@ -343,17 +343,14 @@ static int ensure_partials(pa_ctx* ctx, uint32_t n_cols, uint32_t slots) {
   return PA_OK;
 }
 
-static int prof_begin(pa_ctx* ctx) {
+// an event pair for a kernel-exact timing of the next main-kernel launch (profiling on), else an empty PaTiming
+static int prof_pair(pa_ctx* ctx, PaTiming* t) {
+  *t = PaTiming();
   if (!ctx->profiling) return PA_OK;
   if (ctx->prof_used + 2 > ctx->prof_events.size()) {
     for (int i = 0; i < 2; i++) { hipEvent_t ev; HIPCHK(ctx, hipEventCreate(&ev)); ctx->prof_events.push_back(ev); }
   }
-  HIPCHK(ctx, hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream));
-  return PA_OK;
-}
-static int prof_end(pa_ctx* ctx) {
-  if (!ctx->profiling) return PA_OK;
-  HIPCHK(ctx, hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream));
+  t->start = ctx->prof_events[ctx->prof_used]; t->stop = ctx->prof_events[ctx->prof_used + 1];
   ctx->prof_used += 2;
   return PA_OK;
 }
@@ -389,11 +386,11 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   p.gate_head_stride = c.head_dim;
-  if ((rc = prof_begin(ctx))) return rc;
-  if (pl.kernel == 0) HIPCHK(ctx, pa_launch_decode(p, c.head_dim, pl.row_blocks, pl.waves, pl.col_groups, ctx->stream));
-  else if (getenv("POOLED_ATTN_PREFILL_WIDE")) HIPCHK(ctx, pa_launch_prefill_wide(p, c.head_dim, pl.col_groups, ctx->stream));
-  else HIPCHK(ctx, pa_launch_prefill(p, c.head_dim, pl.row_blocks, pl.col_groups, ctx->stream));
-  if ((rc = prof_end(ctx))) return rc;
+  PaTiming tm;
+  if ((rc = prof_pair(ctx, &tm))) return rc;
+  if (pl.kernel == 0) HIPCHK(ctx, pa_launch_decode(p, c.head_dim, pl.row_blocks, pl.waves, pl.col_groups, ctx->stream, &tm));
+  else if (getenv("POOLED_ATTN_PREFILL_WIDE")) HIPCHK(ctx, pa_launch_prefill_wide(p, c.head_dim, pl.col_groups, ctx->stream, &tm));
+  else HIPCHK(ctx, pa_launch_prefill(p, c.head_dim, pl.row_blocks, pl.col_groups, ctx->stream, &tm));
   if (!direct) HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;
 }
@@ -444,9 +441,9 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
   p.f_q_head_stride = c.head_dim * (gated ? 2 : 1); p.n_rot = c.n_rot; p.eps = c.eps;
   p.gate = gated ? d_q_in + c.head_dim : nullptr;
   p.gate_head_stride = p.f_q_head_stride;
-  if ((rc = prof_begin(ctx))) return rc;
-  HIPCHK(ctx, pa_launch_decode_step(p, c.head_dim, ctx->stream));
-  if ((rc = prof_end(ctx))) return rc;
+  PaTiming tm;
+  if ((rc = prof_pair(ctx, &tm))) return rc;
+  HIPCHK(ctx, pa_launch_decode_step(p, c.head_dim, ctx->stream, &tm));
   HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;
 }

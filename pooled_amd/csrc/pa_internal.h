@@ -1,6 +1,7 @@
 // Internal declarations shared by the host C ABI and the gfx950 kernels.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <string>
 #include <vector>
@@ -50,17 +51,27 @@ struct AttnParams {
 
 // ---- kernel launchers (defined next to their kernels) ------------------------------------------
 
+// Optional kernel-exact timing of a launch: with both events set the kernel goes out through hipExtLaunchKernelGGL,
+// which stamps them with the dispatch's own begin / end timestamps (the clock a kernel trace reports), so
+// hipEventElapsedTime(start, stop) is the kernel's duration without launch or event-handling latency.
+struct PaTiming { hipEvent_t start = nullptr, stop = nullptr; };
+#define PA_LAUNCH(kernel, grid, block, lds, stream, timing, ...)                                                          \
+  do {                                                                                                                    \
+    if ((timing) && (timing)->start) hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, (timing)->start, (timing)->stop, 0, __VA_ARGS__); \
+    else hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                                               \
+  } while (0)
+
 hipError_t pa_launch_glue(const GlueParams& p, hipStream_t s);
 hipError_t pa_launch_rope_table(float2* tab, const float* inv_freq, uint32_t half, uint32_t n_pos, hipStream_t s);
 // waves per workgroup W in {4, 8}; NB = 16-row query blocks per workgroup (1..4); hd in {128, 256}
-hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s);
+hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
 // the same with the pre-step of the one column fused in (p.f_* set; one 16-row block, n_cols == 1)
-hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s);
+hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t = nullptr);
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);
 // MFMA prefill; returns hipErrorNotSupported for shapes it does not cover
-hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s);
+hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
 // the 4-wave, 64-rows-per-wave software-pipelined variant (same contract)
-hipError_t pa_launch_prefill_wide(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s);
+hipError_t pa_launch_prefill_wide(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
 
 // ---- context -----------------------------------------------------------------------------------
 
