@@ -6,9 +6,10 @@
 // the reference runs as consecutive 16-column passes.
 //
 // Work decomposition
-//   * A workgroup (4 wavefronts, one per SIMD) owns one kv head and a block of columns; its 4 x 64 = 256 query
-//     rows are (column, head-in-group) pairs, so every K/V tile it stages serves all G heads of the group
-//     (the reference's "up to 64 rows share a tile", scaled to the MFMA shape).
+//   * A workgroup owns one kv head and a block of columns; its 256 query rows are (column, head-in-group) pairs,
+//     so every K/V tile it stages serves all G heads of the group (the reference's "up to 64 rows share a tile",
+//     scaled to the MFMA shape).  8 wavefronts x 32 rows, two per SIMD: while one wave of a SIMD does its softmax
+//     on the VALU the other one's MFMAs keep the matrix pipe busy.
 //   * K/V tiles of 32 positions go global -> LDS directly (global_load_lds_dwordx4: no staging registers),
 //     double buffered, one barrier a step; the next tile's loads are in flight while the current one is consumed.
 //     An LDS-direct load writes 64 lanes x 16 B contiguously, so rows cannot be padded; bank conflicts are
@@ -17,12 +18,12 @@
 //     c ^ 4 (r & 3) (2-way = optimal ds_read_b64_tr_b16).  Rows at or past the end of the context are fetched
 //     from the cache's zero padding row instead, so 0 x stale bits never reaches O.
 //   * S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_f16.  Q fragments stay in registers for the whole
-//     kernel; K fragments are ds_read_b128, V^T fragments come from the gfx950 LDS transpose read
+//     kernel (at hd 256 half of them, the other half is parked in LDS); K fragments are ds_read_b128, V^T fragments come from the gfx950 LDS transpose read
 //     (ds_read_b64_tr_b16).  The S^T accumulator layout (lane = query row, 16 positions) is the B-operand
 //     layout of the PV product, so P never leaves registers.
 //   * Online softmax in f32 in the exp2 domain with a lazily updated reference maximum: O and l are rescaled
 //     only when some row's maximum grows by more than 2^8, which keeps exp2(x - m_ref) <= 256 (exact enough
-//     in f16) and takes the 256-register O rescale off the common path.
+//     in f16) and takes the 128-register O rescale off the common path.
 //   * Workgroup ids are remapped so that each XCD (ids are dealt round-robin to the 8 XCDs) works on one
 //     contiguous range of (kv head, column block): the K/V stream of a kv head is fetched into one L2.
 //   * Optional split over the context (short chunks on long contexts would otherwise leave CUs idle): partial
@@ -462,9 +463,9 @@ static hipError_t launch_prefill_t(const AttnParams& p, uint32_t col_groups, hip
   return hipGetLastError();
 }
 
-// row_blocks = 32-row query blocks per wavefront (2); the workgroup covers 4 * row_blocks * 32 rows
+// row_blocks = 32-row query blocks per workgroup (8: one per wavefront)
 hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
-  if (row_blocks != 2) return hipErrorNotSupported;
+  if (row_blocks != 8) return hipErrorNotSupported;
   // In-phase waves measure faster than the anti-phase schedule on MI355X (C5: 7.27 ms vs 7.77 ms): with one wave
   // of a SIMD alone on the MFMA pipe, every LDS fragment wait is exposed.  The anti-phase variant stays selectable
   // for measurements.

@@ -290,7 +290,7 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   return PA_OK;
 }
 
-// Prefill (MFMA kernel): a workgroup is 4 wavefronts x 64 query rows = 256 rows of one kv head, i.e.
+// Prefill (MFMA kernel): a workgroup is 8 wavefronts x 32 query rows = 256 rows of one kv head, i.e.
 // floor(256 / G) columns x G heads.  Chunks wide enough to give every CU a workgroup run unsplit and write the
 // output directly; narrower chunks are also split over the context (partials + merge kernel) until about two
 // workgroups per CU exist.  Chunks of fewer rows than one wavefront tile go to the split-K decode kernel.
@@ -308,7 +308,7 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
   if (base_wgs < (uint32_t)ctx->n_cu) splits = std::min(ceil_div(2 * (uint32_t)ctx->n_cu, base_wgs), std::max(1u, seq_max / 256));
   uint32_t sl = ceil_div(ceil_div(seq_max, splits), 32) * 32;
   pl->kernel = 1; pl->split_len = sl; pl->n_splits = ceil_div(seq_max, sl);
-  pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = 4; pl->row_blocks = 2; pl->slots = pl->n_splits;
+  pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = 8; pl->row_blocks = 8; pl->slots = pl->n_splits;
   return PA_OK;
 }
 
