@@ -184,6 +184,8 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (configuration 5) leg")
     ap.add_argument("--unfused", action="store_true", help="decode step as three launches (pa_glue_kv + pa_attn_decode) instead of the fused pa_attn_decode_step")
     ap.add_argument("--prefill-steps", type=int, default=5)
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="only run the device probe: sustained f16 MFMA TFLOP/s and shader clock with constant and with random operands")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 10 device-to-device copies of 256 MiB (the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -194,6 +196,20 @@ def main():
     from pooled_amd.capi import PooledAttn, PA_OUT_F16, load
     L = load()
     log("library:", L.pa_version().decode())
+    if args.mfma_probe:
+        # what the f16 matrix pipe sustains on this part, and at which clock: constant vs random operands, after a
+        # warm-up long enough for the clock to settle
+        pa = PooledAttn(C3, 64, n_layers=1, max_cols=1)
+        res = {}
+        for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+            for _ in range(3):
+                pa.mfma_probe(rnd, 20000)
+            tf, mhz = pa.mfma_probe(rnd, 60000)
+            res[name] = dict(tflops=round(tf, 1), shader_mhz=round(mhz), frac_of_nominal_peak=round(tf / MFMA_F16_PEAK_TFLOPS, 3))
+            log("mfma probe, %s: %.0f TFLOP/s at %.0f MHz" % (name, tf, mhz))
+        pa.close()
+        print(json.dumps({"mfma_probe": res}))
+        return
     if args.copy_calibration:
         pa = PooledAttn(C3, 64, n_layers=1, max_cols=1)
         nbytes = 256 << 20

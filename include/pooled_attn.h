@@ -172,6 +172,14 @@ int pa_timer_stop(pa_ctx* ctx, float* ms);
 int pa_profile_enable(pa_ctx* ctx, int on);
 int pa_profile_read(pa_ctx* ctx, float* ms_sum, uint32_t* count);
 
+/* Device probe (measurement infrastructure, no counterpart in the reference): runs back-to-back
+ * v_mfma_f32_32x32x16_f16 on every CU for iters x 64 instructions per wavefront, with constant operands
+ * (random_operands = 0) or random f16 fragments, and returns the achieved TFLOP/s and the mean shader clock during
+ * the kernel (shader clock counter against the 100 MHz wall clock).  Blocks until done.  It tells what the matrix
+ * pipe of this part sustains under its power limit, which is what an MFMA-bound kernel's roofline fraction has to
+ * be read against. */
+int pa_mfma_probe(pa_ctx* ctx, int random_operands, uint32_t iters, float* tflops, float* shader_mhz);
+
 /* library / device description, e.g. "pooled_attn 0.1 gfx950 256CU" (static storage) */
 const char* pa_version(void);
 

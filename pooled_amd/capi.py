@@ -59,6 +59,7 @@ SYMBOLS = {
     "pa_timer_stop": (c_int, [vp, ctypes.POINTER(ctypes.c_float)]),
     "pa_profile_enable": (c_int, [vp, c_int]),
     "pa_profile_read": (c_int, [vp, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(u32)]),
+    "pa_mfma_probe": (c_int, [vp, c_int, u32, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]),
     "pa_version": (ctypes.c_char_p, []),
 }
 
@@ -241,6 +242,12 @@ class PooledAttn:
         ms, n = ctypes.c_float(), u32()
         self._chk(self.L.pa_profile_read(self.ctx, ctypes.byref(ms), ctypes.byref(n)))
         return ms.value, n.value
+
+    def mfma_probe(self, random_operands, iters):
+        """(TFLOP/s, shader MHz) of back-to-back f16 MFMAs on every CU with constant or random operands."""
+        tf, mhz = ctypes.c_float(), ctypes.c_float()
+        self._chk(self.L.pa_mfma_probe(self.ctx, int(bool(random_operands)), iters, ctypes.byref(tf), ctypes.byref(mhz)))
+        return tf.value, mhz.value
 
     # ---- numpy convenience used by tests / smoke: whole passes from host arrays ----
     def run_glue_kv(self, layer, q_in, k_in, v_in, qw, kw, base_pos):

@@ -505,6 +505,11 @@ extern "C" int pa_timer_stop(pa_ctx* ctx, float* ms) {
   HIPCHK(ctx, hipEventElapsedTime(ms, ctx->t0, ctx->t1));
   return PA_OK;
 }
+extern "C" int pa_mfma_probe(pa_ctx* ctx, int random_operands, uint32_t iters, float* tflops, float* shader_mhz) {
+  if (!ctx || !tflops || !shader_mhz || iters == 0) return PA_ERR_INVALID;
+  HIPCHK(ctx, pa_run_mfma_probe(ctx->n_cu, random_operands != 0, iters, ctx->stream, tflops, shader_mhz));
+  return PA_OK;
+}
 extern "C" int pa_profile_enable(pa_ctx* ctx, int on) {
   if (!ctx) return PA_ERR_INVALID;
   ctx->profiling = on != 0;

@@ -73,6 +73,9 @@ hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_bloc
 // the 4-wave, 64-rows-per-wave software-pipelined variant (same contract)
 hipError_t pa_launch_prefill_wide(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
 
+// device probe (probe.hip): sustained f16 MFMA rate and shader clock, constant or random operands
+hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, uint32_t iters, hipStream_t st, float* tflops, float* shader_mhz);
+
 // ---- context -----------------------------------------------------------------------------------
 
 struct pa_layer { uint16_t* k = nullptr; uint16_t* v = nullptr; };
