@@ -160,6 +160,25 @@ int pa_kv_write(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t 
 /* device address of a cache (read-only use; the head-major device layout described at pa_layer_alloc) */
 const void* pa_kv_device_ptr(pa_ctx* ctx, uint32_t layer, int which);
 
+/* ---- checkpoint slots: the rows written so far, kept on the device or moved to the host ----
+ * Replace the engines' saveSlot / loadSlot / dropSlot (engine/dense.js:20-47, engine/qwen35.js:190-230: a copy of
+ * KV rows [0, pos) per layer, made and restored on the GPU queue) and, for the attention layers, the parts of
+ * exportSlot / exportState / importState (engine/qwen35.js:121-131, :151-190): per layer one K and one V part of
+ * pos * nKV * hd f16, position-major -- the reference's flash-KV part layout, so parts written by either backend
+ * load into the other.  slot is a caller-chosen id (the shim maps names to ids).
+ * pa_slot_save: device copy of rows [0, pos) of every allocated layer, queued on the context's stream (a slot of the
+ *   same id is replaced); pa_slot_load: the copy back, *pos = the saved position; pa_slot_drop frees (unknown id:
+ *   no error, as dropSlot); pa_slot_pos: the saved position.
+ * pa_slot_create + pa_slot_import build a slot from host parts (then pa_slot_load restores it);
+ * pa_slot_export reads one part back.  Host copies block. */
+int pa_slot_save(pa_ctx* ctx, uint32_t slot, uint32_t pos);
+int pa_slot_load(pa_ctx* ctx, uint32_t slot, uint32_t* pos);
+int pa_slot_drop(pa_ctx* ctx, uint32_t slot);
+int pa_slot_pos(pa_ctx* ctx, uint32_t slot, uint32_t* pos);
+int pa_slot_create(pa_ctx* ctx, uint32_t slot, uint32_t pos);
+int pa_slot_export(pa_ctx* ctx, uint32_t slot, uint32_t layer, int which, void* h_dst);
+int pa_slot_import(pa_ctx* ctx, uint32_t slot, uint32_t layer, int which, const void* h_src);
+
 /* ---- timing on the context's stream (HIP events; replaces the reference's timestamp-query passes,
  *      tests/prof/gpuprof.js:1-16) ----
  * pa_timer_start / pa_timer_stop bracket a region; stop blocks and returns milliseconds.

@@ -59,6 +59,13 @@ SYMBOLS = {
     "pa_timer_stop": (c_int, [vp, ctypes.POINTER(ctypes.c_float)]),
     "pa_profile_enable": (c_int, [vp, c_int]),
     "pa_profile_read": (c_int, [vp, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(u32)]),
+    "pa_slot_save": (c_int, [vp, u32, u32]),
+    "pa_slot_load": (c_int, [vp, u32, ctypes.POINTER(u32)]),
+    "pa_slot_drop": (c_int, [vp, u32]),
+    "pa_slot_pos": (c_int, [vp, u32, ctypes.POINTER(u32)]),
+    "pa_slot_create": (c_int, [vp, u32, u32]),
+    "pa_slot_export": (c_int, [vp, u32, u32, c_int, vp]),
+    "pa_slot_import": (c_int, [vp, u32, u32, c_int, vp]),
     "pa_mfma_probe": (c_int, [vp, c_int, u32, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]),
     "pa_version": (ctypes.c_char_p, []),
 }
@@ -242,6 +249,36 @@ class PooledAttn:
         ms, n = ctypes.c_float(), u32()
         self._chk(self.L.pa_profile_read(self.ctx, ctypes.byref(ms), ctypes.byref(n)))
         return ms.value, n.value
+
+    # ---- checkpoint slots ----
+    def slot_save(self, slot, pos):
+        self._chk(self.L.pa_slot_save(self.ctx, slot, pos))
+
+    def slot_load(self, slot):
+        pos = u32()
+        self._chk(self.L.pa_slot_load(self.ctx, slot, ctypes.byref(pos)))
+        return pos.value
+
+    def slot_drop(self, slot):
+        self._chk(self.L.pa_slot_drop(self.ctx, slot))
+
+    def slot_pos(self, slot):
+        pos = u32()
+        self._chk(self.L.pa_slot_pos(self.ctx, slot, ctypes.byref(pos)))
+        return pos.value
+
+    def slot_create(self, slot, pos):
+        self._chk(self.L.pa_slot_create(self.ctx, slot, pos))
+
+    def slot_export(self, slot, layer, which):
+        """One part as f16 bits [pos, nKV * hd] (position-major)."""
+        out = np.empty((self.slot_pos(slot), self.cfg["n_kv_heads"] * self.cfg["head_dim"]), dtype=np.uint16)
+        self._chk(self.L.pa_slot_export(self.ctx, slot, layer, which, out.ctypes.data))
+        return out
+
+    def slot_import(self, slot, layer, which, part):
+        part = np.ascontiguousarray(part, dtype=np.uint16)
+        self._chk(self.L.pa_slot_import(self.ctx, slot, layer, which, part.ctypes.data))
 
     def mfma_probe(self, random_operands, iters):
         """(TFLOP/s, shader MHz) of back-to-back f16 MFMAs on every CU with constant or random operands."""

@@ -90,10 +90,13 @@ extern "C" int pa_create(const pa_config* cfg, pa_ctx** out) {
   return PA_OK;
 }
 
+static void slot_free(pa_slot& sl);
+
 extern "C" int pa_destroy(pa_ctx* ctx) {
   if (!ctx) return PA_OK;
   if (ctx->own_stream) (void)hipStreamSynchronize(ctx->own_stream);
   for (auto& L : ctx->layers) { if (L.k) (void)hipFree(L.k); if (L.v) (void)hipFree(L.v); }
+  for (auto& kv : ctx->slots) slot_free(kv.second);
   if (ctx->q_buf) (void)hipFree(ctx->q_buf);
   if (ctx->gate_buf) (void)hipFree(ctx->gate_buf);
   if (ctx->inv_freq) (void)hipFree(ctx->inv_freq);
@@ -486,6 +489,135 @@ extern "C" int pa_kv_write(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0
   if (!ctx) return PA_ERR_INVALID;
   return kv_copy(ctx, "pa_kv_write", layer, which, row0, n_rows, const_cast<void*>(h_src), false);
 }
+// ---- checkpoint slots ---------------------------------------------------------------------------------
+// Device-side copies of the rows written so far (the reference's saveSlot / loadSlot / dropSlot:
+// engine/dense.js:20-47, engine/qwen35.js:190-230) and their host form (exportSlot / importState parts:
+// engine/qwen35.js:121-131, :151-190): per layer one K part and one V part of pos * kvDim f16, position-major.
+
+static void slot_free(pa_slot& sl) {
+  for (auto p : sl.k) if (p) (void)hipFree(p);
+  for (auto p : sl.v) if (p) (void)hipFree(p);
+  sl.k.clear(); sl.v.clear(); sl.pos = 0;
+}
+
+// a slot with room for rows [0, pos) of every allocated layer (contents undefined)
+static int slot_make(pa_ctx* ctx, const char* who, uint32_t slot, uint32_t pos) {
+  if (pos > ctx->cfg.max_seq) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": pos exceeds max_seq");
+  auto it = ctx->slots.find(slot);
+  if (it != ctx->slots.end() && it->second.pos == pos && it->second.k.size() == ctx->layers.size()) {
+    bool same = true;                                   // same shape: the buffers are reused (the stream orders the copies)
+    for (size_t l = 0; l < ctx->layers.size(); l++) same = same && ((ctx->layers[l].k != nullptr && pos != 0) == (it->second.k[l] != nullptr));
+    if (same) return PA_OK;
+  }
+  if (it != ctx->slots.end()) {
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));     // copies out of the old buffers may still be queued
+    slot_free(it->second); ctx->slots.erase(it);
+  }
+  pa_slot sl; sl.pos = pos;
+  sl.k.assign(ctx->layers.size(), nullptr); sl.v.assign(ctx->layers.size(), nullptr);
+  const size_t bytes = (size_t)pos * ctx->cfg.n_kv_heads * ctx->cfg.head_dim * 2;
+  for (size_t l = 0; l < ctx->layers.size() && bytes; l++) {
+    if (!ctx->layers[l].k) continue;
+    hipError_t e = hipMalloc((void**)&sl.k[l], bytes);
+    if (e == hipSuccess) e = hipMalloc((void**)&sl.v[l], bytes);
+    if (e != hipSuccess) { slot_free(sl); return fail_hip(ctx, e, "slot allocation"); }
+  }
+  ctx->slots[slot] = std::move(sl);
+  return PA_OK;
+}
+
+// rows [0, pos) of one tensor between the cache ([nKV][max_seq + 32][hd]) and a slot ([nKV][pos][hd]): one pitched copy
+static hipError_t slot_copy(const pa_ctx* ctx, uint16_t* cache, uint16_t* slot_buf, uint32_t pos, bool to_slot) {
+  const size_t plane = (size_t)pos * ctx->cfg.head_dim * 2, cache_pitch = ((size_t)ctx->cfg.max_seq + 32) * ctx->cfg.head_dim * 2;
+  return to_slot ? hipMemcpy2DAsync(slot_buf, plane, cache, cache_pitch, plane, ctx->cfg.n_kv_heads, hipMemcpyDeviceToDevice, ctx->stream)
+                 : hipMemcpy2DAsync(cache, cache_pitch, slot_buf, plane, plane, ctx->cfg.n_kv_heads, hipMemcpyDeviceToDevice, ctx->stream);
+}
+
+extern "C" int pa_slot_save(pa_ctx* ctx, uint32_t slot, uint32_t pos) {
+  if (!ctx) return PA_ERR_INVALID;
+  int rc = slot_make(ctx, "pa_slot_save", slot, pos);
+  if (rc) return rc;
+  pa_slot& sl = ctx->slots[slot];
+  for (size_t l = 0; l < ctx->layers.size(); l++) {
+    if (!sl.k[l]) continue;
+    HIPCHK(ctx, slot_copy(ctx, ctx->layers[l].k, sl.k[l], pos, true));
+    HIPCHK(ctx, slot_copy(ctx, ctx->layers[l].v, sl.v[l], pos, true));
+  }
+  return PA_OK;
+}
+
+extern "C" int pa_slot_load(pa_ctx* ctx, uint32_t slot, uint32_t* pos) {
+  if (!ctx || !pos) return PA_ERR_INVALID;
+  auto it = ctx->slots.find(slot);
+  if (it == ctx->slots.end()) return fail(ctx, PA_ERR_INVALID, "pa_slot_load: no saved slot " + std::to_string(slot));
+  pa_slot& sl = it->second;
+  for (size_t l = 0; l < ctx->layers.size(); l++) {
+    if (l >= sl.k.size() || !sl.k[l]) continue;
+    if (!ctx->layers[l].k) return fail(ctx, PA_ERR_INVALID, "pa_slot_load: the slot holds a layer that has no cache now");
+    HIPCHK(ctx, slot_copy(ctx, ctx->layers[l].k, sl.k[l], sl.pos, false));
+    HIPCHK(ctx, slot_copy(ctx, ctx->layers[l].v, sl.v[l], sl.pos, false));
+  }
+  *pos = sl.pos;
+  return PA_OK;
+}
+
+extern "C" int pa_slot_drop(pa_ctx* ctx, uint32_t slot) {
+  if (!ctx) return PA_ERR_INVALID;
+  auto it = ctx->slots.find(slot);
+  if (it == ctx->slots.end()) return PA_OK;               // as dropSlot: dropping an unknown slot is not an error
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  slot_free(it->second); ctx->slots.erase(it);
+  return PA_OK;
+}
+
+extern "C" int pa_slot_pos(pa_ctx* ctx, uint32_t slot, uint32_t* pos) {
+  if (!ctx || !pos) return PA_ERR_INVALID;
+  auto it = ctx->slots.find(slot);
+  if (it == ctx->slots.end()) return fail(ctx, PA_ERR_INVALID, "pa_slot_pos: no saved slot " + std::to_string(slot));
+  *pos = it->second.pos;
+  return PA_OK;
+}
+
+extern "C" int pa_slot_create(pa_ctx* ctx, uint32_t slot, uint32_t pos) {
+  if (!ctx) return PA_ERR_INVALID;
+  return slot_make(ctx, "pa_slot_create", slot, pos);
+}
+
+// one part between a slot and the host, position-major [pos][nKV * hd] on the host side
+static int slot_part(pa_ctx* ctx, const char* who, uint32_t slot, uint32_t layer, int which, void* host, bool to_host) {
+  auto it = ctx->slots.find(slot);
+  if (it == ctx->slots.end()) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": no saved slot " + std::to_string(slot));
+  pa_slot& sl = it->second;
+  if (which != 0 && which != 1) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": which must be 0 (K) or 1 (V)");
+  if (sl.pos == 0) return PA_OK;
+  if (layer >= sl.k.size() || !sl.k[layer]) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": the slot has no such layer");
+  if (!host) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null host buffer");
+  const pa_config& c = ctx->cfg;
+  const size_t hd_bytes = (size_t)c.head_dim * 2, host_pitch = hd_bytes * c.n_kv_heads, plane_bytes = (size_t)sl.pos * hd_bytes;
+  unsigned char* dev = (unsigned char*)(which ? sl.v[layer] : sl.k[layer]);
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  std::vector<unsigned char> plane(plane_bytes);
+  for (uint32_t g = 0; g < c.n_kv_heads; g++) {
+    unsigned char* h = (unsigned char*)host + (size_t)g * hd_bytes;
+    if (to_host) {
+      HIPCHK(ctx, hipMemcpy(plane.data(), dev + g * plane_bytes, plane_bytes, hipMemcpyDeviceToHost));
+      for (uint32_t r = 0; r < sl.pos; r++) memcpy(h + (size_t)r * host_pitch, plane.data() + (size_t)r * hd_bytes, hd_bytes);
+    } else {
+      for (uint32_t r = 0; r < sl.pos; r++) memcpy(plane.data() + (size_t)r * hd_bytes, h + (size_t)r * host_pitch, hd_bytes);
+      HIPCHK(ctx, hipMemcpy(dev + g * plane_bytes, plane.data(), plane_bytes, hipMemcpyHostToDevice));
+    }
+  }
+  return PA_OK;
+}
+extern "C" int pa_slot_export(pa_ctx* ctx, uint32_t slot, uint32_t layer, int which, void* h_dst) {
+  if (!ctx) return PA_ERR_INVALID;
+  return slot_part(ctx, "pa_slot_export", slot, layer, which, h_dst, true);
+}
+extern "C" int pa_slot_import(pa_ctx* ctx, uint32_t slot, uint32_t layer, int which, const void* h_src) {
+  if (!ctx) return PA_ERR_INVALID;
+  return slot_part(ctx, "pa_slot_import", slot, layer, which, const_cast<void*>(h_src), false);
+}
+
 extern "C" const void* pa_kv_device_ptr(pa_ctx* ctx, uint32_t layer, int which) {
   if (!ctx || layer >= ctx->cfg.n_layers) return nullptr;
   return which ? (const void*)ctx->layers[layer].v : (const void*)ctx->layers[layer].k;

@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <string>
 #include <vector>
+#include <map>
 #include "../../include/pooled_attn.h"
 
 // ---- kernel-side parameter blocks -------------------------------------------------------------
@@ -80,6 +81,12 @@ hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, uint32_t iters, hip
 
 struct pa_layer { uint16_t* k = nullptr; uint16_t* v = nullptr; };
 
+// A checkpoint slot: per allocated layer a compact head-major copy [nKV][pos][hd] of K and of V rows [0, pos).
+struct pa_slot {
+  uint32_t pos = 0;
+  std::vector<uint16_t*> k, v;     // indexed by layer; nullptr for layers without a cache (or pos == 0)
+};
+
 struct pa_ctx {
   pa_config cfg{};
   int device = 0;
@@ -87,6 +94,7 @@ struct pa_ctx {
   hipStream_t own_stream = nullptr;
   hipStream_t stream = nullptr;
   std::vector<pa_layer> layers;
+  std::map<uint32_t, pa_slot> slots;
   float* q_buf = nullptr;       // [max_cols][nH*hd]
   float* gate_buf = nullptr;    // [max_cols][nH*hd]
   float* inv_freq = nullptr;    // [n_rot/2]

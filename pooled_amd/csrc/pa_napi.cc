@@ -181,6 +181,22 @@ static napi_value ProfileRead(napi_env env, napi_callback_info info) {
   napi_value o; NAPI_OK(napi_create_object(env, &o)); napi_set_named_property(env, o, "ms", num_value(env, ms)); napi_set_named_property(env, o, "count", num_value(env, n)); return o;
 }
 
+// ---- checkpoint slots: slotSave(ctx, id, pos), slotLoad(ctx, id) -> pos, slotDrop(ctx, id), slotPos(ctx, id) -> pos,
+//      slotCreate(ctx, id, pos), slotExport(ctx, id, layer, which, Uint16Array), slotImport(ctx, id, layer, which, Uint16Array)
+static napi_value SlotSave(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1), pos = a.u32(2); CHECK_ARGS("slotSave"); int rc = pa_slot_save(c, id, pos); if (rc) return throw_pa(env, c, rc, "pa_slot_save"); return undefined(env); }
+static napi_value SlotLoad(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1); CHECK_ARGS("slotLoad"); uint32_t pos = 0; int rc = pa_slot_load(c, id, &pos); if (rc) return throw_pa(env, c, rc, "pa_slot_load"); return num_value(env, pos); }
+static napi_value SlotDrop(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1); CHECK_ARGS("slotDrop"); int rc = pa_slot_drop(c, id); if (rc) return throw_pa(env, c, rc, "pa_slot_drop"); return undefined(env); }
+static napi_value SlotPos(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1); CHECK_ARGS("slotPos"); uint32_t pos = 0; int rc = pa_slot_pos(c, id, &pos); if (rc) return throw_pa(env, c, rc, "pa_slot_pos"); return num_value(env, pos); }
+static napi_value SlotCreate(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1), pos = a.u32(2); CHECK_ARGS("slotCreate"); int rc = pa_slot_create(c, id, pos); if (rc) return throw_pa(env, c, rc, "pa_slot_create"); return undefined(env); }
+static napi_value SlotExport(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1), layer = a.u32(2); int which = (int)a.u32(3); size_t n; void* h = a.host(4, &n); CHECK_ARGS("slotExport");
+  int rc = pa_slot_export(c, id, layer, which, h); if (rc) return throw_pa(env, c, rc, "pa_slot_export"); return undefined(env);
+}
+static napi_value SlotImport(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1), layer = a.u32(2); int which = (int)a.u32(3); size_t n; void* h = a.host(4, &n); CHECK_ARGS("slotImport");
+  int rc = pa_slot_import(c, id, layer, which, h); if (rc) return throw_pa(env, c, rc, "pa_slot_import"); return undefined(env);
+}
+
 static napi_value Init(napi_env env, napi_value exports) {
   struct { const char* name; napi_callback fn; } table[] = {
     {"create", Create}, {"destroy", Destroy}, {"lastError", LastError}, {"version", Version}, {"layerAlloc", LayerAlloc}, {"sync", Sync},
@@ -188,7 +204,8 @@ static napi_value Init(napi_env env, napi_value exports) {
     {"kvStore", KvStore}, {"qBuffer", QBuffer}, {"gateBuffer", GateBuffer}, {"attn", Attn}, {"planQuery", PlanQuery},
     {"setDecodeSplits", SetDecodeSplits}, {"kvRead", KvRead}, {"kvWrite", KvWrite}, {"kvDevicePtr", KvDevicePtr}, {"timerStart", TimerStart},
     {"timerStop", TimerStop}, {"profileEnable", ProfileEnable}, {"profileRead", ProfileRead}, {"attnDecodeStep", AttnDecodeStep},
-    {"copyD2d", CopyD2d},
+    {"copyD2d", CopyD2d}, {"slotSave", SlotSave}, {"slotLoad", SlotLoad}, {"slotDrop", SlotDrop}, {"slotPos", SlotPos},
+    {"slotCreate", SlotCreate}, {"slotExport", SlotExport}, {"slotImport", SlotImport},
   };
   for (auto& t : table) {
     napi_value fn;

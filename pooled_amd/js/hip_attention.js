@@ -125,6 +125,50 @@ class HipAttention {
   sync() { addon.sync(this.ctx); }
   plan(kind, basePos, nCols) { return addon.planQuery(this.ctx, kind === "prefill" ? 1 : 0, basePos, nCols); }
 
+  // ---- session state: the engines' saveSlot / loadSlot / dropSlot (engine/dense.js:20-47, engine/qwen35.js:190-230)
+  //      and the attention layers' share of exportSlot / importState (engine/qwen35.js:121-131, :151-190) ----
+  // this.pos is the number of rows written so far, as in the engines; the callers keep it (the shim's attention
+  // methods take positions as arguments and do not advance it).
+  _slotId(name, make) {
+    this._slotIds = this._slotIds || new Map();
+    if (!this._slotIds.has(name) && make) this._slotIds.set(name, this._slotNext = (this._slotNext || 0) + 1);
+    return this._slotIds.get(name);
+  }
+  saveSlot(name) { addon.slotSave(this.ctx, this._slotId(name, true), this.pos); }
+  loadSlot(name) {
+    const id = this._slotId(name, false);
+    if (id === undefined) throw new Error("no saved slot " + name);
+    this.pos = addon.slotLoad(this.ctx, id);
+  }
+  dropSlot(name) { const id = this._slotId(name, false); if (id !== undefined) { addon.slotDrop(this.ctx, id); this._slotIds.delete(name); } }
+  dropAllSlots() { for (const k of Array.from((this._slotIds || new Map()).keys())) this.dropSlot(k); }
+  // what a saved state must match to be loaded here (the attention-relevant fields of engine/qwen35.js:133-143)
+  stateSignature() { return { v: 1, layers: this.layers.length, flash: true, kvQ8: false, dims: [this.dims.kvDim] }; }
+  // { sig, pos, parts: [ArrayBuffer] }: per layer a K part and a V part of pos * kvDim f16, position-major
+  exportSlot(name) {
+    const id = this._slotId(name, false);
+    if (id === undefined) throw new Error("no saved slot " + name);
+    const pos = addon.slotPos(this.ctx, id), parts = [];
+    for (let l = 0; l < this.layers.length; l++) for (let w = 0; w < 2; w++) {
+      const a = new Uint16Array(pos * this.dims.kvDim);
+      if (pos) addon.slotExport(this.ctx, id, l, w, a);
+      parts.push(a.buffer);
+    }
+    return { sig: this.stateSignature(), pos: pos, parts: parts };
+  }
+  exportState() { this.saveSlot("__export"); try { return this.exportSlot("__export"); } finally { this.dropSlot("__export"); } }
+  importState(st) {
+    if (JSON.stringify(st.sig) !== JSON.stringify(this.stateSignature())) throw new Error("saved state is for a different model, layer range or KV format");
+    const bytes = st.pos * this.dims.kvDim * 2;
+    if (st.parts.length !== 2 * this.layers.length || st.parts.some((p) => p.byteLength !== bytes)) throw new Error("saved state has the wrong shape");
+    const id = this._slotId("__import", true);
+    addon.slotCreate(this.ctx, id, st.pos);
+    try {
+      if (st.pos) st.parts.forEach((p, i) => addon.slotImport(this.ctx, id, i >> 1, i & 1, new Uint16Array(p)));
+      this.pos = addon.slotLoad(this.ctx, id);
+    } finally { this.dropSlot("__import"); }
+  }
+
   _norms(L) { return [L.qNorm || this._ones, L.kNorm || this._ones]; }
   _strideF(b) { return b.stride / 4; }
   _outStride() { return this.outDtype === PA_OUT_F32 ? this.B.attnOut.stride / 4 : this.B.attnOut.stride / 2; }

@@ -3,6 +3,7 @@
 //   1. a full-width pass (prefill kernel)            _encAttnGlue + _encAttnCore
 //   2. the same columns as a verify pass (decode kernel, snapshot set)
 //   3. one token at a time                            encodeLayerAttn
+//   4. session state                                  saveSlot / loadSlot / dropSlot / exportSlot / importState
 // against the expected values (max-abs 2e-3, rel 1e-2) and the written KV rows bit for bit.
 "use strict";
 const fs = require("fs"), path = require("path");
@@ -56,6 +57,25 @@ check("token by token (fused glue + decode)", flat(outs), expect);
 if (!eqBits(A.kvRead(0, 0, base, n), kNew)) { console.log("KV rows written token by token differ FAIL"); fails++; }
 // error path: a readable throw, not an abort
 try { A.encodeLayerAttn(null, 0, base + n); console.log("out-of-range position did not throw FAIL"); fails++; } catch (e) { if (!/max_seq/.test(e.message)) { console.log("unexpected error text: " + e.message + " FAIL"); fails++; } }
+// 4. session state: slot save / overwrite / load, export / import (saveSlot, loadSlot, exportSlot, importState)
+{
+  const rowsK = A.kvRead(0, 0, 0, base + n), rowsV = A.kvRead(0, 1, 0, base + n);
+  A.pos = base + n;
+  A.saveSlot("turn1");
+  const st = A.exportSlot("turn1");
+  if (st.pos !== base + n || st.parts.length !== 2 || !eqBits(new Uint16Array(st.parts[0]), rowsK) || !eqBits(new Uint16Array(st.parts[1]), rowsV)) { console.log("exportSlot parts differ from the cache rows FAIL"); fails++; }
+  A.kvWrite(0, 0, 0, new Uint16Array(rowsK.length).fill(0x7e00)); A.kvWrite(0, 1, 0, new Uint16Array(rowsV.length).fill(0x7e00));
+  A.pos = 0;
+  A.loadSlot("turn1");
+  if (A.pos !== base + n || !eqBits(A.kvRead(0, 0, 0, base + n), rowsK) || !eqBits(A.kvRead(0, 1, 0, base + n), rowsV)) { console.log("loadSlot did not restore the rows FAIL"); fails++; }
+  A.kvWrite(0, 0, 0, new Uint16Array(rowsK.length).fill(0x7e00));
+  A.importState(st);
+  if (A.pos !== base + n || !eqBits(A.kvRead(0, 0, 0, base + n), rowsK)) { console.log("importState did not restore the rows FAIL"); fails++; }
+  A.dropSlot("turn1");
+  try { A.loadSlot("turn1"); console.log("loadSlot of a dropped slot did not throw FAIL"); fails++; } catch (e) { if (!/no saved slot/.test(e.message)) { console.log("unexpected error text: " + e.message + " FAIL"); fails++; } }
+  try { A.importState({ sig: { v: 0 }, pos: 0, parts: [] }); console.log("importState of a foreign signature did not throw FAIL"); fails++; } catch (e) { if (!/different model/.test(e.message)) { console.log("unexpected error text: " + e.message + " FAIL"); fails++; } }
+  console.log("session state (slots, export, import) " + (fails ? "see above" : "ok"));
+}
 A.destroy();
 console.log(fails ? "SHIM FAIL" : "SHIM PASS");
 process.exit(fails ? 1 : 0);
