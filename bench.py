@@ -274,7 +274,7 @@ def main():
     if os.path.exists(tpath):
         traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
-                    traffic=traffic, kernel="pa_decode_kernel<256, 1, 4, %s>" % ("false" if args.unfused else "true"), kernel_us=round(k_ms * 1e3, 3),
+                    traffic=traffic, kernel="pa_decode_kernel<256, 1, 4, %s, false>" % ("false" if args.unfused else "true"), kernel_us=round(k_ms * 1e3, 3),
                     algorithmic_bytes_per_launch=kv_bytes, launches=kcount)
     log("split-K kernel: %.2f us/launch -> %.0f GB/s (%.1f%% of 8 TB/s)" % (k_ms * 1e3, achieved, 100 * achieved / HBM_PEAK_GBS))
     plan = pa.plan("decode", ctx, 1)

@@ -146,6 +146,18 @@ int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_st
  * pa_q_buffer / pa_gate_buffer are not written by this call. */
 int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
                         const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype);
+/* pa_attn_decode_gather: decode / verify attention where every column attends to a list of cache rows instead of
+ * rows [0, base_pos + c] -- the gather mode of the reference's split-K kernel used by its sparse-attention layers:
+ * attn_dec_qsa + attn_dec_qsa_combine(_g) (engine/wgsl/attn_dec.js:33-38, :105, :170-183, :246; dispatch
+ * engine/qsa.js:41-56).  Same q / gate / out contract as pa_attn_decode.
+ *   d_sel: u32 [n_cols][sel_stride]; column c's list is d_sel[c * sel_stride] = n (1 <= n <= max_rows), then n row
+ *          indices < max_seq at d_sel[c * sel_stride + 1 ..], ascending (the reference's QSA_SEL_STRIDE layout)
+ *   max_rows: the longest list of the pass (engine/qsa.js:34 qsaMaxRows); sizes the splits
+ * List position t stands where position t stands in pa_attn_decode: with the list 0 .. pos a single column gives the
+ * same bits as pa_attn_decode at base_pos = pos. */
+int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_stride, const float* d_gate,
+                          uint32_t gate_stride, const uint32_t* d_sel, uint32_t sel_stride, uint32_t max_rows,
+                          uint32_t n_cols, void* d_out, uint32_t out_stride, int out_dtype);
 /* which kernel / split / tile shape the table picks (kind: 0 decode/verify, 1 prefill) */
 int pa_plan_query(const pa_ctx* ctx, int kind, uint32_t base_pos, uint32_t n_cols, pa_plan* out);
 /* override the table's split count for decode passes (0 = table); the reference's attnDecodeSplits

@@ -49,6 +49,7 @@ SYMBOLS = {
     "pa_gate_buffer": (vp, [vp]),
     "pa_attn_decode": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32, vp, u32, c_int]),
     "pa_attn_prefill": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32, vp, u32, c_int]),
+    "pa_attn_decode_gather": (c_int, [vp, u32, f32p, u32, f32p, u32, vp, u32, u32, u32, vp, u32, c_int]),
     "pa_attn_decode_step": (c_int, [vp, u32, f32p, f32p, f32p, f32p, f32p, u32, vp, c_int]),
     "pa_plan_query": (c_int, [vp, c_int, u32, u32, ctypes.POINTER(PaPlan)]),
     "pa_set_decode_splits": (c_int, [vp, u32]),
@@ -307,6 +308,28 @@ class PooledAttn:
         for b in bufs + [dout]:
             b.free(); self._bufs.remove(b)
         return out.reshape(self.cfg["n_heads"], self.cfg["head_dim"])
+
+    def run_attn_gather(self, layer, q, lists, gate=None, out_dtype=PA_OUT_F32):
+        """q [n, nH, hd]; lists: n sequences of cache row indices (ascending) -> out [n, nH, hd]."""
+        n = q.shape[0]
+        max_rows = max(len(l) for l in lists)
+        stride = max_rows + 1
+        sel = np.zeros((n, stride), np.uint32)
+        for c, l in enumerate(lists):
+            sel[c, 0] = len(l); sel[c, 1:1 + len(l)] = np.asarray(l, np.uint32)
+        dq = self.to_device(q.reshape(n, -1).astype(np.float32))
+        dg = self.to_device(gate.reshape(n, -1).astype(np.float32)) if gate is not None else None
+        dsel = self.to_device(sel)
+        esz = 4 if out_dtype == PA_OUT_F32 else 2
+        dout = self.alloc(n * self.q_dim * esz)
+        self._chk(self.L.pa_attn_decode_gather(self.ctx, layer, dq.ptr, self.q_dim, dg.ptr if dg else None, self.q_dim if dg else 0,
+                                               dsel.ptr, stride, max_rows, n, dout.ptr, self.q_dim, out_dtype))
+        self.sync()
+        out = dout.download(np.float32 if out_dtype == PA_OUT_F32 else np.float16, n * self.q_dim)
+        for b in (dq, dg, dsel, dout):
+            if b is not None:
+                b.free(); self._bufs.remove(b)
+        return out.reshape(n, self.cfg["n_heads"], self.cfg["head_dim"])
 
     def run_attn(self, kind, layer, q, base_pos, gate=None, out_dtype=PA_OUT_F32):
         """q [n, nH, hd] f32 (None: the context's q buffer, n from gate or 1) -> out [n, nH, hd]."""

@@ -63,9 +63,16 @@ template <int HD> struct DecShape {
 // its G query heads are normed and roped from the raw projection on the way into LDS, and the wave whose tile
 // holds position base_pos norms / ropes the new key row, writes it and the value row to the cache and patches them
 // into its staged tile (the tile's own load of that row raced the write and is discarded).
-template <int HD, int NB, int W, bool FUSED>
-__global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
+//
+// GATHER (the reference's attn_dec_qsa, engine/wgsl/attn_dec.js:33-38, :105, :170-183): each column attends to a
+// list of cache rows instead of rows 0 .. seqLen - 1.  Column col's list is sel[col * sel_stride] = n, then n row
+// indices (ascending) at sel[col * sel_stride + 1 ..].  List position t stands where position t stands in the dense
+// kernel: splits, tiles and masks are taken over list positions, only the K/V loads go through the list.  One
+// column per workgroup (grid z = column, NB == 1), since the lists differ between columns.
+template <int HD, int NB, int W, bool FUSED, bool GATHER>
+__global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
   static_assert(!FUSED || NB == 1, "the fused pre-step serves one column");
+  static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
   typedef DecShape<HD> S;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]
@@ -80,7 +87,9 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
   const uint32_t c0 = cg * p.cols_per_group;
   const uint32_t ncl = min(p.cols_per_group, p.n_cols - c0);
   const uint32_t R = ncl * G;                                        // live rows (<= 16*NB)
-  const uint32_t seq_max = p.base_pos + c0 + ncl;                    // rows visible to the group's last column
+  const uint32_t sel_base = GATHER ? c0 * p.sel_stride + 1 : 0;      // gather: first list entry of this column
+  // rows visible to the group's last column (gather: the column's list length)
+  const uint32_t seq_max = GATHER ? p.sel[c0 * p.sel_stride] : p.base_pos + c0 + ncl;
   const uint32_t t_begin = sp * p.split_len;
   if (t_begin >= seq_max) return;
   // the last split is open-ended: the plan may hand it up to one split length of remainder
@@ -158,12 +167,33 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
   // A wave with no tile of its own (short splits) loads the split's last tile and discards it: the prologue
   // stays branch-free, so the q staging below waits for the q loads only.
   uint32_t tile = __builtin_amdgcn_readfirstlane(wave);
+  // gather: byte offsets of this lane's rows of a tile, through the list (positions at or past the list's end take
+  // its last row: valid memory, masked or zeroed like any row past t_end)
+  uint32_t goff[GATHER ? S::NLD : 1];
+  auto gather_offsets = [&](uint32_t tpos) {
+    if constexpr (GATHER) {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) {
+        const uint32_t li = min(tpos + i * S::RPL + lrow, seq_max - 1);
+        goff[i] = min(p.sel[sel_base + li], p.max_seq - 1);      // a bad index must not leave the cache
+      }
+    }
+  };
   {
-    const size_t tb = (size_t)(t_begin + min(tile, n_tiles - 1) * TILE) * row_bytes;
+    const uint32_t t0 = t_begin + min(tile, n_tiles - 1) * TILE;
+    if constexpr (GATHER) {
+      gather_offsets(t0);
 #pragma unroll
-    for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
+      for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
 #pragma unroll
-    for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
+      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
+    } else {
+      const size_t tb = (size_t)t0 * row_bytes;
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
+    }
   }
   PA_TP(1);
   __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the K/V load issue
@@ -218,7 +248,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     const uint32_t r = nb * 16 + ln;
-    end_pos[nb] = r < R ? p.base_pos + c0 + r / G + 1 : 0u;
+    end_pos[nb] = r < R ? (GATHER ? seq_max : p.base_pos + c0 + r / G + 1) : 0u;
   }
   __syncthreads();
   PA_TP(2);
@@ -231,8 +261,14 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::KROW + (lane % S::LPR) * 16) = kr[i];
     if (more) {
+      if constexpr (GATHER) {
+        gather_offsets(tp + W * TILE);
 #pragma unroll
-      for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
+        for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
+      } else {
+#pragma unroll
+        for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
+      }
     }
     if (FUSED && own_pos && tile == pos_tile && lane < HD / 4)      // the new key row (in-order LDS: lands after the staged copy)
       *(h4*)(stage + (p.base_pos - tp) * S::KROW + lane * 8) = kpatch;
@@ -293,8 +329,13 @@ __global__ __launch_bounds__(W * 64, (NB == 1 ? 2 : 1)) void pa_decode_kernel(At
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
     if (more) {
+      if constexpr (GATHER) {                         // goff still holds the next tile's rows (set with the K loads above)
 #pragma unroll
-      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
+        for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
+      } else {
+#pragma unroll
+        for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
+      }
     }
     if (FUSED && own_pos && tile == pos_tile && lane < HD / 4)      // the new value row
       *(h4*)(stage + (p.base_pos - tp) * S::VROW + lane * 8) = vpatch;
@@ -384,7 +425,7 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   __shared__ float red[256];
   __shared__ f4 ored[256];
   const uint32_t h = blockIdx.x / CQ, dq = blockIdx.x % CQ, col = blockIdx.y, tid = threadIdx.x;
-  const uint32_t col_end = p.base_pos + col + 1;
+  const uint32_t col_end = p.sel ? p.sel[col * p.sel_stride] : p.base_pos + col + 1;   // gather: the column's list length
   const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits);   // the last split is open-ended
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
   const uint32_t grp = tid >> 4, l4 = tid & 15;
@@ -461,17 +502,17 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   }
 }
 
-template <int HD, int NB, int W, bool FUSED>
+template <int HD, int NB, int W, bool FUSED, bool GATHER = false>
 static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   typedef DecShape<HD> S;
   const size_t lds = 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W, FUSED>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W, FUSED, GATHER>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
+  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
   return hipGetLastError();
 }
 
@@ -497,6 +538,13 @@ hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s
   if (!p.f_q_in || p.n_cols != 1 || p.group > 16) return hipErrorInvalidValue;
   if (hd == 256) return launch_decode_t<256, 1, 4, true>(p, 1, s, t);
   if (hd == 128) return launch_decode_t<128, 1, 4, true>(p, 1, s, t);
+  return hipErrorInvalidValue;
+}
+
+hipError_t pa_launch_decode_gather(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t) {
+  if (!p.sel || p.cols_per_group != 1 || p.group > 16) return hipErrorInvalidValue;
+  if (hd == 256) return launch_decode_t<256, 1, 4, false, true>(p, p.n_cols, s, t);
+  if (hd == 128) return launch_decode_t<128, 1, 4, false, true>(p, p.n_cols, s, t);
   return hipErrorInvalidValue;
 }
 

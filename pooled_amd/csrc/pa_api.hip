@@ -489,6 +489,55 @@ extern "C" int pa_kv_write(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0
   if (!ctx) return PA_ERR_INVALID;
   return kv_copy(ctx, "pa_kv_write", layer, which, row0, n_rows, const_cast<void*>(h_src), false);
 }
+extern "C" int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_stride, const float* d_gate,
+                                     uint32_t gate_stride, const uint32_t* d_sel, uint32_t sel_stride, uint32_t max_rows,
+                                     uint32_t n_cols, void* d_out, uint32_t out_stride, int out_dtype) {
+  const char* who = "pa_attn_decode_gather";
+  if (!ctx) return PA_ERR_INVALID;
+  int rc = check_cols(ctx, who, layer, true, 0, n_cols);
+  if (rc) return rc;
+  const pa_config& c = ctx->cfg;
+  const uint32_t qd = c.n_heads * c.head_dim;
+  if (!d_out || !d_sel) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null buffer");
+  if (max_rows == 0 || max_rows > c.max_seq) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": max_rows must be in [1, max_seq]");
+  if (sel_stride < max_rows + 1) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": sel_stride shorter than a list of max_rows");
+  if (out_dtype != PA_OUT_F32 && out_dtype != PA_OUT_F16) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": bad out_dtype");
+  if (!d_q) { d_q = ctx->q_buf; q_stride = qd; }
+  if (q_stride < qd || out_stride < qd || (d_gate && gate_stride < qd))
+    return fail(ctx, PA_ERR_INVALID, std::string(who) + ": column stride shorter than a column");
+  if ((q_stride & 3) || (out_stride & 3) || (d_gate && (gate_stride & 3)) || ((uintptr_t)d_q & 15) || ((uintptr_t)d_out & 15) || ((uintptr_t)d_gate & 15) || ((uintptr_t)d_sel & 3))
+    return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned with strides a multiple of 4 elements");
+  if (c.n_heads / c.n_kv_heads > 16) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": more than 16 query heads per kv head");
+  // splits over list positions: the table's choice for one column of max_rows rows (an identity list then runs
+  // exactly the dense decode), thinned when several columns share the chip
+  pa_plan pl;
+  rc = plan_decode(ctx, max_rows - 1, 1, &pl);
+  if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
+  if (n_cols > 1 && pl.n_splits > 1) {
+    const uint32_t want = std::max(1u, pl.n_splits / n_cols);
+    pl.split_len = ceil_div(ceil_div(max_rows, want), 128) * 128;
+    pl.n_splits = ceil_div(max_rows, pl.split_len);
+  }
+  pl.slots = pl.n_splits;
+  if ((rc = ensure_partials(ctx, n_cols, pl.slots))) return rc;
+  AttnParams p; memset(&p, 0, sizeof p);
+  p.q = d_q; p.gate = d_gate; p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+  p.part_o = ctx->part_o; p.part_ml = ctx->part_ml; p.out = d_out;
+  p.q_stride = q_stride; p.gate_stride = gate_stride; p.out_stride = out_stride;
+  p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
+  p.base_pos = 0; p.n_cols = n_cols;
+  p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = 1;
+  p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
+  p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
+  p.gate_head_stride = c.head_dim;
+  p.sel = d_sel; p.sel_stride = sel_stride;
+  PaTiming tm;
+  if ((rc = prof_pair(ctx, &tm))) return rc;
+  HIPCHK(ctx, pa_launch_decode_gather(p, c.head_dim, ctx->stream, &tm));
+  HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
+  return PA_OK;
+}
+
 // ---- checkpoint slots ---------------------------------------------------------------------------------
 // Device-side copies of the rows written so far (the reference's saveSlot / loadSlot / dropSlot:
 // engine/dense.js:20-47, engine/qwen35.js:190-230) and their host form (exportSlot / importState parts:

@@ -48,6 +48,8 @@ struct AttnParams {
   const float2* rope_tab; const float* inv_freq;
   uint32_t f_q_head_stride, n_rot;
   float eps;
+  // gather mode (pa_attn_decode_gather): per column sel[col * sel_stride] = n, then n cache rows; nullptr otherwise
+  const uint32_t* sel; uint32_t sel_stride;
 };
 
 // ---- kernel launchers (defined next to their kernels) ------------------------------------------
@@ -66,6 +68,8 @@ hipError_t pa_launch_glue(const GlueParams& p, hipStream_t s);
 hipError_t pa_launch_rope_table(float2* tab, const float* inv_freq, uint32_t half, uint32_t n_pos, hipStream_t s);
 // waves per workgroup W in {4, 8}; NB = 16-row query blocks per workgroup (1..4); hd in {128, 256}
 hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
+// gather mode: every column attends to its own list of cache rows (p.sel set; cols_per_group == 1, grid z = column)
+hipError_t pa_launch_decode_gather(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t = nullptr);
 // the same with the pre-step of the one column fused in (p.f_* set; one 16-row block, n_cols == 1)
 hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t = nullptr);
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);

@@ -152,6 +152,16 @@ static napi_value CopyD2d(napi_env env, napi_callback_info info) {
   ARGS; pa_ctx* c = a.ctx(0); void* dst = a.ptr(1); const void* src = a.ptr(2); size_t n = (size_t)a.num(3); CHECK_ARGS("copyD2d");
   int rc = pa_copy_d2d(c, dst, src, n); if (rc) return throw_pa(env, c, rc, "pa_copy_d2d"); return undefined(env);
 }
+// attnGather(ctx, layer, q|null, qStride, gate|null, gateStride, sel, selStride, maxRows, nCols, out, outStride, outDtype)
+static napi_value AttnGather(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0);
+  uint32_t layer = a.u32(1); const float* q = (const float*)a.ptr(2); uint32_t qs = a.u32(3);
+  const float* g = (const float*)a.ptr(4); uint32_t gs = a.u32(5); const uint32_t* sel = (const uint32_t*)a.ptr(6);
+  uint32_t ss = a.u32(7), mr = a.u32(8), n = a.u32(9); void* out = a.ptr(10); uint32_t os = a.u32(11); int dt = (int)a.u32(12); CHECK_ARGS("attnGather");
+  int rc = pa_attn_decode_gather(c, layer, q, qs, g, gs, sel, ss, mr, n, out, os, dt);
+  if (rc) return throw_pa(env, c, rc, "pa_attn_decode_gather");
+  return undefined(env);
+}
 // planQuery(ctx, kind, basePos, nCols) -> {kernel, splitLen, nSplits, colGroups, colsPerGroup, waves, rowBlocks, slots}
 static napi_value PlanQuery(napi_env env, napi_callback_info info) {
   ARGS; pa_ctx* c = a.ctx(0); int kind = (int)a.u32(1); uint32_t base = a.u32(2), n = a.u32(3); CHECK_ARGS("planQuery");
@@ -204,7 +214,7 @@ static napi_value Init(napi_env env, napi_value exports) {
     {"kvStore", KvStore}, {"qBuffer", QBuffer}, {"gateBuffer", GateBuffer}, {"attn", Attn}, {"planQuery", PlanQuery},
     {"setDecodeSplits", SetDecodeSplits}, {"kvRead", KvRead}, {"kvWrite", KvWrite}, {"kvDevicePtr", KvDevicePtr}, {"timerStart", TimerStart},
     {"timerStop", TimerStop}, {"profileEnable", ProfileEnable}, {"profileRead", ProfileRead}, {"attnDecodeStep", AttnDecodeStep},
-    {"copyD2d", CopyD2d}, {"slotSave", SlotSave}, {"slotLoad", SlotLoad}, {"slotDrop", SlotDrop}, {"slotPos", SlotPos},
+    {"copyD2d", CopyD2d}, {"attnGather", AttnGather}, {"slotSave", SlotSave}, {"slotLoad", SlotLoad}, {"slotDrop", SlotDrop}, {"slotPos", SlotPos},
     {"slotCreate", SlotCreate}, {"slotExport", SlotExport}, {"slotImport", SlotImport},
   };
   for (auto& t : table) {

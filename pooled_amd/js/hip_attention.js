@@ -212,6 +212,14 @@ class HipAttention {
     addon.attn(this.ctx, 0, i, null, 0, gate, this.dims.qDim, pos, 1, B.attnOut.ptr, this._outStride(), this.outDtype);
   }
 
+  // ---- sparse-attention layers: the attn step of a QSA pass (engine/qsa.js:8-14, dispatch :41-56) ----
+  // sel: device address of the per-column row lists qsa_select wrote (u32 [nCols][selStride]: n, then n rows);
+  // maxRows = qsaMaxRows(pos, nCols).  Reads B.q (the context's roped q) and the gate, writes B.attnOut.
+  _encAttnQsa(p, LB, sel, selStride, maxRows, nCols) {
+    const gate = this.gate ? addon.gateBuffer(this.ctx) : null;
+    addon.attnGather(this.ctx, LB.layer, null, 0, gate, this.dims.qDim, sel, selStride, maxRows, nCols, this.B.attnOut.ptr, this._outStride(), this.outDtype);
+  }
+
   // ---- DenseEngine shapes (full RoPE, no gate): the glue writes the cache, then attention ----
   // _encodeAttn(pass, BG, seqLen): BG = { layer }; attention of the token at position seqLen - 1
   _encodeAttn(pass, BG, seqLen) {
