@@ -89,3 +89,27 @@ def test_decode_step_rejects_bad_arguments():
         with pytest.raises(PaError) as e:
             pa.run_decode_step(0, d["qraw"][0], d["kraw"][0], d["vraw"][0], d["qw"], d["kw"], 64)   # pos == max_seq
         assert e.value.code == PA_ERR_INVALID
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(n_heads=32, n_kv_heads=2, head_dim=128, n_rot=128, rope_theta=1e6, eps=1e-6, qk_norm=True, gate=False),   # G = 16: a full MFMA row block
+    dict(n_heads=32, n_kv_heads=2, head_dim=256, n_rot=64, rope_theta=1e7, eps=1e-6, qk_norm=True, gate=True),     # G = 16 at hd 256
+    dict(n_heads=4, n_kv_heads=4, head_dim=256, n_rot=256, rope_theta=1e4, eps=1e-5, qk_norm=False, gate=True),    # G = 1, full RoPE, no norm
+])
+def test_group_sizes_one_and_sixteen(cfg):
+    """Group sizes at both ends of what one 16-row block holds, through the fused step, the unfused pair, a verify
+    block and a prefill chunk."""
+    pos = 1234
+    d, k16, v16, K, V, ref, max_seq = _case(cfg, pos, seed=77)
+    nH, hd = cfg["n_heads"], cfg["head_dim"]
+    with PooledAttn(cfg, max_seq, n_layers=1, max_cols=64) as pa:
+        pa.layer_alloc(0); pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
+        got = pa.run_decode_step(0, d["qraw"][0], d["kraw"][0], d["vraw"][0], d["qw"], d["kw"], pos)
+        assert_parity(got[None], ref, "fused step G=%d" % (nH // cfg["n_kv_heads"]))
+        rng = np.random.default_rng(1)
+        q = rng.standard_normal((48, nH, hd), dtype=np.float32)
+        gate = rng.standard_normal(q.shape, dtype=np.float32) if cfg["gate"] else None
+        base = pos - 47
+        refb = C.attention(q, K, V, base, gate=gate)
+        assert_parity(pa.run_attn("decode", 0, q[:5], base, gate=None if gate is None else gate[:5]), refb[:5], "verify block")
+        assert_parity(pa.run_attn("prefill", 0, q, base, gate=gate), refb, "prefill chunk")
