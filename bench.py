@@ -175,6 +175,42 @@ def prefill_leg(steps, with_cpu):
     return res
 
 
+def other_configs():
+    """Configurations 1, 2 and 4 of the baseline (parity-test cases, not bench lines): steady-state time per call on
+    caches in rotation, for the record in DESIGN.md."""
+    from pooled_amd.capi import PooledAttn, PA_OUT_F16
+    dense = dict(n_heads=16, n_kv_heads=8, head_dim=128, n_rot=128, rope_theta=1e6, eps=1e-6, qk_norm=True, gate=False)
+    b27 = dict(n_heads=24, n_kv_heads=4, head_dim=256, n_rot=64, rope_theta=1e7, eps=1e-6, qk_norm=True, gate=True)
+    out = {}
+    for name, cfg, kind, base, n, layers in (("C1", dense, "decode", 2048, 1, 8), ("C2", dense, "prefill", 1536, 512, 8),
+                                             ("C4", b27, "decode", 65536, 8, 3)):
+        nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+        qd, kvd = nH * hd, nKV * hd
+        pa = PooledAttn(cfg, base + n, n_layers=layers, max_cols=4096)
+        rng = np.random.default_rng(7)
+        for l in range(layers):
+            pa.layer_alloc(l)
+            fill_cache(pa, cfg, l, base + n, seed=100 + l, chunk=4096)
+        dq = pa.to_device(rng.standard_normal((n, qd), dtype=np.float32))
+        dg = pa.to_device(rng.standard_normal((n, qd), dtype=np.float32)) if cfg["gate"] else None
+        dout = pa.alloc(n * qd * 2)
+        call = lambda i: pa.attn(kind, i % layers, dq, qd, dg, qd if dg else 0, base, n, dout, qd, PA_OUT_F16)
+        for i in range(10):
+            call(i)
+        pa.sync()
+        reps = 200
+        pa.timer_start()
+        for i in range(reps):
+            call(i)
+        ms = pa.timer_stop() / reps
+        kv = 2 * (base + n) * kvd * 2
+        fl = causal_flops(cfg, base, n)
+        out[name] = dict(us_per_call=round(ms * 1e3, 2), kv_gb_s=round(kv / ms / 1e6, 1), tflops=round(fl / ms / 1e9, 2), plan=pa.plan(kind, base, n))
+        log("%s: %.2f us/call, %.0f GB/s of KV, %.2f TFLOP/s" % (name, ms * 1e3, kv / ms / 1e6, fl / ms / 1e9))
+        pa.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -184,6 +220,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (configuration 5) leg")
     ap.add_argument("--unfused", action="store_true", help="decode step as three launches (pa_glue_kv + pa_attn_decode) instead of the fused pa_attn_decode_step")
     ap.add_argument("--prefill-steps", type=int, default=5)
+    ap.add_argument("--other-configs", action="store_true", help="only time configurations 1, 2 and 4 (attention call alone, caches in rotation)")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="only run the device probe: sustained f16 MFMA TFLOP/s and shader clock with constant and with random operands")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -196,6 +233,9 @@ def main():
     from pooled_amd.capi import PooledAttn, PA_OUT_F16, load
     L = load()
     log("library:", L.pa_version().decode())
+    if args.other_configs:
+        print(json.dumps({"other_configs": other_configs()}))
+        return
     if args.mfma_probe:
         # what the f16 matrix pipe sustains on this part, and at which clock: constant vs random operands, after a
         # warm-up long enough for the clock to settle

@@ -16,6 +16,8 @@ How each function is pinned (tests/test_oracle.py):
                       row-permutation invariance, brute-force scalar loops on tiny shapes, C oracle
   lse_merge           merging split partials == unsplit attention; one split -> O / l
   split formulas      integer known answers quoted in the reference's own comments
+  q8_quantize         zero block, exact-integer block (scale 1), ties to even, clamp at +-127, the block maximum maps
+                      to +-127, |x - dequant| <= scale / 2, scale from the f32 quotient
 """
 import numpy as np
 
@@ -132,6 +134,34 @@ def glue_kv(q_in, k_in, v_in, qw, kw, base_pos, cfg):
 
 
 # ---------------------------------------------------------------------------------------------
+# int8 KV (one f32 scale per 32 values)
+# ---------------------------------------------------------------------------------------------
+
+def q8_quantize(x):
+    """x [..., n] f32, n % 32 == 0 -> (q int8 [..., n], scale f32 [..., n/32]).
+
+    Reference: engine/wgsl/qwen35.js:908-946 (kv_store_q8): per block of 32 values scale = max|x| / 127,
+    inv = 1 / scale (0 for an all-zero block), value = clamp(round(x * inv), -127, 127), every operation in f32;
+    WGSL round() rounds half-way cases to even.
+    """
+    x = np.asarray(x, dtype=np.float32)
+    b = x.reshape(x.shape[:-1] + (x.shape[-1] // 32, 32))
+    a = np.abs(b).max(axis=-1)
+    sc = (a / np.float32(127.0)).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        inv = np.where(sc > 0, np.float32(1.0) / sc, np.float32(0.0)).astype(np.float32)
+    q = np.clip(np.rint((b * inv[..., None]).astype(np.float32)), -127.0, 127.0).astype(np.int8)
+    return q.reshape(x.shape), sc
+
+
+def q8_dequantize(q, sc):
+    """value * scale in f32, as the attention kernels read an int8 cache (engine/wgsl/qwen35.js:112-126)."""
+    q = np.asarray(q, dtype=np.int8)
+    b = q.reshape(q.shape[:-1] + (q.shape[-1] // 32, 32)).astype(np.float32)
+    return (b * np.asarray(sc, np.float32)[..., None]).astype(np.float32).reshape(q.shape)
+
+
+# ---------------------------------------------------------------------------------------------
 # attention
 # ---------------------------------------------------------------------------------------------
 
@@ -155,17 +185,23 @@ def attention(q, k16, v16, base_pos, gate=None, rows=None):
     One decode token is n = 1; a verify block or a prefill chunk is n > 1 (engine/qwen35.js:2485-2517:
     every column sees seqLen + col rows).
     """
+    return attention_values(q, k16.view(np.float16), v16.view(np.float16), base_pos, gate=gate, rows=rows)
+
+
+def attention_values(q, kf, vf, base_pos, gate=None, rows=None):
+    """attention() over cache rows given as numbers (any float dtype, [S, nKV, hd]) instead of f16 bits: the same
+    arithmetic; used for caches whose stored form is not f16 (the int8 cache after de-quantisation)."""
     q = np.asarray(q, dtype=np.float32)
     n, nH, hd = q.shape
-    nKV = k16.shape[1]
+    nKV = kf.shape[1]
     G = nH // nKV
     out = np.zeros((n, nH, hd), dtype=np.float64)
     cols = range(n) if rows is None else rows
     for c in cols:
         L = base_pos + c + 1
         for g in range(nKV):
-            K = k16[:L, g, :].view(np.float16).astype(np.float64)      # [L, hd]
-            V = v16[:L, g, :].view(np.float16).astype(np.float64)
+            K = kf[:L, g, :].astype(np.float64)                         # [L, hd]
+            V = vf[:L, g, :].astype(np.float64)
             qq = q[c, g * G:(g + 1) * G, :].astype(np.float64)          # [G, hd]
             s = (qq @ K.T) / np.sqrt(np.float64(hd))                    # [G, L]
             s -= s.max(axis=1, keepdims=True)

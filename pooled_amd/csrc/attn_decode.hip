@@ -502,6 +502,44 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   }
 }
 
+// The same merge for wide passes with few splits (a split prefill chunk: hundreds of columns, a handful of splits):
+// one thread per (column, head, 4 dims) walks the splits in order, so a workgroup covers 256 / (HD / 4) (column,
+// head) pairs instead of one 64-dim slice of one.  Same arithmetic, split order fixed.
+template <int HD>
+__global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
+  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const uint32_t d4 = (uint32_t)(e % (HD / 4));
+  const size_t ch = e / (HD / 4);
+  if (ch >= (size_t)p.n_cols * p.n_heads) return;
+  const uint32_t col = (uint32_t)(ch / p.n_heads), h = (uint32_t)(ch % p.n_heads);
+  const uint32_t col_end = p.sel ? p.sel[col * p.sel_stride] : p.base_pos + col + 1;
+  const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits);
+  const size_t base = ch * p.slots;
+  const float* po = p.part_o + base * HD + 4 * d4;
+  float M = NEG_INF;
+  for (uint32_t s = 0; s < ns; s++) M = fmaxf(M, p.part_ml[(base + s) * 2]);
+  float L = 0.f;
+  f4 o = {0.f, 0.f, 0.f, 0.f};
+  for (uint32_t s = 0; s < ns; s++) {
+    const float w = __expf(p.part_ml[(base + s) * 2] - M);
+    L += p.part_ml[(base + s) * 2 + 1] * w;
+    o += *(const f4*)(po + (size_t)s * HD) * w;
+  }
+  f4 r = o / L;
+  const uint32_t d = 4 * d4;
+  if (p.gate) {
+    const f4 gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d);
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] *= 1.f / (1.f + __expf(-gt[i]));
+  }
+  if (p.out_f16) {
+    const h4 hv = { (_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3] };
+    *(h4*)((_Float16*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + d) = hv;
+  } else {
+    *(f4*)((float*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + d) = r;
+  }
+}
+
 template <int HD, int NB, int W, bool FUSED, bool GATHER = false>
 static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   typedef DecShape<HD> S;
@@ -549,6 +587,14 @@ hipError_t pa_launch_decode_gather(const AttnParams& p, uint32_t hd, hipStream_t
 }
 
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s) {
+  // many columns, few splits: one thread per (column, head, 4 dims)
+  if (p.n_cols >= 16 && p.n_splits <= 32 && (hd == 256 || hd == 128)) {
+    const size_t threads = (size_t)p.n_cols * p.n_heads * (hd / 4);
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    if (hd == 256) hipLaunchKernelGGL(pa_combine_wide_kernel<256>, grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(pa_combine_wide_kernel<128>, grid, dim3(256), 0, s, p);
+    return hipGetLastError();
+  }
   const size_t lds = (size_t)p.slots * sizeof(float);
   if (hd == 256) hipLaunchKernelGGL(pa_combine_kernel<256>, dim3(p.n_heads * 4, p.n_cols), dim3(256), lds, s, p);
   else if (hd == 128) hipLaunchKernelGGL(pa_combine_kernel<128>, dim3(p.n_heads * 2, p.n_cols), dim3(256), lds, s, p);

@@ -232,3 +232,26 @@ def test_glue_kv_composition():
     assert np.array_equal(g["gate"][2, 5], d["qraw"][2, 5 * 2 * hd + hd: 5 * 2 * hd + 2 * hd])
     qn = O.head_rmsnorm(O.qsplit(d["qraw"], nH, hd)[0], d["qw"], cfg["eps"])
     assert np.array_equal(g["q"][..., cfg["n_rot"]:], qn[..., cfg["n_rot"]:])                   # un-rotated dims = normed q
+
+
+def test_q8_quantize_known_answers():
+    """int8 KV blocks (engine/wgsl/qwen35.js:908-946): answers fixed by the definition, not by the oracle's code."""
+    z = np.zeros(32, np.float32)
+    q, sc = O.q8_quantize(z)
+    assert sc.shape == (1,) and sc[0] == 0 and not q.any()                       # all-zero block: scale 0, inv 0
+    x = np.zeros(32, np.float32); x[0] = 127.0; x[1:8] = [0.5, 1.5, 2.5, -0.5, -1.5, 3.49, -126.6]
+    q, sc = O.q8_quantize(x)
+    assert sc[0] == 1.0                                                           # max 127 -> scale exactly 1
+    assert q[:8].tolist() == [127, 0, 2, 2, 0, -2, 3, -127]                       # ties to even; -126.6 -> -127
+    x = np.linspace(-3, 3, 64, dtype=np.float32); x[40] = 9.0                     # two blocks with their own scales
+    q, sc = O.q8_quantize(x)
+    assert sc[0] == np.float32(3.0) / np.float32(127.0) and sc[1] == np.float32(9.0) / np.float32(127.0)
+    assert q[0] == -127 and q[40] == 127 and np.abs(q).max() == 127
+    d = O.q8_dequantize(q, sc)
+    assert np.all(np.abs(d - x) <= np.repeat(sc, 32) * 0.5000001)                 # rounding error at most half a step
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((5, 3, 256), dtype=np.float32)
+    q, sc = O.q8_quantize(x)
+    assert q.shape == x.shape and sc.shape == (5, 3, 8)
+    blocks = x.reshape(5, 3, 8, 32)
+    assert np.array_equal(np.abs(q.reshape(5, 3, 8, 32)).max(-1), np.full((5, 3, 8), 127))     # the block maximum maps to +-127
