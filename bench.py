@@ -220,6 +220,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (configuration 5) leg")
     ap.add_argument("--unfused", action="store_true", help="decode step as three launches (pa_glue_kv + pa_attn_decode) instead of the fused pa_attn_decode_step")
     ap.add_argument("--prefill-steps", type=int, default=5)
+    ap.add_argument("--kv-q8", action="store_true", help="run the C3 decode step on int8 caches (one f32 scale per 32 values) instead of f16; implies --unfused")
     ap.add_argument("--other-configs", action="store_true", help="only time configurations 1, 2 and 4 (attention call alone, caches in rotation)")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="only run the device probe: sustained f16 MFMA TFLOP/s and shader clock with constant and with random operands")
@@ -262,6 +263,8 @@ def main():
         print(json.dumps({"copy_calibration": {"bytes_per_copy": nbytes, "copies": 10}}))
         return
     cfg, ctx = C3, C3_CTX
+    if args.kv_q8:
+        cfg = dict(C3, kv_q8=True); args.unfused = True; args.no_cpu = True
     nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
     qd, kvd = nH * hd, nKV * hd
     pa = PooledAttn(cfg, ctx + 1, n_layers=N_LAYERS, max_cols=4096)
@@ -288,6 +291,8 @@ def main():
             pa.attn_decode_step(layer, d_qfull, d_k, d_v, d_qw, d_kw, ctx, d_out, PA_OUT_F16)
 
     kv_bytes = 2 * (ctx + 1) * kvd * 2            # K and V rows [0, 32768], f16
+    if args.kv_q8:
+        kv_bytes = 2 * (ctx + 1) * (kvd + kvd // 32 * 4)          # int8 values + one f32 scale per 32
     for i in range(args.warmup):
         step(i)
     pa.sync()
@@ -314,7 +319,7 @@ def main():
     if os.path.exists(tpath):
         traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
-                    traffic=traffic, kernel="pa_decode_kernel<256, 1, 4, %s, false>" % ("false" if args.unfused else "true"), kernel_us=round(k_ms * 1e3, 3),
+                    traffic=traffic, kernel="pa_decode_kernel<256, 1, 4, %s, false, %s>" % ("false" if args.unfused else "true", "true" if args.kv_q8 else "false"), kernel_us=round(k_ms * 1e3, 3),
                     algorithmic_bytes_per_launch=kv_bytes, launches=kcount)
     log("split-K kernel: %.2f us/launch -> %.0f GB/s (%.1f%% of 8 TB/s)" % (k_ms * 1e3, achieved, 100 * achieved / HBM_PEAK_GBS))
     plan = pa.plan("decode", ctx, 1)
@@ -339,8 +344,8 @@ def main():
         metric="decode attn KV-read GB/s (% HBM peak) @32K ctx; prefill attn TFLOP/s (% MFMA)",
         value=round(value, 1), unit="GB/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
         ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None,
-        dtype="f16", data="synthetic",
-        config=dict(workload="C3 gated decode: 16q/2kv heads, head_dim 256, ctx 32768, 1 token, f16 KV, partial RoPE 64 dims theta 1e7, sigmoid gate, f16 out",
+        dtype="f16 (int8 cache widened to f16)" if args.kv_q8 else "f16", data="synthetic",
+        config=dict(workload="C3 gated decode: 16q/2kv heads, head_dim 256, ctx 32768, 1 token, %s KV," % ("int8 (f32 scale per 32)" if args.kv_q8 else "f16") + " partial RoPE 64 dims theta 1e7, sigmoid gate, f16 out",
                     step="%s on one layer; %d layers' caches in rotation (cold HBM)" % ("pa_glue_kv + pa_attn_decode (pre-step, split-K decode, LSE merge/gate: 3 launches)" if args.unfused else "pa_attn_decode_step (pre-step fused into the split-K decode kernel + LSE merge/gate: 2 launches)", N_LAYERS),
                     kv_bytes_per_step=kv_bytes, plan=plan, pct_hbm_peak=round(100 * value / HBM_PEAK_GBS, 2)),
         roofline=roofline, cpu_baseline=cpu)

@@ -30,6 +30,11 @@ extern "C" {
 #define PA_FLAG_GATE 2u       /* q input is interleaved [q(hd) | gate(hd)] per head and the output is
                                  multiplied by sigmoid(gate) (engine/wgsl/qwen35.js:370-384, :406-416) */
 
+#define PA_FLAG_KV_Q8 4u      /* int8 caches: values rounded to int8 with one f32 scale per 32 (scale = max|x| / 127),
+                                 the reference's kvQ8 mode (kv_store_q8, attn_flash_q8: engine/wgsl/qwen35.js:908-946,
+                                 :99-139).  Served by pa_glue_kv / pa_kv_store / pa_attn_decode / pa_attn_prefill /
+                                 slots; pa_attn_decode_step and pa_attn_decode_gather return PA_ERR_UNSUPPORTED. */
+
 /* output element types */
 #define PA_OUT_F32 0          /* the engine's attnOut feeding wo (engine/qwen35.js:881) */
 #define PA_OUT_F16 1
@@ -166,7 +171,9 @@ int pa_set_decode_splits(pa_ctx* ctx, uint32_t splits);
 
 /* ---- cache access for tests, checkpoints and slot copies (engine/dense.js:20-47 saveSlot/loadSlot
  *      copy rows [0, pos) of each layer) ----  which: 0 = K, 1 = V; the host side is the engine's position-major
- *      view, f16 bits [n_rows][nKV*hd]; the calls translate to and from the device layout and block */
+ *      view, f16 bits [n_rows][nKV*hd]; the calls translate to and from the device layout and block.
+ *      int8 caches: which 0 / 1 are int8 [n_rows][nKV*hd], which 2 / 3 the K / V scales, f32 [n_rows][nKV*hd/32]
+ *      (the reference's kCache / vCache / kScale / vScale parts, engine/qwen35.js:121-131) */
 int pa_kv_read(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, void* h_dst);
 int pa_kv_write(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, const void* h_src);
 /* device address of a cache (read-only use; the head-major device layout described at pa_layer_alloc) */

@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libpooled_attn.so")
 
 PA_OK, PA_ERR_INVALID, PA_ERR_UNSUPPORTED, PA_ERR_HIP, PA_ERR_NOMEM = 0, 1, 2, 3, 4
-PA_FLAG_QK_NORM, PA_FLAG_GATE = 1, 2
+PA_FLAG_QK_NORM, PA_FLAG_GATE, PA_FLAG_KV_Q8 = 1, 2, 4
 PA_OUT_F32, PA_OUT_F16 = 0, 1
 
 u32, c_int, vp, f32p = ctypes.c_uint32, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p
@@ -122,12 +122,13 @@ class DeviceBuffer:
 
 
 class PooledAttn:
-    """One pa_ctx.  cfg keys: n_heads, n_kv_heads, head_dim, n_rot, rope_theta, eps, qk_norm, gate."""
+    """One pa_ctx.  cfg keys: n_heads, n_kv_heads, head_dim, n_rot, rope_theta, eps, qk_norm, gate, kv_q8."""
 
     def __init__(self, cfg, max_seq, n_layers=1, max_cols=16):
         self.L = load()
         self.cfg = dict(cfg)
-        flags = (PA_FLAG_QK_NORM if cfg.get("qk_norm", True) else 0) | (PA_FLAG_GATE if cfg.get("gate", False) else 0)
+        flags = ((PA_FLAG_QK_NORM if cfg.get("qk_norm", True) else 0) | (PA_FLAG_GATE if cfg.get("gate", False) else 0)
+                 | (PA_FLAG_KV_Q8 if cfg.get("kv_q8", False) else 0))
         c = PaConfig(cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["n_rot"], cfg["rope_theta"], cfg["eps"],
                      max_seq, n_layers, max_cols, flags)
         h = vp()
@@ -179,12 +180,23 @@ class PooledAttn:
         self._chk(self.L.pa_sync(self.ctx))
 
     # ---- cache ----
-    def kv_write(self, layer, which, row0, rows16):
-        a = np.ascontiguousarray(rows16, dtype=np.uint16).reshape(-1, self.kv_dim)
+    def _kv_part(self, which):
+        """(dtype, elements per kv head and row) of cache tensor `which` in the host view."""
+        hd = self.cfg["head_dim"]
+        if not self.cfg.get("kv_q8", False):
+            return np.uint16, hd
+        return (np.int8, hd) if which < 2 else (np.float32, hd // 32)
+
+    def kv_write(self, layer, which, row0, rows):
+        dt, per = self._kv_part(which)
+        a = np.ascontiguousarray(rows, dtype=dt).reshape(-1, self.cfg["n_kv_heads"] * per)
         self._chk(self.L.pa_kv_write(self.ctx, layer, which, row0, a.shape[0], a.ctypes.data))
 
     def kv_read(self, layer, which, row0, n_rows):
-        out = np.empty((n_rows, self.cfg["n_kv_heads"], self.cfg["head_dim"]), dtype=np.uint16)
+        """f16 caches: f16 bits [n_rows, nKV, hd]; int8 caches: int8 values (which 0 / 1) or f32 scales
+        [n_rows, nKV, hd / 32] (which 2 / 3)."""
+        dt, per = self._kv_part(which)
+        out = np.empty((n_rows, self.cfg["n_kv_heads"], per), dtype=dt)
         self._chk(self.L.pa_kv_read(self.ctx, layer, which, row0, n_rows, out.ctypes.data))
         return out
 
@@ -272,13 +284,14 @@ class PooledAttn:
         self._chk(self.L.pa_slot_create(self.ctx, slot, pos))
 
     def slot_export(self, slot, layer, which):
-        """One part as f16 bits [pos, nKV * hd] (position-major)."""
-        out = np.empty((self.slot_pos(slot), self.cfg["n_kv_heads"] * self.cfg["head_dim"]), dtype=np.uint16)
+        """One part, position-major [pos, nKV * row]: f16 bits, or int8 values / f32 scales on an int8 cache."""
+        dt, per = self._kv_part(which)
+        out = np.empty((self.slot_pos(slot), self.cfg["n_kv_heads"] * per), dtype=dt)
         self._chk(self.L.pa_slot_export(self.ctx, slot, layer, which, out.ctypes.data))
         return out
 
     def slot_import(self, slot, layer, which, part):
-        part = np.ascontiguousarray(part, dtype=np.uint16)
+        part = np.ascontiguousarray(part, dtype=self._kv_part(which)[0])
         self._chk(self.L.pa_slot_import(self.ctx, slot, layer, which, part.ctypes.data))
 
     def mfma_probe(self, random_operands, iters):

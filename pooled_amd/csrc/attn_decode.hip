@@ -46,6 +46,26 @@ static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
   h4 r; __builtin_memcpy(&r, &t, 8); return r;
 }
 
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+// 16 int8 values x scale -> 16 f16 (see the Q8 note at the kernel)
+static __device__ inline void dq16(const u4 raw, const float sc, h8& lo, h8& hi) {
+  const h2 s2 = { (_Float16)sc, (_Float16)sc };
+  const h2 off = { (_Float16)1152.f, (_Float16)1152.f };
+  h2 o[8];
+#pragma unroll
+  for (int d = 0; d < 4; d++) {
+    const uint32_t w = raw[d] ^ 0x80808080u;
+    const uint32_t a = __builtin_amdgcn_perm(0x64646464u, w, 0x04010400u), b = __builtin_amdgcn_perm(0x64646464u, w, 0x04030402u);
+    h2 xa, xb;
+    __builtin_memcpy(&xa, &a, 4); __builtin_memcpy(&xb, &b, 4);
+    o[2 * d] = (xa - off) * s2;
+    o[2 * d + 1] = (xb - off) * s2;
+  }
+  lo = (h8){ o[0][0], o[0][1], o[1][0], o[1][1], o[2][0], o[2][1], o[3][0], o[3][1] };
+  hi = (h8){ o[4][0], o[4][1], o[5][0], o[5][1], o[6][0], o[6][1], o[7][0], o[7][1] };
+}
+
 template <int HD> struct DecShape {
   static constexpr int LPR = HD / 8;            // lanes per f16 row at 16 bytes a lane
   static constexpr int RPL = 64 / LPR;          // rows per wave-wide load
@@ -55,6 +75,12 @@ template <int HD> struct DecShape {
   static constexpr int STAGE = TILE * VROW;     // wave-private staging bytes (>= 16 x (HD + 4) floats for the merge)
   static constexpr int QROW = HD * 2 + 16;      // staged q row stride (bytes)
   static constexpr int OROW = (HD + 4) * 4;     // merge row stride (bytes)
+  // int8 caches: 16 values a lane
+  static constexpr int LPR8 = HD / 16;          // lanes per int8 row
+  static constexpr int RPL8 = 64 / LPR8;        // rows per wave-wide load
+  static constexpr int NLD8 = TILE / RPL8;      // loads per tile and tensor
+  static constexpr int SPR = HD / 32;           // scales per row
+  static constexpr int LPS = SPR / 4;           // lanes per row of scales at 16 bytes a lane
   static constexpr int KS = HD / 32;            // k-steps of the QK product
   static constexpr int DB = HD / 16;            // 16-dim blocks of the output
 };
@@ -69,10 +95,18 @@ template <int HD> struct DecShape {
 // indices (ascending) at sel[col * sel_stride + 1 ..].  List position t stands where position t stands in the dense
 // kernel: splits, tiles and masks are taken over list positions, only the K/V loads go through the list.  One
 // column per workgroup (grid z = column, NB == 1), since the lists differ between columns.
-template <int HD, int NB, int W, bool FUSED, bool GATHER>
+//
+// Q8 (the reference's kvQ8 caches read by attn_flash_q8, engine/wgsl/qwen35.js:99-139): K and V rows are int8 with one
+// f32 scale per 32 values.  Only the way a tile gets into LDS differs: a lane loads 16 values (16 bytes) and the
+// tile's scales (one 16-byte load), the scales make a round trip through the staging region so that every lane can
+// pick the scale of each of its 16-value pieces, and the pieces are widened to f16 on their way into the staged
+// tile -- int8 -> f16 through the 0x6400 | (v + 128) bit pattern (= 1152 + v exactly), a packed subtract and a
+// packed multiply by the f16-rounded scale.  From there on (MFMA, softmax, merge) it is the f16 kernel.
+template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8>
 __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
   static_assert(!FUSED || NB == 1, "the fused pre-step serves one column");
   static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
+  static_assert(!Q8 || (!FUSED && !GATHER), "int8 caches: plain decode / verify only");
   typedef DecShape<HD> S;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]
@@ -104,6 +138,14 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   const uint32_t voff = lrow * (uint32_t)row_bytes + (lane % S::LPR) * 16;
   const unsigned char* kbase = (const unsigned char*)(p.k_cache + (size_t)g * head_rows * HD);
   const unsigned char* vbase = (const unsigned char*)(p.v_cache + (size_t)g * head_rows * HD);
+  // int8 caches: rows of HD bytes, scales of SPR floats per row
+  const uint32_t lrow8 = lane / S::LPR8, voff8 = lrow8 * HD + (lane % S::LPR8) * 16;
+  const uint32_t srow = min(lane / S::LPS, (uint32_t)TILE - 1), soff = srow * S::SPR * 4 + (lane % S::LPS) * 16;
+  const unsigned char* kbase8 = (const unsigned char*)p.k_cache + (size_t)g * head_rows * HD;
+  const unsigned char* vbase8 = (const unsigned char*)p.v_cache + (size_t)g * head_rows * HD;
+  const unsigned char* ksbase = (const unsigned char*)(p.k_scale + (Q8 ? (size_t)g * head_rows * S::SPR : 0));
+  const unsigned char* vsbase = (const unsigned char*)(p.v_scale + (Q8 ? (size_t)g * head_rows * S::SPR : 0));
+  u4 ksr = {0u, 0u, 0u, 0u}, vsr = {0u, 0u, 0u, 0u};
 
   f4 acc[S::DB][NB];
 #pragma unroll
@@ -187,6 +229,14 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
 #pragma unroll
       for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
+    } else if constexpr (Q8) {
+      const size_t tb = (size_t)t0 * HD, sb = (size_t)t0 * S::SPR * 4;
+#pragma unroll
+      for (int i = 0; i < S::NLD8; i++) kr[i] = *(const u4*)(kbase8 + tb + (size_t)(i * S::RPL8) * HD + voff8);
+      ksr = *(const u4*)(ksbase + sb + soff);
+#pragma unroll
+      for (int i = 0; i < S::NLD8; i++) vr[i] = *(const u4*)(vbase8 + tb + (size_t)(i * S::RPL8) * HD + voff8);
+      vsr = *(const u4*)(vsbase + sb + soff);
     } else {
       const size_t tb = (size_t)t0 * row_bytes;
 #pragma unroll
@@ -258,9 +308,31 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     const size_t tnb = (size_t)(tp + W * TILE) * row_bytes;   // next tile of this wave
     const bool more = tile + W < n_tiles;
     // ---- K tile -> LDS, next K loads ----
+    if constexpr (Q8) {
+      if (lane / S::LPS < TILE) *(u4*)(stage + soff) = ksr;          // the tile's scales, [row][SPR] f32
+      wave_lds_fence();
+      float sc[S::NLD8];
+#pragma unroll
+      for (int i = 0; i < S::NLD8; i++) sc[i] = *(const float*)(stage + ((i * S::RPL8 + lrow8) * S::SPR + (lane % S::LPR8) / 2) * 4);
+      wave_lds_fence();                                              // read before the tile overwrites the region
+#pragma unroll
+      for (int i = 0; i < S::NLD8; i++) {
+        h8 lo, hi;
+        dq16(kr[i], sc[i], lo, hi);
+        unsigned char* d = stage + (i * S::RPL8 + lrow8) * S::KROW + (lane % S::LPR8) * 32;
+        *(h8*)d = lo; *(h8*)(d + 16) = hi;
+      }
+      if (more) {
+        const size_t tb = (size_t)(tp + W * TILE) * HD;
+#pragma unroll
+        for (int i = 0; i < S::NLD8; i++) kr[i] = *(const u4*)(kbase8 + tb + (size_t)(i * S::RPL8) * HD + voff8);
+        ksr = *(const u4*)(ksbase + (size_t)(tp + W * TILE) * S::SPR * 4 + soff);
+      }
+    } else {
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::KROW + (lane % S::LPR) * 16) = kr[i];
-    if (more) {
+    }
+    if (!Q8 && more) {
       if constexpr (GATHER) {
         gather_offsets(tp + W * TILE);
 #pragma unroll
@@ -322,13 +394,36 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       for (int db = 0; db < S::DB; db++) acc[db][nb] *= alpha;
     }
     // ---- V tile -> LDS, after the softmax so that the wait for the V loads comes as late as possible (rows at or past t_end as zeros: 0 x stale bits must not reach O), next V loads ----
+    if constexpr (Q8) {
+      if (lane / S::LPS < TILE) *(u4*)(stage + soff) = vsr;
+      wave_lds_fence();
+      float sc[S::NLD8];
+#pragma unroll
+      for (int i = 0; i < S::NLD8; i++) sc[i] = *(const float*)(stage + ((i * S::RPL8 + lrow8) * S::SPR + (lane % S::LPR8) / 2) * 4);
+      wave_lds_fence();
+#pragma unroll
+      for (int i = 0; i < S::NLD8; i++) {
+        h8 lo, hi;
+        dq16(vr[i], sc[i], lo, hi);
+        if (tp + i * S::RPL8 + lrow8 >= t_end) { lo = (h8){0, 0, 0, 0, 0, 0, 0, 0}; hi = lo; }   // also rows whose scale is not a number
+        unsigned char* d = stage + (i * S::RPL8 + lrow8) * S::VROW + (lane % S::LPR8) * 32;
+        *(h8*)d = lo; *(h8*)(d + 16) = hi;
+      }
+      if (more) {
+        const size_t tb = (size_t)(tp + W * TILE) * HD;
+#pragma unroll
+        for (int i = 0; i < S::NLD8; i++) vr[i] = *(const u4*)(vbase8 + tb + (size_t)(i * S::RPL8) * HD + voff8);
+        vsr = *(const u4*)(vsbase + (size_t)(tp + W * TILE) * S::SPR * 4 + soff);
+      }
+    } else {
     if (tp + TILE > t_end) {
 #pragma unroll
       for (int i = 0; i < S::NLD; i++) if (tp + i * S::RPL + lrow >= t_end) vr[i] = zero4;
     }
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
-    if (more) {
+    }
+    if (!Q8 && more) {
       if constexpr (GATHER) {                         // goff still holds the next tile's rows (set with the K loads above)
 #pragma unroll
         for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
@@ -540,22 +635,31 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
   }
 }
 
-template <int HD, int NB, int W, bool FUSED, bool GATHER = false>
+template <int HD, int NB, int W, bool FUSED, bool GATHER = false, bool Q8 = false>
 static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   typedef DecShape<HD> S;
   const size_t lds = 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W, FUSED, GATHER>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
+  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
   return hipGetLastError();
 }
 
 template <int HD>
 static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
+  if (p.k_scale) {                                // int8 caches
+    switch (nb) {
+      case 1: return launch_decode_t<HD, 1, 4, false, false, true>(p, col_groups, s, t);
+      case 2: return launch_decode_t<HD, 2, 4, false, false, true>(p, col_groups, s, t);
+      case 3: return launch_decode_t<HD, 3, 4, false, false, true>(p, col_groups, s, t);
+      case 4: return launch_decode_t<HD, 4, 4, false, false, true>(p, col_groups, s, t);
+      default: return hipErrorInvalidValue;
+    }
+  }
   switch (nb) {
     case 1: return launch_decode_t<HD, 1, 4, false>(p, col_groups, s, t);
     case 2: return launch_decode_t<HD, 2, 4, false>(p, col_groups, s, t);

@@ -12,6 +12,31 @@
 
 #define GLUE_DO_MATH 0x100u
 
+// int8 cache row (the reference's kv_store_q8, engine/wgsl/qwen35.js:908-946): per block of 32 values
+// scale = max|x| / 127, inv = 1 / scale (0 for an all-zero block), value = clamp(round-half-even(x * inv), -127, 127),
+// every operation a separately rounded f32 one.  One wavefront, 4 consecutive values a lane (8 lanes = one block);
+// src holds the row's hd f32 values (LDS or global), dst the row's hd int8, sc_dst its hd / 32 scales.
+static __device__ inline void store_row_q8(const float* src, uint32_t hd, uint32_t lane, unsigned char* dst, float* sc_dst) {
+#pragma clang fp contract(off)
+  const bool on = 4 * lane < hd;
+  float x[4] = {0.f, 0.f, 0.f, 0.f};
+  if (on) { x[0] = src[4 * lane]; x[1] = src[4 * lane + 1]; x[2] = src[4 * lane + 2]; x[3] = src[4 * lane + 3]; }
+  float a = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+  a = fmaxf(a, __shfl_xor(a, 1, 64)); a = fmaxf(a, __shfl_xor(a, 2, 64)); a = fmaxf(a, __shfl_xor(a, 4, 64));
+  const float sc = a / 127.0f;
+  const float inv = sc > 0.f ? 1.0f / sc : 0.f;
+  uint32_t w = 0;
+#pragma unroll
+  for (int b = 0; b < 4; b++) {
+    const float r = fminf(fmaxf(__builtin_rintf(x[b] * inv), -127.0f), 127.0f);
+    w |= ((uint32_t)(int)r & 255u) << (8 * b);
+  }
+  if (on) {
+    *(uint32_t*)(dst + 4 * lane) = w;
+    if ((lane & 7) == 0) sc_dst[lane >> 3] = sc;
+  }
+}
+
 static __device__ inline uint32_t pack_f16x2(float lo, float hi) {
   return (uint32_t)__half_as_ushort(__float2half_rn(lo)) | ((uint32_t)__half_as_ushort(__float2half_rn(hi)) << 16);
 }
@@ -73,7 +98,11 @@ __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
     return;
   }
   if (p.k_out) for (uint32_t i = lane; i < hd; i += 64) p.k_out[(size_t)col * p.k_stride + h * hd + i] = xs[i];
-  if (p.k_cache) {
+  if (p.k_cache && p.ks_cache) {                                     // int8 caches
+    const size_t row = (size_t)h * p.head_rows + pos;
+    store_row_q8(xs, hd, lane, (unsigned char*)p.k_cache + row * hd, p.ks_cache + row * (hd / 32));
+    store_row_q8(p.v_in + (size_t)col * p.v_stride + (size_t)h * hd, hd, lane, (unsigned char*)p.v_cache + row * hd, p.vs_cache + row * (hd / 32));
+  } else if (p.k_cache) {
     const size_t ro = ((size_t)h * p.head_rows + pos) * hd;           // head-major caches
     uint32_t* kc = (uint32_t*)(p.k_cache + ro);
     uint32_t* vc = (uint32_t*)(p.v_cache + ro);

@@ -92,10 +92,19 @@ extern "C" int pa_create(const pa_config* cfg, pa_ctx** out) {
 
 static void slot_free(pa_slot& sl);
 
+// caches: tensors per layer (K, V [, K scales, V scales]) and the bytes of one kv head's row of each
+static inline bool kv_q8(const pa_ctx* ctx) { return (ctx->cfg.flags & PA_FLAG_KV_Q8) != 0; }
+static inline int n_tensors(const pa_ctx* ctx) { return kv_q8(ctx) ? 4 : 2; }
+static inline size_t head_row_bytes(const pa_ctx* ctx, int which) {
+  const size_t hd = ctx->cfg.head_dim;
+  return which >= 2 ? hd / 32 * sizeof(float) : (kv_q8(ctx) ? hd : hd * 2);
+}
+
+
 extern "C" int pa_destroy(pa_ctx* ctx) {
   if (!ctx) return PA_OK;
   if (ctx->own_stream) (void)hipStreamSynchronize(ctx->own_stream);
-  for (auto& L : ctx->layers) { if (L.k) (void)hipFree(L.k); if (L.v) (void)hipFree(L.v); }
+  for (auto& L : ctx->layers) for (int w = 0; w < 4; w++) if (L.tensor(w)) (void)hipFree(L.tensor(w));
   for (auto& kv : ctx->slots) slot_free(kv.second);
   if (ctx->q_buf) (void)hipFree(ctx->q_buf);
   if (ctx->gate_buf) (void)hipFree(ctx->gate_buf);
@@ -118,13 +127,15 @@ extern "C" int pa_layer_alloc(pa_ctx* ctx, uint32_t layer) {
   if (L.k) return PA_OK;
   // head-major, 32 rows of zero padding after each kv head's max_seq rows: the attention kernels load whole
   // 32-row tiles unconditionally
-  const size_t bytes = ((size_t)ctx->cfg.max_seq + 32) * ctx->cfg.n_kv_heads * ctx->cfg.head_dim * 2;
-  HIPCHK(ctx, hipMalloc((void**)&L.k, bytes));
-  hipError_t e = hipMalloc((void**)&L.v, bytes);
-  if (e != hipSuccess) { (void)hipFree(L.k); L.k = nullptr; return fail_hip(ctx, e, "pa_layer_alloc: V cache"); }
-  HIPCHK(ctx, hipMemsetAsync(L.k, 0, bytes, ctx->stream));
-  HIPCHK(ctx, hipMemsetAsync(L.v, 0, bytes, ctx->stream));
+  void* t[4] = {nullptr, nullptr, nullptr, nullptr};
+  for (int w = 0; w < n_tensors(ctx); w++) {
+    const size_t bytes = ((size_t)ctx->cfg.max_seq + 32) * ctx->cfg.n_kv_heads * head_row_bytes(ctx, w);
+    hipError_t e = hipMalloc(&t[w], bytes);
+    if (e == hipSuccess) e = hipMemsetAsync(t[w], 0, bytes, ctx->stream);
+    if (e != hipSuccess) { for (int x = 0; x < 4; x++) if (t[x]) (void)hipFree(t[x]); return fail_hip(ctx, e, "pa_layer_alloc: cache allocation"); }
+  }
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  L.k = (uint16_t*)t[0]; L.v = (uint16_t*)t[1]; L.ks = (float*)t[2]; L.vs = (float*)t[3];
   return PA_OK;
 }
 
@@ -211,7 +222,7 @@ extern "C" int pa_glue_kv(pa_ctx* ctx, uint32_t layer, const float* d_q_in, uint
   if (q_stride < qcol || k_stride < kvd || v_stride < kvd) return fail(ctx, PA_ERR_INVALID, "pa_glue_kv: column stride shorter than a column");
   GlueParams p; fill_glue(ctx, p);
   p.q_in = d_q_in; p.k_in = d_k; p.v_in = d_v; p.qw = d_qw; p.kw = d_kw;
-  p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+  p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v; p.ks_cache = ctx->layers[layer].ks; p.vs_cache = ctx->layers[layer].vs;
   p.q_stride = q_stride; p.k_stride = k_stride; p.v_stride = v_stride;
   p.base_pos = base_pos; p.n_cols = n_cols;
   HIPCHK(ctx, pa_launch_glue(p, ctx->stream));
@@ -249,7 +260,7 @@ extern "C" int pa_kv_store(pa_ctx* ctx, uint32_t layer, const float* d_k, uint32
   p.n_heads = 0;            // key heads only
   p.flags = 0;              // pack only: no norm, no rope
   p.k_in = d_k; p.v_in = d_v;
-  p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+  p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v; p.ks_cache = ctx->layers[layer].ks; p.vs_cache = ctx->layers[layer].vs;
   p.k_stride = k_stride; p.v_stride = v_stride;
   p.base_pos = base_pos; p.n_cols = n_cols;
   HIPCHK(ctx, pa_launch_glue(p, ctx->stream));
@@ -317,7 +328,7 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
 
 extern "C" int pa_plan_query(const pa_ctx* ctx, int kind, uint32_t base_pos, uint32_t n_cols, pa_plan* out) {
   if (!ctx || !out || n_cols == 0) return PA_ERR_INVALID;
-  return kind == 0 ? plan_decode(ctx, base_pos, n_cols, out) : plan_prefill(ctx, base_pos, n_cols, out);
+  return (kind == 0 || kv_q8(ctx)) ? plan_decode(ctx, base_pos, n_cols, out) : plan_prefill(ctx, base_pos, n_cols, out);
 }
 extern "C" int pa_set_decode_splits(pa_ctx* ctx, uint32_t splits) {
   if (!ctx) return PA_ERR_INVALID;
@@ -374,7 +385,9 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   if ((q_stride & 3) || (out_stride & 3) || (d_gate && (gate_stride & 3)) || ((uintptr_t)d_q & 15) || ((uintptr_t)d_out & 15) || ((uintptr_t)d_gate & 15))
     return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned with strides a multiple of 4 elements");
   pa_plan pl;
-  rc = kind == 0 ? plan_decode(ctx, base_pos, n_cols, &pl) : plan_prefill(ctx, base_pos, n_cols, &pl);
+  // int8 caches are served by the split-K kernel only (the reference has no tiled prefill for them either): a
+  // prefill chunk then runs as column groups of that kernel
+  rc = (kind == 0 || kv_q8(ctx)) ? plan_decode(ctx, base_pos, n_cols, &pl) : plan_prefill(ctx, base_pos, n_cols, &pl);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
   const bool direct = pl.kernel == 1 && pl.n_splits == 1;     // the prefill kernel writes the output itself
@@ -385,6 +398,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   p.q_stride = q_stride; p.gate_stride = gate_stride; p.out_stride = out_stride;
   p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
   p.base_pos = base_pos; p.n_cols = n_cols;
+  p.k_scale = ctx->layers[layer].ks; p.v_scale = ctx->layers[layer].vs;
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
@@ -417,6 +431,7 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
   if (rc) return rc;
   const pa_config& c = ctx->cfg;
   const bool gated = (c.flags & PA_FLAG_GATE) != 0, norm = (c.flags & PA_FLAG_QK_NORM) != 0;
+  if (kv_q8(ctx)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": int8 caches take pa_glue_kv + pa_attn_decode");
   if (!d_q_in || !d_k || !d_v || !d_out) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null buffer");
   if (norm && (!d_qw || !d_kw)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": norm weights required");
   if (out_dtype != PA_OUT_F32 && out_dtype != PA_OUT_F16) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": bad out_dtype");
@@ -458,13 +473,13 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
 // [rows][nKV * hd], so each call is one strided copy per kv head.
 static int kv_copy(pa_ctx* ctx, const char* who, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, void* host, bool to_host) {
   if (layer >= ctx->cfg.n_layers || !ctx->layers[layer].k) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": layer not allocated");
-  if (which != 0 && which != 1) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": which must be 0 (K) or 1 (V)");
+  if (which < 0 || which >= n_tensors(ctx)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": which must be 0 (K) or 1 (V), or 2 / 3 (their scales) on an int8 cache");
   if ((uint64_t)row0 + n_rows > ctx->cfg.max_seq) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": rows exceed max_seq");
   if (!host) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null host buffer");
   if (n_rows == 0) return PA_OK;
   const pa_config& c = ctx->cfg;
-  const size_t hd_bytes = (size_t)c.head_dim * 2, host_pitch = hd_bytes * c.n_kv_heads, head_rows = (size_t)c.max_seq + 32;
-  unsigned char* dev = (unsigned char*)(which ? ctx->layers[layer].v : ctx->layers[layer].k);
+  const size_t hd_bytes = head_row_bytes(ctx, which), host_pitch = hd_bytes * c.n_kv_heads, head_rows = (size_t)c.max_seq + 32;
+  unsigned char* dev = (unsigned char*)ctx->layers[layer].tensor(which);
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   // one contiguous transfer per kv head through a host staging plane (a pitched copy of 512-byte rows is far slower)
   std::vector<unsigned char> plane((size_t)n_rows * hd_bytes);
@@ -498,6 +513,7 @@ extern "C" int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d
   if (rc) return rc;
   const pa_config& c = ctx->cfg;
   const uint32_t qd = c.n_heads * c.head_dim;
+  if (kv_q8(ctx)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": no gather mode on int8 caches");
   if (!d_out || !d_sel) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null buffer");
   if (max_rows == 0 || max_rows > c.max_seq) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": max_rows must be in [1, max_seq]");
   if (sel_stride < max_rows + 1) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": sel_stride shorter than a list of max_rows");
@@ -544,18 +560,17 @@ extern "C" int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d
 // engine/qwen35.js:121-131, :151-190): per layer one K part and one V part of pos * kvDim f16, position-major.
 
 static void slot_free(pa_slot& sl) {
-  for (auto p : sl.k) if (p) (void)hipFree(p);
-  for (auto p : sl.v) if (p) (void)hipFree(p);
-  sl.k.clear(); sl.v.clear(); sl.pos = 0;
+  for (int w = 0; w < 4; w++) { for (auto p : sl.t[w]) if (p) (void)hipFree(p); sl.t[w].clear(); }
+  sl.pos = 0;
 }
 
 // a slot with room for rows [0, pos) of every allocated layer (contents undefined)
 static int slot_make(pa_ctx* ctx, const char* who, uint32_t slot, uint32_t pos) {
   if (pos > ctx->cfg.max_seq) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": pos exceeds max_seq");
   auto it = ctx->slots.find(slot);
-  if (it != ctx->slots.end() && it->second.pos == pos && it->second.k.size() == ctx->layers.size()) {
+  if (it != ctx->slots.end() && it->second.pos == pos && it->second.t[0].size() == ctx->layers.size()) {
     bool same = true;                                   // same shape: the buffers are reused (the stream orders the copies)
-    for (size_t l = 0; l < ctx->layers.size(); l++) same = same && ((ctx->layers[l].k != nullptr && pos != 0) == (it->second.k[l] != nullptr));
+    for (size_t l = 0; l < ctx->layers.size(); l++) same = same && ((ctx->layers[l].k != nullptr && pos != 0) == (it->second.t[0][l] != nullptr));
     if (same) return PA_OK;
   }
   if (it != ctx->slots.end()) {
@@ -563,21 +578,21 @@ static int slot_make(pa_ctx* ctx, const char* who, uint32_t slot, uint32_t pos) 
     slot_free(it->second); ctx->slots.erase(it);
   }
   pa_slot sl; sl.pos = pos;
-  sl.k.assign(ctx->layers.size(), nullptr); sl.v.assign(ctx->layers.size(), nullptr);
-  const size_t bytes = (size_t)pos * ctx->cfg.n_kv_heads * ctx->cfg.head_dim * 2;
-  for (size_t l = 0; l < ctx->layers.size() && bytes; l++) {
+  for (int w = 0; w < 4; w++) sl.t[w].assign(ctx->layers.size(), nullptr);
+  for (size_t l = 0; l < ctx->layers.size() && pos; l++) {
     if (!ctx->layers[l].k) continue;
-    hipError_t e = hipMalloc((void**)&sl.k[l], bytes);
-    if (e == hipSuccess) e = hipMalloc((void**)&sl.v[l], bytes);
-    if (e != hipSuccess) { slot_free(sl); return fail_hip(ctx, e, "slot allocation"); }
+    for (int w = 0; w < n_tensors(ctx); w++) {
+      hipError_t e = hipMalloc(&sl.t[w][l], (size_t)pos * ctx->cfg.n_kv_heads * head_row_bytes(ctx, w));
+      if (e != hipSuccess) { slot_free(sl); return fail_hip(ctx, e, "slot allocation"); }
+    }
   }
   ctx->slots[slot] = std::move(sl);
   return PA_OK;
 }
 
 // rows [0, pos) of one tensor between the cache ([nKV][max_seq + 32][hd]) and a slot ([nKV][pos][hd]): one pitched copy
-static hipError_t slot_copy(const pa_ctx* ctx, uint16_t* cache, uint16_t* slot_buf, uint32_t pos, bool to_slot) {
-  const size_t plane = (size_t)pos * ctx->cfg.head_dim * 2, cache_pitch = ((size_t)ctx->cfg.max_seq + 32) * ctx->cfg.head_dim * 2;
+static hipError_t slot_copy(const pa_ctx* ctx, int which, void* cache, void* slot_buf, uint32_t pos, bool to_slot) {
+  const size_t plane = (size_t)pos * head_row_bytes(ctx, which), cache_pitch = ((size_t)ctx->cfg.max_seq + 32) * head_row_bytes(ctx, which);
   return to_slot ? hipMemcpy2DAsync(slot_buf, plane, cache, cache_pitch, plane, ctx->cfg.n_kv_heads, hipMemcpyDeviceToDevice, ctx->stream)
                  : hipMemcpy2DAsync(cache, cache_pitch, slot_buf, plane, plane, ctx->cfg.n_kv_heads, hipMemcpyDeviceToDevice, ctx->stream);
 }
@@ -588,9 +603,8 @@ extern "C" int pa_slot_save(pa_ctx* ctx, uint32_t slot, uint32_t pos) {
   if (rc) return rc;
   pa_slot& sl = ctx->slots[slot];
   for (size_t l = 0; l < ctx->layers.size(); l++) {
-    if (!sl.k[l]) continue;
-    HIPCHK(ctx, slot_copy(ctx, ctx->layers[l].k, sl.k[l], pos, true));
-    HIPCHK(ctx, slot_copy(ctx, ctx->layers[l].v, sl.v[l], pos, true));
+    if (!sl.t[0][l]) continue;
+    for (int w = 0; w < n_tensors(ctx); w++) HIPCHK(ctx, slot_copy(ctx, w, ctx->layers[l].tensor(w), sl.t[w][l], pos, true));
   }
   return PA_OK;
 }
@@ -601,10 +615,9 @@ extern "C" int pa_slot_load(pa_ctx* ctx, uint32_t slot, uint32_t* pos) {
   if (it == ctx->slots.end()) return fail(ctx, PA_ERR_INVALID, "pa_slot_load: no saved slot " + std::to_string(slot));
   pa_slot& sl = it->second;
   for (size_t l = 0; l < ctx->layers.size(); l++) {
-    if (l >= sl.k.size() || !sl.k[l]) continue;
+    if (l >= sl.t[0].size() || !sl.t[0][l]) continue;
     if (!ctx->layers[l].k) return fail(ctx, PA_ERR_INVALID, "pa_slot_load: the slot holds a layer that has no cache now");
-    HIPCHK(ctx, slot_copy(ctx, ctx->layers[l].k, sl.k[l], sl.pos, false));
-    HIPCHK(ctx, slot_copy(ctx, ctx->layers[l].v, sl.v[l], sl.pos, false));
+    for (int w = 0; w < n_tensors(ctx); w++) HIPCHK(ctx, slot_copy(ctx, w, ctx->layers[l].tensor(w), sl.t[w][l], sl.pos, false));
   }
   *pos = sl.pos;
   return PA_OK;
@@ -637,13 +650,13 @@ static int slot_part(pa_ctx* ctx, const char* who, uint32_t slot, uint32_t layer
   auto it = ctx->slots.find(slot);
   if (it == ctx->slots.end()) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": no saved slot " + std::to_string(slot));
   pa_slot& sl = it->second;
-  if (which != 0 && which != 1) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": which must be 0 (K) or 1 (V)");
+  if (which < 0 || which >= n_tensors(ctx)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": which must be 0 (K) or 1 (V), or 2 / 3 (their scales) on an int8 cache");
   if (sl.pos == 0) return PA_OK;
-  if (layer >= sl.k.size() || !sl.k[layer]) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": the slot has no such layer");
+  if (layer >= sl.t[0].size() || !sl.t[0][layer]) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": the slot has no such layer");
   if (!host) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null host buffer");
   const pa_config& c = ctx->cfg;
-  const size_t hd_bytes = (size_t)c.head_dim * 2, host_pitch = hd_bytes * c.n_kv_heads, plane_bytes = (size_t)sl.pos * hd_bytes;
-  unsigned char* dev = (unsigned char*)(which ? sl.v[layer] : sl.k[layer]);
+  const size_t hd_bytes = head_row_bytes(ctx, which), host_pitch = hd_bytes * c.n_kv_heads, plane_bytes = (size_t)sl.pos * hd_bytes;
+  unsigned char* dev = (unsigned char*)sl.t[which][layer];
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   std::vector<unsigned char> plane(plane_bytes);
   for (uint32_t g = 0; g < c.n_kv_heads; g++) {
@@ -669,7 +682,7 @@ extern "C" int pa_slot_import(pa_ctx* ctx, uint32_t slot, uint32_t layer, int wh
 
 extern "C" const void* pa_kv_device_ptr(pa_ctx* ctx, uint32_t layer, int which) {
   if (!ctx || layer >= ctx->cfg.n_layers) return nullptr;
-  return which ? (const void*)ctx->layers[layer].v : (const void*)ctx->layers[layer].k;
+  return which >= 0 && which < 4 ? (const void*)ctx->layers[layer].tensor(which) : nullptr;
 }
 
 // ---- timing -----------------------------------------------------------------------------------------

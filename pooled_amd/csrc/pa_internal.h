@@ -17,7 +17,8 @@ struct GlueParams {
   const float* inv_freq;                                     // [n_rot/2] f32, theta^(-2i/n_rot)
   const float2* rope_tab;                                    // [max_seq][n_rot/2] (cos, sin) or nullptr
   float* q_out; float* gate_out;                             // [n_cols][nH*hd]
-  uint16_t* k_cache; uint16_t* v_cache;                      // f16 [nKV][head_rows][hd] or nullptr
+  uint16_t* k_cache; uint16_t* v_cache;                      // f16 (or int8) [nKV][head_rows][hd] or nullptr
+  float* ks_cache; float* vs_cache;                          // int8 caches: scales [nKV][head_rows][hd/32]
   uint32_t head_rows;                                        // rows of one kv head's plane (max_seq + padding)
   uint32_t q_stride, k_stride, v_stride;
   uint32_t n_heads, n_kv_heads, head_dim, n_rot;
@@ -29,6 +30,7 @@ struct GlueParams {
 struct AttnParams {
   const float* q; const float* gate;          // f32 [n_cols][stride]
   const uint16_t* k_cache; const uint16_t* v_cache;
+  const float* k_scale; const float* v_scale;   // int8 caches: one f32 scale per 32 values, [nKV][head_rows][hd/32]
   float* part_o; float* part_ml;              // split partials: [(col*nH + h)*slots + sp][hd], [..][2]
   void* out;                                  // [n_cols][out_stride]
   uint32_t q_stride, gate_stride, out_stride;
@@ -83,12 +85,17 @@ hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, uint32_t iters, hip
 
 // ---- context -----------------------------------------------------------------------------------
 
-struct pa_layer { uint16_t* k = nullptr; uint16_t* v = nullptr; };
+// One layer's caches.  f16 caches: k, v.  int8 caches (PA_FLAG_KV_Q8): k, v hold int8 values (hd bytes a row), ks, vs
+// one f32 scale per 32 values.  All head-major [nKV][max_seq + 32][row].
+struct pa_layer {
+  uint16_t* k = nullptr; uint16_t* v = nullptr; float* ks = nullptr; float* vs = nullptr;
+  void* tensor(int which) const { return which == 0 ? (void*)k : which == 1 ? (void*)v : which == 2 ? (void*)ks : (void*)vs; }
+};
 
 // A checkpoint slot: per allocated layer a compact head-major copy [nKV][pos][hd] of K and of V rows [0, pos).
 struct pa_slot {
   uint32_t pos = 0;
-  std::vector<uint16_t*> k, v;     // indexed by layer; nullptr for layers without a cache (or pos == 0)
+  std::vector<void*> t[4];         // per tensor (K, V, K scales, V scales), indexed by layer; nullptr where absent
 };
 
 struct pa_ctx {

@@ -17,7 +17,7 @@
 const path = require("path");
 const addon = require(path.join(__dirname, "..", "lib", "pooled_attn.node"));
 
-const PA_FLAG_QK_NORM = 1, PA_FLAG_GATE = 2, PA_OUT_F32 = 0, PA_OUT_F16 = 1;
+const PA_FLAG_QK_NORM = 1, PA_FLAG_GATE = 2, PA_FLAG_KV_Q8 = 4, PA_OUT_F32 = 0, PA_OUT_F16 = 1;
 
 // ---- the reference's sizing formulas, kept for callers that still size grids or slot buffers with them.
 //      The HIP kernels take their splits from the gfx950 table instead (HipAttention.plan). ----
@@ -64,10 +64,12 @@ class HipAttention {
     this.outDtype = opts.outF16 ? PA_OUT_F16 : PA_OUT_F32;
     this.fusedStep = opts.fusedStep !== false;
     // engine fields the attention dispatch reads (engine/qwen35.js:366, :416-419): always the f16-KV split-K path here
-    this.flash = true; this.kvQ8 = false; this.attnDecode = "v2"; this.attnPrefillTile = true;
+    this.flash = true; this.attnDecode = "v2"; this.attnPrefillTile = true;
     this._snapNow = null;                                          // set by a verify pass (engine/qwen35.js:2960-2965)
     this.pos = 0;
-    const flags = (this.qkNorm ? PA_FLAG_QK_NORM : 0) | (this.gate ? PA_FLAG_GATE : 0);
+    this.kvQ8 = !!opts.kvQ8;                                       // int8 caches (engine option kvQ8): three launches per token
+    if (this.kvQ8) this.fusedStep = false;
+    const flags = (this.qkNorm ? PA_FLAG_QK_NORM : 0) | (this.gate ? PA_FLAG_GATE : 0) | (this.kvQ8 ? PA_FLAG_KV_Q8 : 0);
     // a readable throw at create, like the engine's KV binding check (engine/qwen35.js:378-383)
     this.ctx = addon.create({ nH: nH, nKV: nKV, hd: hd, nRot: this.dims.nRot, ropeTheta: opts.ropeTheta, eps: opts.eps,
       maxSeq: opts.maxSeq, nLayers: opts.nLayers || 1, maxCols: this.NC, flags: flags });
@@ -120,8 +122,13 @@ class HipAttention {
     }
     return out;
   }
-  kvRead(layer, which, row0, nRows) { const a = new Uint16Array(nRows * this.dims.kvDim); addon.kvRead(this.ctx, layer, which, row0, nRows, a); return a; }
-  kvWrite(layer, which, row0, rows) { addon.kvWrite(this.ctx, layer, which, row0, rows.length / this.dims.kvDim, rows); }
+  // which: 0 K, 1 V (f16 bits as Uint16Array; on int8 caches Int8Array), 2 / 3 their scales (int8 caches, Float32Array)
+  _kvPart(which, nRows) {
+    if (!this.kvQ8) return new Uint16Array(nRows * this.dims.kvDim);
+    return which < 2 ? new Int8Array(nRows * this.dims.kvDim) : new Float32Array(nRows * this.dims.kvDim / 32);
+  }
+  kvRead(layer, which, row0, nRows) { const a = this._kvPart(which, nRows); addon.kvRead(this.ctx, layer, which, row0, nRows, a); return a; }
+  kvWrite(layer, which, row0, rows) { addon.kvWrite(this.ctx, layer, which, row0, rows.length / this._kvPart(which, 1).length, rows); }
   sync() { addon.sync(this.ctx); }
   plan(kind, basePos, nCols) { return addon.planQuery(this.ctx, kind === "prefill" ? 1 : 0, basePos, nCols); }
 
@@ -143,14 +150,15 @@ class HipAttention {
   dropSlot(name) { const id = this._slotId(name, false); if (id !== undefined) { addon.slotDrop(this.ctx, id); this._slotIds.delete(name); } }
   dropAllSlots() { for (const k of Array.from((this._slotIds || new Map()).keys())) this.dropSlot(k); }
   // what a saved state must match to be loaded here (the attention-relevant fields of engine/qwen35.js:133-143)
-  stateSignature() { return { v: 1, layers: this.layers.length, flash: true, kvQ8: false, dims: [this.dims.kvDim] }; }
+  stateSignature() { return { v: 1, layers: this.layers.length, flash: true, kvQ8: this.kvQ8, dims: [this.dims.kvDim] }; }
   // { sig, pos, parts: [ArrayBuffer] }: per layer a K part and a V part of pos * kvDim f16, position-major
   exportSlot(name) {
     const id = this._slotId(name, false);
     if (id === undefined) throw new Error("no saved slot " + name);
     const pos = addon.slotPos(this.ctx, id), parts = [];
-    for (let l = 0; l < this.layers.length; l++) for (let w = 0; w < 2; w++) {
-      const a = new Uint16Array(pos * this.dims.kvDim);
+    // per layer kCache, vCache (and, int8 caches, kScale, vScale): the order of the reference's _stateParts
+    for (let l = 0; l < this.layers.length; l++) for (let w = 0; w < (this.kvQ8 ? 4 : 2); w++) {
+      const a = this._kvPart(w, pos);
       if (pos) addon.slotExport(this.ctx, id, l, w, a);
       parts.push(a.buffer);
     }
@@ -159,12 +167,12 @@ class HipAttention {
   exportState() { this.saveSlot("__export"); try { return this.exportSlot("__export"); } finally { this.dropSlot("__export"); } }
   importState(st) {
     if (JSON.stringify(st.sig) !== JSON.stringify(this.stateSignature())) throw new Error("saved state is for a different model, layer range or KV format");
-    const bytes = st.pos * this.dims.kvDim * 2;
-    if (st.parts.length !== 2 * this.layers.length || st.parts.some((p) => p.byteLength !== bytes)) throw new Error("saved state has the wrong shape");
+    const nt = this.kvQ8 ? 4 : 2;
+    if (st.parts.length !== nt * this.layers.length || st.parts.some((p, i) => p.byteLength !== this._kvPart(i % nt, st.pos).byteLength)) throw new Error("saved state has the wrong shape");
     const id = this._slotId("__import", true);
     addon.slotCreate(this.ctx, id, st.pos);
     try {
-      if (st.pos) st.parts.forEach((p, i) => addon.slotImport(this.ctx, id, i >> 1, i & 1, new Uint16Array(p)));
+      if (st.pos) st.parts.forEach((p, i) => addon.slotImport(this.ctx, id, Math.floor(i / nt), i % nt, new Uint8Array(p)));
       this.pos = addon.slotLoad(this.ctx, id);
     } finally { this.dropSlot("__import"); }
   }
@@ -237,4 +245,4 @@ class HipAttention {
 }
 
 module.exports = { HipAttention, addon, attnDecConfig, decSplitLen, decSplits, DEC_CQ, attnTileConfig, tileSplitLen, faSizing,
-  PA_FLAG_QK_NORM, PA_FLAG_GATE, PA_OUT_F32, PA_OUT_F16 };
+  PA_FLAG_QK_NORM, PA_FLAG_GATE, PA_FLAG_KV_Q8, PA_OUT_F32, PA_OUT_F16 };
