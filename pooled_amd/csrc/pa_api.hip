@@ -369,6 +369,10 @@ static int prof_pair(pa_ctx* ctx, PaTiming* t) {
   return PA_OK;
 }
 
+// POOLED_ATTN_PREFILL_WIDE selects the 4-wave prefill kernel for measurements; read at every call (a getenv is
+// nothing next to a kernel launch) so that a test can switch it inside one process
+static bool prefill_wide_selected() { return getenv("POOLED_ATTN_PREFILL_WIDE") != nullptr; }
+
 static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, const float* d_q, uint32_t q_stride,
                        const float* d_gate, uint32_t gate_stride, uint32_t base_pos, uint32_t n_cols, void* d_out,
                        uint32_t out_stride, int out_dtype) {
@@ -406,7 +410,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   PaTiming tm;
   if ((rc = prof_pair(ctx, &tm))) return rc;
   if (pl.kernel == 0) HIPCHK(ctx, pa_launch_decode(p, c.head_dim, pl.row_blocks, pl.waves, pl.col_groups, ctx->stream, &tm));
-  else if (getenv("POOLED_ATTN_PREFILL_WIDE")) HIPCHK(ctx, pa_launch_prefill_wide(p, c.head_dim, pl.col_groups, ctx->stream, &tm));
+  else if (prefill_wide_selected()) HIPCHK(ctx, pa_launch_prefill_wide(p, c.head_dim, pl.col_groups, ctx->stream, &tm));
   else HIPCHK(ctx, pa_launch_prefill(p, c.head_dim, pl.row_blocks, pl.col_groups, ctx->stream, &tm));
   if (!direct) HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;
