@@ -350,15 +350,38 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     f4 s[2][NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) { s[0][nb] = (f4){0.f, 0.f, 0.f, 0.f}; s[1][nb] = (f4){0.f, 0.f, 0.f, 0.f}; }
+    {
+      // fragments are fetched FD k-steps ahead of the MFMAs that use them, and the issue order is pinned: left to
+      // itself the compiler waits for each k-step's three LDS reads right before its MFMAs, one LDS latency a step
+      constexpr int FD = HD == 256 ? 1 : 3;
+      h8 a0r[FD], a1r[FD], br[FD][NB];
+      auto fetch = [&](int ks, int slot) __attribute__((always_inline)) {
+        a0r[slot] = *(const h8*)(stage + ln * S::KROW + ks * 64 + kg * 16);
+        a1r[slot] = *(const h8*)(stage + (16 + ln) * S::KROW + ks * 64 + kg * 16);
 #pragma unroll
-    for (int ks = 0; ks < S::KS; ks++) {
-      const h8 a0 = *(const h8*)(stage + ln * S::KROW + ks * 64 + kg * 16);
-      const h8 a1 = *(const h8*)(stage + (16 + ln) * S::KROW + ks * 64 + kg * 16);
+        for (int nb = 0; nb < NB; nb++) br[slot][nb] = *(const h8*)(q_lds + (nb * 16 + ln) * S::QROW + ks * 64 + kg * 16);
+      };
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++) {
-        const h8 b = *(const h8*)(q_lds + (nb * 16 + ln) * S::QROW + ks * 64 + kg * 16);
-        s[0][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b, s[0][nb], 0, 0, 0);
-        s[1][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b, s[1][nb], 0, 0, 0);
+      for (int ks = 0; ks < FD; ks++) fetch(ks, ks);
+#pragma unroll
+      for (int ks = 0; ks < S::KS; ks++) {
+        const h8 a0 = a0r[ks % FD], a1 = a1r[ks % FD];
+        h8 b[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) b[nb] = br[ks % FD][nb];
+        if (ks + FD < S::KS) fetch(ks + FD, ks % FD);
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+          s[0][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b[nb], s[0][nb], 0, 0, 0);
+          s[1][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b[nb], s[1][nb], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int ks = 0; ks < FD; ks++) __builtin_amdgcn_sched_group_barrier(0x100, 2 + NB, 0);
+#pragma unroll
+      for (int ks = 0; ks < S::KS; ks++) {
+        if (ks + FD < S::KS) __builtin_amdgcn_sched_group_barrier(0x100, 2 + NB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
       }
     }
     wave_lds_fence();
@@ -438,14 +461,32 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     wave_lds_fence();
     PA_TP(6);
     // ---- O^T += V^T P^T ----
+    {
+      // the same for the V^T fragments (two transpose reads each), VD blocks ahead
+      constexpr int VD = 4;
+      h4 lor[VD], hir[VD];
+      auto fetch = [&](int db, int slot) __attribute__((always_inline)) {
+        const unsigned char* vp = stage + (4 * kg + (ln >> 2)) * S::VROW + (db * 16 + 4 * (ln & 3)) * 2;
+        lor[slot] = lds_read_tr16(vp);
+        hir[slot] = lds_read_tr16(vp + 16 * S::VROW);
+      };
 #pragma unroll
-    for (int db = 0; db < S::DB; db++) {
-      const unsigned char* vp = stage + (4 * kg + (ln >> 2)) * S::VROW + (db * 16 + 4 * (ln & 3)) * 2;
-      const h4 lo = lds_read_tr16(vp);
-      const h4 hi = lds_read_tr16(vp + 16 * S::VROW);
-      const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+      for (int db = 0; db < VD; db++) fetch(db, db);
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++) acc[db][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pfrag[nb], acc[db][nb], 0, 0, 0);
+      for (int db = 0; db < S::DB; db++) {
+        const h4 lo = lor[db % VD], hi = hir[db % VD];
+        if (db + VD < S::DB) fetch(db + VD, db % VD);
+        const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[db][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pfrag[nb], acc[db][nb], 0, 0, 0);
+      }
+#pragma unroll
+      for (int db = 0; db < VD; db++) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+#pragma unroll
+      for (int db = 0; db < S::DB; db++) {
+        if (db + VD < S::DB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+        __builtin_amdgcn_sched_group_barrier(0x008, NB, 1);
+      }
     }
     wave_lds_fence();
     PA_TP(7);
@@ -476,29 +517,52 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     }
     __syncthreads();
     PA_TP(10);
-    // rows nb*16 .. nb*16+15, HD/4 float4 each, summed over waves in wave order
-    for (uint32_t e = tid; e < 16 * (HD / 4); e += W * 64) {
+    // rows nb*16 .. nb*16+15, HD/4 float4 each, summed over waves in wave order.  Every thread first issues all
+    // its LDS reads (the accumulators are dead, registers are free), then adds and stores: one LDS latency, not one
+    // per element.  The (m, l) of a row is merged by one of the first 16 threads.
+    constexpr int EPT = 16 * (HD / 4) / (W * 64);
+    f4 part[EPT][W];
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+      const uint32_t e = tid + j * W * 64;
+      const uint32_t rr = e / (HD / 4), d4 = e % (HD / 4);
+      if (nb * 16 + rr < R) {
+#pragma unroll
+        for (int w = 0; w < W; w++) part[j][w] = *(const f4*)(stage_all + w * S::STAGE + rr * S::OROW + d4 * 16);
+      }
+    }
+    float mw[W], lw[W];
+    const bool ml_thread = tid < 16 && nb * 16 + tid < R;
+    if (ml_thread) {
+#pragma unroll
+      for (int w = 0; w < W; w++) { mw[w] = mex[w * 16 * NB + nb * 16 + tid]; lw[w] = lex[w * 16 * NB + nb * 16 + tid]; }
+    }
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+      const uint32_t e = tid + j * W * 64;
       const uint32_t rr = e / (HD / 4), d4 = e % (HD / 4);
       const uint32_t r = nb * 16 + rr;
       if (r < R) {
-        f4 o = *(const f4*)(stage_all + rr * S::OROW + d4 * 16);
+        f4 o = part[j][0];
 #pragma unroll
-        for (int w = 1; w < W; w++) o += *(const f4*)(stage_all + w * S::STAGE + rr * S::OROW + d4 * 16);
+        for (int w = 1; w < W; w++) o += part[j][w];
         const uint32_t col = c0 + r / G, hq = g * G + r % G;
         const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
         *(f4*)(p.part_o + slot * HD + 4 * d4) = o;
-        if (d4 == 0) {
-          float Mr = NEG_INF;
-#pragma unroll
-          for (int w = 0; w < W; w++) Mr = fmaxf(Mr, mex[w * 16 * NB + r]);
-          const float ms = Mr == NEG_INF ? 0.f : Mr;
-          float L = 0.f;
-#pragma unroll
-          for (int w = 0; w < W; w++) L += lex[w * 16 * NB + r] * __expf(mex[w * 16 * NB + r] - ms);
-          p.part_ml[slot * 2] = Mr;
-          p.part_ml[slot * 2 + 1] = L;
-        }
       }
+    }
+    if (ml_thread) {
+      const uint32_t r = nb * 16 + tid;
+      float Mr = NEG_INF;
+#pragma unroll
+      for (int w = 0; w < W; w++) Mr = fmaxf(Mr, mw[w]);
+      const float ms = Mr == NEG_INF ? 0.f : Mr;
+      float L = 0.f;
+#pragma unroll
+      for (int w = 0; w < W; w++) L += lw[w] * __expf(mw[w] - ms);
+      const uint32_t col = c0 + r / G, hq = g * G + r % G;
+      const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
+      *(float2*)(p.part_ml + slot * 2) = make_float2(Mr, L);
     }
     if (nb + 1 < NB) __syncthreads();                                  // the regions are rewritten by the next row block
   }
