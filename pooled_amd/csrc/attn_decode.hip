@@ -66,6 +66,30 @@ static __device__ inline void dq16(const u4 raw, const float sc, h8& lo, h8& hi)
   hi = (h8){ o[4][0], o[4][1], o[5][0], o[5][1], o[6][0], o[6][1], o[7][0], o[7][1] };
 }
 
+// Fused pre-step of N query heads of one wave (heads wave, wave + W, ...): norm + rope side by side, then the heads
+// as f16 rows of the q tile.  xs: wave-private LDS scratch of N x HD floats.
+template <int N, int HD, int W, int QROW>
+static __device__ inline void fused_q_rows(const float (&xq)[16 / W][4], const float (&wq)[4], bool norm, float eps, uint32_t half,
+                                           const float2 (&cs)[2], float* xs, unsigned char* q_lds, uint32_t G, uint32_t wave, uint32_t lane) {
+  static_assert(N <= 16 / W, "at most 16 query heads per kv head");
+  float x[N][4];
+#pragma unroll
+  for (int n = 0; n < N; n++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) x[n][j] = xq[n][j];
+  glue_heads_wave<N>(x, wq, norm, eps, HD, half, cs, xs, HD, lane);
+#pragma unroll
+  for (int n = 0; n < N; n++) {
+    const uint32_t r = wave + W * n;
+    if (r < G && lane < HD / 4) {
+      const f4 v = *(const f4*)(xs + n * HD + 4 * lane);
+      const h4 hv = { (_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3] };
+      *(h4*)(q_lds + r * QROW + lane * 8) = hv;
+    }
+  }
+  wave_lds_fence();
+}
+
 template <int HD> struct DecShape {
   static constexpr int LPR = HD / 8;            // lanes per f16 row at 16 bytes a lane
   static constexpr int RPL = 64 / LPR;          // rows per wave-wide load
@@ -85,10 +109,13 @@ template <int HD> struct DecShape {
   static constexpr int DB = HD / 16;            // 16-dim blocks of the output
 };
 
-// FUSED: the workgroup also runs the pre-step of its kv head for the one column at base_pos (n_cols == 1, NB == 1):
-// its G query heads are normed and roped from the raw projection on the way into LDS, and the wave whose tile
-// holds position base_pos norms / ropes the new key row, writes it and the value row to the cache and patches them
-// into its staged tile (the tile's own load of that row raced the write and is discarded).
+// FUSED: the workgroup also runs the pre-step of its kv head for the one column at base_pos (n_cols == 1, NB == 1,
+// self_row set): its G query heads are normed and roped from the raw projection on the way into LDS, and wave 0 of
+// split 0 norms / ropes the new key row and writes it and the value row to the cache.
+//
+// self_row (every one-column decode on f16 caches, fused or not): the column's own row base_pos is not streamed with
+// rows 0 .. base_pos - 1; wave 0 of split 0 holds it in registers (from the pre-step above, or loaded), scores it
+// against the G query rows and writes it as one more split partial, which the merge kernel folds in like any other.
 //
 // GATHER (the reference's attn_dec_qsa, engine/wgsl/attn_dec.js:33-38, :105, :170-183): each column attends to a
 // list of cache rows instead of rows 0 .. seqLen - 1.  Column col's list is sel[col * sel_stride] = n, then n row
@@ -102,8 +129,14 @@ template <int HD> struct DecShape {
 // pick the scale of each of its 16-value pieces, and the pieces are widened to f16 on their way into the staged
 // tile -- int8 -> f16 through the 0x6400 | (v + 128) bit pattern (= 1152 + v exactly), a packed subtract and a
 // packed multiply by the f16-rounded scale.  From there on (MFMA, softmax, merge) it is the f16 kernel.
-template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8>
+//
+// SR (single-round splits; one 16-row block): splits are one tile per wave (split_len = W x 32) and a workgroup takes
+// splits blockIdx.x, blockIdx.x + gridDim.x, ... one after the other, each with a partial of its own; the product
+// O^T = V^T P^T of a split is divided over the waves by output dims, see the code.  Without SR a workgroup owns one
+// split of any length and every wave loops over its own tiles.
+template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
 __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
+  static_assert(!SR || NB == 1, "single-round splits: one 16-row block");
   static_assert(!FUSED || NB == 1, "the fused pre-step serves one column");
   static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
   static_assert(!Q8 || (!FUSED && !GATHER), "int8 caches: plain decode / verify only");
@@ -123,11 +156,16 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   const uint32_t R = ncl * G;                                        // live rows (<= 16*NB)
   const uint32_t sel_base = GATHER ? c0 * p.sel_stride + 1 : 0;      // gather: first list entry of this column
   // rows visible to the group's last column (gather: the column's list length)
-  const uint32_t seq_max = GATHER ? p.sel[c0 * p.sel_stride] : p.base_pos + c0 + ncl;
-  const uint32_t t_begin = sp * p.split_len;
-  if (t_begin >= seq_max) return;
+  // self_row (one-column decode): the column's own row base_pos is not streamed with the others -- see below
+  const uint32_t seq_max = GATHER ? p.sel[c0 * p.sel_stride] : p.base_pos + c0 + ncl - p.self_row;
+  uint32_t t_begin = sp * p.split_len;                               // SR: of the workgroup's current split
+  // The workgroup of split 0 turns the column's own row into a partial of its own (wave 0, while the tile loads are
+  // in flight), so it runs even when no other row exists (base_pos == 0).
+  const bool self_wg = !GATHER && !Q8 && p.self_row && sp == 0;
+  if (t_begin >= seq_max && !self_wg) return;
+  const bool has_rows = t_begin < seq_max;
   // the last split is open-ended: the plan may hand it up to one split length of remainder
-  const uint32_t t_end = sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
+  uint32_t t_end = !SR && sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
   const size_t head_rows = (size_t)p.max_seq + TILE;              // rows of one kv head's plane, padding included
   PA_TP(0);
 
@@ -147,19 +185,20 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   const unsigned char* vsbase = (const unsigned char*)(p.v_scale + (Q8 ? (size_t)g * head_rows * S::SPR : 0));
   u4 ksr = {0u, 0u, 0u, 0u}, vsr = {0u, 0u, 0u, 0u};
 
-  f4 acc[S::DB][NB];
-#pragma unroll
-  for (int db = 0; db < S::DB; db++)
-#pragma unroll
-    for (int nb = 0; nb < NB; nb++) acc[db][nb] = (f4){0.f, 0.f, 0.f, 0.f};
-  float m_run[NB], l_run[NB];
-#pragma unroll
-  for (int nb = 0; nb < NB; nb++) { m_run[nb] = NEG_INF; l_run[nb] = 0.f; }
-
-  const uint32_t n_tiles = (t_end - t_begin + TILE - 1) / TILE;
+  uint32_t n_tiles = has_rows ? (t_end - t_begin + TILE - 1) / TILE : 0;
   u4 kr[S::NLD], vr[S::NLD];
   const u4 zero4 = {0u, 0u, 0u, 0u};
 
+  // the column's own K / V row, 4 dims a lane: loaded here (the pre-step wrote it), or made below by the fused pre-step
+  const bool self_wave = self_wg && wave == 0;
+  h4 kx = {0, 0, 0, 0}, vx = {0, 0, 0, 0};
+  if constexpr (!FUSED && !GATHER && !Q8) {
+    if (self_wave) {
+      const size_t ro = (size_t)p.base_pos * row_bytes + min(lane, (uint32_t)HD / 4 - 1) * 8;
+      kx = *(const h4*)(kbase + ro);
+      vx = *(const h4*)(vbase + ro);
+    }
+  }
   // q loads first (they return first), then the first tile's K/V loads; staging q below overlaps the K/V latency.
   constexpr int QPT = 16 * NB * (HD / 4) / (W * 64);               // float4 of q per thread
   constexpr int HPW = 16 / W;                                      // fused: query heads per wave (G <= 16)
@@ -222,7 +261,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     }
   };
   {
-    const uint32_t t0 = t_begin + min(tile, n_tiles - 1) * TILE;
+    const uint32_t t0 = t_begin + min(tile, max(n_tiles, 1u) - 1) * TILE;
     if constexpr (GATHER) {
       gather_offsets(t0);
 #pragma unroll
@@ -248,39 +287,26 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   PA_TP(1);
   __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the K/V load issue
   // ---- q -> f16 rows in LDS; waits only for the q loads, which were issued first ----
-  h4 kpatch = {0, 0, 0, 0}, vpatch = {0, 0, 0, 0};
-  bool own_pos = false;              // this wave's tile sequence holds position base_pos
-  uint32_t pos_tile = 0;
   if constexpr (FUSED) {
     float* xs = (float*)stage;       // wave-private scratch (the staging region is not in use yet)
-#pragma unroll
-    for (int t = 0; t < HPW; t++) {
-      const uint32_t r = wave + W * t;
-      if (r < G) {
-        glue_head_wave(xq[t], wq, p.f_qw != nullptr, p.eps, HD, half, cs, xs, lane);
-        if (lane < HD / 4) {
-          const f4 v = *(const f4*)(xs + 4 * lane);
-          const h4 hv = { (_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3] };
-          *(h4*)(q_lds + r * S::QROW + lane * 8) = hv;
-        }
-        wave_lds_fence();
-      }
+    // this wave's query heads wave, wave + W, ... side by side (ceil(G / W) of them; one past G is computed and dropped)
+    switch ((G + W - 1) / W) {
+      case 1: fused_q_rows<1, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
+      case 2: fused_q_rows<2, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
+      case 3: fused_q_rows<3, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
+      default: fused_q_rows<4, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
     }
     for (uint32_t e = tid; e < (16 - G) * (HD / 4); e += W * 64)     // padding rows (masked out later)
       *(h4*)(q_lds + (G + e / (HD / 4)) * S::QROW + (e % (HD / 4)) * 8) = (h4){0, 0, 0, 0};
-    if (p.base_pos >= t_begin && p.base_pos < t_end) {
-      pos_tile = (p.base_pos - t_begin) / TILE;
-      own_pos = pos_tile % W == wave;
-    }
-    if (own_pos) {
+    if (self_wave) {                 // the new key row: normed, roped, rounded; it and the value row go to the cache
       glue_head_wave(xk, wk, p.f_kw != nullptr, p.eps, HD, half, cs, xs, lane);
       if (lane < HD / 4) {
         const f4 v = *(const f4*)(xs + 4 * lane);
-        kpatch = (h4){ (_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3] };
-        vpatch = (h4){ (_Float16)xv4[0], (_Float16)xv4[1], (_Float16)xv4[2], (_Float16)xv4[3] };
+        kx = (h4){ (_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3] };
+        vx = (h4){ (_Float16)xv4[0], (_Float16)xv4[1], (_Float16)xv4[2], (_Float16)xv4[3] };
         const size_t ro = ((size_t)g * head_rows + p.base_pos) * HD + 4 * lane;
-        *(h4*)((_Float16*)const_cast<uint16_t*>(p.k_cache) + ro) = kpatch;
-        *(h4*)((_Float16*)const_cast<uint16_t*>(p.v_cache) + ro) = vpatch;
+        *(h4*)((_Float16*)const_cast<uint16_t*>(p.k_cache) + ro) = kx;
+        *(h4*)((_Float16*)const_cast<uint16_t*>(p.v_cache) + ro) = vx;
       }
       wave_lds_fence();
     }
@@ -298,16 +324,37 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     const uint32_t r = nb * 16 + ln;
-    end_pos[nb] = r < R ? (GATHER ? seq_max : p.base_pos + c0 + r / G + 1) : 0u;
+    end_pos[nb] = r < R ? (GATHER ? seq_max : p.base_pos + c0 + r / G + 1 - p.self_row) : 0u;
   }
   __syncthreads();
   PA_TP(2);
+  // ---- the column's own row as a partial of its own (slot = number of splits that hold rows): m = its score,
+  // l = 1, O = its value row.  The scores run on the VALU over the f16 operands the MFMA path would see, f32 sums in a
+  // fixed order; the work hides under the latency of the tile loads.  Decoding a token at a position that is a
+  // multiple of the split length therefore streams whole tiles only.
+  if (self_wave) {
+    const uint32_t self_slot = min((seq_max + p.split_len - 1) / p.split_len, p.n_splits);
+    const bool on = lane < HD / 4;
+    const f4 vxf = { (float)vx[0], (float)vx[1], (float)vx[2], (float)vx[3] };
+    for (uint32_t r = 0; r < G; r++) {                                 // one column: row r is head g * G + r
+      const h4 qv = *(const h4*)(q_lds + r * S::QROW + min(lane, (uint32_t)HD / 4 - 1) * 8);
+      float d = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; i++) d = __builtin_fmaf((float)qv[i], (float)kx[i], d);
+      if (!on) d = 0.f;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+      const size_t slot = ((size_t)c0 * nH + g * G + r) * p.slots + self_slot;
+      if (on) *(f4*)(p.part_o + slot * HD + 4 * lane) = vxf;
+      if (lane == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(d * p.scale, 1.f);
+    }
+  }
+  if (!has_rows) return;
 
-  for (; tile < n_tiles; tile += W) {
-    const uint32_t tp = t_begin + tile * TILE;
-    const size_t tnb = (size_t)(tp + W * TILE) * row_bytes;   // next tile of this wave
-    const bool more = tile + W < n_tiles;
-    // ---- K tile -> LDS, next K loads ----
+  // The three staging / product steps of a tile, shared by the tile loop and the single-round path below.
+  // stage_k: the K registers of the tile at position tp -> LDS (int8: widened), then the loads of the wave's next tile.
+  auto stage_k = [&](const uint32_t tp, const bool more, const uint32_t tpn) __attribute__((always_inline)) {
+    const size_t tnb = (size_t)tpn * row_bytes;               // next tile of this wave
     if constexpr (Q8) {
       if (lane / S::LPS < TILE) *(u4*)(stage + soff) = ksr;          // the tile's scales, [row][SPR] f32
       wave_lds_fence();
@@ -323,10 +370,10 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
         *(h8*)d = lo; *(h8*)(d + 16) = hi;
       }
       if (more) {
-        const size_t tb = (size_t)(tp + W * TILE) * HD;
+        const size_t tb = (size_t)tpn * HD;
 #pragma unroll
         for (int i = 0; i < S::NLD8; i++) kr[i] = *(const u4*)(kbase8 + tb + (size_t)(i * S::RPL8) * HD + voff8);
-        ksr = *(const u4*)(ksbase + (size_t)(tp + W * TILE) * S::SPR * 4 + soff);
+        ksr = *(const u4*)(ksbase + (size_t)tpn * S::SPR * 4 + soff);
       }
     } else {
 #pragma unroll
@@ -334,7 +381,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     }
     if (!Q8 && more) {
       if constexpr (GATHER) {
-        gather_offsets(tp + W * TILE);
+        gather_offsets(tpn);
 #pragma unroll
         for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
       } else {
@@ -342,12 +389,10 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
         for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
       }
     }
-    if (FUSED && own_pos && tile == pos_tile && lane < HD / 4)      // the new key row (in-order LDS: lands after the staged copy)
-      *(h4*)(stage + (p.base_pos - tp) * S::KROW + lane * 8) = kpatch;
     wave_lds_fence();
-    PA_TP(3);
-    // ---- S^T = K Q^T ----
-    f4 s[2][NB];
+  };
+  // qk: S^T = K Q^T of the staged tile
+  auto qk = [&](f4 (&s)[2][NB]) __attribute__((always_inline)) {
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) { s[0][nb] = (f4){0.f, 0.f, 0.f, 0.f}; s[1][nb] = (f4){0.f, 0.f, 0.f, 0.f}; }
     {
@@ -385,6 +430,178 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       }
     }
     wave_lds_fence();
+  };
+  // stage_v: the V registers -> LDS (rows at or past t_end as zeros: 0 x stale bits must not reach O), next V loads;
+  // the caller fences
+  auto stage_v = [&](const uint32_t tp, const bool more, const uint32_t tpn) __attribute__((always_inline)) {
+    const size_t tnb = (size_t)tpn * row_bytes;
+    if constexpr (Q8) {
+      if (lane / S::LPS < TILE) *(u4*)(stage + soff) = vsr;
+      wave_lds_fence();
+      float sc[S::NLD8];
+#pragma unroll
+      for (int i = 0; i < S::NLD8; i++) sc[i] = *(const float*)(stage + ((i * S::RPL8 + lrow8) * S::SPR + (lane % S::LPR8) / 2) * 4);
+      wave_lds_fence();
+#pragma unroll
+      for (int i = 0; i < S::NLD8; i++) {
+        h8 lo, hi;
+        dq16(vr[i], sc[i], lo, hi);
+        if (tp + i * S::RPL8 + lrow8 >= t_end) { lo = (h8){0, 0, 0, 0, 0, 0, 0, 0}; hi = lo; }   // also rows whose scale is not a number
+        unsigned char* d = stage + (i * S::RPL8 + lrow8) * S::VROW + (lane % S::LPR8) * 32;
+        *(h8*)d = lo; *(h8*)(d + 16) = hi;
+      }
+      if (more) {
+        const size_t tb = (size_t)tpn * HD;
+#pragma unroll
+        for (int i = 0; i < S::NLD8; i++) vr[i] = *(const u4*)(vbase8 + tb + (size_t)(i * S::RPL8) * HD + voff8);
+        vsr = *(const u4*)(vsbase + (size_t)tpn * S::SPR * 4 + soff);
+      }
+    } else {
+    if (tp + TILE > t_end) {
+#pragma unroll
+      for (int i = 0; i < S::NLD; i++) if (tp + i * S::RPL + lrow >= t_end) vr[i] = zero4;
+    }
+#pragma unroll
+    for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
+    }
+    if (!Q8 && more) {
+      if constexpr (GATHER) {                         // goff still holds the next tile's rows (set with the K loads above)
+#pragma unroll
+        for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
+      } else {
+#pragma unroll
+        for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
+      }
+    }
+  };
+
+  // ---- SR: the product O^T = V^T P^T of a split is divided over the waves by OUTPUT DIMS instead of by positions.
+  // Every wave scores its own tile (own maximum m_w, probabilities P_w relative to it), publishes P_w -- in the 32
+  // padding bytes of its staged V rows -- and (m_w, l_w); after one barrier wave w multiplies all tiles' V^T by their
+  // P for dims [w * HD/W, (w + 1) * HD/W), re-weights the per-tile products by exp(m_w' - M) in registers and stores
+  // its slice of the split's partial.  Nothing but P crosses waves, so the tail after the last V bytes is one barrier,
+  // the MFMAs and a store (the tile loop further down merges the waves' O through LDS: two more LDS round trips).
+  if constexpr (SR) {
+    constexpr int DBW = S::DB / W;                                      // 16-dim output blocks per wave
+    for (uint32_t split = sp;;) {
+      const uint32_t nsplit = split + gridDim.x;                        // this workgroup's next split, if any
+      const uint32_t nb_begin = nsplit * p.split_len;
+      const bool more = nb_begin < seq_max;
+      const uint32_t n_tiles_next = more ? (min(nb_begin + p.split_len, seq_max) - nb_begin + TILE - 1) / TILE : 1;
+      const uint32_t tpn = nb_begin + min(wave, n_tiles_next - 1) * TILE;
+      const bool has_tile = wave < n_tiles;
+      const uint32_t tp = t_begin + min(wave, n_tiles - 1) * TILE;      // the tile this wave holds in registers
+      stage_k(tp, more, tpn);
+      PA_TP(3);
+      f4 s[2][NB];
+      qk(s);
+      PA_TP(4);
+      const uint32_t row_end = has_tile ? end_pos[0] : 0u;              // a wave without a tile contributes nothing
+      float v[8], mx = NEG_INF;
+#pragma unroll
+      for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const uint32_t pos = tp + pb * 16 + 4 * kg + i;
+          const float x = pos < row_end ? s[pb][0][i] * p.scale : NEG_INF;
+          v[pb * 4 + i] = x;
+          mx = fmaxf(mx, x);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mw_safe = mx == NEG_INF ? 0.f : mx;
+      float ps = 0.f;
+      h8 pf;
+#pragma unroll
+      for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
+      ps += __shfl_xor(ps, 16, 64);
+      ps += __shfl_xor(ps, 32, 64);
+      stage_v(tp, more, tpn);
+      *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pf;
+      if (kg == 0) { mex[wave * 16 + ln] = mx; lex[wave * 16 + ln] = ps; }
+      PA_TP(5);
+      __syncthreads();
+      PA_TP(6);
+      {
+        // V^T fragments (two transpose reads each) and the tile's P are fetched VD steps ahead of their MFMA
+        constexpr int NS = W * DBW, VD = 4;
+        h4 lor[VD], hir[VD];
+        h8 pfr[VD];
+        f4 pr[W][DBW];
+        auto fetch = [&](int st, int slot) __attribute__((always_inline)) {
+          const int w2 = st / DBW, db = wave * DBW + st % DBW;
+          const unsigned char* sw = stage_all + w2 * S::STAGE;
+          const unsigned char* vp = sw + (4 * kg + (ln >> 2)) * S::VROW + (db * 16 + 4 * (ln & 3)) * 2;
+          lor[slot] = lds_read_tr16(vp);
+          hir[slot] = lds_read_tr16(vp + 16 * S::VROW);
+          pfr[slot] = *(const h8*)(sw + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16);
+        };
+#pragma unroll
+        for (int st = 0; st < VD; st++) fetch(st, st);
+#pragma unroll
+        for (int st = 0; st < NS; st++) {
+          const h4 lo = lor[st % VD], hi = hir[st % VD];
+          const h8 pb = pfr[st % VD];
+          if (st + VD < NS) fetch(st + VD, st % VD);
+          const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+          pr[st / DBW][st % DBW] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pb, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        }
+#pragma unroll
+        for (int st = 0; st < VD; st++) __builtin_amdgcn_sched_group_barrier(0x100, 3, 1);
+#pragma unroll
+        for (int st = 0; st < NS; st++) {
+          if (st + VD < NS) __builtin_amdgcn_sched_group_barrier(0x100, 3, 1);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+        }
+        // a wave without a tile staged stale rows: its m is -inf, and its products must not reach O even as 0 x NaN
+        float mw[W], lw[W], M = NEG_INF;
+#pragma unroll
+        for (int w2 = 0; w2 < W; w2++) { mw[w2] = mex[w2 * 16 + ln]; lw[w2] = lex[w2 * 16 + ln]; M = fmaxf(M, mw[w2]); }
+        const float m_safe = M == NEG_INF ? 0.f : M;
+        float Lr = 0.f;
+        f4 o[DBW];
+#pragma unroll
+        for (int j = 0; j < DBW; j++) o[j] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w2 = 0; w2 < W; w2++) {
+          const bool dead = mw[w2] == NEG_INF;
+          const float c = dead ? 0.f : __expf(mw[w2] - m_safe);
+          Lr += lw[w2] * c;
+#pragma unroll
+          for (int j = 0; j < DBW; j++) o[j] += (dead ? (f4){0.f, 0.f, 0.f, 0.f} : pr[w2][j]) * c;
+        }
+        PA_TP(7); PA_TP(8); PA_TP(10);
+        if (ln < R) {
+          const uint32_t col = c0 + ln / G, hq = g * G + ln % G;
+          const size_t slot = ((size_t)col * nH + hq) * p.slots + split;
+#pragma unroll
+          for (int j = 0; j < DBW; j++) *(f4*)(p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = o[j];
+          if (wave == 0 && kg == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(M, Lr);
+        }
+      }
+      if (!more) break;
+      __syncthreads();                                                  // the staged tiles and (m, l) are rewritten
+      split = nsplit; t_begin = nb_begin; t_end = min(t_begin + p.split_len, seq_max); n_tiles = n_tiles_next;
+    }
+    PA_TP(9);
+    return;
+  }
+  // ---- tile loop: every wave streams its own tiles and keeps its own (m, l, O) ----
+  f4 acc[S::DB][NB];
+#pragma unroll
+  for (int db = 0; db < S::DB; db++)
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) acc[db][nb] = (f4){0.f, 0.f, 0.f, 0.f};
+  float m_run[NB], l_run[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) { m_run[nb] = NEG_INF; l_run[nb] = 0.f; }
+  for (; tile < n_tiles; tile += W) {
+    const uint32_t tp = t_begin + tile * TILE;
+    const bool more = tile + W < n_tiles;
+    stage_k(tp, more, tp + W * TILE);
+    PA_TP(3);
+    f4 s[2][NB];
+    qk(s);
     PA_TP(4);
     // ---- online softmax; lane holds row nb*16 + ln, positions tp + pb*16 + 4*kg + i ----
     h8 pfrag[NB];
@@ -416,47 +633,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
 #pragma unroll
       for (int db = 0; db < S::DB; db++) acc[db][nb] *= alpha;
     }
-    // ---- V tile -> LDS, after the softmax so that the wait for the V loads comes as late as possible (rows at or past t_end as zeros: 0 x stale bits must not reach O), next V loads ----
-    if constexpr (Q8) {
-      if (lane / S::LPS < TILE) *(u4*)(stage + soff) = vsr;
-      wave_lds_fence();
-      float sc[S::NLD8];
-#pragma unroll
-      for (int i = 0; i < S::NLD8; i++) sc[i] = *(const float*)(stage + ((i * S::RPL8 + lrow8) * S::SPR + (lane % S::LPR8) / 2) * 4);
-      wave_lds_fence();
-#pragma unroll
-      for (int i = 0; i < S::NLD8; i++) {
-        h8 lo, hi;
-        dq16(vr[i], sc[i], lo, hi);
-        if (tp + i * S::RPL8 + lrow8 >= t_end) { lo = (h8){0, 0, 0, 0, 0, 0, 0, 0}; hi = lo; }   // also rows whose scale is not a number
-        unsigned char* d = stage + (i * S::RPL8 + lrow8) * S::VROW + (lane % S::LPR8) * 32;
-        *(h8*)d = lo; *(h8*)(d + 16) = hi;
-      }
-      if (more) {
-        const size_t tb = (size_t)(tp + W * TILE) * HD;
-#pragma unroll
-        for (int i = 0; i < S::NLD8; i++) vr[i] = *(const u4*)(vbase8 + tb + (size_t)(i * S::RPL8) * HD + voff8);
-        vsr = *(const u4*)(vsbase + (size_t)(tp + W * TILE) * S::SPR * 4 + soff);
-      }
-    } else {
-    if (tp + TILE > t_end) {
-#pragma unroll
-      for (int i = 0; i < S::NLD; i++) if (tp + i * S::RPL + lrow >= t_end) vr[i] = zero4;
-    }
-#pragma unroll
-    for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
-    }
-    if (!Q8 && more) {
-      if constexpr (GATHER) {                         // goff still holds the next tile's rows (set with the K loads above)
-#pragma unroll
-        for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
-      } else {
-#pragma unroll
-        for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tnb + (size_t)(i * S::RPL) * row_bytes + voff);
-      }
-    }
-    if (FUSED && own_pos && tile == pos_tile && lane < HD / 4)      // the new value row
-      *(h4*)(stage + (p.base_pos - tp) * S::VROW + lane * 8) = vpatch;
+    // V after the softmax, so that the wait for the V loads comes as late as possible
+    stage_v(tp, more, tp + W * TILE);
     PA_TP(5);
     wave_lds_fence();
     PA_TP(6);
@@ -573,19 +751,20 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
 // One workgroup per (head, 64-dim slice, column) -- the reference's layout (engine/wgsl/attn_dec.js:215-287,
 // DEC_CQ slices per head) -- so the merge of a decode token runs on nH * HD/64 workgroups instead of nH.
 // 256 threads = 16 split groups x 16 float4 lanes.  The kernel is latency-bound (a few KB per workgroup, read
-// once, from the memory side), so it is written as one round trip: a thread issues all 16 output-partial loads of
-// its first 256-split chunk and its (m, l) loads before anything waits; the maximum and the weighted sum of l are
+// once, from the memory side), so it is written as one round trip: a thread issues all 17 output-partial loads of
+// its first 272-split chunk and its (m, l) loads before anything waits; the maximum and the weighted sum of l are
 // fixed-order tree reductions, a group's splits are accumulated in split order and the 16 groups in group order.
 template <int HD>
 __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
-  constexpr int CQ = HD / 64, CH = 16;      // CH loads in flight per thread = 256 splits per chunk
+  constexpr int CQ = HD / 64, CH = 17;      // CH loads in flight per thread = 272 splits per chunk (256 + the own-row partial)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* wl = (float*)smem;                 // [slots] split weights exp(m_s - M)
   __shared__ float red[256];
   __shared__ f4 ored[256];
   const uint32_t h = blockIdx.x / CQ, dq = blockIdx.x % CQ, col = blockIdx.y, tid = threadIdx.x;
-  const uint32_t col_end = p.sel ? p.sel[col * p.sel_stride] : p.base_pos + col + 1;   // gather: the column's list length
-  const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits);   // the last split is open-ended
+  const uint32_t col_end = p.sel ? p.sel[col * p.sel_stride] : p.base_pos + col + 1 - p.self_row;   // gather: the column's list length
+  // the last split is open-ended; a one-column decode's own row is one more partial after the splits that hold rows
+  const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
   const uint32_t grp = tid >> 4, l4 = tid & 15;
   const float* po = p.part_o + base * HD + dq * 64 + 4 * l4;
@@ -600,10 +779,11 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   const uint32_t d_out = dq * 64 + 4 * (tid & 15);
   f4 gt = zero;
   if (p.gate && tid < 16) gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d_out);
-  // (m, l) of this thread's first split; further ones (more than 256 splits) in the loops below
+  // (m, l) of this thread's first two splits; further ones (more than 512 splits) in the loops below
   const float2 ml0 = tid < ns ? *(const float2*)(p.part_ml + (base + tid) * 2) : make_float2(NEG_INF, 0.f);
-  float lm = ml0.x;
-  for (uint32_t s = tid + 256; s < ns; s += 256) lm = fmaxf(lm, p.part_ml[(base + s) * 2]);
+  const float2 ml1 = tid + 256 < ns ? *(const float2*)(p.part_ml + (base + tid + 256) * 2) : make_float2(NEG_INF, 0.f);
+  float lm = fmaxf(ml0.x, ml1.x);
+  for (uint32_t s = tid + 512; s < ns; s += 256) lm = fmaxf(lm, p.part_ml[(base + s) * 2]);
   // maximum: xor-shuffle tree inside each wave, then the 4 waves' values in wave order
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) lm = fmaxf(lm, __shfl_xor(lm, o, 64));
@@ -612,7 +792,8 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   float ll = 0.f;
   if (tid < ns) { const float w = __expf(ml0.x - M); wl[tid] = w; ll = ml0.y * w; }
-  for (uint32_t s = tid + 256; s < ns; s += 256) {
+  if (tid + 256 < ns) { const float w = __expf(ml1.x - M); wl[tid + 256] = w; ll += ml1.y * w; }
+  for (uint32_t s = tid + 512; s < ns; s += 256) {
     const float w = __expf(p.part_ml[(base + s) * 2] - M);
     wl[s] = w;
     ll += p.part_ml[(base + s) * 2 + 1] * w;
@@ -628,7 +809,7 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
     const uint32_t s = grp + 16 * k;
     if (s < ns) o += ov[k] * wl[s];
   }
-  for (uint32_t s0 = 16 * CH; s0 < ns; s0 += 16 * CH) {          // contexts with more than 256 splits
+  for (uint32_t s0 = 16 * CH; s0 < ns; s0 += 16 * CH) {          // contexts with more than 272 splits
 #pragma unroll
     for (int k = 0; k < CH; k++) {
       const uint32_t s = s0 + grp + 16 * k;
@@ -671,8 +852,8 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
   const size_t ch = e / (HD / 4);
   if (ch >= (size_t)p.n_cols * p.n_heads) return;
   const uint32_t col = (uint32_t)(ch / p.n_heads), h = (uint32_t)(ch % p.n_heads);
-  const uint32_t col_end = p.sel ? p.sel[col * p.sel_stride] : p.base_pos + col + 1;
-  const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits);
+  const uint32_t col_end = p.sel ? p.sel[col * p.sel_stride] : p.base_pos + col + 1 - p.self_row;
+  const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
   const size_t base = ch * p.slots;
   const float* po = p.part_o + base * HD + 4 * d4;
   float M = NEG_INF;
@@ -699,18 +880,29 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
   }
 }
 
-template <int HD, int NB, int W, bool FUSED, bool GATHER = false, bool Q8 = false>
-static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
+template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
+static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   typedef DecShape<HD> S;
   const size_t lds = 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
+  const uint32_t gx = SR && p.n_wgs ? p.n_wgs : p.n_splits;
+  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), dim3(gx, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
   return hipGetLastError();
+}
+
+// one 16-row block with splits of one tile per wave: the single-round kernel (a workgroup may take several splits)
+template <int HD, int NB, int W, bool FUSED, bool GATHER = false, bool Q8 = false>
+static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
+  if constexpr (NB == 1) {
+    if (p.split_len == W * TILE) return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, true>(p, col_groups, s, t);
+  }
+  if (p.n_wgs && p.n_wgs != p.n_splits) return hipErrorInvalidValue;   // only the single-round kernel loops over splits
+  return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, false>(p, col_groups, s, t);
 }
 
 template <int HD>
@@ -741,7 +933,7 @@ hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint3
 }
 
 hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t) {
-  if (!p.f_q_in || p.n_cols != 1 || p.group > 16) return hipErrorInvalidValue;
+  if (!p.f_q_in || p.n_cols != 1 || p.group > 16 || !p.self_row) return hipErrorInvalidValue;
   if (hd == 256) return launch_decode_t<256, 1, 4, true>(p, 1, s, t);
   if (hd == 128) return launch_decode_t<128, 1, 4, true>(p, 1, s, t);
   return hipErrorInvalidValue;

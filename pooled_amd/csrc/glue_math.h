@@ -21,10 +21,25 @@ static __device__ inline void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Sum over the 64 lanes, the same value in every lane, in a fixed order: quads, half rows and rows through DPP
+// lane permutations (a lane adds its partner's value, so both partners end up with the same bits), then the four
+// row sums as (r0 + r1) + (r2 + r3).  No LDS traffic: 8 moves + 4 adds + 8 lane reads, against 12 dependent
+// ds_bpermute round trips for a shuffle butterfly.
+template <int CTRL> static __device__ inline double dpp_f64(double v) {
+  int lo = __double2loint(v), hi = __double2hiint(v);
+  lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, 0xF, 0xF, false);
+  hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, 0xF, 0xF, false);
+  return __hiloint2double(hi, lo);
+}
+static __device__ inline double readlane_f64(double v, int l) {
+  return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), l), __builtin_amdgcn_readlane(__double2loint(v), l));
+}
 static __device__ inline double wave_sum_f64(double v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+  v += dpp_f64<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  v += dpp_f64<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  v += dpp_f64<0x141>(v);     // row_half_mirror: lane i <-> 7 - i of each 8
+  v += dpp_f64<0x140>(v);     // row_mirror: lane i <-> 15 - i of each 16
+  return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
 }
 
 // c, s of the f32 angle f32(pos) * inv_freq, evaluated in f64 and rounded once
@@ -45,45 +60,72 @@ static __device__ inline float2 rope_pair(const float2* rope_tab, const float* i
   return make_float2(c, s);
 }
 
-// One wavefront, one head of hd <= 256 values: x[j] is element lane + 64 j (0 past hd).  Optional RMSNorm with
-// weights w[j] (of element lane + 64 j; norm == false: none), optional rotation of pairs (i, i + half), i < half,
-// by cs[j] = (cos, sin) of pair lane + 64 j (half == 0: none).  xs is a wave-private LDS scratch of hd floats; on
-// return xs[0, hd) holds the head and the wave's LDS accesses are fenced.
-static __device__ inline void glue_head_wave(const float (&x_in)[4], const float (&w)[4], bool norm, float eps, uint32_t hd,
-                                             uint32_t half, const float2 (&cs)[2], float* xs, uint32_t lane) {
+// One wavefront, N heads of hd <= 256 values side by side (their dependent chains -- reduction, 1 / sqrt, the LDS
+// exchanges -- overlap): x[n][j] is element lane + 64 j of head n (0 past hd).  Optional RMSNorm with weights w[j]
+// (of element lane + 64 j, shared by the heads; norm == false: none), optional rotation of pairs (i, i + half),
+// i < half, by cs[j] = (cos, sin) of pair lane + 64 j (half == 0: none).  xs[n] = xs0 + n * xs_stride is a wave-private LDS
+// scratch of hd floats; on return xs[n][0, hd) holds head n and the wave's LDS accesses are fenced.
+template <int N>
+static __device__ inline void glue_heads_wave(const float (&x_in)[N][4], const float (&w)[4], bool norm, float eps, uint32_t hd,
+                                              uint32_t half, const float2 (&cs)[2], float* xs0, uint32_t xs_stride, uint32_t lane) {
 #pragma clang fp contract(off)
-  float x[4];
-  double ss = 0.0;
+  float* xs[N];
 #pragma unroll
-  for (int j = 0; j < 4; j++) { x[j] = x_in[j]; ss += (double)x[j] * (double)x[j]; }
+  for (int n = 0; n < N; n++) xs[n] = xs0 + n * xs_stride;
+  float x[N][4];
+  double ss[N];
+#pragma unroll
+  for (int n = 0; n < N; n++) {
+    ss[n] = 0.0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) { x[n][j] = x_in[n][j]; ss[n] += (double)x[n][j] * (double)x[n][j]; }
+  }
   if (norm) {
-    ss = wave_sum_f64(ss);
-    const float inv = (float)(1.0 / sqrt(ss / (double)hd + (double)eps));
 #pragma unroll
-    for (int j = 0; j < 4; j++) { const float sw = inv * w[j]; x[j] = x[j] * sw; }
+    for (int n = 0; n < N; n++) ss[n] = wave_sum_f64(ss[n]);
+    float inv[N];
+#pragma unroll
+    for (int n = 0; n < N; n++) inv[n] = (float)(1.0 / sqrt(ss[n] / (double)hd + (double)eps));
+#pragma unroll
+    for (int n = 0; n < N; n++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) { const float sw = inv[n] * w[j]; x[n][j] = x[n][j] * sw; }
   }
 #pragma unroll
-  for (int j = 0; j < 4; j++) { const uint32_t i = lane + 64 * j; if (i < hd) xs[i] = x[j]; }
+  for (int n = 0; n < N; n++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) { const uint32_t i = lane + 64 * j; if (i < hd) xs[n][i] = x[n][j]; }
   wave_lds_fence();
   if (half) {
-    float ra[2], rb[2];
+    float ra[N][2], rb[N][2];
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const uint32_t i = lane + 64 * j;
-      if (i < half) {
-        const float c = cs[j].x, s = cs[j].y;
-        const float a = xs[i], b = xs[i + half];
-        const float ac = a * c, bs = b * s, bc = b * c, as = a * s;   // rounded one by one
-        ra[j] = ac - bs;
-        rb[j] = bc + as;
+    for (int n = 0; n < N; n++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const uint32_t i = lane + 64 * j;
+        if (i < half) {
+          const float c = cs[j].x, s = cs[j].y;
+          const float a = xs[n][i], b = xs[n][i + half];
+          const float ac = a * c, bs = b * s, bc = b * c, as = a * s;   // rounded one by one
+          ra[n][j] = ac - bs;
+          rb[n][j] = bc + as;
+        }
       }
-    }
     wave_lds_fence();
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const uint32_t i = lane + 64 * j;
-      if (i < half) { xs[i] = ra[j]; xs[i + half] = rb[j]; }
-    }
+    for (int n = 0; n < N; n++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const uint32_t i = lane + 64 * j;
+        if (i < half) { xs[n][i] = ra[n][j]; xs[n][i + half] = rb[n][j]; }
+      }
     wave_lds_fence();
   }
+}
+
+// one head
+static __device__ inline void glue_head_wave(const float (&x_in)[4], const float (&w)[4], bool norm, float eps, uint32_t hd,
+                                             uint32_t half, const float2 (&cs)[2], float* xs, uint32_t lane) {
+  const float x1[1][4] = { { x_in[0], x_in[1], x_in[2], x_in[3] } };
+  glue_heads_wave<1>(x1, w, norm, eps, hd, half, cs, xs, 0, lane);
 }

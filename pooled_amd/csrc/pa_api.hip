@@ -273,7 +273,12 @@ extern "C" int pa_kv_store(pa_ctx* ctx, uint32_t layer, const float* d_k, uint32
 // further column groups).  Splits are sized so that about two workgroups (one when the row blocks need the
 // whole register file) land on each CU, but never shorter than the tiles-per-wave floor that keeps the
 // partial (m, l, O) traffic a few percent of the K/V bytes.
-static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl) {
+// self_ok: a one-column decode on f16 caches keeps the column's own row out of the streamed rows (the kernel turns it
+// into one more partial: slots = n_splits + 1), so a token at a multiple of the split length streams whole tiles only.
+static bool plan_self_row(const pa_plan& pl) { return pl.kernel == 0 && pl.slots == pl.n_splits + 1; }
+// wgs (optional): workgroups per kv head and column group that the launch uses; fewer than n_splits when the
+// single-round kernel hands some workgroups a second split.
+static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, bool self_ok = true, uint32_t* wgs = nullptr) {
   const pa_config& c = ctx->cfg;
   const uint32_t G = c.n_heads / c.n_kv_heads;
   // rows per workgroup: 16-row blocks whose O^T accumulators still fit the register file next to the
@@ -283,7 +288,8 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   if (n_cols * G > max_rows) { cw = max_rows / G; if (cw == 0) return PA_ERR_UNSUPPORTED; groups = ceil_div(n_cols, cw); }
   const uint32_t nb = ceil_div(cw * G, 16);
   const uint32_t W = 4;
-  const uint32_t seq_max = base_pos + n_cols;
+  const uint32_t self = self_ok && n_cols == 1 && !kv_q8(ctx) ? 1 : 0;
+  const uint32_t seq_max = std::max(base_pos + n_cols - self, 1u);   // streamed rows (position 0 alone: one empty split)
   const uint32_t tiles = ceil_div(seq_max, 32);
   const uint32_t occ = nb == 1 ? 2 : 1;
   uint32_t target = ctx->decode_splits_override ? ctx->decode_splits_override
@@ -299,8 +305,13 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
     const uint32_t tpw_lo = std::max(tiles / (target * W), floor_tiles[nb]), sl_lo = 32 * W * tpw_lo;
     if ((uint64_t)seq_max < (uint64_t)(target + 1) * sl_lo) { sl = sl_lo; ns = std::max(1u, std::min(target, seq_max / sl_lo)); }
   }
+  uint32_t n_wg = ns;
+  // One 16-row block and one tile per wave: the single-round kernel.  Its splits are all whole (no open-ended last
+  // one); a remainder past the workgroup slots is one more split that the first workgroup takes after its own.
+  if (nb == 1 && sl == 32 * W) { ns = ceil_div(seq_max, sl); n_wg = std::min(ns, target); }
+  if (wgs) *wgs = n_wg;
   pl->kernel = 0; pl->split_len = sl; pl->n_splits = ns;
-  pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = W; pl->row_blocks = nb; pl->slots = pl->n_splits;
+  pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = W; pl->row_blocks = nb; pl->slots = pl->n_splits + self;
   return PA_OK;
 }
 
@@ -308,10 +319,10 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
 // floor(256 / G) columns x G heads.  Chunks wide enough to give every CU a workgroup run unsplit and write the
 // output directly; narrower chunks are also split over the context (partials + merge kernel) until about two
 // workgroups per CU exist.  Chunks of fewer rows than one wavefront tile go to the split-K decode kernel.
-static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl) {
+static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, uint32_t* wgs = nullptr) {
   const pa_config& c = ctx->cfg;
   const uint32_t G = c.n_heads / c.n_kv_heads;
-  if (n_cols * G <= (c.head_dim == 256 ? 32u : 64u)) return plan_decode(ctx, base_pos, n_cols, pl);
+  if (n_cols * G <= (c.head_dim == 256 ? 32u : 64u)) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
   const uint32_t rows_wg = 256;
   const uint32_t cw = rows_wg / G;
   if (cw == 0) return PA_ERR_UNSUPPORTED;
@@ -391,7 +402,8 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   pa_plan pl;
   // int8 caches are served by the split-K kernel only (the reference has no tiled prefill for them either): a
   // prefill chunk then runs as column groups of that kernel
-  rc = (kind == 0 || kv_q8(ctx)) ? plan_decode(ctx, base_pos, n_cols, &pl) : plan_prefill(ctx, base_pos, n_cols, &pl);
+  uint32_t n_wgs = 0;
+  rc = (kind == 0 || kv_q8(ctx)) ? plan_decode(ctx, base_pos, n_cols, &pl, true, &n_wgs) : plan_prefill(ctx, base_pos, n_cols, &pl, &n_wgs);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
   const bool direct = pl.kernel == 1 && pl.n_splits == 1;     // the prefill kernel writes the output itself
@@ -404,6 +416,8 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   p.base_pos = base_pos; p.n_cols = n_cols;
   p.k_scale = ctx->layers[layer].ks; p.v_scale = ctx->layers[layer].vs;
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
+  p.self_row = plan_self_row(pl) ? 1 : 0;
+  p.n_wgs = pl.kernel == 0 ? n_wgs : 0;
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   p.gate_head_stride = c.head_dim;
@@ -443,10 +457,11 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
     return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned");
   if (c.n_heads / c.n_kv_heads > 16) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": more than 16 query heads per kv head");
   pa_plan pl;
-  rc = plan_decode(ctx, pos, 1, &pl);
+  uint32_t n_wgs = 0;
+  rc = plan_decode(ctx, pos, 1, &pl, true, &n_wgs);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
-  if (pl.row_blocks != 1 || pl.waves != 4 || pl.col_groups != 1) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": plan is not a one-block decode");
+  if (pl.row_blocks != 1 || pl.waves != 4 || pl.col_groups != 1 || !plan_self_row(pl)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": plan is not a one-block decode");
   if ((rc = ensure_partials(ctx, 1, pl.slots))) return rc;
   AttnParams p; memset(&p, 0, sizeof p);
   p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
@@ -454,6 +469,7 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
   p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
   p.base_pos = pos; p.n_cols = 1;
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
+  p.self_row = 1; p.n_wgs = n_wgs;
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   // the pre-step inputs; the gate is read in place from the interleaved [q | gate] heads
@@ -531,12 +547,14 @@ extern "C" int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d
   // splits over list positions: the table's choice for one column of max_rows rows (an identity list then runs
   // exactly the dense decode), thinned when several columns share the chip
   pa_plan pl;
-  rc = plan_decode(ctx, max_rows - 1, 1, &pl);
+  uint32_t n_wgs = 0;
+  rc = plan_decode(ctx, max_rows - 1, 1, &pl, false, &n_wgs);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (n_cols > 1 && pl.n_splits > 1) {
     const uint32_t want = std::max(1u, pl.n_splits / n_cols);
     pl.split_len = ceil_div(ceil_div(max_rows, want), 128) * 128;
     pl.n_splits = ceil_div(max_rows, pl.split_len);
+    n_wgs = 0;                                  // one workgroup per split
   }
   pl.slots = pl.n_splits;
   if ((rc = ensure_partials(ctx, n_cols, pl.slots))) return rc;
@@ -550,7 +568,7 @@ extern "C" int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   p.gate_head_stride = c.head_dim;
-  p.sel = d_sel; p.sel_stride = sel_stride;
+  p.sel = d_sel; p.sel_stride = sel_stride; p.n_wgs = n_wgs;
   PaTiming tm;
   if ((rc = prof_pair(ctx, &tm))) return rc;
   HIPCHK(ctx, pa_launch_decode_gather(p, c.head_dim, ctx->stream, &tm));

@@ -37,8 +37,12 @@ struct AttnParams {
   uint32_t n_heads, n_kv_heads, group;        // group = nH / nKV
   uint32_t base_pos, n_cols;                  // column c sees rows [0, base_pos + c]
   uint32_t split_len, n_splits, slots;
+  uint32_t n_wgs;                             // single-round decode kernel: workgroups along x (each takes splits x,
+                                              // x + n_wgs, ...); 0 = n_splits
   uint32_t cols_per_group;                    // columns per workgroup (grid z = column groups)
   uint32_t max_seq;
+  uint32_t self_row;                          // 1: one-column decode whose own row base_pos is a partial of its own (slot
+                                              // = number of splits that hold rows) instead of a streamed row; else 0
   int out_f16;
   float scale;                                // 1 / sqrt(hd)
   unsigned long long* trace;                  // per-wave timestamps when built with PA_TRACE (else unused, nullptr)

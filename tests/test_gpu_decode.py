@@ -73,7 +73,8 @@ def test_decode_split_invariance_and_plan():
         for s in (0, 1, 3, 16, 40):
             pa.set_decode_splits(s)
             pl = pa.plan("decode", L - 1, 1)
-            assert pl["n_splits"] * pl["split_len"] >= L and pl["split_len"] % 32 == 0
+            # a one-column decode streams rows 0 .. L - 2; its own row L - 1 is one more partial (slots = splits + 1)
+            assert pl["n_splits"] * pl["split_len"] >= L - 1 and pl["split_len"] % 32 == 0 and pl["slots"] == pl["n_splits"] + 1
             if s:
                 assert pl["n_splits"] <= s
             outs.append(pa.run_attn("decode", 0, q, L - 1))
@@ -169,16 +170,17 @@ def test_c3_gated_decode_32k():
         pa.attn("decode", 0, None, 0, pa.gate_buffer_ptr(), pa.q_dim, ctx, 1, dout, pa.q_dim)
         pa.sync()
         got = dout.download(np.float32, pa.q_dim).reshape(ref.shape)
-        # 32769 rows over 256 workgroup slots per kv head: the last split takes the one row past 256 x 128
+        # 32768 streamed rows over 256 workgroup slots per kv head = whole 128-row splits; the token's own row is
+        # the 257th partial
         pl = pa.plan("decode", ctx, 1)
-        assert (pl["n_splits"] + 1) * pl["split_len"] > ctx + 1 >= pl["n_splits"] * pl["split_len"] and pl["split_len"] % 32 == 0
+        assert pl["n_splits"] * pl["split_len"] == ctx and pl["split_len"] % 32 == 0 and pl["slots"] == pl["n_splits"] + 1
     assert_parity(got, ref, "C3")
 
 
-@pytest.mark.parametrize("extra", [1, 2, 31, 32, 33, 127])
-def test_decode_open_ended_last_split(extra):
-    """Contexts a little past a whole number of splits: the last split also serves the remainder, which may add
-    tiles to some of its waves (the new row included: poisoned rows past the context must stay unused)."""
+@pytest.mark.parametrize("extra", [1, 2, 3, 32, 33, 34, 128])
+def test_decode_remainder_past_the_workgroup_slots(extra):
+    """Contexts a little past a whole number of splits: the remainder is one more split, which the first workgroup
+    takes after its own (poisoned rows past the context must stay unused)."""
     cfg = SHAPES["qwen36_moe"]
     L = 32768 + extra
     rng = np.random.default_rng(40 + extra)
@@ -187,7 +189,11 @@ def test_decode_open_ended_last_split(extra):
     ref = C.attention(q, k16, v16, L - 1)
     with _ctx_with_cache(cfg, k16, v16, L + 40, poison_from=L) as pa:
         pl = pa.plan("decode", L - 1, 1)
-        assert pl["n_splits"] * pl["split_len"] < L, "this case is meant to exercise the open-ended last split"
+        if extra == 1:
+            assert pl["n_splits"] * pl["split_len"] == L - 1      # whole splits + the token's own row
+        else:
+            # one split more than the 256 workgroup slots of a kv head: a workgroup takes a second split
+            assert pl["n_splits"] == 257 and pl["split_len"] == 128, "this case is meant to exercise a second round"
         got = pa.run_attn("decode", 0, q, L - 1)
     assert_parity(got, ref, "open-ended last split, +%d rows" % extra)
 

@@ -46,9 +46,10 @@ def test_gather_lists_of_many_lengths(shape):
 
 
 @pytest.mark.parametrize("pos", [0, 40, 2050, 6000])
-def test_identity_list_equals_dense_decode_bits(pos):
-    """With the list 0 .. pos the gathered kernel does the dense kernel's arithmetic in the same order
-    (engine/wgsl/attn_dec.js:35-37)."""
+def test_identity_list_equals_dense_decode(pos):
+    """With the list 0 .. pos the gathered kernel computes what the dense kernel computes
+    (engine/wgsl/attn_dec.js:35-37).  Not bit for bit: a dense one-column decode folds the column's own row in as a
+    partial of its own (f32 products), the gathered kernel streams every listed row through the f16 MFMA path."""
     cfg = SHAPES["qwen36_moe"]
     rng = np.random.default_rng(pos + 1)
     k16, v16 = random_cache(cfg, pos + 1, seed=pos + 2)
@@ -58,7 +59,7 @@ def test_identity_list_equals_dense_decode_bits(pos):
         pa.layer_alloc(0); pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
         dense = pa.run_attn("decode", 0, q, pos, gate=gate)
         gath = pa.run_attn_gather(0, q, [np.arange(pos + 1)], gate=gate)
-    assert np.array_equal(dense.view(np.uint32), gath.view(np.uint32))
+    assert np.abs(dense - gath).max() < 2e-5
 
 
 def test_gather_f16_out_and_bad_arguments():
