@@ -260,32 +260,38 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       }
     }
   };
-  {
-    const uint32_t t0 = t_begin + min(tile, max(n_tiles, 1u) - 1) * TILE;
-    if constexpr (GATHER) {
-      gather_offsets(t0);
+  const uint32_t t0 = t_begin + min(tile, max(n_tiles, 1u) - 1) * TILE;
+  if constexpr (GATHER) {
+    gather_offsets(t0);
 #pragma unroll
-      for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
+    for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
+  } else if constexpr (Q8) {
+#pragma unroll
+    for (int i = 0; i < S::NLD8; i++) kr[i] = *(const u4*)(kbase8 + (size_t)t0 * HD + (size_t)(i * S::RPL8) * HD + voff8);
+    ksr = *(const u4*)(ksbase + (size_t)t0 * S::SPR * 4 + soff);
+  } else {
+#pragma unroll
+    for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)t0 * row_bytes + (size_t)(i * S::RPL) * row_bytes + voff);
+  }
+  auto first_v_loads = [&]() __attribute__((always_inline)) {
+    if constexpr (GATHER) {
 #pragma unroll
       for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
     } else if constexpr (Q8) {
-      const size_t tb = (size_t)t0 * HD, sb = (size_t)t0 * S::SPR * 4;
 #pragma unroll
-      for (int i = 0; i < S::NLD8; i++) kr[i] = *(const u4*)(kbase8 + tb + (size_t)(i * S::RPL8) * HD + voff8);
-      ksr = *(const u4*)(ksbase + sb + soff);
-#pragma unroll
-      for (int i = 0; i < S::NLD8; i++) vr[i] = *(const u4*)(vbase8 + tb + (size_t)(i * S::RPL8) * HD + voff8);
-      vsr = *(const u4*)(vsbase + sb + soff);
+      for (int i = 0; i < S::NLD8; i++) vr[i] = *(const u4*)(vbase8 + (size_t)t0 * HD + (size_t)(i * S::RPL8) * HD + voff8);
+      vsr = *(const u4*)(vsbase + (size_t)t0 * S::SPR * 4 + soff);
     } else {
-      const size_t tb = (size_t)t0 * row_bytes;
 #pragma unroll
-      for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
-#pragma unroll
-      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + tb + (size_t)(i * S::RPL) * row_bytes + voff);
+      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)t0 * row_bytes + (size_t)(i * S::RPL) * row_bytes + voff);
     }
-  }
+  };
+  // The fused pre-step computes between the K and the V loads: a wave sits in the issue of its tile loads for
+  // microseconds (the memory pipeline is full), so arithmetic placed after all of them starts that much later, while
+  // the K requests already queued keep the pipeline fed during the arithmetic.
+  if constexpr (!FUSED) first_v_loads();
   PA_TP(1);
-  __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the K/V load issue
+  __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the load issue
   // ---- q -> f16 rows in LDS; waits only for the q loads, which were issued first ----
   if constexpr (FUSED) {
     float* xs = (float*)stage;       // wave-private scratch (the staging region is not in use yet)
@@ -318,6 +324,11 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       const h4 hv = { (_Float16)qv[j][0], (_Float16)qv[j][1], (_Float16)qv[j][2], (_Float16)qv[j][3] };
       *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
     }
+  }
+  if constexpr (FUSED) {
+    __builtin_amdgcn_sched_barrier(0);
+    first_v_loads();
+    __builtin_amdgcn_sched_barrier(0);
   }
   // per-lane row bookkeeping: row nb*16 + ln ends (exclusive) at end_pos[nb]; 0 for padding rows
   uint32_t end_pos[NB];
