@@ -316,13 +316,16 @@ def main():
     achieved = kv_bytes / (k_ms * 1e-3) / 1e9
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "decode_c3_traffic.json")
-    if os.path.exists(tpath):
+    if os.path.exists(tpath) and not args.kv_q8 and not args.unfused:      # measured for the default (fused, f16) kernel
         traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+    plan = pa.plan("decode", ctx, 1)
+    # template arguments: head_dim, row blocks, waves, fused pre-step, gather, int8 caches, single-round splits
+    kname = "pa_decode_kernel<256, 1, 4, %s, false, %s, %s>" % ("false" if args.unfused else "true", "true" if args.kv_q8 else "false",
+                                                               "true" if plan["split_len"] == 128 and plan["row_blocks"] == 1 else "false")
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
-                    traffic=traffic, kernel="pa_decode_kernel<256, 1, 4, %s, false, %s>" % ("false" if args.unfused else "true", "true" if args.kv_q8 else "false"), kernel_us=round(k_ms * 1e3, 3),
+                    traffic=traffic, kernel=kname, kernel_us=round(k_ms * 1e3, 3),
                     algorithmic_bytes_per_launch=kv_bytes, launches=kcount)
     log("split-K kernel: %.2f us/launch -> %.0f GB/s (%.1f%% of 8 TB/s)" % (k_ms * 1e3, achieved, 100 * achieved / HBM_PEAK_GBS))
-    plan = pa.plan("decode", ctx, 1)
 
     cpu = None
     if not args.no_cpu:

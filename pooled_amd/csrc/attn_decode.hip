@@ -113,7 +113,7 @@ template <int HD> struct DecShape {
 // self_row set): its G query heads are normed and roped from the raw projection on the way into LDS, and wave 0 of
 // split 0 norms / ropes the new key row and writes it and the value row to the cache.
 //
-// self_row (every one-column decode on f16 caches, fused or not): the column's own row base_pos is not streamed with
+// self_row (every one-column decode, fused or not, f16 or int8 caches): the column's own row base_pos is not streamed with
 // rows 0 .. base_pos - 1; wave 0 of split 0 holds it in registers (from the pre-step above, or loaded), scores it
 // against the G query rows and writes it as one more split partial, which the merge kernel folds in like any other.
 //
@@ -130,10 +130,9 @@ template <int HD> struct DecShape {
 // tile -- int8 -> f16 through the 0x6400 | (v + 128) bit pattern (= 1152 + v exactly), a packed subtract and a
 // packed multiply by the f16-rounded scale.  From there on (MFMA, softmax, merge) it is the f16 kernel.
 //
-// SR (single-round splits; one 16-row block): splits are one tile per wave (split_len = W x 32) and a workgroup takes
-// splits blockIdx.x, blockIdx.x + gridDim.x, ... one after the other, each with a partial of its own; the product
-// O^T = V^T P^T of a split is divided over the waves by output dims, see the code.  Without SR a workgroup owns one
-// split of any length and every wave loops over its own tiles.
+// SR (single-round splits; one 16-row block): splits are one tile per wave (split_len = W x 32); the product
+// O^T = V^T P^T of a split is divided over the waves by output dims, see the code.  Without SR a split has any length
+// and every wave loops over its own tiles.
 template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
 __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
   static_assert(!SR || NB == 1, "single-round splits: one 16-row block");
@@ -147,7 +146,17 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   float* mex = (float*)(stage_all + W * S::STAGE);                   // [W][16*NB]
   float* lex = mex + W * 16 * NB;                                    // [W][16*NB]
 
-  const uint32_t sp = blockIdx.x, g = blockIdx.y, cg = blockIdx.z;
+  // SR: a context a little past the workgroup slots of the chip has a few more splits than slots.  Their workgroups
+  // come last in dispatch order (ids past n_wgs x kv heads) whatever the kv head, so that the ones that wait for a
+  // free slot are the short remainder splits; they start when the first workgroups retire and end under the tail of
+  // the others.
+  uint32_t sp = blockIdx.x, g = blockIdx.y;
+  if constexpr (SR) {
+    const uint32_t nf = p.n_wgs ? min(p.n_wgs, gridDim.x) : gridDim.x, lin = blockIdx.x + gridDim.x * blockIdx.y;
+    if (lin < nf * gridDim.y) { g = lin / nf; sp = lin % nf; }
+    else { const uint32_t e = lin - nf * gridDim.y; g = e % gridDim.y; sp = nf + e / gridDim.y; }
+  }
+  const uint32_t cg = blockIdx.z;
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t ln = lane & 15, kg = lane >> 4;
   const uint32_t G = p.group, nH = p.n_heads;
@@ -158,14 +167,14 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   // rows visible to the group's last column (gather: the column's list length)
   // self_row (one-column decode): the column's own row base_pos is not streamed with the others -- see below
   const uint32_t seq_max = GATHER ? p.sel[c0 * p.sel_stride] : p.base_pos + c0 + ncl - p.self_row;
-  uint32_t t_begin = sp * p.split_len;                               // SR: of the workgroup's current split
+  const uint32_t t_begin = sp * p.split_len;
   // The workgroup of split 0 turns the column's own row into a partial of its own (wave 0, while the tile loads are
   // in flight), so it runs even when no other row exists (base_pos == 0).
-  const bool self_wg = !GATHER && !Q8 && p.self_row && sp == 0;
+  const bool self_wg = !GATHER && p.self_row && sp == 0;
   if (t_begin >= seq_max && !self_wg) return;
   const bool has_rows = t_begin < seq_max;
   // the last split is open-ended: the plan may hand it up to one split length of remainder
-  uint32_t t_end = !SR && sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
+  const uint32_t t_end = !SR && sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
   const size_t head_rows = (size_t)p.max_seq + TILE;              // rows of one kv head's plane, padding included
   PA_TP(0);
 
@@ -185,7 +194,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   const unsigned char* vsbase = (const unsigned char*)(p.v_scale + (Q8 ? (size_t)g * head_rows * S::SPR : 0));
   u4 ksr = {0u, 0u, 0u, 0u}, vsr = {0u, 0u, 0u, 0u};
 
-  uint32_t n_tiles = has_rows ? (t_end - t_begin + TILE - 1) / TILE : 0;
+  const uint32_t n_tiles = has_rows ? (t_end - t_begin + TILE - 1) / TILE : 0;
   u4 kr[S::NLD], vr[S::NLD];
   const u4 zero4 = {0u, 0u, 0u, 0u};
 
@@ -197,6 +206,19 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       const size_t ro = (size_t)p.base_pos * row_bytes + min(lane, (uint32_t)HD / 4 - 1) * 8;
       kx = *(const h4*)(kbase + ro);
       vx = *(const h4*)(vbase + ro);
+    }
+  }
+  if constexpr (Q8) {                   // int8 row: widened as the tile path widens it (exact integer x f16-rounded scale, one rounding)
+    if (self_wave) {
+      const uint32_t l4 = min(lane, (uint32_t)HD / 4 - 1);
+      const size_t ro = (size_t)p.base_pos * HD + 4 * l4, so = ((size_t)p.base_pos * S::SPR + l4 / 8) * 4;
+      const uint32_t kq = *(const uint32_t*)(kbase8 + ro), vq = *(const uint32_t*)(vbase8 + ro);
+      const _Float16 ksc = (_Float16)*(const float*)(ksbase + so), vsc = (_Float16)*(const float*)(vsbase + so);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        kx[i] = (_Float16)(int)(signed char)(kq >> (8 * i)) * ksc;
+        vx[i] = (_Float16)(int)(signed char)(vq >> (8 * i)) * vsc;
+      }
     }
   }
   // q loads first (they return first), then the first tile's K/V loads; staging q below overlaps the K/V latency.
@@ -347,14 +369,14 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     const uint32_t self_slot = min((seq_max + p.split_len - 1) / p.split_len, p.n_splits);
     const bool on = lane < HD / 4;
     const f4 vxf = { (float)vx[0], (float)vx[1], (float)vx[2], (float)vx[3] };
+#pragma unroll 4
     for (uint32_t r = 0; r < G; r++) {                                 // one column: row r is head g * G + r
       const h4 qv = *(const h4*)(q_lds + r * S::QROW + min(lane, (uint32_t)HD / 4 - 1) * 8);
       float d = 0.f;
 #pragma unroll
       for (int i = 0; i < 4; i++) d = __builtin_fmaf((float)qv[i], (float)kx[i], d);
       if (!on) d = 0.f;
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+      d = wave_sum_f32(d);
       const size_t slot = ((size_t)c0 * nH + g * G + r) * p.slots + self_slot;
       if (on) *(f4*)(p.part_o + slot * HD + 4 * lane) = vxf;
       if (lane == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(d * p.scale, 1.f);
@@ -494,15 +516,10 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   // the MFMAs and a store (the tile loop further down merges the waves' O through LDS: two more LDS round trips).
   if constexpr (SR) {
     constexpr int DBW = S::DB / W;                                      // 16-dim output blocks per wave
-    for (uint32_t split = sp;;) {
-      const uint32_t nsplit = split + gridDim.x;                        // this workgroup's next split, if any
-      const uint32_t nb_begin = nsplit * p.split_len;
-      const bool more = nb_begin < seq_max;
-      const uint32_t n_tiles_next = more ? (min(nb_begin + p.split_len, seq_max) - nb_begin + TILE - 1) / TILE : 1;
-      const uint32_t tpn = nb_begin + min(wave, n_tiles_next - 1) * TILE;
+    {
       const bool has_tile = wave < n_tiles;
       const uint32_t tp = t_begin + min(wave, n_tiles - 1) * TILE;      // the tile this wave holds in registers
-      stage_k(tp, more, tpn);
+      stage_k(tp, false, 0);
       PA_TP(3);
       f4 s[2][NB];
       qk(s);
@@ -527,7 +544,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
       ps += __shfl_xor(ps, 16, 64);
       ps += __shfl_xor(ps, 32, 64);
-      stage_v(tp, more, tpn);
+      stage_v(tp, false, 0);
       *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pf;
       if (kg == 0) { mex[wave * 16 + ln] = mx; lex[wave * 16 + ln] = ps; }
       PA_TP(5);
@@ -584,15 +601,12 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
         PA_TP(7); PA_TP(8); PA_TP(10);
         if (ln < R) {
           const uint32_t col = c0 + ln / G, hq = g * G + ln % G;
-          const size_t slot = ((size_t)col * nH + hq) * p.slots + split;
+          const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
 #pragma unroll
           for (int j = 0; j < DBW; j++) *(f4*)(p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = o[j];
           if (wave == 0 && kg == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(M, Lr);
         }
       }
-      if (!more) break;
-      __syncthreads();                                                  // the staged tiles and (m, l) are rewritten
-      split = nsplit; t_begin = nb_begin; t_end = min(t_begin + p.split_len, seq_max); n_tiles = n_tiles_next;
     }
     PA_TP(9);
     return;
@@ -901,18 +915,16 @@ static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipS
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  const uint32_t gx = SR && p.n_wgs ? p.n_wgs : p.n_splits;
-  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), dim3(gx, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
+  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
   return hipGetLastError();
 }
 
-// one 16-row block with splits of one tile per wave: the single-round kernel (a workgroup may take several splits)
+// one 16-row block with splits of one tile per wave: the single-round kernel
 template <int HD, int NB, int W, bool FUSED, bool GATHER = false, bool Q8 = false>
 static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   if constexpr (NB == 1) {
     if (p.split_len == W * TILE) return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, true>(p, col_groups, s, t);
   }
-  if (p.n_wgs && p.n_wgs != p.n_splits) return hipErrorInvalidValue;   // only the single-round kernel loops over splits
   return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, false>(p, col_groups, s, t);
 }
 

@@ -42,6 +42,19 @@ static __device__ inline double wave_sum_f64(double v) {
   return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
 }
 
+// the same for a float
+template <int CTRL> static __device__ inline float dpp_f32(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+static __device__ inline float readlane_f32(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
+static __device__ inline float wave_sum_f32(float v) {
+  v += dpp_f32<0xB1>(v);
+  v += dpp_f32<0x4E>(v);
+  v += dpp_f32<0x141>(v);
+  v += dpp_f32<0x140>(v);
+  return (readlane_f32(v, 0) + readlane_f32(v, 16)) + (readlane_f32(v, 32) + readlane_f32(v, 48));
+}
+
 // c, s of the f32 angle f32(pos) * inv_freq, evaluated in f64 and rounded once
 static __device__ inline void rope_cos_sin(uint32_t pos, float inv_freq, float& c, float& s) {
   // every product below is rounded on its own (plain operators: the __fmul_rn family is compiled with contraction on)

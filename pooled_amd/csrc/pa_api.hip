@@ -273,11 +273,11 @@ extern "C" int pa_kv_store(pa_ctx* ctx, uint32_t layer, const float* d_k, uint32
 // further column groups).  Splits are sized so that about two workgroups (one when the row blocks need the
 // whole register file) land on each CU, but never shorter than the tiles-per-wave floor that keeps the
 // partial (m, l, O) traffic a few percent of the K/V bytes.
-// self_ok: a one-column decode on f16 caches keeps the column's own row out of the streamed rows (the kernel turns it
+// self_ok: a one-column decode keeps the column's own row out of the streamed rows (the kernel turns it
 // into one more partial: slots = n_splits + 1), so a token at a multiple of the split length streams whole tiles only.
 static bool plan_self_row(const pa_plan& pl) { return pl.kernel == 0 && pl.slots == pl.n_splits + 1; }
-// wgs (optional): workgroups per kv head and column group that the launch uses; fewer than n_splits when the
-// single-round kernel hands some workgroups a second split.
+// wgs (optional): splits per kv head and column group that fit the chip at once; the single-round kernel dispatches
+// the workgroups of further splits (a short remainder) last.
 static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, bool self_ok = true, uint32_t* wgs = nullptr) {
   const pa_config& c = ctx->cfg;
   const uint32_t G = c.n_heads / c.n_kv_heads;
@@ -288,7 +288,7 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   if (n_cols * G > max_rows) { cw = max_rows / G; if (cw == 0) return PA_ERR_UNSUPPORTED; groups = ceil_div(n_cols, cw); }
   const uint32_t nb = ceil_div(cw * G, 16);
   const uint32_t W = 4;
-  const uint32_t self = self_ok && n_cols == 1 && !kv_q8(ctx) ? 1 : 0;
+  const uint32_t self = self_ok && n_cols == 1 ? 1 : 0;
   const uint32_t seq_max = std::max(base_pos + n_cols - self, 1u);   // streamed rows (position 0 alone: one empty split)
   const uint32_t tiles = ceil_div(seq_max, 32);
   const uint32_t occ = nb == 1 ? 2 : 1;
@@ -304,10 +304,13 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   if (!ctx->decode_splits_override && tpw > floor_tiles[nb]) {
     const uint32_t tpw_lo = std::max(tiles / (target * W), floor_tiles[nb]), sl_lo = 32 * W * tpw_lo;
     if ((uint64_t)seq_max < (uint64_t)(target + 1) * sl_lo) { sl = sl_lo; ns = std::max(1u, std::min(target, seq_max / sl_lo)); }
+    // one tile per wave: up to an eighth more splits than slots stay single-round splits (their workgroups start as
+    // the first ones retire and end under the tail of the rest)
+    else if (nb == 1 && tpw_lo == 1 && (uint64_t)seq_max <= (uint64_t)(target + target / 8) * sl_lo) sl = sl_lo;
   }
   uint32_t n_wg = ns;
   // One 16-row block and one tile per wave: the single-round kernel.  Its splits are all whole (no open-ended last
-  // one); a remainder past the workgroup slots is one more split that the first workgroup takes after its own.
+  // one); a remainder past the workgroup slots is a few more splits.
   if (nb == 1 && sl == 32 * W) { ns = ceil_div(seq_max, sl); n_wg = std::min(ns, target); }
   if (wgs) *wgs = n_wg;
   pl->kernel = 0; pl->split_len = sl; pl->n_splits = ns;

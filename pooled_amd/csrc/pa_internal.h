@@ -37,8 +37,8 @@ struct AttnParams {
   uint32_t n_heads, n_kv_heads, group;        // group = nH / nKV
   uint32_t base_pos, n_cols;                  // column c sees rows [0, base_pos + c]
   uint32_t split_len, n_splits, slots;
-  uint32_t n_wgs;                             // single-round decode kernel: workgroups along x (each takes splits x,
-                                              // x + n_wgs, ...); 0 = n_splits
+  uint32_t n_wgs;                             // single-round decode kernel: splits per kv head whose workgroups are
+                                              // dispatched first (the rest, a remainder past the chip's slots, last); 0 = all
   uint32_t cols_per_group;                    // columns per workgroup (grid z = column groups)
   uint32_t max_seq;
   uint32_t self_row;                          // 1: one-column decode whose own row base_pos is a partial of its own (slot
