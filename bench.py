@@ -211,6 +211,54 @@ def other_configs():
     return out
 
 
+def layer_leg(pa, cfg, ctx, steps, warmup, attn_ms):
+    """The attention half of a layer for one token, projections included (pa_attn_layer_decode: normed [q | k | v]
+    GEMV, fused decode step, accumulating output GEMV; Q4_0 weights of the MoE model's shape, a set per layer and
+    three sets in rotation so that weights and caches come from HBM), and the two GEMVs on their own."""
+    from pooled_amd.capi import PA_W_Q4_0
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    qd, kvd, dim = nH * hd, nKV * hd, 2048
+    rows_qkv = 2 * qd + 2 * kvd
+    rng = np.random.default_rng(0x5EED00F1)
+
+    def mk(d_out, d_in):
+        sc = np.asarray(rng.uniform(0.001, 0.003, (d_out, d_in // 32)), np.float16).view(np.uint16)
+        return pa.weight(PA_W_Q4_0, rng.integers(0, 256, (d_out, d_in // 2), dtype=np.uint8), sc)
+    n_sets = 3 * N_LAYERS
+    wq = [mk(rows_qkv, dim) for _ in range(n_sets)]
+    wo = [mk(dim, qd) for _ in range(n_sets)]
+    d_x = pa.to_device(rng.standard_normal(dim).astype(np.float32))
+    d_nw = pa.to_device((1 + 0.1 * rng.standard_normal(dim)).astype(np.float32))
+    d_hw = pa.to_device((1 + 0.1 * rng.standard_normal(hd)).astype(np.float32))
+    d_y = pa.alloc(rows_qkv * 4)
+    d_a = pa.to_device((rng.standard_normal(qd) * 0.01).astype(np.float32))
+
+    def timed(f):
+        for i in range(warmup):
+            f(i)
+        pa.sync()
+        pa.timer_start()
+        for i in range(steps):
+            f(i)
+        return pa.timer_stop() / steps
+    t_qkv = timed(lambda i: pa.gemv_norm(wq[i % n_sets], d_x, d_nw, d_y))
+    t_o = timed(lambda i: pa.gemv(wo[i % n_sets], d_a, d_x, acc=True))
+    d_x.upload(rng.standard_normal(dim).astype(np.float32))
+    t_layer = timed(lambda i: pa.attn_layer_decode(i % N_LAYERS, wq[i % n_sets], wo[i % n_sets], d_nw, d_hw, d_hw, d_x, ctx))
+    b_qkv = rows_qkv * dim // 2 + rows_qkv * (dim // 32) * 2
+    b_o = dim * qd // 2 + dim * (qd // 32) * 2
+    kv_bytes = 2 * (ctx + 1) * kvd * 2
+    log("layer: [q|k|v] GEMV %.2f us, wo GEMV %.2f us, whole attention half %.2f us" % (t_qkv * 1e3, t_o * 1e3, t_layer * 1e3))
+    return dict(workload="one token through the attention half of a full-attention layer (engine/qwen35.js:1586-1641): rmsnorm + [q|k|v] "
+                         "GEMV %dx%d, pre-step + split-K attention over %d rows + merge/gate, wo GEMV %dx%d accumulated into the residual; "
+                         "Q4_0 weights, 4 launches; weights and caches in rotation (cold HBM)" % (rows_qkv, dim, ctx, dim, qd),
+                us_per_step=round(t_layer * 1e3, 2), attention_us=round(attn_ms * 1e3, 2),
+                gemv_qkv_norm=dict(us=round(t_qkv * 1e3, 2), weight_bytes=b_qkv, gbs=round(b_qkv / t_qkv / 1e6, 1)),
+                gemv_o_acc=dict(us=round(t_o * 1e3, 2), weight_bytes=b_o, gbs=round(b_o / t_o / 1e6, 1)),
+                bytes_per_step=kv_bytes + b_qkv + b_o, gbs=round((kv_bytes + b_qkv + b_o) / t_layer / 1e6, 1),
+                pct_hbm_peak=round(100 * (kv_bytes + b_qkv + b_o) / t_layer / 1e6 / HBM_PEAK_GBS, 2))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -221,6 +269,7 @@ def main():
     ap.add_argument("--unfused", action="store_true", help="decode step as three launches (pa_glue_kv + pa_attn_decode) instead of the fused pa_attn_decode_step")
     ap.add_argument("--prefill-steps", type=int, default=5)
     ap.add_argument("--kv-q8", action="store_true", help="run the C3 decode step on int8 caches (one f32 scale per 32 values) instead of f16; implies --unfused")
+    ap.add_argument("--no-layer", action="store_true", help="skip the whole-layer leg (projections + attention, pa_attn_layer_decode)")
     ap.add_argument("--other-configs", action="store_true", help="only time configurations 1, 2 and 4 (attention call alone, caches in rotation)")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="only run the device probe: sustained f16 MFMA TFLOP/s and shader clock with constant and with random operands")
@@ -352,6 +401,8 @@ def main():
                     step="%s on one layer; %d layers' caches in rotation (cold HBM)" % ("pa_glue_kv + pa_attn_decode (pre-step, split-K decode, LSE merge/gate: 3 launches)" if args.unfused else "pa_attn_decode_step (pre-step fused into the split-K decode kernel + LSE merge/gate: 2 launches)", N_LAYERS),
                     kv_bytes_per_step=kv_bytes, plan=plan, pct_hbm_peak=round(100 * value / HBM_PEAK_GBS, 2)),
         roofline=roofline, cpu_baseline=cpu)
+    if not args.no_layer and not args.kv_q8 and not args.unfused:
+        line["layer_decode"] = layer_leg(pa, cfg, ctx, args.steps, args.warmup, ms_per_step)
     pa.close()
     if not args.no_prefill:
         line["prefill"] = prefill_leg(args.prefill_steps, not args.no_cpu)

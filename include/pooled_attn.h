@@ -211,6 +211,35 @@ int pa_timer_stop(pa_ctx* ctx, float* ms);
 int pa_profile_enable(pa_ctx* ctx, int on);
 int pa_profile_read(pa_ctx* ctx, float* ms_sum, uint32_t* count);
 
+/* ---- projections either side of the attention block, one-token passes.  Replace the reference's matvec /
+ *      matvec_q8 / matvec_q4 dispatches and their cooperative, accumulating and normed forms
+ *      (engine/wgsl/base.js:15-118, engine/wgsl/coop.js:236-420); built by the engine's mv() / mvN() helpers
+ *      (engine/qwen35.js:906-922) and recorded around the attention block at engine/qwen35.js:1591-1597 and :1641.
+ *      Weight kinds are the reference's split planes (engine/qwen35.js:894-903): ---- */
+#define PA_W_F32 0    /* f32 [d_out][d_in] row-major (engine/wgsl/base.js:15-30) */
+#define PA_W_Q8_0 1   /* int8 [d_out][d_in] + one f16 scale per 32 values, [d_out][d_in / 32] (base.js:32-63) */
+#define PA_W_Q4_0 2   /* nibbles [d_out][d_in / 2]: byte j of a block's 16 = element j (low) and j + 16 (high), value =
+                         nibble - 8; scales as Q8_0 (base.js:81-118) */
+typedef struct pa_weight pa_weight;
+/* copies a weight matrix to the device.  h_w: the values plane (f32 / int8 / packed nibbles), h_scales: f16 bits
+ * (NULL for PA_W_F32).  d_in must be a multiple of 32 and at most 8192 (4096 for PA_W_F32). */
+int pa_weight_create(pa_ctx* ctx, int kind, uint32_t d_out, uint32_t d_in, const void* h_w, const void* h_scales, pa_weight** out);
+int pa_weight_destroy(pa_ctx* ctx, pa_weight* w);
+/* y[d_out] = W x[d_in]; acc != 0: y += W x (matvec*_coop_acc: the residual add folded into the GEMV) */
+int pa_gemv(pa_ctx* ctx, const pa_weight* w, const float* d_x, float* d_y, int acc);
+/* y = W rmsnorm(x_raw) with xn = (x * inv) * norm_w, inv = 1 / sqrt(mean(x^2) + eps), eps from pa_config
+ * (matvec*_coop_n; rmsnorm: engine/wgsl/base.js:119-152).  d_xn_out != NULL: xn is also written there, as
+ * workgroup 0 of the reference's kernel does for the layer's later dispatches. */
+int pa_gemv_norm(pa_ctx* ctx, const pa_weight* w, const float* d_x_raw, const float* d_norm_w, float* d_xn_out, float* d_y);
+/* One token through the attention half of a full-attention layer, as _encodeLayerR records it
+ * (engine/qwen35.js:1586-1641): input rmsnorm -> [q | k | v] projections -> pre-step + cache write -> split-K
+ * attention -> merge + gate -> output projection accumulated into the residual.  w_qkv: rows [q (n_heads x head_dim,
+ * x 2 with PA_FLAG_GATE: q | gate interleaved per head) | k | v] x dim, one fused weight (the reference fuses k | v,
+ * engine/qwen35.js:1109-1114); w_o: dim x (n_heads x head_dim).  d_x [dim] is read and updated in place.  Four
+ * launches: normed GEMV, fused decode step (2), accumulating GEMV.  f16 caches only. */
+int pa_attn_layer_decode(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
+                         const float* d_qw, const float* d_kw, float* d_x, uint32_t pos);
+
 /* Device probe (measurement infrastructure, no counterpart in the reference): runs back-to-back
  * v_mfma_f32_32x32x16_f16 on every CU for iters x 64 instructions per wavefront, with constant operands
  * (random_operands = 0) or random f16 fragments, and returns the achieved TFLOP/s and the mean shader clock during

@@ -18,6 +18,9 @@ How each function is pinned (tests/test_oracle.py):
   split formulas      integer known answers quoted in the reference's own comments
   q8_quantize         zero block, exact-integer block (scale 1), ties to even, clamp at +-127, the block maximum maps
                       to +-127, |x - dequant| <= scale / 2, scale from the f32 quotient
+  w_dequant / gemv    hand-made Q4_0 / Q8_0 blocks with known values (nibble order, sign, scale), the reference's scalar
+                      matvec loops restated element by element on small shapes, linearity, unit vectors pick columns
+  rmsnorm             closed form on a constant vector, unit-RMS invariant, eps = 0 scale invariance
 """
 import numpy as np
 
@@ -162,6 +165,101 @@ def q8_dequantize(q, sc):
 
 
 # ---------------------------------------------------------------------------------------------
+# projections either side of the attention block (one-token GEMVs over the reference's weight planes)
+# ---------------------------------------------------------------------------------------------
+
+W_F32, W_Q8_0, W_Q4_0 = 0, 1, 2
+
+
+def w_dequant(kind, w, scales=None):
+    """Weight planes -> f64 matrix [d_out, d_in].
+
+    Reference: engine/wgsl/base.js:15-30 (f32 row-major), :32-63 (Q8_0: int8 packed 4 a word, value index = byte
+    index; one f16 scale per 32 values, unpack2x16float), :81-118 (Q4_0: "byte j holds elem j (low nibble) and elem
+    j+16 (high)", value = nibble - 8).  kind W_F32: w f32 [d_out, d_in]; W_Q8_0: w int8 [d_out, d_in];
+    W_Q4_0: w uint8 [d_out, d_in / 2]; scales: f16 bits (uint16) [d_out, d_in / 32].
+    """
+    if kind == W_F32:
+        return np.asarray(w, dtype=np.float32).astype(np.float64)
+    sc = np.asarray(scales, dtype=np.uint16).view(np.float16).astype(np.float64)          # [d_out, nb]
+    if kind == W_Q8_0:
+        q = np.asarray(w, dtype=np.int8).astype(np.float64)
+        d_out, d_in = q.shape
+        return (q.reshape(d_out, d_in // 32, 32) * sc[:, :, None]).reshape(d_out, d_in)
+    if kind == W_Q4_0:
+        b = np.asarray(w, dtype=np.uint8)
+        d_out, half = b.shape
+        blk = b.reshape(d_out, half // 16, 16)
+        vals = np.concatenate([(blk & 15).astype(np.float64) - 8.0, (blk >> 4).astype(np.float64) - 8.0], axis=2)   # [.., 32]
+        return (vals * sc[:, :, None]).reshape(d_out, half * 2)
+    raise ValueError("unknown weight kind")
+
+
+def gemv(kind, w, scales, x):
+    """y = W x in f64 (the reference accumulates in f32 in an order of its own; tests use its tolerance).
+
+    Reference: engine/wgsl/base.js:20-30, :40-63, :90-118; cooperative forms engine/wgsl/coop.js:236-345.
+    """
+    return w_dequant(kind, w, scales) @ np.asarray(x, dtype=np.float32).astype(np.float64)
+
+
+def gemv_reference_loops(kind, w, scales, x):
+    """The reference's scalar kernels restated loop for loop (small shapes only): pins w_dequant / gemv.
+
+    Reference: engine/wgsl/base.js:40-63 (matvec_q8: sum over words of extractBits(word, 8k, 8) * x, times the block
+    scale), :90-118 (matvec_q4: word w of a block, nibble pairs (4k, 4k + 4) -> elements (4w + k, 4w + k + 16)).
+    """
+    x = np.asarray(x, dtype=np.float32).astype(np.float64)
+    if kind == W_F32:
+        wf = np.asarray(w, dtype=np.float32)
+        return np.array([sum(float(wf[r, c]) * x[c] for c in range(wf.shape[1])) for r in range(wf.shape[0])])
+    sc = np.asarray(scales, dtype=np.uint16).view(np.float16).astype(np.float64)
+    d_out = w.shape[0]
+    y = np.zeros(d_out)
+    if kind == W_Q8_0:
+        words = np.ascontiguousarray(np.asarray(w, dtype=np.int8)).view(np.uint32)       # [d_out, d_in / 4]
+        nb = words.shape[1] // 8
+        for r in range(d_out):
+            acc = 0.0
+            for b in range(nb):
+                s_ = 0.0
+                for wi in range(8):
+                    word = int(words[r, b * 8 + wi])
+                    for k in range(4):
+                        v = (word >> (8 * k)) & 255
+                        v = v - 256 if v >= 128 else v                                   # extractBits on an i32: sign-extended
+                        s_ += v * x[b * 32 + wi * 4 + k]
+                acc += sc[r, b] * s_
+            y[r] = acc
+        return y
+    words = np.ascontiguousarray(np.asarray(w, dtype=np.uint8)).view(np.uint32)          # [d_out, d_in / 8]
+    nb = words.shape[1] // 4
+    for r in range(d_out):
+        acc = 0.0
+        for b in range(nb):
+            s_ = 0.0
+            for wi in range(4):
+                word = int(words[r, b * 4 + wi])
+                j = b * 32 + wi * 4
+                for k in range(4):
+                    s_ += (((word >> (8 * k)) & 15) - 8.0) * x[j + k]
+                    s_ += (((word >> (8 * k + 4)) & 15) - 8.0) * x[j + 16 + k]
+            acc += sc[r, b] * s_
+        y[r] = acc
+    return y
+
+
+def rmsnorm(x, w, eps):
+    """xn = (x * inv) * w, inv = 1 / sqrt(mean(x^2) + eps): f32 in, f64 arithmetic, f32 out.
+
+    Reference: engine/wgsl/base.js:119-152 (rmsnorm), engine/wgsl/coop.js:389-411 (the same inside a GEMV).
+    """
+    x = np.asarray(x, dtype=np.float32).astype(np.float64)
+    inv = 1.0 / np.sqrt(np.mean(x * x) + eps)
+    return ((x * inv) * np.asarray(w, dtype=np.float32).astype(np.float64)).astype(np.float32)
+
+
+# ---------------------------------------------------------------------------------------------
 # attention
 # ---------------------------------------------------------------------------------------------
 
@@ -299,3 +397,24 @@ def make_inputs(cfg, ctx, n_cols, seed, with_cache_rows=True):
         kw=(1.0 + 0.1 * rng.standard_normal(hd)).astype(np.float32),
     )
     return d
+
+
+def attn_layer_decode(x, kind_qkv, w_qkv, sc_qkv, kind_o, w_o, sc_o, attn_norm_w, qw, kw, k16, v16, pos, cfg):
+    """One token through the attention half of a full-attention layer; returns (x_out f32 [dim], k16 row, v16 row).
+
+    Reference: engine/qwen35.js:1586-1641 (_encodeLayerR, L.isFull): rmsnorm -> q / [k | v] GEMVs -> pre-step ->
+    KV write -> attention over rows [0, pos] -> sigmoid gate -> wo GEMV -> residual add.  k16 / v16: cache rows
+    [0, pos) as f16 bits [pos, nKV, hd].  f32 hand-offs between the stages, as the engine's buffers are.
+    """
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    gated = cfg.get("gate", False)
+    xn = rmsnorm(x, attn_norm_w, cfg["eps"])
+    qkv = gemv(kind_qkv, w_qkv, sc_qkv, xn).astype(np.float32)
+    q_rows = nH * hd * (2 if gated else 1)
+    kvd = nKV * hd
+    g = glue_kv(qkv[None, :q_rows], qkv[None, q_rows:q_rows + kvd], qkv[None, q_rows + kvd:], qw, kw, pos, cfg)
+    kall = np.concatenate([np.asarray(k16).reshape(pos, nKV, hd), g["k16"].reshape(1, nKV, hd)])
+    vall = np.concatenate([np.asarray(v16).reshape(pos, nKV, hd), g["v16"].reshape(1, nKV, hd)])
+    out = attention(g["q"], kall, vall, pos, gate=g["gate"] if gated else None)            # [1, nH, hd]
+    y = gemv(kind_o, w_o, sc_o, np.asarray(out, dtype=np.float32).reshape(-1))
+    return (np.asarray(x, dtype=np.float32).astype(np.float64) + y).astype(np.float32), g["k16"], g["v16"]

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libpooled_attn.so")
 
 PA_OK, PA_ERR_INVALID, PA_ERR_UNSUPPORTED, PA_ERR_HIP, PA_ERR_NOMEM = 0, 1, 2, 3, 4
 PA_FLAG_QK_NORM, PA_FLAG_GATE, PA_FLAG_KV_Q8 = 1, 2, 4
+PA_W_F32, PA_W_Q8_0, PA_W_Q4_0 = 0, 1, 2
 PA_OUT_F32, PA_OUT_F16 = 0, 1
 
 u32, c_int, vp, f32p = ctypes.c_uint32, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p
@@ -68,6 +69,11 @@ SYMBOLS = {
     "pa_slot_export": (c_int, [vp, u32, u32, c_int, vp]),
     "pa_slot_import": (c_int, [vp, u32, u32, c_int, vp]),
     "pa_mfma_probe": (c_int, [vp, c_int, u32, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]),
+    "pa_weight_create": (c_int, [vp, c_int, u32, u32, vp, vp, ctypes.POINTER(vp)]),
+    "pa_weight_destroy": (c_int, [vp, vp]),
+    "pa_gemv": (c_int, [vp, vp, f32p, f32p, c_int]),
+    "pa_gemv_norm": (c_int, [vp, vp, f32p, f32p, f32p, f32p]),
+    "pa_attn_layer_decode": (c_int, [vp, u32, vp, vp, f32p, f32p, f32p, f32p, u32]),
     "pa_version": (ctypes.c_char_p, []),
 }
 
@@ -148,6 +154,9 @@ class PooledAttn:
 
     def close(self):
         if self.ctx:
+            for w in getattr(self, "_weights", []):
+                self.L.pa_weight_destroy(self.ctx, w)
+            self._weights = []
             for b in self._bufs:
                 b.free()
             self._bufs = []
@@ -293,6 +302,31 @@ class PooledAttn:
     def slot_import(self, slot, layer, which, part):
         part = np.ascontiguousarray(part, dtype=self._kv_part(which)[0])
         self._chk(self.L.pa_slot_import(self.ctx, slot, layer, which, part.ctypes.data))
+
+    # ---- projections (one-token passes) ----
+    def weight(self, kind, w, scales=None):
+        """Upload a weight matrix: kind PA_W_F32 (w f32 [d_out, d_in]), PA_W_Q8_0 (w int8 [d_out, d_in]) or PA_W_Q4_0
+        (w uint8 [d_out, d_in / 2]); scales: f16 bits (uint16) [d_out, d_in / 32].  Returns an opaque handle."""
+        w = np.ascontiguousarray(w)
+        d_out = w.shape[0]
+        d_in = w.shape[1] * (2 if kind == PA_W_Q4_0 else 1)
+        sc = None if scales is None else np.ascontiguousarray(scales, dtype=np.uint16)
+        h = vp()
+        self._chk(self.L.pa_weight_create(self.ctx, kind, d_out, d_in, w.ctypes.data, sc.ctypes.data if sc is not None else None, ctypes.byref(h)))
+        if not hasattr(self, "_weights"):
+            self._weights = []
+        self._weights.append(h)
+        return h
+
+    def gemv(self, w, d_x, d_y, acc=False):
+        self._chk(self.L.pa_gemv(self.ctx, w, d_x.ptr, d_y.ptr, int(bool(acc))))
+
+    def gemv_norm(self, w, d_x_raw, d_norm_w, d_y, d_xn_out=None):
+        self._chk(self.L.pa_gemv_norm(self.ctx, w, d_x_raw.ptr, d_norm_w.ptr, d_xn_out.ptr if d_xn_out else None, d_y.ptr))
+
+    def attn_layer_decode(self, layer, w_qkv, w_o, d_attn_norm_w, d_qw, d_kw, d_x, pos):
+        self._chk(self.L.pa_attn_layer_decode(self.ctx, layer, w_qkv, w_o, d_attn_norm_w.ptr, d_qw.ptr if d_qw else None,
+                                              d_kw.ptr if d_kw else None, d_x.ptr, pos))
 
     def mfma_probe(self, random_operands, iters):
         """(TFLOP/s, shader MHz) of back-to-back f16 MFMAs on every CU with constant or random operands."""

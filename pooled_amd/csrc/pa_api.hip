@@ -112,6 +112,7 @@ extern "C" int pa_destroy(pa_ctx* ctx) {
   if (ctx->rope_tab) (void)hipFree(ctx->rope_tab);
   if (ctx->part_o) (void)hipFree(ctx->part_o);
   if (ctx->part_ml) (void)hipFree(ctx->part_ml);
+  if (ctx->proj_buf) (void)hipFree(ctx->proj_buf);
   for (auto ev : ctx->prof_events) (void)hipEventDestroy(ev);
   if (ctx->t0) (void)hipEventDestroy(ctx->t0);
   if (ctx->t1) (void)hipEventDestroy(ctx->t1);
@@ -487,6 +488,91 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
   HIPCHK(ctx, pa_launch_decode_step(p, c.head_dim, ctx->stream, &tm));
   HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;
+}
+
+// ---- projections (one-token passes) -------------------------------------------------------------
+
+extern "C" int pa_weight_create(pa_ctx* ctx, int kind, uint32_t d_out, uint32_t d_in, const void* h_w, const void* h_scales, pa_weight** out) {
+  const char* who = "pa_weight_create";
+  if (!ctx || !out) return PA_ERR_INVALID;
+  *out = nullptr;
+  if (kind != PA_W_F32 && kind != PA_W_Q8_0 && kind != PA_W_Q4_0) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": unknown weight kind");
+  if (!h_w || (kind != PA_W_F32 && !h_scales)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null plane");
+  if (d_out == 0 || d_in == 0 || (d_in & 31)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": d_in must be a positive multiple of 32");
+  if (d_in > (kind == PA_W_F32 ? 4096u : 8192u)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": d_in beyond the gfx950 table");
+  pa_weight* w = new (std::nothrow) pa_weight();
+  if (!w) return fail(ctx, PA_ERR_NOMEM, std::string(who) + ": out of host memory");
+  w->kind = kind; w->d_out = d_out; w->d_in = d_in;
+  const size_t wbytes = kind == PA_W_F32 ? (size_t)d_out * d_in * 4 : kind == PA_W_Q8_0 ? (size_t)d_out * d_in : (size_t)d_out * d_in / 2;
+  const size_t sbytes = kind == PA_W_F32 ? 0 : (size_t)d_out * (d_in / 32) * 2;
+  hipError_t e = hipMalloc(&w->w, wbytes);
+  if (e == hipSuccess && sbytes) e = hipMalloc((void**)&w->scales, sbytes);
+  if (e == hipSuccess) e = hipMemcpyAsync(w->w, h_w, wbytes, hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess && sbytes) e = hipMemcpyAsync(w->scales, h_scales, sbytes, hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) {
+    if (w->w) (void)hipFree(w->w);
+    if (w->scales) (void)hipFree(w->scales);
+    delete w;
+    return fail_hip(ctx, e, "pa_weight_create: upload");
+  }
+  *out = w;
+  return PA_OK;
+}
+
+extern "C" int pa_weight_destroy(pa_ctx* ctx, pa_weight* w) {
+  if (!ctx) return PA_ERR_INVALID;
+  if (!w) return PA_OK;
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  if (w->w) (void)hipFree(w->w);
+  if (w->scales) (void)hipFree(w->scales);
+  delete w;
+  return PA_OK;
+}
+
+static int gemv_common(pa_ctx* ctx, const char* who, const pa_weight* w, const float* d_x, const float* d_norm_w, float* d_xn_out, float* d_y, int acc) {
+  if (!ctx) return PA_ERR_INVALID;
+  if (!w || !d_x || !d_y) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null argument");
+  if (((uintptr_t)d_x & 15) || ((uintptr_t)d_norm_w & 15) || ((uintptr_t)d_xn_out & 15))
+    return fail(ctx, PA_ERR_INVALID, std::string(who) + ": vectors must be 16-byte aligned");
+  GemvParams p; memset(&p, 0, sizeof p);
+  p.w = w->w; p.scales = w->scales; p.x = d_x; p.norm_w = d_norm_w; p.xn_out = d_xn_out; p.y = d_y;
+  p.d_out = w->d_out; p.d_in = w->d_in; p.eps = ctx->cfg.eps; p.acc = acc; p.kind = w->kind;
+  HIPCHK(ctx, pa_launch_gemv(p, ctx->n_cu, ctx->stream));
+  return PA_OK;
+}
+
+extern "C" int pa_gemv(pa_ctx* ctx, const pa_weight* w, const float* d_x, float* d_y, int acc) {
+  return gemv_common(ctx, "pa_gemv", w, d_x, nullptr, nullptr, d_y, acc);
+}
+extern "C" int pa_gemv_norm(pa_ctx* ctx, const pa_weight* w, const float* d_x_raw, const float* d_norm_w, float* d_xn_out, float* d_y) {
+  if (ctx && !d_norm_w) return fail(ctx, PA_ERR_INVALID, "pa_gemv_norm: null norm weight");
+  return gemv_common(ctx, "pa_gemv_norm", w, d_x_raw, d_norm_w, d_xn_out, d_y, 0);
+}
+
+extern "C" int pa_attn_layer_decode(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
+                                    const float* d_qw, const float* d_kw, float* d_x, uint32_t pos) {
+  const char* who = "pa_attn_layer_decode";
+  if (!ctx) return PA_ERR_INVALID;
+  const pa_config& c = ctx->cfg;
+  if (!w_qkv || !w_o || !d_attn_norm_w || !d_x) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null argument");
+  const uint32_t qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim;
+  const uint32_t q_rows = qd * ((c.flags & PA_FLAG_GATE) ? 2 : 1);
+  if (w_qkv->d_out != q_rows + 2 * kvd) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": w_qkv must have q (+ gate), k and v rows");
+  if (w_o->d_in != qd || w_o->d_out != w_qkv->d_in) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": w_o must map n_heads x head_dim back to the model width");
+  const size_t need = (size_t)w_qkv->d_out + qd;
+  if (need > ctx->proj_buf_floats) {
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->proj_buf) { HIPCHK(ctx, hipFree(ctx->proj_buf)); ctx->proj_buf = nullptr; ctx->proj_buf_floats = 0; }
+    HIPCHK(ctx, hipMalloc((void**)&ctx->proj_buf, need * sizeof(float)));
+    ctx->proj_buf_floats = need;
+  }
+  float* qkv = ctx->proj_buf;
+  float* attn_out = ctx->proj_buf + w_qkv->d_out;
+  int rc = gemv_common(ctx, who, w_qkv, d_x, d_attn_norm_w, nullptr, qkv, 0);
+  if (rc) return rc;
+  if ((rc = pa_attn_decode_step(ctx, layer, qkv, qkv + q_rows, qkv + q_rows + kvd, d_qw, d_kw, pos, attn_out, PA_OUT_F32))) return rc;
+  return gemv_common(ctx, who, w_o, attn_out, nullptr, nullptr, d_x, 1);
 }
 
 // ---- cache access ---------------------------------------------------------------------------------

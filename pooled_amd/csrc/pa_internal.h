@@ -84,6 +84,17 @@ hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_bloc
 // the 4-wave, 64-rows-per-wave software-pipelined variant (same contract)
 hipError_t pa_launch_prefill_wide(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
 
+// one-token projection y = W x (proj_gemv.hip): kind PA_W_*, w = f32 [d_out][d_in] / int8 [d_out][d_in] / nibbles
+// [d_out][d_in / 2], scales = f16 bits [d_out][d_in / 32] (quantised kinds); norm_w != nullptr: x is the raw vector and
+// the kernel applies rmsnorm with that weight (xn_out != nullptr: also written); acc: y += W x
+struct GemvParams {
+  const void* w; const uint16_t* scales;
+  const float* x; const float* norm_w; float* xn_out; float* y;
+  uint32_t d_out, d_in;
+  float eps; int acc; int kind;
+};
+hipError_t pa_launch_gemv(const GemvParams& p, int n_cu, hipStream_t s);
+
 // device probe (probe.hip): sustained f16 MFMA rate and shader clock, constant or random operands
 hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, uint32_t iters, hipStream_t st, float* tflops, float* shader_mhz);
 
@@ -102,6 +113,13 @@ struct pa_slot {
   std::vector<void*> t[4];         // per tensor (K, V, K scales, V scales), indexed by layer; nullptr where absent
 };
 
+struct pa_weight {
+  int kind = 0;
+  uint32_t d_out = 0, d_in = 0;
+  void* w = nullptr;              // values plane on the device
+  uint16_t* scales = nullptr;     // f16 bits [d_out][d_in / 32]; nullptr for f32 weights
+};
+
 struct pa_ctx {
   pa_config cfg{};
   int device = 0;
@@ -116,6 +134,8 @@ struct pa_ctx {
   float2* rope_tab = nullptr;   // [max_seq][n_rot/2] (cos, sin); nullptr when it would exceed 1 GiB
   float* part_o = nullptr; float* part_ml = nullptr;
   size_t part_o_bytes = 0, part_ml_bytes = 0;
+  float* proj_buf = nullptr;    // pa_attn_layer_decode: [q(+gate) | k | v] projections, then attnOut [nH*hd]
+  size_t proj_buf_floats = 0;
   uint32_t decode_splits_override = 0;
   // timing
   hipEvent_t t0 = nullptr, t1 = nullptr;

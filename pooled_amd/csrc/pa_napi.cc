@@ -207,6 +207,46 @@ static napi_value SlotImport(napi_env env, napi_callback_info info) {
   int rc = pa_slot_import(c, id, layer, which, h); if (rc) return throw_pa(env, c, rc, "pa_slot_import"); return undefined(env);
 }
 
+// ---- projections (one-token passes) ----
+// weightCreate(ctx, kind, dOut, dIn, valuesTypedArray, scalesUint16Array | null) -> weight handle (a number)
+static napi_value WeightCreate(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); int kind = (int)a.u32(1); uint32_t d_out = a.u32(2), d_in = a.u32(3);
+  size_t nw = 0, ns = 0; void* hw = a.host(4, &nw);
+  void* hs = nullptr;
+  if (a.argc > 5) { napi_valuetype t; napi_typeof(env, a.argv[5], &t); if (t != napi_null && t != napi_undefined) hs = a.host(5, &ns); }
+  CHECK_ARGS("weightCreate");
+  const size_t want_w = kind == PA_W_F32 ? (size_t)d_out * d_in * 4 : kind == PA_W_Q8_0 ? (size_t)d_out * d_in : (size_t)d_out * d_in / 2;
+  const size_t want_s = kind == PA_W_F32 ? 0 : (size_t)d_out * (d_in / 32) * 2;
+  if (nw < want_w || (want_s && ns < want_s)) { napi_throw_range_error(env, nullptr, "weightCreate: plane shorter than dOut x dIn needs"); return nullptr; }
+  pa_weight* w = nullptr;
+  int rc = pa_weight_create(c, kind, d_out, d_in, hw, hs, &w);
+  if (rc) return throw_pa(env, c, rc, "pa_weight_create");
+  return num_value(env, (double)(uintptr_t)w);
+}
+static napi_value WeightDestroy(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); pa_weight* w = (pa_weight*)a.ptr(1); CHECK_ARGS("weightDestroy");
+  int rc = pa_weight_destroy(c, w); if (rc) return throw_pa(env, c, rc, "pa_weight_destroy"); return undefined(env);
+}
+// gemv(ctx, weight, x, y, acc)
+static napi_value Gemv(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); pa_weight* w = (pa_weight*)a.ptr(1); const float* x = (const float*)a.ptr(2); float* y = (float*)a.ptr(3); int acc = (int)a.u32(4);
+  CHECK_ARGS("gemv");
+  int rc = pa_gemv(c, w, x, y, acc); if (rc) return throw_pa(env, c, rc, "pa_gemv"); return undefined(env);
+}
+// gemvNorm(ctx, weight, xRaw, normW, xnOut | null, y)
+static napi_value GemvNorm(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); pa_weight* w = (pa_weight*)a.ptr(1); const float* x = (const float*)a.ptr(2); const float* nw = (const float*)a.ptr(3);
+  float* xn = (float*)a.ptr(4); float* y = (float*)a.ptr(5); CHECK_ARGS("gemvNorm");
+  int rc = pa_gemv_norm(c, w, x, nw, xn, y); if (rc) return throw_pa(env, c, rc, "pa_gemv_norm"); return undefined(env);
+}
+// attnLayerDecode(ctx, layer, wQkv, wO, attnNormW, qNormW, kNormW, x, pos)
+static napi_value AttnLayerDecode(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); uint32_t layer = a.u32(1); pa_weight* wqkv = (pa_weight*)a.ptr(2); pa_weight* wo = (pa_weight*)a.ptr(3);
+  const float* nw = (const float*)a.ptr(4); const float* qw = (const float*)a.ptr(5); const float* kw = (const float*)a.ptr(6);
+  float* x = (float*)a.ptr(7); uint32_t pos = a.u32(8); CHECK_ARGS("attnLayerDecode");
+  int rc = pa_attn_layer_decode(c, layer, wqkv, wo, nw, qw, kw, x, pos); if (rc) return throw_pa(env, c, rc, "pa_attn_layer_decode"); return undefined(env);
+}
+
 static napi_value Init(napi_env env, napi_value exports) {
   struct { const char* name; napi_callback fn; } table[] = {
     {"create", Create}, {"destroy", Destroy}, {"lastError", LastError}, {"version", Version}, {"layerAlloc", LayerAlloc}, {"sync", Sync},
@@ -215,7 +255,8 @@ static napi_value Init(napi_env env, napi_value exports) {
     {"setDecodeSplits", SetDecodeSplits}, {"kvRead", KvRead}, {"kvWrite", KvWrite}, {"kvDevicePtr", KvDevicePtr}, {"timerStart", TimerStart},
     {"timerStop", TimerStop}, {"profileEnable", ProfileEnable}, {"profileRead", ProfileRead}, {"attnDecodeStep", AttnDecodeStep},
     {"copyD2d", CopyD2d}, {"attnGather", AttnGather}, {"slotSave", SlotSave}, {"slotLoad", SlotLoad}, {"slotDrop", SlotDrop}, {"slotPos", SlotPos},
-    {"slotCreate", SlotCreate}, {"slotExport", SlotExport}, {"slotImport", SlotImport},
+    {"slotCreate", SlotCreate}, {"slotExport", SlotExport}, {"slotImport", SlotImport}, {"weightCreate", WeightCreate},
+    {"weightDestroy", WeightDestroy}, {"gemv", Gemv}, {"gemvNorm", GemvNorm}, {"attnLayerDecode", AttnLayerDecode},
   };
   for (auto& t : table) {
     napi_value fn;

@@ -18,6 +18,7 @@ const path = require("path");
 const addon = require(path.join(__dirname, "..", "lib", "pooled_attn.node"));
 
 const PA_FLAG_QK_NORM = 1, PA_FLAG_GATE = 2, PA_FLAG_KV_Q8 = 4, PA_OUT_F32 = 0, PA_OUT_F16 = 1;
+const PA_W_F32 = 0, PA_W_Q8_0 = 1, PA_W_Q4_0 = 2;             // weight kinds of the projections (include/pooled_attn.h)
 
 // ---- the reference's sizing formulas, kept for callers that still size grids or slot buffers with them.
 //      The HIP kernels take their splits from the gfx950 table instead (HipAttention.plan). ----
@@ -88,7 +89,8 @@ class HipAttention {
   destroy() {
     if (!this.ctx) return;
     for (const k of Object.keys(this.B)) addon.free(this.ctx, this.B[k].ptr);
-    for (const L of this.layers) { if (L.qNorm) addon.free(this.ctx, L.qNorm); if (L.kNorm) addon.free(this.ctx, L.kNorm); }
+    for (const L of this.layers) { if (L.qNorm) addon.free(this.ctx, L.qNorm); if (L.kNorm) addon.free(this.ctx, L.kNorm); if (L.attnNorm) addon.free(this.ctx, L.attnNorm); }
+    for (const w of this._weights || []) addon.weightDestroy(this.ctx, w);
     addon.free(this.ctx, this._ones);
     addon.destroy(this.ctx);
     this.ctx = null;
@@ -218,6 +220,44 @@ class HipAttention {
     addon.glueKv(this.ctx, i, B.qFull.ptr, this._strideF(B.qFull), B.k.ptr, this._strideF(B.k), B.v.ptr, this._strideF(B.v), n[0], n[1], pos, 1);
     const gate = this.gate ? addon.gateBuffer(this.ctx) : null;
     addon.attn(this.ctx, 0, i, null, 0, gate, this.dims.qDim, pos, 1, B.attnOut.ptr, this._outStride(), this.outDtype);
+  }
+
+  // ---- projections either side of the attention block, one token (engine/qwen35.js:894-922 up / mv / mvN) ----
+  // e: a weight entry as the engine's loaders make them: { kind: "q4" | "q8", qs, scales, dOut, dIn } (qs: Uint8Array /
+  // Int8Array / Uint32Array words, scales: Uint16Array of f16 bits) or { kind: "f32", data, dOut, dIn }
+  up(e) {
+    const kind = e.kind === "q4" ? PA_W_Q4_0 : e.kind === "q8" ? PA_W_Q8_0 : e.kind === "f32" ? PA_W_F32 : -1;
+    if (kind < 0) throw new Error("up: unknown weight kind " + e.kind);
+    const h = addon.weightCreate(this.ctx, kind, e.dOut, e.dIn, kind === PA_W_F32 ? e.data : e.qs, kind === PA_W_F32 ? null : e.scales);
+    (this._weights = this._weights || []).push(h);
+    return { kind: e.kind, handle: h, dOut: e.dOut, dIn: e.dIn };
+  }
+  // the engine's fuse() (engine/qwen35.js:1001-1019): several weights of one kind and width as one, rows concatenated
+  fuse(parts) {
+    const k = parts[0].kind, dIn = parts[0].dIn;
+    if (!parts.every((p) => p.kind === k && p.dIn === dIn)) throw new Error("fuse: parts must share kind and dIn");
+    const cat = (arrs) => { const out = new arrs[0].constructor(arrs.reduce((n, x) => n + x.length, 0)); let o = 0; for (const x of arrs) { out.set(x, o); o += x.length; } return out; };
+    const dOut = parts.reduce((n, p) => n + p.dOut, 0);
+    return k === "f32" ? { kind: k, data: cat(parts.map((p) => p.data)), dOut: dOut, dIn: dIn }
+                       : { kind: k, qs: cat(parts.map((p) => p.qs)), scales: cat(parts.map((p) => p.scales)), dOut: dOut, dIn: dIn };
+  }
+  // mv: y = W x (acc: y += W x); mvN: y = W rmsnorm(x) with norm weight nw (xnOut: also keep the normed vector)
+  mv(p, w, x, y, acc) { addon.gemv(this.ctx, w.handle, x, y, acc ? 1 : 0); }
+  mvN(p, w, x, nw, y, xnOut) { addon.gemvNorm(this.ctx, w.handle, x, nw, xnOut || null, y); }
+  // per-layer projection weights: wqkv = fuse([wq, wk, wv]) uploaded, wo, attnNorm (Float32Array [dim])
+  setLayerProj(i, wqkv, wo, attnNorm) {
+    const L = this.layers[i];
+    L.wqkv = wqkv; L.wo = wo;
+    if (!L.attnNorm) L.attnNorm = addon.malloc(this.ctx, attnNorm.length * 4);
+    addon.upload(this.ctx, L.attnNorm, Float32Array.from(attnNorm));
+    if (!this.B.x) this.B.x = { ptr: addon.malloc(this.ctx, attnNorm.length * 4), stride: attnNorm.length * 4, n: attnNorm.length };
+  }
+  // one token through the attention half of full-attention layer i, as _encodeLayerR records it
+  // (engine/qwen35.js:1586-1641): B.x (the residual) is read and updated in place
+  encodeLayerR(p, i, pos) {
+    const L = this.layers[i], n = this._norms(L);
+    if (!L.wqkv) throw new Error("encodeLayerR: layer " + i + " has no projection weights (setLayerProj)");
+    addon.attnLayerDecode(this.ctx, i, L.wqkv.handle, L.wo.handle, L.attnNorm, n[0], n[1], this.B.x.ptr, pos);
   }
 
   // ---- sparse-attention layers: the attn step of a QSA pass (engine/qsa.js:8-14, dispatch :41-56) ----

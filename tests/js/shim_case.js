@@ -76,6 +76,54 @@ try { A.encodeLayerAttn(null, 0, base + n); console.log("out-of-range position d
   try { A.importState({ sig: { v: 0 }, pos: 0, parts: [] }); console.log("importState of a foreign signature did not throw FAIL"); fails++; } catch (e) { if (!/different model/.test(e.message)) { console.log("unexpected error text: " + e.message + " FAIL"); fails++; } }
   console.log("session state (slots, export, import) " + (fails ? "see above" : "ok"));
 }
+// 5. projections either side: up / fuse / mv / mvN and the whole attention half of a layer (encodeLayerR) against
+//    the same stages called one by one through the shim, and the GEMV alone against a float64 product
+{
+  let seed = 12345;
+  const rnd = () => { seed = (seed * 1664525 + 1013904223) >>> 0; return seed / 4294967296; };
+  const dim = 256, kvd = D.kvDim;
+  const f16bits = (x) => { const f = new Float32Array([x]), u = new Uint32Array(f.buffer)[0]; const s = (u >>> 16) & 0x8000, e = ((u >>> 23) & 255) - 112, m = u & 0x7fffff; return s | (e << 10) | (m >>> 13); };  // exact for the values below
+  const mkQ8 = (dOut, dIn) => { const qs = new Int8Array(dOut * dIn), sc = new Uint16Array(dOut * dIn / 32);
+    for (let i = 0; i < qs.length; i++) qs[i] = Math.floor(rnd() * 255) - 127;
+    for (let i = 0; i < sc.length; i++) sc[i] = f16bits((1 + Math.floor(rnd() * 8)) / 4096);
+    return { kind: "q8", qs: qs, scales: sc, dOut: dOut, dIn: dIn }; };
+  const scaleOf = (bits) => (bits & 0x3ff | 0x400) * Math.pow(2, ((bits >> 10) & 31) - 25);
+  const eq = mkQ8(qIn, dim), ek = mkQ8(kvd, dim), ev = mkQ8(kvd, dim), eo = mkQ8(dim, D.qDim);
+  const wqkv = A.up(A.fuse([eq, ek, ev])), wo = A.up(eo);
+  const nw = new Float32Array(dim).map(() => 0.9 + 0.2 * rnd()), x0 = new Float32Array(dim).map(() => 2 * rnd() - 1);
+  A.setLayerProj(0, wqkv, wo, nw);
+  const pos = base + n - 1;                                      // rewrite the last token's row
+  // (a) stage by stage: normed [q | k | v] GEMV into one buffer, then the columns the attention step reads
+  const addon = require(path.join(__dirname, "..", "..", "pooled_amd", "lib", "pooled_attn.node"));
+  const malloc = (nf) => addon.malloc(A.ctx, nf * 4);
+  const dQkv = malloc(qIn + 2 * kvd), dX = malloc(dim), dXn = malloc(dim);
+  addon.upload(A.ctx, dX, x0);
+  A.mvN(null, wqkv, dX, A.layers[0].attnNorm, dQkv, dXn);
+  A.sync();
+  const qkv = new Float32Array(qIn + 2 * kvd); addon.download(A.ctx, qkv, dQkv, 0);
+  const xn = new Float32Array(dim); addon.download(A.ctx, xn, dXn, 0);
+  // GEMV alone against float64 over the same normed vector
+  const refRow = (e, r, xv) => { let acc = 0; for (let b = 0; b < e.dIn / 32; b++) { let t = 0; for (let j = 0; j < 32; j++) t += e.qs[r * e.dIn + b * 32 + j] * xv[b * 32 + j]; acc += scaleOf(e.scales[r * e.dIn / 32 + b]) * t; } return acc; };
+  const want = new Float32Array(qkv.length);
+  for (let r = 0; r < qIn; r++) want[r] = refRow(eq, r, xn);
+  for (let r = 0; r < kvd; r++) { want[qIn + r] = refRow(ek, r, xn); want[qIn + kvd + r] = refRow(ev, r, xn); }
+  check("mvN over fuse([q, k, v]) vs float64", qkv, want);
+  A.writeColumn(A.B.qFull, 0, qkv.subarray(0, qIn)); A.writeColumn(A.B.k, 0, qkv.subarray(qIn, qIn + kvd)); A.writeColumn(A.B.v, 0, qkv.subarray(qIn + kvd));
+  A.encodeLayerAttn(null, 0, pos);
+  A.mv(null, wo, A.B.attnOut.ptr, dX, true);
+  A.sync();
+  const xSteps = new Float32Array(dim); addon.download(A.ctx, xSteps, dX, 0);
+  // (b) the same token through encodeLayerR
+  A.writeColumn(A.B.x, 0, x0);
+  A.encodeLayerR(null, 0, pos);
+  A.sync();
+  const xLayer = A.readColumn(A.B.x, 0);
+  if (!eqBits(new Uint32Array(xLayer.buffer), new Uint32Array(xSteps.buffer))) { console.log("encodeLayerR differs from its stages called one by one FAIL"); fails++; }
+  let moved = 0; for (let i = 0; i < dim; i++) moved = Math.max(moved, Math.abs(xLayer[i] - x0[i]));
+  if (!(moved > 1e-4)) { console.log("encodeLayerR left the residual unchanged FAIL"); fails++; }
+  for (const p of [dQkv, dX, dXn]) addon.free(A.ctx, p);
+  console.log("projections (up, fuse, mv, mvN, encodeLayerR) " + (fails ? "see above" : "ok"));
+}
 A.destroy();
 console.log(fails ? "SHIM FAIL" : "SHIM PASS");
 process.exit(fails ? 1 : 0);

@@ -1,0 +1,118 @@
+"""GPU tests of the one-token projections either side of the attention block (pa_gemv, pa_gemv_norm,
+pa_attn_layer_decode) through the C ABI, against the oracle's dequantise-and-multiply in f64.
+
+The reference checks its GEMVs against a CPU product of the dequantised weights with a tolerance relative to the
+output scale (engine/selftest.js:120-139: max-abs / scale < 2e-3; tests/test_gemm.js:13-14, :105: ~1e-6 for
+summation order alone).  Here: 2e-5 of the largest output for a GEMV alone, the path's 2e-3 / 1e-2 gate for the layer.
+"""
+import numpy as np
+import pytest
+from oracle import attn_oracle as O
+from pooled_amd.capi import PooledAttn, PaError, PA_W_F32, PA_W_Q8_0, PA_W_Q4_0, PA_ERR_INVALID, PA_ERR_UNSUPPORTED
+from helpers import SHAPES, assert_parity, oracle_cache
+
+pytestmark = pytest.mark.gpu
+
+
+def _weights(kind, d_out, d_in, rng, scale=0.02):
+    """Random weight planes of a kind: (w, scales-or-None)."""
+    if kind == PA_W_F32:
+        return (rng.standard_normal((d_out, d_in)) * scale).astype(np.float32), None
+    sc = np.asarray(rng.uniform(0.5, 1.5, (d_out, d_in // 32)) * scale / (127 if kind == PA_W_Q8_0 else 8) * 3, np.float16).view(np.uint16)
+    if kind == PA_W_Q8_0:
+        return rng.integers(-127, 128, (d_out, d_in)).astype(np.int8), sc
+    return rng.integers(0, 256, (d_out, d_in // 2)).astype(np.uint8), sc
+
+
+def _rel(got, ref):
+    return np.abs(np.asarray(got, np.float64) - ref).max() / max(np.abs(ref).max(), 1e-30)
+
+
+@pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q8_0, PA_W_Q4_0])
+@pytest.mark.parametrize("d_out,d_in", [(9216, 2048), (2048, 4096), (1, 32), (37, 96), (5000, 6144), (130, 8192)])
+def test_gemv_matches_oracle(kind, d_out, d_in):
+    if kind == PA_W_F32 and d_in > 4096:
+        pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
+    rng = np.random.default_rng(d_out * 7 + d_in + kind)
+    w, sc = _weights(kind, d_out, d_in, rng)
+    x = rng.standard_normal(d_in).astype(np.float32)
+    y0 = rng.standard_normal(d_out).astype(np.float32)
+    ref = O.gemv(kind, w, sc, x)
+    with PooledAttn(SHAPES["qwen36_moe"], 64, n_layers=1, max_cols=1) as pa:
+        wh = pa.weight(kind, w, sc)
+        dx = pa.to_device(x); dy = pa.to_device(y0)
+        pa.gemv(wh, dx, dy); pa.sync()
+        got = dy.download(np.float32, d_out)
+        assert _rel(got, ref) < 2e-5, "plain"
+        pa.gemv(wh, dx, dy, acc=True); pa.sync()                      # y = W x, then y += W x
+        assert _rel(dy.download(np.float32, d_out), 2.0 * ref) < 2e-5, "accumulate"
+        # deterministic run to run
+        pa.gemv(wh, dx, dy); pa.sync()
+        assert np.array_equal(dy.download(np.float32, d_out), got)
+
+
+@pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q4_0])
+def test_gemv_norm_matches_rmsnorm_then_gemv(kind):
+    cfg = SHAPES["qwen36_moe"]
+    d_out, d_in = 1024 + 3, 2048
+    rng = np.random.default_rng(11 + kind)
+    w, sc = _weights(kind, d_out, d_in, rng)
+    x = (rng.standard_normal(d_in) * 3.0).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(d_in)).astype(np.float32)
+    xn_ref = O.rmsnorm(x, nw, cfg["eps"])
+    ref = O.gemv(kind, w, sc, xn_ref)
+    with PooledAttn(cfg, 64, n_layers=1, max_cols=1) as pa:
+        wh = pa.weight(kind, w, sc)
+        dx = pa.to_device(x); dnw = pa.to_device(nw); dy = pa.alloc(d_out * 4); dxn = pa.alloc(d_in * 4)
+        pa.gemv_norm(wh, dx, dnw, dy, dxn); pa.sync()
+        assert _rel(dxn.download(np.float32, d_in), xn_ref.astype(np.float64)) < 1e-6
+        assert _rel(dy.download(np.float32, d_out), ref) < 2e-5
+        pa.gemv_norm(wh, dx, dnw, dy); pa.sync()                      # without the xn copy
+        assert _rel(dy.download(np.float32, d_out), ref) < 2e-5
+
+
+def test_weight_and_gemv_errors():
+    with PooledAttn(SHAPES["qwen36_moe"], 64, n_layers=1, max_cols=1) as pa:
+        with pytest.raises(PaError) as e:
+            pa.weight(PA_W_Q8_0, np.zeros((4, 48), np.int8), np.zeros((4, 1), np.uint16))       # d_in not a multiple of 32
+        assert e.value.code == PA_ERR_INVALID
+        with pytest.raises(PaError) as e:
+            pa.weight(PA_W_Q4_0, np.zeros((4, 8192), np.uint8), np.zeros((4, 512), np.uint16))  # d_in 16384
+        assert e.value.code == PA_ERR_UNSUPPORTED
+        with pytest.raises(PaError) as e:
+            pa.weight(7, np.zeros((4, 32), np.float32))
+        assert e.value.code == PA_ERR_INVALID
+
+
+@pytest.mark.parametrize("shape,dim,kind,pos", [("qwen36_moe", 2048, PA_W_Q4_0, 777), ("qwen36_moe", 2048, PA_W_Q8_0, 0),
+                                                 ("qwen3_1p7b", 2048, PA_W_Q4_0, 300), ("qwen38_27b", 5120, PA_W_Q8_0, 1029)])
+def test_attn_layer_decode_matches_oracle(shape, dim, kind, pos):
+    """rmsnorm -> [q | k | v] -> pre-step -> attention over the cache -> gate -> wo, accumulated into x: the residual
+    and the new cache rows against the oracle's composition of the same stages."""
+    cfg = SHAPES[shape]
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    qd, kvd = nH * hd, nKV * hd
+    q_rows = qd * (2 if cfg["gate"] else 1)
+    rng = np.random.default_rng(pos + dim)
+    w_qkv, s_qkv = _weights(kind, q_rows + 2 * kvd, dim, rng, scale=0.03)
+    w_o, s_o = _weights(kind, dim, qd, rng, scale=0.03)
+    x = rng.standard_normal(dim).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
+    qw = (1 + 0.1 * rng.standard_normal(hd)).astype(np.float32); kw = (1 + 0.1 * rng.standard_normal(hd)).astype(np.float32)
+    k16, v16 = oracle_cache(cfg, rng.standard_normal((pos, kvd)).astype(np.float32), rng.standard_normal((pos, kvd)).astype(np.float32), kw)
+    x_ref, k_row, v_row = O.attn_layer_decode(x, kind, w_qkv, s_qkv, kind, w_o, s_o, nw, qw, kw, k16, v16, pos, cfg)
+    with PooledAttn(cfg, pos + 8, n_layers=1, max_cols=1) as pa:
+        pa.layer_alloc(0)
+        if pos:
+            pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
+        wq = pa.weight(kind, w_qkv, s_qkv); wo = pa.weight(kind, w_o, s_o)
+        dx = pa.to_device(x); dnw = pa.to_device(nw); dqw = pa.to_device(qw); dkw = pa.to_device(kw)
+        pa.attn_layer_decode(0, wq, wo, dnw, dqw, dkw, dx, pos); pa.sync()
+        got = dx.download(np.float32, dim)
+        kc = pa.kv_read(0, 0, pos, 1).view(np.float16).astype(np.float64); vc = pa.kv_read(0, 1, pos, 1).view(np.float16).astype(np.float64)
+    assert_parity(got, x_ref, "layer %s pos %d" % (shape, pos))
+    # the new cache rows: f16 of GEMV outputs that differ from the oracle's f64 products in the last f32 bits, so a
+    # value next to a rounding boundary may land one f16 step away
+    for a, b in ((kc, k_row), (vc, v_row)):
+        ref = np.asarray(b).reshape(a.shape).view(np.float16).astype(np.float64)
+        assert np.abs(a - ref).max() <= np.abs(ref).max() * 2.0 ** -10

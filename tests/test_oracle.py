@@ -255,3 +255,57 @@ def test_q8_quantize_known_answers():
     assert q.shape == x.shape and sc.shape == (5, 3, 8)
     blocks = x.reshape(5, 3, 8, 32)
     assert np.array_equal(np.abs(q.reshape(5, 3, 8, 32)).max(-1), np.full((5, 3, 8), 127))     # the block maximum maps to +-127
+
+
+# ---- projections: weight planes, GEMV, rmsnorm ------------------------------------------------------------------
+
+def _f16b(x):
+    return np.asarray(x, np.float16).view(np.uint16)
+
+
+def test_w_dequant_known_blocks():
+    """Hand-made blocks: nibble order and sign of Q4_0 (engine/wgsl/base.js:81-83), byte order and sign of Q8_0."""
+    # Q4_0, one row of one block, scale 0.5: byte j = (low nibble -> element j, high nibble -> element j + 16)
+    b = np.zeros((1, 16), np.uint8)
+    b[0, 0] = 0xF0          # element 0: nibble 0 -> -8;  element 16: nibble 15 -> +7
+    b[0, 3] = 0x89          # element 3: nibble 9 -> +1;  element 19: nibble 8 -> 0
+    b[0, 15] = 0x08         # element 15: nibble 8 -> 0;  element 31: nibble 0 -> -8
+    w = O.w_dequant(O.W_Q4_0, b, _f16b([[0.5]]))
+    want = np.full(32, -8.0 * 0.5)            # untouched bytes are 0x00: both nibbles 0 -> -8
+    want[0], want[16], want[3], want[19], want[15], want[31] = -4.0, 3.5, 0.5, 0.0, 0.0, -4.0
+    assert np.array_equal(w[0], want)
+    # Q8_0: two blocks with different scales, negative values
+    q = np.zeros((1, 64), np.int8); q[0, 0], q[0, 31], q[0, 32], q[0, 63] = -128, 127, 5, -1
+    w = O.w_dequant(O.W_Q8_0, q, _f16b([[0.25, 2.0]]))
+    assert w[0, 0] == -32.0 and w[0, 31] == 31.75 and w[0, 32] == 10.0 and w[0, 63] == -2.0 and np.count_nonzero(w) == 4
+
+
+def test_gemv_matches_the_reference_loops_and_is_linear():
+    rng = np.random.default_rng(3)
+    d_out, d_in = 5, 96
+    x = rng.standard_normal(d_in).astype(np.float32)
+    sc = _f16b(rng.uniform(0.01, 0.2, (d_out, d_in // 32)))
+    cases = [(O.W_F32, rng.standard_normal((d_out, d_in)).astype(np.float32), None),
+             (O.W_Q8_0, rng.integers(-128, 128, (d_out, d_in)).astype(np.int8), sc),
+             (O.W_Q4_0, rng.integers(0, 256, (d_out, d_in // 2)).astype(np.uint8), sc)]
+    for kind, w, s in cases:
+        y = O.gemv(kind, w, s, x)
+        assert np.allclose(y, O.gemv_reference_loops(kind, w, s, x), rtol=1e-12, atol=1e-12)
+        # unit vectors pick columns of the dequantised matrix; linearity
+        e = np.zeros(d_in, np.float32); e[37] = 1.0
+        assert np.array_equal(O.gemv(kind, w, s, e), O.w_dequant(kind, w, s)[:, 37])
+        x2 = rng.standard_normal(d_in).astype(np.float32)
+        lhs = O.gemv(kind, w, s, x) * 2.0 + O.gemv(kind, w, s, x2)
+        assert np.allclose(lhs, O.w_dequant(kind, w, s) @ (2.0 * x.astype(np.float64) + x2), rtol=1e-12)
+
+
+def test_rmsnorm_closed_forms():
+    n, eps = 64, 1e-6
+    w = np.linspace(0.5, 1.5, n).astype(np.float32)
+    x = np.full(n, 3.0, np.float32)
+    assert np.allclose(O.rmsnorm(x, w, eps), w * 3.0 / np.sqrt(9.0 + eps), rtol=1e-6)
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(n).astype(np.float32)
+    y = O.rmsnorm(x, np.ones(n, np.float32), 0.0)
+    assert abs(np.mean(y.astype(np.float64) ** 2) - 1.0) < 1e-6                      # unit RMS
+    assert np.allclose(O.rmsnorm(4.0 * x, w, 0.0), O.rmsnorm(x, w, 0.0), rtol=1e-6)  # scale invariance at eps = 0
