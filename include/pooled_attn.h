@@ -240,6 +240,24 @@ int pa_gemv_norm(pa_ctx* ctx, const pa_weight* w, const float* d_x_raw, const fl
 int pa_attn_layer_decode(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
                          const float* d_qw, const float* d_kw, float* d_x, uint32_t pos);
 
+/* ---- the same projections for column-batched passes (prefill chunks, verify blocks) on the f16 matrix cores.
+ *      Replace the reference's batched GEMMs over the same weight planes (engine/wgsl/gemm.js, gemm_sgm.js,
+ *      gemm_wide.js; dispatched at engine/qwen35.js:2142-2170, :2600-2620) with its "f16" prefill math
+ *      (gemm.js:31-36): dequantised weights and activations rounded to f16, products and sums f32. ---- */
+/* xn[c] = f16(rmsnorm(x[c]) * norm_w) for n_cols columns of dim floats (strides in elements); eps from pa_config */
+int pa_rmsnorm_f16(pa_ctx* ctx, const float* d_x, uint32_t x_stride, const float* d_norm_w, uint32_t dim, uint32_t n_cols,
+                   void* d_xn_f16, uint32_t xn_stride);
+/* y[c][0 .. d_out) = W x[c] for n_cols columns; x: f16 bits, stride in f16 elements (>= d_in, multiple of 8);
+ * y: f32, stride in floats; acc != 0: y += W x */
+int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uint32_t x_stride, uint32_t n_cols, float* d_y, uint32_t y_stride, int acc);
+/* n_cols tokens at positions base_pos .. through the attention half of a full-attention layer, as
+ * _encodeLayerBatch / _encodeLayerWide record it (engine/qwen35.js:2416-2425, :2827): rmsnorm -> [q | k | v] GEMM ->
+ * pre-step + cache write -> causal attention -> gate -> wo GEMM accumulated into the residual columns d_x
+ * [n_cols][x_stride] (f32, read and updated in place).  Weights as pa_attn_layer_decode.  Five launches (six when
+ * the attention pass is split).  f16 caches only; n_cols <= max_cols. */
+int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
+                          const float* d_qw, const float* d_kw, float* d_x, uint32_t x_stride, uint32_t base_pos, uint32_t n_cols);
+
 /* Device probe (measurement infrastructure, no counterpart in the reference): runs back-to-back
  * v_mfma_f32_32x32x16_f16 on every CU for iters x 64 instructions per wavefront, with constant operands
  * (random_operands = 0) or random f16 fragments, and returns the achieved TFLOP/s and the mean shader clock during

@@ -418,3 +418,39 @@ def attn_layer_decode(x, kind_qkv, w_qkv, sc_qkv, kind_o, w_o, sc_o, attn_norm_w
     out = attention(g["q"], kall, vall, pos, gate=g["gate"] if gated else None)            # [1, nH, hd]
     y = gemv(kind_o, w_o, sc_o, np.asarray(out, dtype=np.float32).reshape(-1))
     return (np.asarray(x, dtype=np.float32).astype(np.float64) + y).astype(np.float32), g["k16"], g["v16"]
+
+
+def gemm_f16(kind, w, scales, x):
+    """Y[c] = W x[c] with the reference's "f16" prefill math: every dequantised weight and every activation rounded
+    to f16, products and sums exact (f64 here, f32 in the kernels).  x: [n, d_in] f32 (or f16-representable) -> [n, d_out].
+
+    Reference: engine/wgsl/gemm.js:31-36 (the r16 twins: "every dequantized weight and every activation rounded to f16
+    (pack2x16float), products and sums still f32 ... the operand precision of the tensor-core path"), gemm_sgm.js.
+    """
+    w16 = w_dequant(kind, w, scales).astype(np.float32).astype(np.float16).astype(np.float64)     # the product is exact in f32
+    x16 = np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float64)
+    return x16 @ w16.T
+
+
+def attn_layer_prefill(x, kind_qkv, w_qkv, sc_qkv, kind_o, w_o, sc_o, attn_norm_w, qw, kw, k16, v16, base_pos, cfg):
+    """n tokens at positions base_pos .. through the attention half of a full-attention layer; returns (x_out f32
+    [n, dim], new k16 rows, new v16 rows).  k16 / v16: cache rows [0, base_pos).
+
+    Reference: engine/qwen35.js:2416-2425 (_encodeLayerBatch), :2827 (_encodeLayerWide): per-column rmsnorm -> batched
+    q / k / v GEMMs -> pre-step + KV write -> causal attention -> gate -> wo GEMM -> residual add, with the f16 operand
+    rounding of gemm_f16 on both GEMMs (the attention output is handed over as f16).
+    """
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    gated = cfg.get("gate", False)
+    x = np.asarray(x, dtype=np.float32)
+    n = x.shape[0]
+    xn = np.stack([rmsnorm(x[c], attn_norm_w, cfg["eps"]) for c in range(n)])
+    qkv = gemm_f16(kind_qkv, w_qkv, sc_qkv, xn).astype(np.float32)
+    q_rows = nH * hd * (2 if gated else 1)
+    kvd = nKV * hd
+    g = glue_kv(qkv[:, :q_rows], qkv[:, q_rows:q_rows + kvd], qkv[:, q_rows + kvd:], qw, kw, base_pos, cfg)
+    kall = np.concatenate([np.asarray(k16).reshape(base_pos, nKV, hd), g["k16"].reshape(n, nKV, hd)])
+    vall = np.concatenate([np.asarray(v16).reshape(base_pos, nKV, hd), g["v16"].reshape(n, nKV, hd)])
+    out = attention(g["q"], kall, vall, base_pos, gate=g["gate"] if gated else None)       # [n, nH, hd]
+    y = gemm_f16(kind_o, w_o, sc_o, np.asarray(out, dtype=np.float32).reshape(n, -1))
+    return (x.astype(np.float64) + y).astype(np.float32), g["k16"], g["v16"]

@@ -74,6 +74,9 @@ SYMBOLS = {
     "pa_gemv": (c_int, [vp, vp, f32p, f32p, c_int]),
     "pa_gemv_norm": (c_int, [vp, vp, f32p, f32p, f32p, f32p]),
     "pa_attn_layer_decode": (c_int, [vp, u32, vp, vp, f32p, f32p, f32p, f32p, u32]),
+    "pa_rmsnorm_f16": (c_int, [vp, f32p, u32, f32p, u32, u32, vp, u32]),
+    "pa_gemm": (c_int, [vp, vp, vp, u32, u32, f32p, u32, c_int]),
+    "pa_attn_layer_prefill": (c_int, [vp, u32, vp, vp, f32p, f32p, f32p, f32p, u32, u32, u32]),
     "pa_version": (ctypes.c_char_p, []),
 }
 
@@ -327,6 +330,16 @@ class PooledAttn:
     def attn_layer_decode(self, layer, w_qkv, w_o, d_attn_norm_w, d_qw, d_kw, d_x, pos):
         self._chk(self.L.pa_attn_layer_decode(self.ctx, layer, w_qkv, w_o, d_attn_norm_w.ptr, d_qw.ptr if d_qw else None,
                                               d_kw.ptr if d_kw else None, d_x.ptr, pos))
+
+    def rmsnorm_f16(self, d_x, x_stride, d_norm_w, dim, n_cols, d_xn, xn_stride):
+        self._chk(self.L.pa_rmsnorm_f16(self.ctx, d_x.ptr, x_stride, d_norm_w.ptr, dim, n_cols, d_xn.ptr, xn_stride))
+
+    def gemm(self, w, d_x16, x_stride, n_cols, d_y, y_stride, acc=False):
+        self._chk(self.L.pa_gemm(self.ctx, w, d_x16.ptr, x_stride, n_cols, d_y.ptr, y_stride, int(bool(acc))))
+
+    def attn_layer_prefill(self, layer, w_qkv, w_o, d_attn_norm_w, d_qw, d_kw, d_x, x_stride, base_pos, n_cols):
+        self._chk(self.L.pa_attn_layer_prefill(self.ctx, layer, w_qkv, w_o, d_attn_norm_w.ptr, d_qw.ptr if d_qw else None,
+                                               d_kw.ptr if d_kw else None, d_x.ptr, x_stride, base_pos, n_cols))
 
     def mfma_probe(self, random_operands, iters):
         """(TFLOP/s, shader MHz) of back-to-back f16 MFMAs on every CU with constant or random operands."""

@@ -113,6 +113,7 @@ extern "C" int pa_destroy(pa_ctx* ctx) {
   if (ctx->part_o) (void)hipFree(ctx->part_o);
   if (ctx->part_ml) (void)hipFree(ctx->part_ml);
   if (ctx->proj_buf) (void)hipFree(ctx->proj_buf);
+  if (ctx->chunk_buf) (void)hipFree(ctx->chunk_buf);
   for (auto ev : ctx->prof_events) (void)hipEventDestroy(ev);
   if (ctx->t0) (void)hipEventDestroy(ctx->t0);
   if (ctx->t1) (void)hipEventDestroy(ctx->t1);
@@ -573,6 +574,66 @@ extern "C" int pa_attn_layer_decode(pa_ctx* ctx, uint32_t layer, const pa_weight
   if (rc) return rc;
   if ((rc = pa_attn_decode_step(ctx, layer, qkv, qkv + q_rows, qkv + q_rows + kvd, d_qw, d_kw, pos, attn_out, PA_OUT_F32))) return rc;
   return gemv_common(ctx, who, w_o, attn_out, nullptr, nullptr, d_x, 1);
+}
+
+extern "C" int pa_rmsnorm_f16(pa_ctx* ctx, const float* d_x, uint32_t x_stride, const float* d_norm_w, uint32_t dim, uint32_t n_cols,
+                              void* d_xn_f16, uint32_t xn_stride) {
+  const char* who = "pa_rmsnorm_f16";
+  if (!ctx) return PA_ERR_INVALID;
+  if (!d_x || !d_norm_w || !d_xn_f16) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null argument");
+  if (dim == 0 || (dim & 3) || n_cols == 0 || x_stride < dim || xn_stride < dim || (x_stride & 3) || (xn_stride & 3))
+    return fail(ctx, PA_ERR_INVALID, std::string(who) + ": dim and strides must be positive multiples of 4, strides >= dim");
+  if (((uintptr_t)d_x & 15) || ((uintptr_t)d_norm_w & 15) || ((uintptr_t)d_xn_f16 & 7))
+    return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned");
+  HIPCHK(ctx, pa_launch_rmsnorm_f16(d_x, x_stride, d_norm_w, dim, ctx->cfg.eps, n_cols, (uint16_t*)d_xn_f16, xn_stride, ctx->stream));
+  return PA_OK;
+}
+
+extern "C" int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uint32_t x_stride, uint32_t n_cols, float* d_y, uint32_t y_stride, int acc) {
+  const char* who = "pa_gemm";
+  if (!ctx) return PA_ERR_INVALID;
+  if (!w || !d_x_f16 || !d_y) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null argument");
+  if (n_cols == 0 || x_stride < w->d_in || (x_stride & 7) || y_stride < w->d_out || ((uintptr_t)d_x_f16 & 15) || ((uintptr_t)d_y & 3))
+    return fail(ctx, PA_ERR_INVALID, std::string(who) + ": x stride must be a multiple of 8 halves and >= d_in, y stride >= d_out, x 16-byte aligned");
+  GemmParams p; memset(&p, 0, sizeof p);
+  p.w = w->w; p.scales = w->scales; p.x = (const uint16_t*)d_x_f16; p.y = d_y; p.x_stride = x_stride; p.y_stride = y_stride;
+  p.d_out = w->d_out; p.d_in = w->d_in; p.n_cols = n_cols; p.acc = acc; p.kind = w->kind;
+  HIPCHK(ctx, pa_launch_gemm(p, ctx->stream));
+  return PA_OK;
+}
+
+extern "C" int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
+                                     const float* d_qw, const float* d_kw, float* d_x, uint32_t x_stride, uint32_t base_pos, uint32_t n_cols) {
+  const char* who = "pa_attn_layer_prefill";
+  if (!ctx) return PA_ERR_INVALID;
+  const pa_config& c = ctx->cfg;
+  if (!w_qkv || !w_o || !d_attn_norm_w || !d_x) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null argument");
+  if (kv_q8(ctx)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": f16 caches only");
+  int rc = check_cols(ctx, who, layer, true, base_pos, n_cols);
+  if (rc) return rc;
+  const uint32_t qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim, dim = w_qkv->d_in;
+  const bool gated = (c.flags & PA_FLAG_GATE) != 0;
+  const uint32_t q_rows = qd * (gated ? 2 : 1), rows = q_rows + 2 * kvd;
+  if (w_qkv->d_out != rows) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": w_qkv must have q (+ gate), k and v rows");
+  if (w_o->d_in != qd || w_o->d_out != dim) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": w_o must map n_heads x head_dim back to the model width");
+  if (x_stride < dim || (x_stride & 3) || (dim & 7)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": residual stride must be a multiple of 4 floats and >= the model width");
+  // chunk scratch: xn f16 [cols][dim] | qkv f32 [cols][rows] | attnOut f16 [cols][qd], each 256-byte aligned
+  auto up256 = [](size_t b) { return (b + 255) & ~(size_t)255; };
+  const size_t b_xn = up256((size_t)n_cols * dim * 2), b_qkv = up256((size_t)n_cols * rows * 4), b_at = up256((size_t)n_cols * qd * 2);
+  if (b_xn + b_qkv + b_at > ctx->chunk_buf_bytes) {
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->chunk_buf) { HIPCHK(ctx, hipFree(ctx->chunk_buf)); ctx->chunk_buf = nullptr; ctx->chunk_buf_bytes = 0; }
+    HIPCHK(ctx, hipMalloc(&ctx->chunk_buf, b_xn + b_qkv + b_at));
+    ctx->chunk_buf_bytes = b_xn + b_qkv + b_at;
+  }
+  uint16_t* xn = (uint16_t*)ctx->chunk_buf;
+  float* qkv = (float*)((unsigned char*)ctx->chunk_buf + b_xn);
+  uint16_t* at = (uint16_t*)((unsigned char*)ctx->chunk_buf + b_xn + b_qkv);
+  if ((rc = pa_rmsnorm_f16(ctx, d_x, x_stride, d_attn_norm_w, dim, n_cols, xn, dim))) return rc;
+  if ((rc = pa_gemm(ctx, w_qkv, xn, dim, n_cols, qkv, rows, 0))) return rc;
+  if ((rc = pa_glue_kv(ctx, layer, qkv, rows, qkv + q_rows, rows, qkv + q_rows + kvd, rows, d_qw, d_kw, base_pos, n_cols))) return rc;
+  if ((rc = pa_attn_prefill(ctx, layer, nullptr, 0, gated ? ctx->gate_buf : nullptr, qd, base_pos, n_cols, at, qd, PA_OUT_F16))) return rc;
+  return pa_gemm(ctx, w_o, at, qd, n_cols, d_x, x_stride, 1);
 }
 
 // ---- cache access ---------------------------------------------------------------------------------

@@ -95,6 +95,20 @@ struct GemvParams {
 };
 hipError_t pa_launch_gemv(const GemvParams& p, int n_cu, hipStream_t s);
 
+// column-batched projection Y[c][r] = sum_k W[r][k] X[c][k] (proj_gemm.hip): x = f16 bits [n_cols][x_stride], y = f32
+// [n_cols][y_stride]; weights as GemvParams; acc: y += W x
+struct GemmParams {
+  const void* w; const uint16_t* scales;
+  const uint16_t* x; float* y;
+  uint32_t x_stride, y_stride;
+  uint32_t d_out, d_in, n_cols;
+  int acc; int kind;
+};
+hipError_t pa_launch_gemm(const GemmParams& p, hipStream_t s);
+// rmsnorm of n_cols f32 columns, written as f16 (the GEMM's activation operand)
+hipError_t pa_launch_rmsnorm_f16(const float* x, uint32_t x_stride, const float* w, uint32_t dim, float eps, uint32_t n_cols,
+                                 uint16_t* out, uint32_t out_stride, hipStream_t s);
+
 // device probe (probe.hip): sustained f16 MFMA rate and shader clock, constant or random operands
 hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, uint32_t iters, hipStream_t st, float* tflops, float* shader_mhz);
 
@@ -136,6 +150,8 @@ struct pa_ctx {
   size_t part_o_bytes = 0, part_ml_bytes = 0;
   float* proj_buf = nullptr;    // pa_attn_layer_decode: [q(+gate) | k | v] projections, then attnOut [nH*hd]
   size_t proj_buf_floats = 0;
+  void* chunk_buf = nullptr;    // pa_attn_layer_prefill: xn f16 [cols][dim], qkv f32 [cols][rows], attnOut f16 [cols][nH*hd]
+  size_t chunk_buf_bytes = 0;
   uint32_t decode_splits_override = 0;
   // timing
   hipEvent_t t0 = nullptr, t1 = nullptr;

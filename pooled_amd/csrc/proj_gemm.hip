@@ -1,0 +1,207 @@
+// Column-batched projections either side of the attention block on gfx950 (prefill chunks, verify blocks):
+// Y[c][r] = sum_k W[r][k] X[c][k] for f32, Q8_0 and Q4_0 weights on the f16 matrix cores, and the input rmsnorm of a
+// chunk written as the f16 operand the GEMM reads.
+//
+// Replaces the reference's batched GEMMs over the same weight planes (engine/wgsl/gemm.js:1-60 row-stationary ALU
+// GEMM, engine/wgsl/gemm_sgm.js tensor-core path, dispatched by engine/qwen35.js:2142-2170 and :2600-2620) and the
+// per-column rmsnorm in front of them.  Operand precision is the reference's "f16" prefill math (gemm.js:31-36, the
+// r16 twins = what its tensor-core path computes): every dequantised weight (nibble - 8) * scale and every activation
+// rounded to f16, products and sums in f32.
+//
+// Workgroup = 128 columns x 128 weight rows, 4 wavefronts of 64 x 64 (2 x 2 v_mfma_f32_32x32x16_f16 tiles), K in
+// steps of one quantisation block (32): the 256 threads fetch the next step's 128 x 32 activations (f16) and 128 x 32
+// weights (packed, one scale a row) into registers while the matrix cores work on the current step out of LDS,
+// widen the weights to f16 on the way into LDS (0x6400 | nibble is the f16 1024 + nibble: one byte permute, a packed
+// subtract and a packed multiply by the scale for two weights), and swap two LDS buffers with one barrier a step.
+// Rows of the LDS tiles are 80 bytes apart so that the 128-bit fragment reads are bank-conflict free.  The activation
+// is the MFMA A operand and the weight the B operand: a lane then owns one weight row and four consecutive columns per
+// accumulator quad, and a wave-wide store covers 32 consecutive rows of a column (128 bytes).
+#include "pa_internal.h"
+#include "glue_math.h"
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+
+#define GT 128          // tile edge (columns and rows per workgroup)
+#define GK 32           // K per step = one quantisation block
+#define GROW 80         // LDS row stride in bytes (64 of data + 16 of padding)
+
+static __device__ inline h2 as_h2(uint32_t u) { h2 r; __builtin_memcpy(&r, &u, 4); return r; }
+
+// two bytes of a word (byte indices by the selector) -> two f16 = (byte - bias) * scale
+static __device__ inline h2 bytes_to_h2(uint32_t w, uint32_t sel, h2 bias, h2 sc) {
+  return (as_h2(__builtin_amdgcn_perm(0x64646464u, w, sel)) - bias) * sc;
+}
+
+// 16 weights of one (row, block half) as two h8, from the packed registers of a kind
+template <int KIND> struct WRegs;
+template <> struct WRegs<PA_W_Q4_0> { u2 q; uint16_t sc; };      // bytes 8h .. 8h + 7: elements 8h + j (low), 16 + 8h + j (high)
+template <> struct WRegs<PA_W_Q8_0> { u4 q; uint16_t sc; };      // elements 16h .. 16h + 15
+template <> struct WRegs<PA_W_F32> { f4 q[4]; uint16_t sc; };    // elements 16h .. 16h + 15
+
+template <int KIND>
+static __device__ inline void w_load(WRegs<KIND>& r, const GemmParams& p, size_t row, uint32_t nb, uint32_t kb, uint32_t half) {
+  const unsigned char* base = (const unsigned char*)p.w;
+  if constexpr (KIND == PA_W_Q4_0) {
+    r.q = *(const u2*)(base + (row * nb + kb) * 16 + 8 * half);
+    r.sc = p.scales[row * nb + kb];
+  } else if constexpr (KIND == PA_W_Q8_0) {
+    r.q = *(const u4*)(base + (row * nb + kb) * 32 + 16 * half);
+    r.sc = p.scales[row * nb + kb];
+  } else {
+    const f4* s = (const f4*)(base + ((row * nb + kb) * 32 + 16 * half) * 4);
+#pragma unroll
+    for (int i = 0; i < 4; i++) r.q[i] = s[i];
+    r.sc = 0;
+  }
+}
+
+// widen and store: dst = the row's 32 halves in LDS
+template <int KIND>
+static __device__ inline void w_store(const WRegs<KIND>& r, unsigned char* dst, uint32_t half) {
+  if constexpr (KIND == PA_W_Q4_0) {
+    const _Float16 s = __ushort_as_half(r.sc);
+    const h2 sc = { s, s }, bias = { (_Float16)1032.f, (_Float16)1032.f };      // 0x6400 | n = 1024 + n; n - 8
+    h2 lo[4], hi[4];
+#pragma unroll
+    for (int w = 0; w < 2; w++) {
+      const uint32_t l = r.q[w] & 0x0F0F0F0Fu, h = (r.q[w] >> 4) & 0x0F0F0F0Fu;
+      lo[2 * w] = bytes_to_h2(l, 0x04010400u, bias, sc); lo[2 * w + 1] = bytes_to_h2(l, 0x04030402u, bias, sc);
+      hi[2 * w] = bytes_to_h2(h, 0x04010400u, bias, sc); hi[2 * w + 1] = bytes_to_h2(h, 0x04030402u, bias, sc);
+    }
+    *(h8*)(dst + (8 * half) * 2) = (h8){ lo[0][0], lo[0][1], lo[1][0], lo[1][1], lo[2][0], lo[2][1], lo[3][0], lo[3][1] };
+    *(h8*)(dst + (16 + 8 * half) * 2) = (h8){ hi[0][0], hi[0][1], hi[1][0], hi[1][1], hi[2][0], hi[2][1], hi[3][0], hi[3][1] };
+  } else if constexpr (KIND == PA_W_Q8_0) {
+    const _Float16 s = __ushort_as_half(r.sc);
+    const h2 sc = { s, s }, bias = { (_Float16)1152.f, (_Float16)1152.f };      // 0x6400 | (v + 128) = 1152 + v
+    h2 o[8];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      const uint32_t x = r.q[w] ^ 0x80808080u;
+      o[2 * w] = bytes_to_h2(x, 0x04010400u, bias, sc); o[2 * w + 1] = bytes_to_h2(x, 0x04030402u, bias, sc);
+    }
+    *(h8*)(dst + (16 * half) * 2) = (h8){ o[0][0], o[0][1], o[1][0], o[1][1], o[2][0], o[2][1], o[3][0], o[3][1] };
+    *(h8*)(dst + (16 * half + 8) * 2) = (h8){ o[4][0], o[4][1], o[5][0], o[5][1], o[6][0], o[6][1], o[7][0], o[7][1] };
+  } else {
+    h8 a, b;
+#pragma unroll
+    for (int j = 0; j < 4; j++) { a[j] = (_Float16)r.q[0][j]; a[4 + j] = (_Float16)r.q[1][j]; b[j] = (_Float16)r.q[2][j]; b[4 + j] = (_Float16)r.q[3][j]; }
+    *(h8*)(dst + (16 * half) * 2) = a;
+    *(h8*)(dst + (16 * half + 8) * 2) = b;
+  }
+}
+
+template <int KIND>
+__global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
+  __shared__ __attribute__((aligned(16))) unsigned char xs[2][GT * GROW];
+  __shared__ __attribute__((aligned(16))) unsigned char ws[2][GT * GROW];
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t wm = wave >> 1, wn = wave & 1;                       // the wave's 64 columns x 64 rows
+  const uint32_t r0 = blockIdx.x * GT, c0 = blockIdx.y * GT;
+  const uint32_t nb = p.d_in / GK;
+  // loaders: thread t fetches half a row of each tile
+  const uint32_t lrow = tid >> 1, half = tid & 1;
+  const size_t wrow = min((size_t)r0 + lrow, (size_t)p.d_out - 1);    // past the end: the last row again (never stored)
+  const size_t xcol = min((size_t)c0 + lrow, (size_t)p.n_cols - 1);
+  const unsigned char* xsrc = (const unsigned char*)(p.x + xcol * p.x_stride) + 32 * half;
+  WRegs<KIND> wr;
+  u4 xr[2];
+  auto fetch = [&](uint32_t kb) __attribute__((always_inline)) {
+    w_load<KIND>(wr, p, wrow, nb, kb, half);
+    xr[0] = *(const u4*)(xsrc + (size_t)kb * 64);
+    xr[1] = *(const u4*)(xsrc + (size_t)kb * 64 + 16);
+  };
+  auto stage = [&](int buf) __attribute__((always_inline)) {
+    w_store<KIND>(wr, ws[buf] + lrow * GROW, half);
+    *(u4*)(xs[buf] + lrow * GROW + 32 * half) = xr[0];
+    *(u4*)(xs[buf] + lrow * GROW + 32 * half + 16) = xr[1];
+  };
+  f16v acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  const uint32_t fl = lane & 31, fk = lane >> 5;                      // fragment row and 8-wide k group of this lane
+  for (uint32_t kb = 0; kb < nb; kb++) {
+    const int cur = kb & 1;
+    if (kb + 1 < nb) fetch(kb + 1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      h8 af[2], bf[2];
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        af[t] = *(const h8*)(xs[cur] + (wm * 64 + t * 32 + fl) * GROW + (ks * 16 + fk * 8) * 2);
+        bf[t] = *(const h8*)(ws[cur] + (wn * 64 + t * 32 + fl) * GROW + (ks * 16 + fk * 8) * 2);
+      }
+#pragma unroll
+      for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[a], bf[b], acc[a][b], 0, 0, 0);
+    }
+    if (kb + 1 < nb) stage(cur ^ 1);
+    __syncthreads();
+  }
+  // accumulator i of a tile: column 8 (i / 4) + 4 (lane / 32) + i % 4, row lane % 32
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+      const uint32_t row = r0 + wn * 64 + b * 32 + fl;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const uint32_t col = c0 + wm * 64 + a * 32 + 8 * (i / 4) + 4 * fk + (i % 4);
+        if (row < p.d_out && col < p.n_cols) {
+          float* y = p.y + (size_t)col * p.y_stride + row;
+          *y = p.acc ? *y + acc[a][b][i] : acc[a][b][i];
+        }
+      }
+    }
+}
+
+hipError_t pa_launch_gemm(const GemmParams& p, hipStream_t s) {
+  if (p.d_out == 0 || p.d_in == 0 || (p.d_in & 31) || p.n_cols == 0) return hipErrorInvalidValue;
+  const dim3 grid((p.d_out + GT - 1) / GT, (p.n_cols + GT - 1) / GT), block(256);
+  switch (p.kind) {
+    case PA_W_F32: hipLaunchKernelGGL(pa_gemm_kernel<PA_W_F32>, grid, block, 0, s, p); break;
+    case PA_W_Q8_0: hipLaunchKernelGGL(pa_gemm_kernel<PA_W_Q8_0>, grid, block, 0, s, p); break;
+    case PA_W_Q4_0: hipLaunchKernelGGL(pa_gemm_kernel<PA_W_Q4_0>, grid, block, 0, s, p); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+// rmsnorm of n_cols columns, written as f16: one workgroup per column.  xn = f16((x * inv) * w),
+// inv = 1 / sqrt(mean(x^2) + eps) (engine/wgsl/base.js:119-152); the sum of squares is a fixed-order tree.
+__global__ __launch_bounds__(256) void pa_rmsnorm_f16_kernel(const float* x, uint32_t x_stride, const float* w, uint32_t dim, float eps,
+                                                            uint16_t* out, uint32_t out_stride) {
+  __shared__ float red[4];
+  const uint32_t col = blockIdx.x, tid = threadIdx.x;
+  const f4* xs = (const f4*)(x + (size_t)col * x_stride);
+  float ss = 0.f;
+  for (uint32_t e = tid; e < dim / 4; e += 256) { const f4 v = xs[e]; ss = __builtin_fmaf(v[0], v[0], ss); ss = __builtin_fmaf(v[1], v[1], ss); ss = __builtin_fmaf(v[2], v[2], ss); ss = __builtin_fmaf(v[3], v[3], ss); }
+  ss = wave_sum_f32(ss);
+  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  __syncthreads();
+  const float inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)dim + eps);
+  for (uint32_t e = tid; e < dim / 4; e += 256) {
+    const f4 v = xs[e], wv = ((const f4*)w)[e];
+    const _Float16 o[4] = { (_Float16)((v[0] * inv) * wv[0]), (_Float16)((v[1] * inv) * wv[1]), (_Float16)((v[2] * inv) * wv[2]), (_Float16)((v[3] * inv) * wv[3]) };
+    __builtin_memcpy(out + (size_t)col * out_stride + 4 * e, o, 8);
+  }
+}
+
+hipError_t pa_launch_rmsnorm_f16(const float* x, uint32_t x_stride, const float* w, uint32_t dim, float eps, uint32_t n_cols,
+                                 uint16_t* out, uint32_t out_stride, hipStream_t s) {
+  if (dim == 0 || (dim & 3) || n_cols == 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(pa_rmsnorm_f16_kernel, dim3(n_cols), dim3(256), 0, s, x, x_stride, w, dim, eps, out, out_stride);
+  return hipGetLastError();
+}

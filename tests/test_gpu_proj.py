@@ -116,3 +116,74 @@ def test_attn_layer_decode_matches_oracle(shape, dim, kind, pos):
     for a, b in ((kc, k_row), (vc, v_row)):
         ref = np.asarray(b).reshape(a.shape).view(np.float16).astype(np.float64)
         assert np.abs(a - ref).max() <= np.abs(ref).max() * 2.0 ** -10
+
+
+# ---- column-batched passes: rmsnorm -> f16, GEMM on the matrix cores, the whole attention half of a layer ----
+
+@pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q8_0, PA_W_Q4_0])
+@pytest.mark.parametrize("d_out,d_in,n", [(9216, 2048, 300), (2048, 4096, 129), (37, 96, 5), (130, 8192, 17), (256, 32, 128)])
+def test_gemm_matches_oracle(kind, d_out, d_in, n):
+    if kind == PA_W_F32 and d_in > 4096:
+        pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
+    rng = np.random.default_rng(d_out + 3 * d_in + n + kind)
+    w, sc = _weights(kind, d_out, d_in, rng)
+    x16 = rng.standard_normal((n, d_in)).astype(np.float16)
+    ref = O.gemm_f16(kind, w, sc, x16.astype(np.float32))
+    xs, ys = d_in + 8, d_out + 5                                      # padded strides
+    xpad = np.zeros((n, xs), np.float16); xpad[:, :d_in] = x16
+    y0 = rng.standard_normal((n, ys)).astype(np.float32)
+    with PooledAttn(SHAPES["qwen36_moe"], 64, n_layers=1, max_cols=1) as pa:
+        wh = pa.weight(kind, w, sc)
+        dx = pa.to_device(xpad.view(np.uint16)); dy = pa.to_device(y0)
+        pa.gemm(wh, dx, xs, n, dy, ys); pa.sync()
+        got = dy.download(np.float32, n * ys).reshape(n, ys)
+        assert _rel(got[:, :d_out], ref) < 2e-5, "plain"
+        assert np.array_equal(got[:, d_out:], y0[:, d_out:]), "the stride padding of y must stay untouched"
+        pa.gemm(wh, dx, xs, n, dy, ys, acc=True); pa.sync()
+        assert _rel(dy.download(np.float32, n * ys).reshape(n, ys)[:, :d_out], 2.0 * ref) < 2e-5, "accumulate"
+
+
+def test_rmsnorm_f16_columns():
+    cfg = SHAPES["qwen36_moe"]
+    dim, n = 2048, 37
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal((n, dim)) * rng.uniform(0.1, 10, (n, 1))).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
+    ref = np.stack([O.rmsnorm(x[c], nw, cfg["eps"]) for c in range(n)]).astype(np.float64)
+    with PooledAttn(cfg, 64, n_layers=1, max_cols=1) as pa:
+        dx = pa.to_device(x); dnw = pa.to_device(nw); do = pa.alloc(n * dim * 2)
+        pa.rmsnorm_f16(dx, dim, dnw, dim, n, do, dim); pa.sync()
+        got = do.download(np.uint16, n * dim).view(np.float16).astype(np.float64).reshape(n, dim)
+    assert np.abs(got - ref).max() <= np.abs(ref).max() * 2.0 ** -10          # f16 rounding of an f32 result
+
+
+@pytest.mark.parametrize("shape,dim,kind,base,n", [("qwen36_moe", 512, PA_W_Q4_0, 100, 64), ("qwen36_moe", 1024, PA_W_Q8_0, 0, 33),
+                                                    ("qwen3_1p7b", 512, PA_W_Q4_0, 300, 160), ("qwen38_27b", 1024, PA_W_Q8_0, 77, 40)])
+def test_attn_layer_prefill_matches_oracle(shape, dim, kind, base, n):
+    cfg = SHAPES[shape]
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    qd, kvd = nH * hd, nKV * hd
+    q_rows = qd * (2 if cfg["gate"] else 1)
+    rng = np.random.default_rng(base + dim + n)
+    w_qkv, s_qkv = _weights(kind, q_rows + 2 * kvd, dim, rng, scale=0.05)
+    w_o, s_o = _weights(kind, dim, qd, rng, scale=0.005)              # keeps the residual O(1): the gate below is absolute
+    x = rng.standard_normal((n, dim)).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
+    qw = (1 + 0.1 * rng.standard_normal(hd)).astype(np.float32); kw = (1 + 0.1 * rng.standard_normal(hd)).astype(np.float32)
+    k16, v16 = oracle_cache(cfg, rng.standard_normal((base, kvd)).astype(np.float32), rng.standard_normal((base, kvd)).astype(np.float32), kw)
+    x_ref, k_rows, v_rows = O.attn_layer_prefill(x, kind, w_qkv, s_qkv, kind, w_o, s_o, nw, qw, kw, k16, v16, base, cfg)
+    xs = dim + 4
+    xpad = np.zeros((n, xs), np.float32); xpad[:, :dim] = x
+    with PooledAttn(cfg, base + n + 8, n_layers=1, max_cols=n) as pa:
+        pa.layer_alloc(0)
+        if base:
+            pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
+        wq = pa.weight(kind, w_qkv, s_qkv); wo = pa.weight(kind, w_o, s_o)
+        dx = pa.to_device(xpad); dnw = pa.to_device(nw); dqw = pa.to_device(qw); dkw = pa.to_device(kw)
+        pa.attn_layer_prefill(0, wq, wo, dnw, dqw, dkw, dx, xs, base, n); pa.sync()
+        got = dx.download(np.float32, n * xs).reshape(n, xs)[:, :dim]
+        kc = pa.kv_read(0, 0, base, n).view(np.float16).astype(np.float64); vc = pa.kv_read(0, 1, base, n).view(np.float16).astype(np.float64)
+    assert_parity(got, x_ref, "layer prefill %s base %d n %d" % (shape, base, n))
+    for a, b in ((kc, k_rows), (vc, v_rows)):
+        ref = np.asarray(b).reshape(a.shape).view(np.float16).astype(np.float64)
+        assert np.abs(a - ref).max() <= np.abs(ref).max() * 2.0 ** -9
