@@ -171,6 +171,38 @@ def prefill_leg(steps, with_cpu):
             log("prefill cpu baseline: %.0f ms for %.2f GFLOP -> %.5f TFLOP/s; max |gpu - cpu| = %.2e" % (info["ms"], sub_flops / 1e9, res["cpu_baseline"]["value"], res["cpu_baseline"]["max_abs_diff_vs_gpu"]))
         except Exception as e:
             res["cpu_baseline"] = dict(value=None, unit="TFLOP/s", cores=1, kind="port", sample="failed: %s" % e)
+    # the whole attention half of a layer for the same chunk: rmsnorm + [q|k|v] GEMM + pre-step + attention + wo GEMM
+    try:
+        from pooled_amd.capi import PA_W_Q4_0
+        dim, rows_qkv = 2048, 2 * qd + 2 * kvd
+
+        def mk(d_out, d_in):
+            sc = np.asarray(rng.uniform(0.001, 0.003, (d_out, d_in // 32)), np.float16).view(np.uint16)
+            return pa.weight(PA_W_Q4_0, rng.integers(0, 256, (d_out, d_in // 2), dtype=np.uint8), sc)
+        wq, wo = mk(rows_qkv, dim), mk(dim, qd)
+        d_x = pa.to_device(rng.standard_normal((n, dim), dtype=np.float32))
+        d_nw = pa.to_device((1 + 0.1 * rng.standard_normal(dim)).astype(np.float32))
+        d_x16 = pa.to_device(rng.standard_normal((n, dim)).astype(np.float16).view(np.uint16))
+        d_y = pa.alloc(n * rows_qkv * 4)
+
+        def timed(f, reps):
+            f(); pa.sync()
+            pa.timer_start()
+            for _ in range(reps):
+                f()
+            return pa.timer_stop() / reps
+        t_g1 = timed(lambda: pa.gemm(wq, d_x16, dim, n, d_y, rows_qkv), 10)
+        t_g2 = timed(lambda: pa.gemm(wo, d_out, qd, n, d_x, dim, acc=True), 10)
+        d_x.upload(rng.standard_normal((n, dim), dtype=np.float32))
+        t_layer = timed(lambda: pa.attn_layer_prefill(0, wq, wo, d_nw, d_qw, d_kw, d_x, dim, base, n), max(2, steps // 2))
+        f1, f2 = 2.0 * n * rows_qkv * dim, 2.0 * n * dim * qd
+        log("prefill layer: [q|k|v] GEMM %.3f ms (%.0f TFLOP/s), wo GEMM %.3f ms (%.0f TFLOP/s), whole attention half %.3f ms" % (t_g1, f1 / t_g1 / 1e9, t_g2, f2 / t_g2 / 1e9, t_layer))
+        res["layer_prefill"] = dict(workload="the same chunk through the attention half of a layer (engine/qwen35.js:2416-2425): rmsnorm -> f16, [q|k|v] GEMM "
+                                             "%dx%dx%d, pre-step, causal attention, wo GEMM %dx%dx%d accumulated into the residual; Q4_0 weights, f16 operands" % (n, rows_qkv, dim, n, dim, qd),
+                                    ms_per_step=round(t_layer, 4), tflops=round((flops + f1 + f2) / (t_layer * 1e-3) / 1e12, 1),
+                                    gemm_qkv=dict(ms=round(t_g1, 4), tflops=round(f1 / t_g1 / 1e9, 1)), gemm_o=dict(ms=round(t_g2, 4), tflops=round(f2 / t_g2 / 1e9, 1)))
+    except Exception as e:                       # a reported extra; never let it sink the headline legs
+        log("prefill layer leg failed:", e)
     pa.close()
     return res
 
