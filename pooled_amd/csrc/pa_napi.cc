@@ -247,6 +247,26 @@ static napi_value AttnLayerDecode(napi_env env, napi_callback_info info) {
   int rc = pa_attn_layer_decode(c, layer, wqkv, wo, nw, qw, kw, x, pos); if (rc) return throw_pa(env, c, rc, "pa_attn_layer_decode"); return undefined(env);
 }
 
+// rmsnormF16(ctx, x, xStride, normW, dim, nCols, xnF16, xnStride)
+static napi_value RmsnormF16(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); const float* x = (const float*)a.ptr(1); uint32_t xs = a.u32(2); const float* nw = (const float*)a.ptr(3);
+  uint32_t dim = a.u32(4), n = a.u32(5); void* out = a.ptr(6); uint32_t os = a.u32(7); CHECK_ARGS("rmsnormF16");
+  int rc = pa_rmsnorm_f16(c, x, xs, nw, dim, n, out, os); if (rc) return throw_pa(env, c, rc, "pa_rmsnorm_f16"); return undefined(env);
+}
+// gemm(ctx, weight, xF16, xStride, nCols, y, yStride, acc)
+static napi_value Gemm(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); pa_weight* w = (pa_weight*)a.ptr(1); const void* x = a.ptr(2); uint32_t xs = a.u32(3), n = a.u32(4);
+  float* y = (float*)a.ptr(5); uint32_t ys = a.u32(6); int acc = (int)a.u32(7); CHECK_ARGS("gemm");
+  int rc = pa_gemm(c, w, x, xs, n, y, ys, acc); if (rc) return throw_pa(env, c, rc, "pa_gemm"); return undefined(env);
+}
+// attnLayerPrefill(ctx, layer, wQkv, wO, attnNormW, qNormW, kNormW, x, xStride, basePos, nCols)
+static napi_value AttnLayerPrefill(napi_env env, napi_callback_info info) {
+  ARGS; pa_ctx* c = a.ctx(0); uint32_t layer = a.u32(1); pa_weight* wqkv = (pa_weight*)a.ptr(2); pa_weight* wo = (pa_weight*)a.ptr(3);
+  const float* nw = (const float*)a.ptr(4); const float* qw = (const float*)a.ptr(5); const float* kw = (const float*)a.ptr(6);
+  float* x = (float*)a.ptr(7); uint32_t xs = a.u32(8), base = a.u32(9), n = a.u32(10); CHECK_ARGS("attnLayerPrefill");
+  int rc = pa_attn_layer_prefill(c, layer, wqkv, wo, nw, qw, kw, x, xs, base, n); if (rc) return throw_pa(env, c, rc, "pa_attn_layer_prefill"); return undefined(env);
+}
+
 static napi_value Init(napi_env env, napi_value exports) {
   struct { const char* name; napi_callback fn; } table[] = {
     {"create", Create}, {"destroy", Destroy}, {"lastError", LastError}, {"version", Version}, {"layerAlloc", LayerAlloc}, {"sync", Sync},
@@ -257,6 +277,7 @@ static napi_value Init(napi_env env, napi_value exports) {
     {"copyD2d", CopyD2d}, {"attnGather", AttnGather}, {"slotSave", SlotSave}, {"slotLoad", SlotLoad}, {"slotDrop", SlotDrop}, {"slotPos", SlotPos},
     {"slotCreate", SlotCreate}, {"slotExport", SlotExport}, {"slotImport", SlotImport}, {"weightCreate", WeightCreate},
     {"weightDestroy", WeightDestroy}, {"gemv", Gemv}, {"gemvNorm", GemvNorm}, {"attnLayerDecode", AttnLayerDecode},
+    {"rmsnormF16", RmsnormF16}, {"gemm", Gemm}, {"attnLayerPrefill", AttnLayerPrefill},
   };
   for (auto& t : table) {
     napi_value fn;

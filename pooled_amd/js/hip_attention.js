@@ -260,6 +260,20 @@ class HipAttention {
     addon.attnLayerDecode(this.ctx, i, L.wqkv.handle, L.wo.handle, L.attnNorm, n[0], n[1], this.B.x.ptr, pos);
   }
 
+  // nCols tokens at basePos .. through the attention half of full-attention layer i, as _encodeLayerBatch /
+  // _encodeLayerWide record it (engine/qwen35.js:2416-2425, :2827): B.xCols (residual columns, f32, 256-byte aligned
+  // stride; allocated on first use for batchCols columns) in and out
+  residualCols(dim) {
+    if (!this.B.xCols) { const st = Math.ceil(dim * 4 / 256) * 256; this.B.xCols = { ptr: addon.malloc(this.ctx, this.NC * st), stride: st, n: dim }; }
+    return this.B.xCols;
+  }
+  encodeLayerBatchR(p, i, basePos, nCols) {
+    const L = this.layers[i], n = this._norms(L);
+    if (!L.wqkv) throw new Error("encodeLayerBatchR: layer " + i + " has no projection weights (setLayerProj)");
+    const X = this.residualCols(L.wqkv.dIn);
+    addon.attnLayerPrefill(this.ctx, i, L.wqkv.handle, L.wo.handle, L.attnNorm, n[0], n[1], X.ptr, X.stride / 4, basePos, nCols);
+  }
+
   // ---- sparse-attention layers: the attn step of a QSA pass (engine/qsa.js:8-14, dispatch :41-56) ----
   // sel: device address of the per-column row lists qsa_select wrote (u32 [nCols][selStride]: n, then n rows);
   // maxRows = qsaMaxRows(pos, nCols).  Reads B.q (the context's roped q) and the gate, writes B.attnOut.

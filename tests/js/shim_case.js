@@ -121,6 +121,18 @@ try { A.encodeLayerAttn(null, 0, base + n); console.log("out-of-range position d
   if (!eqBits(new Uint32Array(xLayer.buffer), new Uint32Array(xSteps.buffer))) { console.log("encodeLayerR differs from its stages called one by one FAIL"); fails++; }
   let moved = 0; for (let i = 0; i < dim; i++) moved = Math.max(moved, Math.abs(xLayer[i] - x0[i]));
   if (!(moved > 1e-4)) { console.log("encodeLayerR left the residual unchanged FAIL"); fails++; }
+  // (c) two columns through encodeLayerBatchR: column 0 at pos - 1, column 1 at pos; f16 operands on the GEMMs, so
+  //     it equals the one-token path only to the f16 rounding of activations and weights
+  {
+    const X = A.residualCols(dim);
+    A.writeColumn(X, 0, x0); A.writeColumn(X, 1, x0);
+    A.encodeLayerBatchR(null, 0, pos - 1, 2);
+    A.sync();
+    const c1 = A.readColumn(X, 1);
+    // the one-token reference for column 1: position pos after column 0's row (same x0) was written at pos - 1
+    A.writeColumn(A.B.x, 0, x0); A.encodeLayerR(null, 0, pos - 1); A.writeColumn(A.B.x, 0, x0); A.encodeLayerR(null, 0, pos); A.sync();
+    check("encodeLayerBatchR column vs encodeLayerR", c1, A.readColumn(A.B.x, 0));
+  }
   for (const p of [dQkv, dX, dXn]) addon.free(A.ctx, p);
   console.log("projections (up, fuse, mv, mvN, encodeLayerR) " + (fails ? "see above" : "ok"));
 }
