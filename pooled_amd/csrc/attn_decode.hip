@@ -177,6 +177,25 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   const uint32_t t_end = !SR && sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
   const size_t head_rows = (size_t)p.max_seq + TILE;              // rows of one kv head's plane, padding included
   PA_TP(0);
+  // SR on f16 caches: the whole splits of a kv head are interleaved.  With nw = (whole splits) x W waves, wave v of
+  // them takes rows [(c nw + v) 8, + 8), c = 0 .. 3, instead of 32 consecutive ones: at any moment the loads in
+  // flight on the chip then sweep a compact range of the cache (4 KB pieces, neighbouring waves on neighbouring
+  // pieces) instead of 2048 separate 32 KB streams -- the memory controllers see open pages.  Measured on read-only
+  // stand-ins of this launch shape: 11.9 -> 11.2 us for 64 MiB.  Any partition of the rows is a valid set of
+  // splits; masks go by position.  A trailing partial split and the remainder splits keep consecutive rows.
+  constexpr bool ILV = SR && !GATHER && !Q8;
+  uint32_t ilv_nw = 0, ilv_wv = 0;
+  bool ilv = false;
+  if constexpr (ILV) {
+    const uint32_t nfull = min(p.n_wgs ? p.n_wgs : p.n_splits, seq_max / p.split_len);
+    ilv = sp < nfull;
+    ilv_nw = nfull * W;
+    ilv_wv = sp * W + (threadIdx.x >> 6);
+  }
+  // cache row of row r (0 .. 31) of the tile at tile_pos
+  auto row_pos = [&](uint32_t tile_pos, uint32_t r) __attribute__((always_inline)) -> uint32_t {
+    return ILV && ilv ? (((r >> 3) * ilv_nw + ilv_wv) << 3) + (r & 7) : tile_pos + r;
+  };
 
   unsigned char* stage = stage_all + wave * S::STAGE;
   const size_t row_bytes = (size_t)HD * 2;                         // head-major caches: a kv head's rows are contiguous
@@ -293,7 +312,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     ksr = *(const u4*)(ksbase + (size_t)t0 * S::SPR * 4 + soff);
   } else {
 #pragma unroll
-    for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)t0 * row_bytes + (size_t)(i * S::RPL) * row_bytes + voff);
+    for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)row_pos(t0, i * S::RPL) * row_bytes + voff);
   }
   auto first_v_loads = [&]() __attribute__((always_inline)) {
     if constexpr (GATHER) {
@@ -305,7 +324,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       vsr = *(const u4*)(vsbase + (size_t)t0 * S::SPR * 4 + soff);
     } else {
 #pragma unroll
-      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)t0 * row_bytes + (size_t)(i * S::RPL) * row_bytes + voff);
+      for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)row_pos(t0, i * S::RPL) * row_bytes + voff);
     }
   };
   // The fused pre-step computes between the K and the V loads: a wave sits in the issue of its tile loads for
@@ -530,7 +549,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       for (int pb = 0; pb < 2; pb++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          const uint32_t pos = tp + pb * 16 + 4 * kg + i;
+          const uint32_t pos = row_pos(tp, pb * 16 + 4 * kg + i);
           const float x = pos < row_end ? s[pb][0][i] * p.scale : NEG_INF;
           v[pb * 4 + i] = x;
           mx = fmaxf(mx, x);
@@ -544,7 +563,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
       ps += __shfl_xor(ps, 16, 64);
       ps += __shfl_xor(ps, 32, 64);
-      stage_v(tp, false, 0);
+      stage_v(ILV && ilv ? 0u : tp, false, 0);                          // interleaved splits are whole: no row past the end to zero
       *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pf;
       if (kg == 0) { mex[wave * 16 + ln] = mx; lex[wave * 16 + ln] = ps; }
       PA_TP(5);
