@@ -300,7 +300,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (configuration 5) leg")
     ap.add_argument("--unfused", action="store_true", help="decode step as three launches (pa_glue_kv + pa_attn_decode) instead of the fused pa_attn_decode_step")
     ap.add_argument("--prefill-steps", type=int, default=5)
-    ap.add_argument("--kv-q8", action="store_true", help="run the C3 decode step on int8 caches (one f32 scale per 32 values) instead of f16; implies --unfused")
+    ap.add_argument("--kv-q8", action="store_true", help="run the C3 decode step on int8 caches (one f32 scale per 32 values) instead of f16")
     ap.add_argument("--no-layer", action="store_true", help="skip the whole-layer leg (projections + attention, pa_attn_layer_decode)")
     ap.add_argument("--other-configs", action="store_true", help="only time configurations 1, 2 and 4 (attention call alone, caches in rotation)")
     ap.add_argument("--mfma-probe", action="store_true",
@@ -345,7 +345,7 @@ def main():
         return
     cfg, ctx = C3, C3_CTX
     if args.kv_q8:
-        cfg = dict(C3, kv_q8=True); args.unfused = True; args.no_cpu = True
+        cfg = dict(C3, kv_q8=True); args.no_cpu = True
     nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
     qd, kvd = nH * hd, nKV * hd
     pa = PooledAttn(cfg, ctx + 1, n_layers=N_LAYERS, max_cols=4096)

@@ -33,7 +33,8 @@ extern "C" {
 #define PA_FLAG_KV_Q8 4u      /* int8 caches: values rounded to int8 with one f32 scale per 32 (scale = max|x| / 127),
                                  the reference's kvQ8 mode (kv_store_q8, attn_flash_q8: engine/wgsl/qwen35.js:908-946,
                                  :99-139).  Served by pa_glue_kv / pa_kv_store / pa_attn_decode / pa_attn_prefill /
-                                 slots; pa_attn_decode_step and pa_attn_decode_gather return PA_ERR_UNSUPPORTED. */
+                                 pa_attn_decode_step / slots and the layer calls; pa_attn_decode_gather returns
+                                 PA_ERR_UNSUPPORTED. */
 
 /* output element types */
 #define PA_OUT_F32 0          /* the engine's attnOut feeding wo (engine/qwen35.js:881) */
@@ -236,7 +237,7 @@ int pa_gemv_norm(pa_ctx* ctx, const pa_weight* w, const float* d_x_raw, const fl
  * attention -> merge + gate -> output projection accumulated into the residual.  w_qkv: rows [q (n_heads x head_dim,
  * x 2 with PA_FLAG_GATE: q | gate interleaved per head) | k | v] x dim, one fused weight (the reference fuses k | v,
  * engine/qwen35.js:1109-1114); w_o: dim x (n_heads x head_dim).  d_x [dim] is read and updated in place.  Four
- * launches: normed GEMV, fused decode step (2), accumulating GEMV.  f16 caches only. */
+ * launches: normed GEMV, fused decode step (2), accumulating GEMV.  f16 or int8 caches. */
 int pa_attn_layer_decode(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
                          const float* d_qw, const float* d_kw, float* d_x, uint32_t pos);
 
@@ -254,7 +255,8 @@ int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uint32_t x_str
  * _encodeLayerBatch / _encodeLayerWide record it (engine/qwen35.js:2416-2425, :2827): rmsnorm -> [q | k | v] GEMM ->
  * pre-step + cache write -> causal attention -> gate -> wo GEMM accumulated into the residual columns d_x
  * [n_cols][x_stride] (f32, read and updated in place).  Weights as pa_attn_layer_decode.  Five launches (six when
- * the attention pass is split).  f16 caches only; n_cols <= max_cols. */
+ * the attention pass is split).  n_cols <= max_cols.  On int8 caches the attention pass is the split-K kernel in
+ * column groups (as pa_attn_prefill on such caches). */
 int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
                           const float* d_qw, const float* d_kw, float* d_x, uint32_t x_stride, uint32_t base_pos, uint32_t n_cols);
 

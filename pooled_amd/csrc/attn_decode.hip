@@ -138,7 +138,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   static_assert(!SR || NB == 1, "single-round splits: one 16-row block");
   static_assert(!FUSED || NB == 1, "the fused pre-step serves one column");
   static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
-  static_assert(!Q8 || (!FUSED && !GATHER), "int8 caches: plain decode / verify only");
+  static_assert(!Q8 || !GATHER, "int8 caches: no gather mode");
   typedef DecShape<HD> S;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       vx = *(const h4*)(vbase + ro);
     }
   }
-  if constexpr (Q8) {                   // int8 row: widened as the tile path widens it (exact integer x f16-rounded scale, one rounding)
+  if constexpr (Q8 && !FUSED) {         // int8 row: widened as the tile path widens it (exact integer x f16-rounded scale, one rounding)
     if (self_wave) {
       const uint32_t l4 = min(lane, (uint32_t)HD / 4 - 1);
       const size_t ro = (size_t)p.base_pos * HD + 4 * l4, so = ((size_t)p.base_pos * S::SPR + l4 / 8) * 4;
@@ -347,7 +347,31 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       *(h4*)(q_lds + (G + e / (HD / 4)) * S::QROW + (e % (HD / 4)) * 8) = (h4){0, 0, 0, 0};
     if (self_wave) {                 // the new key row: normed, roped, rounded; it and the value row go to the cache
       glue_head_wave(xk, wk, p.f_kw != nullptr, p.eps, HD, half, cs, xs, lane);
-      if (lane < HD / 4) {
+      if constexpr (Q8) {
+        // int8 caches: both rows quantised as the stand-alone pre-step does (same bits), written with their scales,
+        // and kept as the widened values the tile path would read back
+        const bool on = lane < HD / 4;
+        float kq[4] = {0.f, 0.f, 0.f, 0.f}, vq[4] = {0.f, 0.f, 0.f, 0.f};
+        if (on) { const f4 v = *(const f4*)(xs + 4 * lane); kq[0] = v[0]; kq[1] = v[1]; kq[2] = v[2]; kq[3] = v[3]; vq[0] = xv4[0]; vq[1] = xv4[1]; vq[2] = xv4[2]; vq[3] = xv4[3]; }
+        uint32_t kw8, vw8; float ksc, vsc;
+        quant4_q8(kq, kw8, ksc);
+        quant4_q8(vq, vw8, vsc);
+        if (on) {
+          const size_t row = (size_t)g * head_rows + p.base_pos;
+          *(uint32_t*)((unsigned char*)const_cast<uint16_t*>(p.k_cache) + row * HD + 4 * lane) = kw8;
+          *(uint32_t*)((unsigned char*)const_cast<uint16_t*>(p.v_cache) + row * HD + 4 * lane) = vw8;
+          if ((lane & 7) == 0) {
+            const_cast<float*>(p.k_scale)[row * S::SPR + (lane >> 3)] = ksc;
+            const_cast<float*>(p.v_scale)[row * S::SPR + (lane >> 3)] = vsc;
+          }
+        }
+        const _Float16 ks16 = (_Float16)ksc, vs16 = (_Float16)vsc;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          kx[i] = (_Float16)(int)(signed char)(kw8 >> (8 * i)) * ks16;
+          vx[i] = (_Float16)(int)(signed char)(vw8 >> (8 * i)) * vs16;
+        }
+      } else if (lane < HD / 4) {
         const f4 v = *(const f4*)(xs + 4 * lane);
         kx = (h4){ (_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3] };
         vx = (h4){ (_Float16)xv4[0], (_Float16)xv4[1], (_Float16)xv4[2], (_Float16)xv4[3] };
@@ -976,6 +1000,11 @@ hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint3
 
 hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t) {
   if (!p.f_q_in || p.n_cols != 1 || p.group > 16 || !p.self_row) return hipErrorInvalidValue;
+  if (p.k_scale) {                                // int8 caches
+    if (hd == 256) return launch_decode_t<256, 1, 4, true, false, true>(p, 1, s, t);
+    if (hd == 128) return launch_decode_t<128, 1, 4, true, false, true>(p, 1, s, t);
+    return hipErrorInvalidValue;
+  }
   if (hd == 256) return launch_decode_t<256, 1, 4, true>(p, 1, s, t);
   if (hd == 128) return launch_decode_t<128, 1, 4, true>(p, 1, s, t);
   return hipErrorInvalidValue;

@@ -13,24 +13,14 @@
 #define GLUE_DO_MATH 0x100u
 
 // int8 cache row (the reference's kv_store_q8, engine/wgsl/qwen35.js:908-946): per block of 32 values
-// scale = max|x| / 127, inv = 1 / scale (0 for an all-zero block), value = clamp(round-half-even(x * inv), -127, 127),
-// every operation a separately rounded f32 one.  One wavefront, 4 consecutive values a lane (8 lanes = one block);
+// the arithmetic is quant4_q8 (glue_math.h).  One wavefront, 4 consecutive values a lane (8 lanes = one block);
 // src holds the row's hd f32 values (LDS or global), dst the row's hd int8, sc_dst its hd / 32 scales.
 static __device__ inline void store_row_q8(const float* src, uint32_t hd, uint32_t lane, unsigned char* dst, float* sc_dst) {
-#pragma clang fp contract(off)
   const bool on = 4 * lane < hd;
   float x[4] = {0.f, 0.f, 0.f, 0.f};
   if (on) { x[0] = src[4 * lane]; x[1] = src[4 * lane + 1]; x[2] = src[4 * lane + 2]; x[3] = src[4 * lane + 3]; }
-  float a = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
-  a = fmaxf(a, __shfl_xor(a, 1, 64)); a = fmaxf(a, __shfl_xor(a, 2, 64)); a = fmaxf(a, __shfl_xor(a, 4, 64));
-  const float sc = a / 127.0f;
-  const float inv = sc > 0.f ? 1.0f / sc : 0.f;
-  uint32_t w = 0;
-#pragma unroll
-  for (int b = 0; b < 4; b++) {
-    const float r = fminf(fmaxf(__builtin_rintf(x[b] * inv), -127.0f), 127.0f);
-    w |= ((uint32_t)(int)r & 255u) << (8 * b);
-  }
+  uint32_t w; float sc;
+  quant4_q8(x, w, sc);
   if (on) {
     *(uint32_t*)(dst + 4 * lane) = w;
     if ((lane & 7) == 0) sc_dst[lane >> 3] = sc;

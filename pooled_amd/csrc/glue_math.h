@@ -142,3 +142,21 @@ static __device__ inline void glue_head_wave(const float (&x_in)[4], const float
   const float x1[1][4] = { { x_in[0], x_in[1], x_in[2], x_in[3] } };
   glue_heads_wave<1>(x1, w, norm, eps, hd, half, cs, xs, 0, lane);
 }
+
+// int8 cache row, the lane's 4 consecutive values of a 32-value block (8 lanes = one block; the reference's
+// kv_store_q8, engine/wgsl/qwen35.js:908-946): scale = max|x| / 127 over the block, inv = 1 / scale (0 for an all-zero
+// block), value = clamp(round-half-even(x * inv), -127, 127), every operation a separately rounded f32 one.  Returns
+// the 4 values packed low byte first and the block's scale (the same in its 8 lanes).  All 64 lanes must call.
+static __device__ inline void quant4_q8(const float (&x)[4], uint32_t& w, float& sc) {
+#pragma clang fp contract(off)
+  float a = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+  a = fmaxf(a, __shfl_xor(a, 1, 64)); a = fmaxf(a, __shfl_xor(a, 2, 64)); a = fmaxf(a, __shfl_xor(a, 4, 64));
+  sc = a / 127.0f;
+  const float inv = sc > 0.f ? 1.0f / sc : 0.f;
+  w = 0;
+#pragma unroll
+  for (int b = 0; b < 4; b++) {
+    const float r = fminf(fmaxf(__builtin_rintf(x[b] * inv), -127.0f), 127.0f);
+    w |= ((uint32_t)(int)r & 255u) << (8 * b);
+  }
+}

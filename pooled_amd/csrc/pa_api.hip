@@ -454,7 +454,6 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
   if (rc) return rc;
   const pa_config& c = ctx->cfg;
   const bool gated = (c.flags & PA_FLAG_GATE) != 0, norm = (c.flags & PA_FLAG_QK_NORM) != 0;
-  if (kv_q8(ctx)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": int8 caches take pa_glue_kv + pa_attn_decode");
   if (!d_q_in || !d_k || !d_v || !d_out) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null buffer");
   if (norm && (!d_qw || !d_kw)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": norm weights required");
   if (out_dtype != PA_OUT_F32 && out_dtype != PA_OUT_F16) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": bad out_dtype");
@@ -470,6 +469,7 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
   if ((rc = ensure_partials(ctx, 1, pl.slots))) return rc;
   AttnParams p; memset(&p, 0, sizeof p);
   p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+  p.k_scale = ctx->layers[layer].ks; p.v_scale = ctx->layers[layer].vs;
   p.part_o = ctx->part_o; p.part_ml = ctx->part_ml; p.out = d_out;
   p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
   p.base_pos = pos; p.n_cols = 1;
@@ -608,7 +608,6 @@ extern "C" int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weigh
   if (!ctx) return PA_ERR_INVALID;
   const pa_config& c = ctx->cfg;
   if (!w_qkv || !w_o || !d_attn_norm_w || !d_x) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null argument");
-  if (kv_q8(ctx)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": f16 caches only");
   int rc = check_cols(ctx, who, layer, true, base_pos, n_cols);
   if (rc) return rc;
   const uint32_t qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim, dim = w_qkv->d_in;

@@ -68,8 +68,7 @@ class HipAttention {
     this.flash = true; this.attnDecode = "v2"; this.attnPrefillTile = true;
     this._snapNow = null;                                          // set by a verify pass (engine/qwen35.js:2960-2965)
     this.pos = 0;
-    this.kvQ8 = !!opts.kvQ8;                                       // int8 caches (engine option kvQ8): three launches per token
-    if (this.kvQ8) this.fusedStep = false;
+    this.kvQ8 = !!opts.kvQ8;                                       // int8 caches (engine option kvQ8)
     const flags = (this.qkNorm ? PA_FLAG_QK_NORM : 0) | (this.gate ? PA_FLAG_GATE : 0) | (this.kvQ8 ? PA_FLAG_KV_Q8 : 0);
     // a readable throw at create, like the engine's KV binding check (engine/qwen35.js:378-383)
     this.ctx = addon.create({ nH: nH, nKV: nKV, hd: hd, nRot: this.dims.nRot, ropeTheta: opts.ropeTheta, eps: opts.eps,

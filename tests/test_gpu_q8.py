@@ -93,11 +93,41 @@ def test_q8_verify_block_prefill_chunk_and_slots():
         for w, a in enumerate((kq, vq, ks, vs)):
             assert np.array_equal(pa.kv_read(0, w, 0, base + n), a)
             assert np.array_equal(pa.slot_export(1, 0, w).reshape(a.shape), a)
-        # the fused one-token call and the gather mode are f16-cache paths
-        d = O.make_inputs(cfg, 0, 1, 1)
-        with pytest.raises(PaError) as e:
-            pa.run_decode_step(0, d["qraw"][0], d["kraw"][0], d["vraw"][0], d["qw"], d["kw"], 5)
-        assert e.value.code == PA_ERR_UNSUPPORTED
+        # the gather mode is an f16-cache path
         with pytest.raises(PaError) as e:
             pa.run_attn_gather(0, q[:1], [np.arange(10)])
         assert e.value.code == PA_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("shape,pos", [("qwen36_moe", 0), ("qwen36_moe", 1), ("qwen36_moe", 777), ("qwen36_moe", 4096), ("qwen3_1p7b", 300), ("qwen38_27b", 129)])
+def test_q8_fused_decode_step(shape, pos):
+    """pa_attn_decode_step on int8 caches: the row it writes (values and scales) and its output equal pa_glue_kv +
+    pa_attn_decode bit for bit, neighbouring rows stay untouched, and the output matches the oracle over the
+    dequantised cache."""
+    cfg = _q8cfg(shape)
+    nKV, hd = cfg["n_kv_heads"], cfg["head_dim"]
+    d = O.make_inputs(cfg, pos, 1, seed=pos + 3)
+    kq, ks, vq, vs, kf, vf = _quantised_cache(cfg, pos + 2, seed=pos + 4)
+    with PooledAttn(cfg, pos + 2, n_layers=1, max_cols=1) as pa:
+        pa.layer_alloc(0)
+        for w, a in enumerate((kq, vq, ks, vs)):
+            pa.kv_write(0, w, 0, a)
+        pa.run_glue_kv(0, d["qraw"], d["kraw"][pos:], d["vraw"][pos:], d["qw"], d["kw"], pos)
+        rows = [pa.kv_read(0, w, pos, 1).copy() for w in range(4)]
+        dout = pa.alloc(pa.q_dim * 4)
+        pa.attn("decode", 0, None, 0, pa.gate_buffer_ptr() if cfg["gate"] else None, pa.q_dim, pos, 1, dout, pa.q_dim); pa.sync()
+        unfused = dout.download(np.float32, pa.q_dim)
+        for w, a in enumerate((kq, vq, ks, vs)):                         # the cache as it was, row pos included
+            pa.kv_write(0, w, 0, a)
+        fused = pa.run_decode_step(0, d["qraw"][0], d["kraw"][pos], d["vraw"][pos], d["qw"], d["kw"], pos)
+        for w in range(4):
+            assert np.array_equal(pa.kv_read(0, w, pos, 1), rows[w]), "tensor %d of the written row" % w
+            assert np.array_equal(pa.kv_read(0, w, pos + 1, 1), (kq, vq, ks, vs)[w][pos + 1:pos + 2]), "row after the written one"
+            if pos:
+                assert np.array_equal(pa.kv_read(0, w, pos - 1, 1), (kq, vq, ks, vs)[w][pos - 1:pos]), "row before the written one"
+    assert np.array_equal(fused.reshape(-1).view(np.uint32), unfused.view(np.uint32))
+    # oracle: attention over the dequantised rows, the new row dequantised from what the pre-step wrote
+    g = O.glue_kv(d["qraw"], d["kraw"][pos:], d["vraw"][pos:], d["qw"], d["kw"], pos, cfg)
+    knew = O.q8_dequantize(rows[0].reshape(1, nKV, hd), rows[2].reshape(1, nKV, hd // 32)); vnew = O.q8_dequantize(rows[1].reshape(1, nKV, hd), rows[3].reshape(1, nKV, hd // 32))
+    ref = O.attention_values(g["q"], np.concatenate([kf[:pos], knew]), np.concatenate([vf[:pos], vnew]), pos, gate=g["gate"] if cfg["gate"] else None)
+    assert_parity(fused.reshape(ref.shape), ref, "q8 fused step %s pos %d" % (shape, pos))
