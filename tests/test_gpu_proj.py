@@ -187,3 +187,58 @@ def test_attn_layer_prefill_matches_oracle(shape, dim, kind, base, n):
     for a, b in ((kc, k_rows), (vc, v_rows)):
         ref = np.asarray(b).reshape(a.shape).view(np.float16).astype(np.float64)
         assert np.abs(a - ref).max() <= np.abs(ref).max() * 2.0 ** -9
+
+
+def test_layer_calls_on_int8_caches_equal_their_stages():
+    """pa_attn_layer_decode / pa_attn_layer_prefill on int8 caches: the same bits as their stages called one by one
+    (each stage has its own parity test)."""
+    from pooled_amd.capi import PA_OUT_F16
+    cfg = dict(SHAPES["qwen36_moe"], kv_q8=True)
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    qd, kvd, dim = nH * hd, nKV * hd, 512
+    q_rows = 2 * qd
+    rng = np.random.default_rng(21)
+    w_qkv, s_qkv = _weights(PA_W_Q4_0, q_rows + 2 * kvd, dim, rng, scale=0.05)
+    w_o, s_o = _weights(PA_W_Q4_0, dim, qd, rng, scale=0.005)
+    nw = (1 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
+    hw = (1 + 0.1 * rng.standard_normal(hd)).astype(np.float32)
+    base, n = 200, 24
+    xs = rng.standard_normal((base + n + 1, dim)).astype(np.float32)
+    with PooledAttn(cfg, base + n + 1, n_layers=2, max_cols=base) as pa:
+        pa.layer_alloc(0); pa.layer_alloc(1)
+        wq = pa.weight(PA_W_Q4_0, w_qkv, s_qkv); wo = pa.weight(PA_W_Q4_0, w_o, s_o)
+        dnw = pa.to_device(nw); dhw = pa.to_device(hw)
+        rows = q_rows + 2 * kvd
+        for layer, staged in ((0, False), (1, True)):
+            # a chunk of `base` tokens, then a chunk of n, then one token
+            outs = []
+            for b0, cnt in ((0, base), (base, n)):
+                dx = pa.to_device(xs[b0:b0 + cnt])
+                if not staged:
+                    pa.attn_layer_prefill(layer, wq, wo, dnw, dhw, dhw, dx, dim, b0, cnt)
+                else:
+                    dxn = pa.alloc(cnt * dim * 2); dqkv = pa.alloc(cnt * rows * 4); dat = pa.alloc(cnt * qd * 2)
+                    pa.rmsnorm_f16(dx, dim, dnw, dim, cnt, dxn, dim)
+                    pa.gemm(wq, dxn, dim, cnt, dqkv, rows)
+                    pa.L.pa_glue_kv(pa.ctx, layer, dqkv.ptr, rows, dqkv.ptr + q_rows * 4, rows, dqkv.ptr + (q_rows + kvd) * 4, rows, dhw.ptr, dhw.ptr, b0, cnt)
+                    pa.attn("prefill", layer, None, 0, pa.gate_buffer_ptr(), qd, b0, cnt, dat, qd, PA_OUT_F16)
+                    pa.gemm(wo, dat, qd, cnt, dx, dim, acc=True)
+                pa.sync()
+                outs.append(dx.download(np.float32, cnt * dim))
+            dx = pa.to_device(xs[base + n])
+            if not staged:
+                pa.attn_layer_decode(layer, wq, wo, dnw, dhw, dhw, dx, base + n)
+            else:
+                dqkv = pa.alloc(rows * 4); dat = pa.alloc(qd * 4)
+                pa.gemv_norm(wq, dx, dnw, dqkv)
+                pa.L.pa_attn_decode_step(pa.ctx, layer, dqkv.ptr, dqkv.ptr + q_rows * 4, dqkv.ptr + (q_rows + kvd) * 4, dhw.ptr, dhw.ptr, base + n, dat.ptr, 0)
+                pa.gemv(wo, dat, dx, acc=True)
+            pa.sync()
+            outs.append(dx.download(np.float32, dim))
+            if not staged:
+                first = outs
+        for a, b in zip(first, outs):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+            assert np.all(np.isfinite(a))
+        for w in range(4):
+            assert np.array_equal(pa.kv_read(0, w, 0, base + n + 1), pa.kv_read(1, w, 0, base + n + 1))
