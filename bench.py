@@ -104,12 +104,12 @@ def causal_flops(cfg, base, n):
     return 4.0 * cfg["n_heads"] * cfg["head_dim"] * (n * base + n * (n + 1) // 2)
 
 
-def prefill_leg(steps, with_cpu):
+def prefill_leg(steps, with_cpu, kv_q8=False):
     """Configuration 5: a 4096-token causal chunk at positions 126976-131071 over a 126976-token f16 prefix,
     Qwen3.6-35B-MoE attention shape, sigmoid gate, f16 output.  A step = pre-step for the 4096 columns
     (QK-RMSNorm + partial RoPE + KV write) + the MFMA prefill kernel."""
     from pooled_amd.capi import PooledAttn, PA_OUT_F16
-    cfg, base, n = C5, C5_BASE, C5_COLS
+    cfg, base, n = dict(C5, kv_q8=True) if kv_q8 else C5, C5_BASE, C5_COLS
     nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
     qd, kvd = nH * hd, nKV * hd
     pa = PooledAttn(cfg, base + n, n_layers=1, max_cols=n)
@@ -138,7 +138,8 @@ def prefill_leg(steps, with_cpu):
     flops = causal_flops(cfg, base, n)
     tf_step, tf_kernel = flops / (ms_step * 1e-3) / 1e12, flops / (k_ms * 1e-3) / 1e12
     log("prefill C5: %.3f ms/step -> %.1f TFLOP/s; kernel %.3f ms -> %.1f TFLOP/s (%.1f%% of f16 MFMA peak)" % (ms_step, tf_step, k_ms, tf_kernel, 100 * tf_kernel / MFMA_F16_PEAK_TFLOPS))
-    res = dict(workload="C5 causal chunked prefill: 4096 columns at positions 126976-131071 over a 126976-token f16 prefix, 16q/2kv heads, head_dim 256, partial RoPE, sigmoid gate, f16 out",
+    res = dict(workload="C5 causal chunked prefill: 4096 columns at positions 126976-131071 over a 126976-token %s prefix, 16q/2kv heads, head_dim 256, partial RoPE, sigmoid gate, f16 out"
+                        % ("int8 (widened once per chunk into an f16 staging cache, inside the step)" if kv_q8 else "f16"),
                value=round(tf_step, 1), unit="TFLOP/s", ms_per_step=round(ms_step, 4), steps=steps, flops_per_step=flops, plan=pa.plan("prefill", base, n),
                roofline=dict(bound="mfma", achieved=round(tf_kernel, 1), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s", frac=round(tf_kernel / MFMA_F16_PEAK_TFLOPS, 4),
                              traffic=None, kernel="pa_prefill_kernel<256, 1, 8, false>", kernel_ms=round(k_ms, 4), algorithmic_flops_per_launch=flops, launches=kcount))
@@ -437,7 +438,7 @@ def main():
         line["layer_decode"] = layer_leg(pa, cfg, ctx, args.steps, args.warmup, ms_per_step)
     pa.close()
     if not args.no_prefill:
-        line["prefill"] = prefill_leg(args.prefill_steps, not args.no_cpu)
+        line["prefill"] = prefill_leg(args.prefill_steps, not args.no_cpu, args.kv_q8)
     print(json.dumps(line), flush=True)
 
 

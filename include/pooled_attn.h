@@ -34,7 +34,10 @@ extern "C" {
                                  the reference's kvQ8 mode (kv_store_q8, attn_flash_q8: engine/wgsl/qwen35.js:908-946,
                                  :99-139).  Served by pa_glue_kv / pa_kv_store / pa_attn_decode / pa_attn_prefill /
                                  pa_attn_decode_step / slots and the layer calls; pa_attn_decode_gather returns
-                                 PA_ERR_UNSUPPORTED. */
+                                 PA_ERR_UNSUPPORTED (as the reference: attnDecConfig, engine/wgsl/attn_dec.js:40-41).  A wide
+                                 pa_attn_prefill chunk widens the rows it can see into an f16 staging cache the
+                                 context allocates on first use (one layer's f16 cache in size) and runs the
+                                 matrix-core prefill kernel on it. */
 
 /* output element types */
 #define PA_OUT_F32 0          /* the engine's attnOut feeding wo (engine/qwen35.js:881) */
@@ -255,8 +258,8 @@ int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uint32_t x_str
  * _encodeLayerBatch / _encodeLayerWide record it (engine/qwen35.js:2416-2425, :2827): rmsnorm -> [q | k | v] GEMM ->
  * pre-step + cache write -> causal attention -> gate -> wo GEMM accumulated into the residual columns d_x
  * [n_cols][x_stride] (f32, read and updated in place).  Weights as pa_attn_layer_decode.  Five launches (six when
- * the attention pass is split).  n_cols <= max_cols.  On int8 caches the attention pass is the split-K kernel in
- * column groups (as pa_attn_prefill on such caches). */
+ * the attention pass is split).  n_cols <= max_cols.  On int8 caches one more launch widens the visible rows for the
+ * prefill kernel (as pa_attn_prefill on such caches). */
 int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
                           const float* d_qw, const float* d_kw, float* d_x, uint32_t x_stride, uint32_t base_pos, uint32_t n_cols);
 

@@ -110,3 +110,41 @@ hipError_t pa_launch_glue(const GlueParams& p, hipStream_t s) {
   hipLaunchKernelGGL(pa_glue_kernel, dim3(heads, p.n_cols), dim3(64), 0, s, p);
   return hipGetLastError();
 }
+
+// int8 caches -> an f16 staging cache of the same head-major geometry, rows [0, n_rows) of every kv head; rows from
+// n_live up to n_rows are written as zeros (their scales need not be numbers).  A value is widened as the split-K
+// kernel widens it: exact integer times the f16-rounded scale, rounded once.  One thread = 16 values.
+__global__ __launch_bounds__(256) void pa_widen_q8_kernel(const unsigned char* k8, const unsigned char* v8, const float* ks, const float* vs,
+                                                          uint16_t* ko, uint16_t* vo, uint32_t hd, uint32_t head_rows, uint32_t n_live,
+                                                          uint32_t n_rows) {
+  typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+  const uint32_t ppr = hd / 16;                                       // pieces per row
+  const uint32_t idx = blockIdx.x * 256 + threadIdx.x, row = idx / ppr, pc = idx % ppr, h = blockIdx.y;
+  if (row >= n_rows) return;
+  const bool isV = blockIdx.z != 0;
+  const size_t r = (size_t)h * head_rows + row;
+  uint16_t* dst = (isV ? vo : ko) + r * hd + pc * 16;
+  h8 lo = {0, 0, 0, 0, 0, 0, 0, 0}, hi = lo;
+  if (row < n_live) {
+    const uint4 q = *(const uint4*)((isV ? v8 : k8) + r * hd + pc * 16);
+    const _Float16 sc = (_Float16)(isV ? vs : ks)[r * (hd / 32) + pc / 2];
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      lo[i] = (_Float16)(int)(signed char)(w[i / 4] >> (8 * (i & 3))) * sc;
+      hi[i] = (_Float16)(int)(signed char)(w[2 + i / 4] >> (8 * (i & 3))) * sc;
+    }
+  }
+  *(h8*)dst = lo;
+  *(h8*)(dst + 8) = hi;
+}
+
+hipError_t pa_launch_widen_q8(const void* k8, const void* v8, const float* ks, const float* vs, uint16_t* ko, uint16_t* vo,
+                              uint32_t n_kv_heads, uint32_t hd, uint32_t head_rows, uint32_t n_live, uint32_t n_rows, hipStream_t s) {
+  if (n_rows == 0) return hipSuccess;
+  if (hd % 32 || n_rows > head_rows || n_live > n_rows) return hipErrorInvalidValue;
+  const uint32_t threads = n_rows * (hd / 16);
+  hipLaunchKernelGGL(pa_widen_q8_kernel, dim3((threads + 255) / 256, n_kv_heads, 2), dim3(256), 0, s, (const unsigned char*)k8,
+                     (const unsigned char*)v8, ks, vs, ko, vo, hd, head_rows, n_live, n_rows);
+  return hipGetLastError();
+}

@@ -114,6 +114,8 @@ extern "C" int pa_destroy(pa_ctx* ctx) {
   if (ctx->part_ml) (void)hipFree(ctx->part_ml);
   if (ctx->proj_buf) (void)hipFree(ctx->proj_buf);
   if (ctx->chunk_buf) (void)hipFree(ctx->chunk_buf);
+  if (ctx->wide_k) (void)hipFree(ctx->wide_k);
+  if (ctx->wide_v) (void)hipFree(ctx->wide_v);
   for (auto ev : ctx->prof_events) (void)hipEventDestroy(ev);
   if (ctx->t0) (void)hipEventDestroy(ctx->t0);
   if (ctx->t1) (void)hipEventDestroy(ctx->t1);
@@ -344,7 +346,7 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
 
 extern "C" int pa_plan_query(const pa_ctx* ctx, int kind, uint32_t base_pos, uint32_t n_cols, pa_plan* out) {
   if (!ctx || !out || n_cols == 0) return PA_ERR_INVALID;
-  return (kind == 0 || kv_q8(ctx)) ? plan_decode(ctx, base_pos, n_cols, out) : plan_prefill(ctx, base_pos, n_cols, out);
+  return kind == 0 ? plan_decode(ctx, base_pos, n_cols, out) : plan_prefill(ctx, base_pos, n_cols, out);
 }
 extern "C" int pa_set_decode_splits(pa_ctx* ctx, uint32_t splits) {
   if (!ctx) return PA_ERR_INVALID;
@@ -405,10 +407,8 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   if ((q_stride & 3) || (out_stride & 3) || (d_gate && (gate_stride & 3)) || ((uintptr_t)d_q & 15) || ((uintptr_t)d_out & 15) || ((uintptr_t)d_gate & 15))
     return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned with strides a multiple of 4 elements");
   pa_plan pl;
-  // int8 caches are served by the split-K kernel only (the reference has no tiled prefill for them either): a
-  // prefill chunk then runs as column groups of that kernel
   uint32_t n_wgs = 0;
-  rc = (kind == 0 || kv_q8(ctx)) ? plan_decode(ctx, base_pos, n_cols, &pl, true, &n_wgs) : plan_prefill(ctx, base_pos, n_cols, &pl, &n_wgs);
+  rc = kind == 0 ? plan_decode(ctx, base_pos, n_cols, &pl, true, &n_wgs) : plan_prefill(ctx, base_pos, n_cols, &pl, &n_wgs);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
   const bool direct = pl.kernel == 1 && pl.n_splits == 1;     // the prefill kernel writes the output itself
@@ -420,6 +420,25 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
   p.base_pos = base_pos; p.n_cols = n_cols;
   p.k_scale = ctx->layers[layer].ks; p.v_scale = ctx->layers[layer].vs;
+  if (pl.kernel == 1 && kv_q8(ctx)) {
+    // int8 caches under the MFMA prefill kernel (the reference has no tiled prefill for them): the rows the chunk can
+    // see are widened once into a context-owned f16 staging cache of one layer's size -- a few percent of the
+    // chunk's attention time -- and the f16 kernel runs on that.  Rows past the chunk's last position up to the
+    // next multiple of 32 are staged as zeros.
+    const size_t wide_elems = ((size_t)c.max_seq + 32) * c.n_kv_heads * c.head_dim;
+    for (uint16_t** w : {&ctx->wide_k, &ctx->wide_v}) {
+      if (*w) continue;
+      uint16_t* mem = nullptr;                       // the padding rows from max_seq on stay zero for good
+      HIPCHK(ctx, hipMalloc((void**)&mem, wide_elems * sizeof(uint16_t)));
+      hipError_t e = hipMemsetAsync(mem, 0, wide_elems * sizeof(uint16_t), ctx->stream);
+      if (e != hipSuccess) { (void)hipFree(mem); HIPCHK(ctx, e); }
+      *w = mem;
+    }
+    const uint32_t live = base_pos + n_cols, staged = std::min(ceil_div(live, 32) * 32, c.max_seq + 32);
+    HIPCHK(ctx, pa_launch_widen_q8(ctx->layers[layer].k, ctx->layers[layer].v, ctx->layers[layer].ks, ctx->layers[layer].vs, ctx->wide_k,
+                                   ctx->wide_v, c.n_kv_heads, c.head_dim, c.max_seq + 32, live, staged, ctx->stream));
+    p.k_cache = ctx->wide_k; p.v_cache = ctx->wide_v; p.k_scale = nullptr; p.v_scale = nullptr;
+  }
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
   p.self_row = plan_self_row(pl) ? 1 : 0;
   p.n_wgs = pl.kernel == 0 ? n_wgs : 0;

@@ -109,6 +109,10 @@ hipError_t pa_launch_gemm(const GemmParams& p, hipStream_t s);
 hipError_t pa_launch_rmsnorm_f16(const float* x, uint32_t x_stride, const float* w, uint32_t dim, float eps, uint32_t n_cols,
                                  uint16_t* out, uint32_t out_stride, hipStream_t s);
 
+// int8 caches -> f16 staging cache of the same geometry (glue_kv.hip): rows [0, n_live) widened, [n_live, n_rows) zeroed
+hipError_t pa_launch_widen_q8(const void* k8, const void* v8, const float* ks, const float* vs, uint16_t* ko, uint16_t* vo,
+                              uint32_t n_kv_heads, uint32_t hd, uint32_t head_rows, uint32_t n_live, uint32_t n_rows, hipStream_t s);
+
 // device probe (probe.hip): sustained f16 MFMA rate and shader clock, constant or random operands
 hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, uint32_t iters, hipStream_t st, float* tflops, float* shader_mhz);
 
@@ -152,6 +156,7 @@ struct pa_ctx {
   size_t proj_buf_floats = 0;
   void* chunk_buf = nullptr;    // pa_attn_layer_prefill: xn f16 [cols][dim], qkv f32 [cols][rows], attnOut f16 [cols][nH*hd]
   size_t chunk_buf_bytes = 0;
+  uint16_t* wide_k = nullptr; uint16_t* wide_v = nullptr;   // int8 caches: f16 staging cache of one layer for the prefill kernel
   uint32_t decode_splits_override = 0;
   // timing
   hipEvent_t t0 = nullptr, t1 = nullptr;

@@ -83,7 +83,9 @@ def test_q8_verify_block_prefill_chunk_and_slots():
         for w, a in enumerate((kq, vq, ks, vs)):
             pa.kv_write(0, w, 0, a)
         assert_parity(pa.run_attn("decode", 0, q[:8], base, gate=gate[:8]), ref[:8], "q8 verify block")
-        assert pa.plan("prefill", base, n)["kernel"] == 0                   # int8 caches: the split-K kernel serves prefill chunks too
+        # a narrow chunk runs on the split-K kernel, a wide one on the MFMA prefill kernel over rows widened to f16
+        assert pa.plan("prefill", base, 4)["kernel"] == 0 and pa.plan("prefill", base, n)["kernel"] == 1
+        assert_parity(pa.run_attn("prefill", 0, q[:4], base, gate=gate[:4]), ref[:4], "q8 narrow prefill chunk")
         assert_parity(pa.run_attn("prefill", 0, q, base, gate=gate, out_dtype=PA_OUT_F16).astype(np.float32), ref, "q8 prefill chunk")
         # slots carry the four tensors
         pa.slot_save(1, base + n)
@@ -131,3 +133,30 @@ def test_q8_fused_decode_step(shape, pos):
     knew = O.q8_dequantize(rows[0].reshape(1, nKV, hd), rows[2].reshape(1, nKV, hd // 32)); vnew = O.q8_dequantize(rows[1].reshape(1, nKV, hd), rows[3].reshape(1, nKV, hd // 32))
     ref = O.attention_values(g["q"], np.concatenate([kf[:pos], knew]), np.concatenate([vf[:pos], vnew]), pos, gate=g["gate"] if cfg["gate"] else None)
     assert_parity(fused.reshape(ref.shape), ref, "q8 fused step %s pos %d" % (shape, pos))
+
+
+@pytest.mark.parametrize("shape,base,n", [("qwen36_moe", 0, 33), ("qwen36_moe", 1, 100), ("qwen36_moe", 2017, 300), ("qwen3_1p7b", 500, 257), ("qwen38_27b", 95, 64)])
+def test_q8_prefill_on_the_matrix_cores(shape, base, n):
+    """Wide chunks on int8 caches: rows [0, base + n) widened into the context's f16 staging cache, then the f16
+    prefill kernel.  Rows past the chunk hold NaN scales (they must not leak); a second, shorter chunk on the same
+    context is not disturbed by the rows the first one staged."""
+    cfg = _q8cfg(shape)
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    rng = np.random.default_rng(base * 7 + n)
+    L = base + n
+    kq, ks, vq, vs, kf, vf = _quantised_cache(cfg, L, seed=base + n)
+    q = rng.standard_normal((n, nH, hd), dtype=np.float32)
+    gate = rng.standard_normal(q.shape, dtype=np.float32) if cfg.get("gate") else None
+    with PooledAttn(cfg, L + 64, n_layers=1, max_cols=n) as pa:
+        pa.layer_alloc(0)
+        for w, a in enumerate((kq, vq, ks, vs)):
+            pa.kv_write(0, w, 0, a)
+        bad = np.full((64, nKV, hd // 32), np.nan, np.float32)
+        pa.kv_write(0, 2, L, bad); pa.kv_write(0, 3, L, bad)
+        assert pa.plan("prefill", base, n)["kernel"] == 1
+        ref = O.attention_values(q, kf, vf, base, gate=gate)
+        assert_parity(pa.run_attn("prefill", 0, q, base, gate=gate), ref, "q8 wide prefill %s base %d n %d" % (shape, base, n))
+        m = n // 2
+        if pa.plan("prefill", base, m)["kernel"] == 1:
+            got = pa.run_attn("prefill", 0, q[:m], base, gate=None if gate is None else gate[:m])
+            assert_parity(got, ref[:m], "q8 wide prefill, shorter chunk after a longer one")
