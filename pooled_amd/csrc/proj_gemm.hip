@@ -95,6 +95,9 @@ static __device__ inline void w_store(const WRegs<KIND>& r, unsigned char* dst, 
   }
 }
 
+// lane <-> lane ^ 1
+static __device__ inline uint32_t pair_swap(uint32_t v) { return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, false); }
+
 template <int KIND>
 __global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(16))) unsigned char xs[2][GT * GROW];
@@ -103,22 +106,41 @@ __global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
   const uint32_t wm = wave >> 1, wn = wave & 1;                       // the wave's 64 columns x 64 rows
   const uint32_t r0 = blockIdx.x * GT, c0 = blockIdx.y * GT;
   const uint32_t nb = p.d_in / GK;
-  // loaders: thread t fetches half a row of each tile
+  // The memory pipeline takes a wave-wide load one cache line (128 bytes) at a time, so what a step's loads cost
+  // is the number of lines they touch.  Activations: four lanes fetch the 64 bytes of a column's step (16 lines a
+  // wave-wide load, two loads a step).  Weights: thread t widens half `t & 1` of row `t >> 1`; Q4_0 rows are fetched
+  // as whole 16-byte blocks, two steps at a time -- the even lane of a pair holds the block of the even step, the odd
+  // lane the next one (32 contiguous bytes a row) -- and each step the holder hands its partner the other half.
+  const uint32_t xrow = tid >> 2, xch = tid & 3;
+  const unsigned char* xsrc[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+    xsrc[i] = (const unsigned char*)(p.x + min((size_t)c0 + xrow + 64 * i, (size_t)p.n_cols - 1) * p.x_stride) + 16 * xch;   // past the end: the last column again (never stored)
   const uint32_t lrow = tid >> 1, half = tid & 1;
-  const size_t wrow = min((size_t)r0 + lrow, (size_t)p.d_out - 1);    // past the end: the last row again (never stored)
-  const size_t xcol = min((size_t)c0 + lrow, (size_t)p.n_cols - 1);
-  const unsigned char* xsrc = (const unsigned char*)(p.x + xcol * p.x_stride) + 32 * half;
+  const size_t wrow = min((size_t)r0 + lrow, (size_t)p.d_out - 1);
   WRegs<KIND> wr;
+  u4 wq4 = {0, 0, 0, 0}; uint16_t wsc4 = 0;                           // Q4_0: the pair's block and scale held by this lane
   u4 xr[2];
-  auto fetch = [&](uint32_t kb) __attribute__((always_inline)) {
-    w_load<KIND>(wr, p, wrow, nb, kb, half);
-    xr[0] = *(const u4*)(xsrc + (size_t)kb * 64);
-    xr[1] = *(const u4*)(xsrc + (size_t)kb * 64 + 16);
+  auto fetch_x = [&](uint32_t kb) __attribute__((always_inline)) {
+    xr[0] = *(const u4*)(xsrc[0] + (size_t)kb * 64);
+    xr[1] = *(const u4*)(xsrc[1] + (size_t)kb * 64);
   };
-  auto stage = [&](int buf) __attribute__((always_inline)) {
+  // Q4_0: blocks kb0 + half of the row (kb0 = the step the even lane's block belongs to)
+  auto fetch_w4 = [&](uint32_t kb0) __attribute__((always_inline)) {
+    const size_t b = wrow * nb + min(kb0 + half, nb - 1);
+    wq4 = *(const u4*)((const unsigned char*)p.w + b * 16);
+    wsc4 = p.scales[b];
+  };
+  auto stage = [&](int buf, uint32_t kb) __attribute__((always_inline)) {
+    if constexpr (KIND == PA_W_Q4_0) {
+      const bool holder = half == (kb & 1);
+      const uint32_t m0 = half ? wq4[2] : wq4[0], m1 = half ? wq4[3] : wq4[1];        // my half of my own block
+      const uint32_t g0 = pair_swap(half ? wq4[0] : wq4[2]), g1 = pair_swap(half ? wq4[1] : wq4[3]), gs = pair_swap((uint32_t)wsc4);   // my half of the partner's
+      wr.q[0] = holder ? m0 : g0; wr.q[1] = holder ? m1 : g1; wr.sc = holder ? wsc4 : (uint16_t)gs;
+    }
     w_store<KIND>(wr, ws[buf] + lrow * GROW, half);
-    *(u4*)(xs[buf] + lrow * GROW + 32 * half) = xr[0];
-    *(u4*)(xs[buf] + lrow * GROW + 32 * half + 16) = xr[1];
+    *(u4*)(xs[buf] + xrow * GROW + 16 * xch) = xr[0];
+    *(u4*)(xs[buf] + (xrow + 64) * GROW + 16 * xch) = xr[1];
   };
   f16v acc[2][2];
 #pragma unroll
@@ -127,13 +149,12 @@ __global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
     for (int b = 0; b < 2; b++)
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
-  fetch(0);
-  stage(0);
+  fetch_x(0);
+  if constexpr (KIND == PA_W_Q4_0) fetch_w4(0); else w_load<KIND>(wr, p, wrow, nb, 0, half);
+  stage(0, 0);
   __syncthreads();
   const uint32_t fl = lane & 31, fk = lane >> 5;                      // fragment row and 8-wide k group of this lane
-  for (uint32_t kb = 0; kb < nb; kb++) {
-    const int cur = kb & 1;
-    if (kb + 1 < nb) fetch(kb + 1);
+  auto mma = [&](int cur) __attribute__((always_inline)) {
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
       h8 af[2], bf[2];
@@ -147,8 +168,25 @@ __global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int b = 0; b < 2; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[a], bf[b], acc[a][b], 0, 0, 0);
     }
-    if (kb + 1 < nb) stage(cur ^ 1);
-    __syncthreads();
+  };
+  // Steps two at a time (buffer 0 then 1); every load is issued whatever the step -- past the last step the last block
+  // again, staged into the buffer nobody reads -- so that the waits can count loads instead of draining them.
+  // A compiler-level memory fence between a step's MFMAs and its staging code keeps the step's global loads above
+  // the fence (left alone, the compiler sinks them next to the staging code that consumes them, and every step waits
+  // out a full memory round trip) while the widening arithmetic may still be scheduled among the MFMAs; a full
+  // scheduling barrier there costs 20 %.
+  for (uint32_t kb = 0; kb < nb; kb += 2) {
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+      if (kb + hh >= nb) break;
+      fetch_x(min(kb + 1 + hh, nb - 1));
+      if constexpr (KIND == PA_W_Q4_0) { if (hh == 1) fetch_w4(kb + 2); }     // block kb + 1 sits in the odd lanes since step kb - 1
+      else w_load<KIND>(wr, p, wrow, nb, min(kb + 1 + hh, nb - 1), half);
+      mma(hh);
+      asm volatile("" ::: "memory");
+      stage(hh ^ 1, kb + 1 + hh);
+      __syncthreads();
+    }
   }
   // accumulator i of a tile: column 8 (i / 4) + 4 (lane / 32) + i % 4, row lane % 32
 #pragma unroll
