@@ -618,7 +618,7 @@ extern "C" int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uin
   GemmParams p; memset(&p, 0, sizeof p);
   p.w = w->w; p.scales = w->scales; p.x = (const uint16_t*)d_x_f16; p.y = d_y; p.x_stride = x_stride; p.y_stride = y_stride;
   p.d_out = w->d_out; p.d_in = w->d_in; p.n_cols = n_cols; p.acc = acc; p.kind = w->kind;
-  HIPCHK(ctx, pa_launch_gemm(p, ctx->stream));
+  HIPCHK(ctx, pa_launch_gemm(p, ctx->n_cu, ctx->stream));
   return PA_OK;
 }
 

@@ -104,7 +104,7 @@ struct GemmParams {
   uint32_t d_out, d_in, n_cols;
   int acc; int kind;
 };
-hipError_t pa_launch_gemm(const GemmParams& p, hipStream_t s);
+hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s);
 // rmsnorm of n_cols f32 columns, written as f16 (the GEMM's activation operand)
 hipError_t pa_launch_rmsnorm_f16(const float* x, uint32_t x_stride, const float* w, uint32_t dim, float eps, uint32_t n_cols,
                                  uint16_t* out, uint32_t out_stride, hipStream_t s);

@@ -98,13 +98,15 @@ static __device__ inline void w_store(const WRegs<KIND>& r, unsigned char* dst, 
 // lane <-> lane ^ 1
 static __device__ inline uint32_t pair_swap(uint32_t v) { return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, false); }
 
-template <int KIND>
-__global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char xs[2][GT * GROW];
+// XT: the workgroup covers 128 XT columns (a wave 64 XT columns x 64 rows): with XT = 2 every weight fragment read from
+// LDS feeds four MFMAs instead of two and the LDS traffic per flop drops by a quarter.
+template <int KIND, int XT>
+__global__ __launch_bounds__(256, XT == 2 ? 2 : 1) void pa_gemm_kernel(GemmParams p) {
+  __shared__ __attribute__((aligned(16))) unsigned char xs[2][GT * XT * GROW];
   __shared__ __attribute__((aligned(16))) unsigned char ws[2][GT * GROW];
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const uint32_t wm = wave >> 1, wn = wave & 1;                       // the wave's 64 columns x 64 rows
-  const uint32_t r0 = blockIdx.x * GT, c0 = blockIdx.y * GT;
+  const uint32_t wm = wave >> 1, wn = wave & 1;                       // the wave's 64 XT columns x 64 rows
+  const uint32_t r0 = blockIdx.x * GT, c0 = blockIdx.y * GT * XT;
   const uint32_t nb = p.d_in / GK;
   // The memory pipeline takes a wave-wide load one cache line (128 bytes) at a time, so what a step's loads cost
   // is the number of lines they touch.  Activations: four lanes fetch the 64 bytes of a column's step (16 lines a
@@ -112,18 +114,18 @@ __global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
   // as whole 16-byte blocks, two steps at a time -- the even lane of a pair holds the block of the even step, the odd
   // lane the next one (32 contiguous bytes a row) -- and each step the holder hands its partner the other half.
   const uint32_t xrow = tid >> 2, xch = tid & 3;
-  const unsigned char* xsrc[2];
+  const unsigned char* xsrc[2 * XT];
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < 2 * XT; i++)
     xsrc[i] = (const unsigned char*)(p.x + min((size_t)c0 + xrow + 64 * i, (size_t)p.n_cols - 1) * p.x_stride) + 16 * xch;   // past the end: the last column again (never stored)
   const uint32_t lrow = tid >> 1, half = tid & 1;
   const size_t wrow = min((size_t)r0 + lrow, (size_t)p.d_out - 1);
   WRegs<KIND> wr;
   u4 wq4 = {0, 0, 0, 0}; uint16_t wsc4 = 0;                           // Q4_0: the pair's block and scale held by this lane
-  u4 xr[2];
+  u4 xr[2 * XT];
   auto fetch_x = [&](uint32_t kb) __attribute__((always_inline)) {
-    xr[0] = *(const u4*)(xsrc[0] + (size_t)kb * 64);
-    xr[1] = *(const u4*)(xsrc[1] + (size_t)kb * 64);
+#pragma unroll
+    for (int i = 0; i < 2 * XT; i++) xr[i] = *(const u4*)(xsrc[i] + (size_t)kb * 64);
   };
   // Q4_0: blocks kb0 + half of the row (kb0 = the step the even lane's block belongs to)
   auto fetch_w4 = [&](uint32_t kb0) __attribute__((always_inline)) {
@@ -139,12 +141,12 @@ __global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
       wr.q[0] = holder ? m0 : g0; wr.q[1] = holder ? m1 : g1; wr.sc = holder ? wsc4 : (uint16_t)gs;
     }
     w_store<KIND>(wr, ws[buf] + lrow * GROW, half);
-    *(u4*)(xs[buf] + xrow * GROW + 16 * xch) = xr[0];
-    *(u4*)(xs[buf] + (xrow + 64) * GROW + 16 * xch) = xr[1];
-  };
-  f16v acc[2][2];
 #pragma unroll
-  for (int a = 0; a < 2; a++)
+    for (int i = 0; i < 2 * XT; i++) *(u4*)(xs[buf] + (xrow + 64 * i) * GROW + 16 * xch) = xr[i];
+  };
+  f16v acc[2 * XT][2];
+#pragma unroll
+  for (int a = 0; a < 2 * XT; a++)
 #pragma unroll
     for (int b = 0; b < 2; b++)
 #pragma unroll
@@ -157,14 +159,13 @@ __global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
   auto mma = [&](int cur) __attribute__((always_inline)) {
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
-      h8 af[2], bf[2];
+      h8 af[2 * XT], bf[2];
 #pragma unroll
-      for (int t = 0; t < 2; t++) {
-        af[t] = *(const h8*)(xs[cur] + (wm * 64 + t * 32 + fl) * GROW + (ks * 16 + fk * 8) * 2);
-        bf[t] = *(const h8*)(ws[cur] + (wn * 64 + t * 32 + fl) * GROW + (ks * 16 + fk * 8) * 2);
-      }
+      for (int t = 0; t < 2 * XT; t++) af[t] = *(const h8*)(xs[cur] + (wm * 64 * XT + t * 32 + fl) * GROW + (ks * 16 + fk * 8) * 2);
 #pragma unroll
-      for (int a = 0; a < 2; a++)
+      for (int t = 0; t < 2; t++) bf[t] = *(const h8*)(ws[cur] + (wn * 64 + t * 32 + fl) * GROW + (ks * 16 + fk * 8) * 2);
+#pragma unroll
+      for (int a = 0; a < 2 * XT; a++)
 #pragma unroll
         for (int b = 0; b < 2; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[a], bf[b], acc[a][b], 0, 0, 0);
     }
@@ -190,13 +191,13 @@ __global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
   }
   // accumulator i of a tile: column 8 (i / 4) + 4 (lane / 32) + i % 4, row lane % 32
 #pragma unroll
-  for (int a = 0; a < 2; a++)
+  for (int a = 0; a < 2 * XT; a++)
 #pragma unroll
     for (int b = 0; b < 2; b++) {
       const uint32_t row = r0 + wn * 64 + b * 32 + fl;
 #pragma unroll
       for (int i = 0; i < 16; i++) {
-        const uint32_t col = c0 + wm * 64 + a * 32 + 8 * (i / 4) + 4 * fk + (i % 4);
+        const uint32_t col = c0 + wm * 64 * XT + a * 32 + 8 * (i / 4) + 4 * fk + (i % 4);
         if (row < p.d_out && col < p.n_cols) {
           float* y = p.y + (size_t)col * p.y_stride + row;
           *y = p.acc ? *y + acc[a][b][i] : acc[a][b][i];
@@ -205,16 +206,25 @@ __global__ __launch_bounds__(256) void pa_gemm_kernel(GemmParams p) {
     }
 }
 
-hipError_t pa_launch_gemm(const GemmParams& p, hipStream_t s) {
-  if (p.d_out == 0 || p.d_in == 0 || (p.d_in & 31) || p.n_cols == 0) return hipErrorInvalidValue;
-  const dim3 grid((p.d_out + GT - 1) / GT, (p.n_cols + GT - 1) / GT), block(256);
+template <int XT>
+static hipError_t launch_gemm_xt(const GemmParams& p, hipStream_t s) {
+  const dim3 grid((p.d_out + GT - 1) / GT, (p.n_cols + GT * XT - 1) / (GT * XT)), block(256);
   switch (p.kind) {
-    case PA_W_F32: hipLaunchKernelGGL(pa_gemm_kernel<PA_W_F32>, grid, block, 0, s, p); break;
-    case PA_W_Q8_0: hipLaunchKernelGGL(pa_gemm_kernel<PA_W_Q8_0>, grid, block, 0, s, p); break;
-    case PA_W_Q4_0: hipLaunchKernelGGL(pa_gemm_kernel<PA_W_Q4_0>, grid, block, 0, s, p); break;
+    case PA_W_F32: hipLaunchKernelGGL((pa_gemm_kernel<PA_W_F32, 1>), dim3(grid.x, (p.n_cols + GT - 1) / GT), block, 0, s, p); break;
+    case PA_W_Q8_0: hipLaunchKernelGGL((pa_gemm_kernel<PA_W_Q8_0, XT>), grid, block, 0, s, p); break;
+    case PA_W_Q4_0: hipLaunchKernelGGL((pa_gemm_kernel<PA_W_Q4_0, XT>), grid, block, 0, s, p); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
+}
+
+hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s) {
+  if (p.d_out == 0 || p.d_in == 0 || (p.d_in & 31) || p.n_cols == 0) return hipErrorInvalidValue;
+  // 256-column workgroups (two fit a CU) when they still give every CU four: otherwise 128-column ones (three a CU)
+  const size_t wgs2 = (size_t)((p.d_out + GT - 1) / GT) * ((p.n_cols + 2 * GT - 1) / (2 * GT));
+  const char* e = getenv("POOLED_ATTN_GEMM_XT");
+  const bool xt2 = e ? atoi(e) == 2 : wgs2 >= (size_t)4 * (n_cu > 0 ? n_cu : 256);
+  return xt2 ? launch_gemm_xt<2>(p, s) : launch_gemm_xt<1>(p, s);
 }
 
 // rmsnorm of n_cols columns, written as f16: one workgroup per column.  xn = f16((x * inv) * w),
