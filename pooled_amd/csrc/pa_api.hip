@@ -287,8 +287,7 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   const uint32_t G = c.n_heads / c.n_kv_heads;
   // rows per workgroup: 16-row blocks whose O^T accumulators still fit the register file next to the
   // in-flight K/V tile (hd 256: 2 blocks, hd 128: 4 blocks)
-  uint32_t max_rows = c.head_dim == 256 ? 32 : 64;
-  if (const char* e = getenv("POOLED_ATTN_DECODE_MAX_ROWS")) { const int v = atoi(e); if (v == 16 || v == 32 || v == 48 || v == 64) max_rows = v; }
+  const uint32_t max_rows = c.head_dim == 256 ? 32 : 64;
   uint32_t cw = n_cols, groups = 1;
   if (n_cols * G > max_rows) { cw = max_rows / G; if (cw == 0) return PA_ERR_UNSUPPORTED; groups = ceil_div(n_cols, cw); }
   const uint32_t nb = ceil_div(cw * G, 16);

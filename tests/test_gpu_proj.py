@@ -121,8 +121,11 @@ def test_attn_layer_decode_matches_oracle(shape, dim, kind, pos):
 # ---- column-batched passes: rmsnorm -> f16, GEMM on the matrix cores, the whole attention half of a layer ----
 
 @pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q8_0, PA_W_Q4_0])
-@pytest.mark.parametrize("d_out,d_in,n", [(9216, 2048, 300), (2048, 4096, 129), (37, 96, 5), (130, 8192, 17), (256, 32, 128)])
-def test_gemm_matches_oracle(kind, d_out, d_in, n):
+@pytest.mark.parametrize("d_out,d_in,n", [(9216, 2048, 300), (2048, 4096, 129), (37, 96, 5), (130, 8192, 17), (256, 32, 128), (384, 96, 700)])
+@pytest.mark.parametrize("wide", [False, True])
+def test_gemm_matches_oracle(kind, d_out, d_in, n, wide, monkeypatch):
+    # wide: force the 256-column workgroups that large chunks get (the library reads the switch at every call)
+    monkeypatch.setenv("POOLED_ATTN_GEMM_XT", "2" if wide else "1")
     if kind == PA_W_F32 and d_in > 4096:
         pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
     rng = np.random.default_rng(d_out + 3 * d_in + n + kind)
