@@ -177,13 +177,13 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   const uint32_t t_end = !SR && sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
   const size_t head_rows = (size_t)p.max_seq + TILE;              // rows of one kv head's plane, padding included
   PA_TP(0);
-  // SR on f16 caches: the whole splits of a kv head are interleaved.  With nw = (whole splits) x W waves, wave v of
+  // SR: the whole splits of a kv head are interleaved.  With nw = (whole splits) x W waves, wave v of
   // them takes rows [(c nw + v) 8, + 8), c = 0 .. 3, instead of 32 consecutive ones: at any moment the loads in
   // flight on the chip then sweep a compact range of the cache (4 KB pieces, neighbouring waves on neighbouring
   // pieces) instead of 2048 separate 32 KB streams -- the memory controllers see open pages.  Measured on read-only
   // stand-ins of this launch shape: 11.9 -> 11.2 us for 64 MiB.  Any partition of the rows is a valid set of
   // splits; masks go by position.  A trailing partial split and the remainder splits keep consecutive rows.
-  constexpr bool ILV = SR && !GATHER && !Q8;
+  constexpr bool ILV = SR && !GATHER;
   uint32_t ilv_nw = 0, ilv_wv = 0;
   bool ilv = false;
   if constexpr (ILV) {
@@ -308,8 +308,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
   } else if constexpr (Q8) {
 #pragma unroll
-    for (int i = 0; i < S::NLD8; i++) kr[i] = *(const u4*)(kbase8 + (size_t)t0 * HD + (size_t)(i * S::RPL8) * HD + voff8);
-    ksr = *(const u4*)(ksbase + (size_t)t0 * S::SPR * 4 + soff);
+    for (int i = 0; i < S::NLD8; i++) kr[i] = *(const u4*)(kbase8 + (size_t)row_pos(t0, i * S::RPL8) * HD + voff8);   // a load's rows share an 8-row piece
+    ksr = *(const u4*)(ksbase + (size_t)row_pos(t0, srow) * S::SPR * 4 + (lane % S::LPS) * 16);
   } else {
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)row_pos(t0, i * S::RPL) * row_bytes + voff);
@@ -320,8 +320,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
     } else if constexpr (Q8) {
 #pragma unroll
-      for (int i = 0; i < S::NLD8; i++) vr[i] = *(const u4*)(vbase8 + (size_t)t0 * HD + (size_t)(i * S::RPL8) * HD + voff8);
-      vsr = *(const u4*)(vsbase + (size_t)t0 * S::SPR * 4 + soff);
+      for (int i = 0; i < S::NLD8; i++) vr[i] = *(const u4*)(vbase8 + (size_t)row_pos(t0, i * S::RPL8) * HD + voff8);
+      vsr = *(const u4*)(vsbase + (size_t)row_pos(t0, srow) * S::SPR * 4 + (lane % S::LPS) * 16);
     } else {
 #pragma unroll
       for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)row_pos(t0, i * S::RPL) * row_bytes + voff);
