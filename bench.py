@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Headline workload (BASELINE.json's metric, "decode attn KV-read GB/s @32K ctx"): configuration 3 --
+Headline workload (metric "decode attn KV-read GB/s @32K ctx"): configuration 3 --
 single-token gated decode attention, Qwen3.6-35B-MoE attention shape (16 q heads, 2 kv heads, head_dim 256),
 context 32768.  A step is one pass of the hot path for one token on one attention layer: pre-step (q
 de-interleave + QK-RMSNorm + partial RoPE + f16 KV write at position 32768), split-K decode kernel, log-sum-exp
@@ -210,7 +210,7 @@ def prefill_leg(steps, with_cpu, kv_q8=False):
 
 def other_configs():
     """Configurations 1, 2 and 4 of the baseline (parity-test cases, not bench lines): steady-state time per call on
-    caches in rotation, for the record in DESIGN.md."""
+    caches in rotation, printed for the record."""
     from pooled_amd.capi import PooledAttn, PA_OUT_F16
     dense = dict(n_heads=16, n_kv_heads=8, head_dim=128, n_rot=128, rope_theta=1e6, eps=1e-6, qk_norm=True, gate=False)
     b27 = dict(n_heads=24, n_kv_heads=4, head_dim=256, n_rot=64, rope_theta=1e7, eps=1e-6, qk_norm=True, gate=True)
