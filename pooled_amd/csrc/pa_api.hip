@@ -324,12 +324,23 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
 
 // Prefill (MFMA kernel): a workgroup is 8 wavefronts x 32 query rows = 256 rows of one kv head, i.e.
 // floor(256 / G) columns x G heads.  Chunks wide enough to give every CU a workgroup run unsplit and write the
-// output directly; narrower chunks are also split over the context (partials + merge kernel) until about two
-// workgroups per CU exist.  Chunks of fewer rows than one wavefront tile go to the split-K decode kernel.
+// output directly; narrower chunks are also split over the context (partials + merge kernel) until every CU has a
+// workgroup (one is resident per CU; a second round of a few workgroups costs more than longer splits).  Chunks of fewer rows than one wavefront tile go to the split-K decode kernel.
 static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, uint32_t* wgs = nullptr) {
   const pa_config& c = ctx->cfg;
   const uint32_t G = c.n_heads / c.n_kv_heads;
-  if (n_cols * G <= (c.head_dim == 256 ? 32u : 64u)) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
+  const uint32_t max_rows_sk = c.head_dim == 256 ? 32u : 64u;
+  if (n_cols * G <= max_rows_sk) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
+  // A chunk of a few column groups over a long context (the reference's own prefill passes are 16 columns wide) is
+  // bound by the K/V stream, not by the matrix cores: the split-K kernel serves it in column groups, whose workgroups
+  // share the stream through L2, for as long as groups x K/V bytes stays below what the MFMA kernel's fixed costs
+  // (Q staging, one partial per split and row, the merge) amount to.  Measured crossover on the MoE and 27B shapes
+  // at 32K - 64K rows: about 1.4 GB of L2-level K/V traffic; below 4096 rows both kernels take 25 - 40 us.
+  if (n_cols * G <= 512 && base_pos + n_cols >= 4096 && max_rows_sk >= G) {
+    const uint64_t groups_sk = ceil_div(n_cols, max_rows_sk / G);
+    const uint64_t kv_bytes = 2ull * (base_pos + n_cols) * c.n_kv_heads * c.head_dim * (kv_q8(ctx) ? 1 : 2);
+    if (groups_sk * kv_bytes <= 1400000000ull) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
+  }
   const uint32_t rows_wg = 256;
   const uint32_t cw = rows_wg / G;
   if (cw == 0) return PA_ERR_UNSUPPORTED;
@@ -337,7 +348,7 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
   const uint32_t seq_max = base_pos + n_cols;
   const uint32_t base_wgs = groups * c.n_kv_heads;
   uint32_t splits = 1;
-  if (base_wgs < (uint32_t)ctx->n_cu) splits = std::min(ceil_div(2 * (uint32_t)ctx->n_cu, base_wgs), std::max(1u, seq_max / 256));
+  if (base_wgs < (uint32_t)ctx->n_cu) splits = std::min(std::max(1u, (uint32_t)ctx->n_cu / base_wgs), std::max(1u, seq_max / 256));
   uint32_t sl = ceil_div(ceil_div(seq_max, splits), 32) * 32;
   pl->kernel = 1; pl->split_len = sl; pl->n_splits = ceil_div(seq_max, sl);
   pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = 8; pl->row_blocks = 8; pl->slots = pl->n_splits;

@@ -61,11 +61,20 @@ def test_prefill_equals_decode_columns():
 
 
 def test_prefill_split_path_and_f16_out():
-    """A narrow chunk on a long context is split over the context (partials + merge kernel)."""
+    """A chunk of a few column blocks on a long context is split over the context (partials + merge kernel)."""
     cfg = SHAPES["qwen36_moe"]
-    got, ref, plan = _prefill(cfg, 20000, 64, seed=5, out_dtype=PA_OUT_F16)
+    got, ref, plan = _prefill(cfg, 20000, 80, seed=5, out_dtype=PA_OUT_F16)
     assert plan["kernel"] == 1 and plan["n_splits"] > 1
     assert_parity(got, ref, "split prefill")
+
+
+@pytest.mark.parametrize("shape,base,n", [("qwen36_moe", 20000, 16), ("qwen36_moe", 20000, 64), ("qwen38_27b", 9000, 40), ("qwen3_1p7b", 5000, 100)])
+def test_prefill_narrow_chunk_on_a_long_context_takes_the_stream_kernel(shape, base, n):
+    """Chunks of at most 512 stacked rows over 4096 or more cache rows (the reference's own passes are 16 columns wide)
+    are bound by the K/V stream: the plan hands them to the split-K kernel in column groups."""
+    got, ref, plan = _prefill(SHAPES[shape], base, n, seed=base + n)
+    assert plan["kernel"] == 0 and plan["col_groups"] > 1
+    assert_parity(got, ref, "narrow chunk")
 
 
 def test_prefill_peaked_softmax():
@@ -79,7 +88,7 @@ def test_prefill_peaked_softmax():
 
 @pytest.mark.parametrize("shape,base,n,k_scale", [
     ("qwen36_moe", 301, 16, 1.0), ("qwen36_moe", 1000, 200, 1.0), ("qwen3_1p7b", 219, 257, 1.0),
-    ("qwen38_27b", 500, 96, 3.0), ("qwen36_moe", 20000, 64, 1.0),
+    ("qwen38_27b", 500, 96, 3.0), ("qwen36_moe", 20000, 80, 1.0),
 ])
 def test_prefill_wide_variant(shape, base, n, k_scale, monkeypatch):
     """The 4-wave, 64-rows-per-wave variant of the prefill kernel (selected by an environment variable read at
