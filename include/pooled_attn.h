@@ -163,8 +163,9 @@ int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const 
  *   d_sel: u32 [n_cols][sel_stride]; column c's list is d_sel[c * sel_stride] = n (1 <= n <= max_rows), then n row
  *          indices < max_seq at d_sel[c * sel_stride + 1 ..], ascending (the reference's QSA_SEL_STRIDE layout)
  *   max_rows: the longest list of the pass (engine/qsa.js:34 qsaMaxRows); sizes the splits
- * List position t stands where position t stands in pa_attn_decode: with the list 0 .. pos a single column gives the
- * same bits as pa_attn_decode at base_pos = pos. */
+ * List position t stands where position t stands in pa_attn_decode: with the list 0 .. pos a single column gives
+ * pa_attn_decode's result at base_pos = pos to rounding (2e-5; the dense call keeps the column's own row out of the
+ * streamed rows, so the two sum in a different order). */
 int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_stride, const float* d_gate,
                           uint32_t gate_stride, const uint32_t* d_sel, uint32_t sel_stride, uint32_t max_rows,
                           uint32_t n_cols, void* d_out, uint32_t out_stride, int out_dtype);
