@@ -135,7 +135,9 @@ float* pa_gate_buffer(pa_ctx* ctx);
  *   d_q   : f32 [n_cols][q_stride], a column holds roped q [nH][hd]; NULL = pa_q_buffer
  *   d_gate: f32 [n_cols][gate_stride] gate pre-activations [nH][hd]; NULL = no gate
  *   d_out : [n_cols][out_stride] of out_dtype, a column holds [nH][hd]
- * pa_attn_prefill: the same contract for a causal prefill chunk of any width on the f16 MFMA kernel.
+ * pa_attn_prefill: the same contract for a causal prefill chunk of any width: the f16 MFMA kernel, or, for a chunk of
+ * few columns (at most one 32- / 64-row block, or a few column groups over a long context, where the K/V stream and
+ * not the matrix cores bound the pass), the split-K kernel; pa_plan_query tells which.
  * Replaces attn_flash_tile + attn_combine_tile + sigmoid_mul_mc (engine/wgsl/attn_tile.js:108-193;
  * call site engine/qwen35.js:2489-2493, :2516); one call covers what the reference runs as
  * ceil(n_cols / 16) consecutive 16-column passes (engine/qwen35.js:3843-3860). */
