@@ -255,7 +255,9 @@ int pa_attn_layer_decode(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, co
 int pa_rmsnorm_f16(pa_ctx* ctx, const float* d_x, uint32_t x_stride, const float* d_norm_w, uint32_t dim, uint32_t n_cols,
                    void* d_xn_f16, uint32_t xn_stride);
 /* y[c][0 .. d_out) = W x[c] for n_cols columns; x: f16 bits, stride in f16 elements (>= d_in, multiple of 8);
- * y: f32, stride in floats; acc != 0: y += W x */
+ * y: f32, stride in floats; acc != 0: y += W x.  Chunks of up to 32 columns (verify blocks, the reference's 16-column
+ * passes through its batched matvec, engine/wgsl/coop.js) are served by a kernel that streams the weights once per
+ * 16 columns instead of the tiled one; same operand precision either way. */
 int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uint32_t x_stride, uint32_t n_cols, float* d_y, uint32_t y_stride, int acc);
 /* n_cols tokens at positions base_pos .. through the attention half of a full-attention layer, as
  * _encodeLayerBatch / _encodeLayerWide record it (engine/qwen35.js:2416-2425, :2827): rmsnorm -> [q | k | v] GEMM ->

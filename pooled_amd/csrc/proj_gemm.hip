@@ -206,6 +206,137 @@ __global__ __launch_bounds__(256, XT == 2 ? 2 : 1) void pa_gemm_kernel(GemmParam
     }
 }
 
+// ---- skinny chunks (a verify block, the reference's 16-column passes: engine/wgsl/coop.js batched matvec) ----
+// With a handful of columns the tiled kernel leaves the chip empty (d_out / 128 workgroups, each walking all of K)
+// while the work is one pass over the weights.  This kernel streams the weights GEMV-style -- a wave owns RW rows, a
+// lane the 32-value blocks lane + 64 i of each -- widens them once into f16 pairs in registers, stages all the
+// chunk's columns in LDS (80-byte block stride: conflict-free 128-bit reads) and runs one v_dot2_f32_f16 per two
+// weights and column.  Same operand precision as the tiled kernel (weights and activations f16, sums f32), so a
+// result does not depend on which kernel served the chunk beyond the order of the sums.  The lanes' partial sums go
+// through LDS (the staging area, free by then): lane t of a wave adds up the 64 partials of its (row, column).
+#define SK_NC 16        // columns a launch serves at most
+template <int KIND, int BPL, int RW>
+__global__ __launch_bounds__(256) void pa_gemm_skinny_kernel(GemmParams p) {
+  static_assert(KIND == PA_W_Q4_0 || KIND == PA_W_Q8_0, "quantised weights");
+  extern __shared__ __attribute__((aligned(16))) unsigned char sk_lds[];
+  const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t nb = p.d_in / GK, ncol = p.n_cols;
+  const uint32_t xcol = nb * GROW;                                    // bytes of a staged column
+  const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * RW;
+  // the wave's weights first: they are what the kernel waits for
+  constexpr int WQ = KIND == PA_W_Q4_0 ? 1 : 2;                       // 16-byte words of a packed block
+  u4 wq[RW][BPL][WQ];
+  uint16_t wsc[RW][BPL];
+#pragma unroll
+  for (int r = 0; r < RW; r++) {
+    const size_t row = min(row0 + r, (size_t)p.d_out - 1);            // rows past the end repeat the last one (not stored)
+#pragma unroll
+    for (int i = 0; i < BPL; i++) {
+      const uint32_t b = min(lane + 64 * i, nb - 1);                   // blocks past the end likewise (scale forced to 0)
+      const u4* src = (const u4*)((const unsigned char*)p.w + (row * nb + b) * (16 * WQ));
+#pragma unroll
+      for (int w = 0; w < WQ; w++) wq[r][i][w] = src[w];
+      wsc[r][i] = p.scales[row * nb + b];
+    }
+  }
+  // the chunk's columns -> LDS, 16 bytes a thread and turn
+  const uint32_t cpc = p.d_in / 8;                                    // 16-byte pieces of a column
+  for (uint32_t e = tid; e < ncol * cpc; e += 256) {
+    const uint32_t c = e / cpc, k8 = e % cpc;
+    *(u4*)(sk_lds + c * xcol + (k8 >> 2) * GROW + (k8 & 3) * 16) = *(const u4*)((const unsigned char*)(p.x + (size_t)c * p.x_stride) + k8 * 16);
+  }
+  // widen: pair k of a block = elements 2k, 2k + 1
+  h2 wv[RW][BPL][16];
+#pragma unroll
+  for (int r = 0; r < RW; r++)
+#pragma unroll
+    for (int i = 0; i < BPL; i++) {
+      const _Float16 s1 = __ushort_as_half(lane + 64 * i < nb ? wsc[r][i] : (uint16_t)0);
+      const h2 sc = { s1, s1 };
+      if constexpr (KIND == PA_W_Q4_0) {
+        const h2 bias = { (_Float16)1032.f, (_Float16)1032.f };
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+          const uint32_t l = wq[r][i][0][d] & 0x0F0F0F0Fu, h = (wq[r][i][0][d] >> 4) & 0x0F0F0F0Fu;
+          wv[r][i][2 * d] = bytes_to_h2(l, 0x04010400u, bias, sc); wv[r][i][2 * d + 1] = bytes_to_h2(l, 0x04030402u, bias, sc);
+          wv[r][i][8 + 2 * d] = bytes_to_h2(h, 0x04010400u, bias, sc); wv[r][i][8 + 2 * d + 1] = bytes_to_h2(h, 0x04030402u, bias, sc);
+        }
+      } else {
+        const h2 bias = { (_Float16)1152.f, (_Float16)1152.f };
+#pragma unroll
+        for (int w = 0; w < 2; w++)
+#pragma unroll
+          for (int d = 0; d < 4; d++) {
+            const uint32_t x = wq[r][i][w][d] ^ 0x80808080u;
+            wv[r][i][8 * w + 2 * d] = bytes_to_h2(x, 0x04010400u, bias, sc); wv[r][i][8 * w + 2 * d + 1] = bytes_to_h2(x, 0x04030402u, bias, sc);
+          }
+      }
+    }
+  __syncthreads();
+  float part[SK_NC][RW];
+#pragma unroll
+  for (int c = 0; c < SK_NC; c++) {
+#pragma unroll
+    for (int r = 0; r < RW; r++) part[c][r] = 0.f;
+    if ((uint32_t)c < ncol) {
+#pragma unroll
+      for (int i = 0; i < BPL; i++) {
+        const unsigned char* xb = sk_lds + c * xcol + min(lane + 64 * i, nb - 1) * GROW;
+        h2 xv[16];
+#pragma unroll
+        for (int q = 0; q < 4; q++) { const h8 v = *(const h8*)(xb + 16 * q); xv[4 * q] = (h2){ v[0], v[1] }; xv[4 * q + 1] = (h2){ v[2], v[3] }; xv[4 * q + 2] = (h2){ v[4], v[5] }; xv[4 * q + 3] = (h2){ v[6], v[7] }; }
+#pragma unroll
+        for (int r = 0; r < RW; r++)
+#pragma unroll
+          for (int k = 0; k < 16; k++) part[c][r] = __builtin_amdgcn_fdot2(wv[r][i][k], xv[k], part[c][r], false);
+      }
+    }
+  }
+  __syncthreads();                                                    // every wave is done with the staged columns
+  // partials -> LDS [wave][lane][SK_NC * RW + 1], then lane t sums column t of its wave's 64 x (SK_NC * RW) table
+  constexpr int PV = SK_NC * RW, PS = PV + 1;
+  float* ps = (float*)sk_lds + (size_t)wave * 64 * PS;
+#pragma unroll
+  for (int c = 0; c < SK_NC; c++)
+    if ((uint32_t)c < ncol)
+#pragma unroll
+      for (int r = 0; r < RW; r++) ps[lane * PS + c * RW + r] = part[c][r];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  for (uint32_t t = lane; t < ncol * RW; t += 64) {
+    float a = 0.f;
+    for (int l = 0; l < 64; l++) a += ps[l * PS + t];
+    const uint32_t c = t / RW, r = t % RW;
+    if (row0 + r < p.d_out) {
+      float* y = p.y + (size_t)c * p.y_stride + row0 + r;
+      *y = p.acc ? *y + a : a;
+    }
+  }
+}
+
+// LDS the skinny kernel needs: the staged columns, or the four waves' partial tables if those are larger
+static size_t skinny_lds(const GemmParams& p, int rw) {
+  const size_t x = (size_t)p.n_cols * (p.d_in / GK) * GROW, ps = (size_t)4 * 64 * (SK_NC * rw + 1) * sizeof(float);
+  return x > ps ? x : ps;
+}
+template <int KIND, int BPL, int RW>
+static hipError_t launch_skinny(const GemmParams& p, hipStream_t s) {
+  const size_t lds = skinny_lds(p, RW);
+  static size_t attr = 0;
+  if (lds > attr) {
+    hipError_t e = hipFuncSetAttribute((const void*)pa_gemm_skinny_kernel<KIND, BPL, RW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    attr = lds;
+  }
+  hipLaunchKernelGGL((pa_gemm_skinny_kernel<KIND, BPL, RW>), dim3((p.d_out + 4 * RW - 1) / (4 * RW)), dim3(256), lds, s, p);
+  return hipGetLastError();
+}
+template <int KIND>
+static hipError_t launch_skinny_kind(const GemmParams& p, hipStream_t s) {
+  if (p.d_in <= 2048) return launch_skinny<KIND, 1, 4>(p, s);
+  if (p.d_in <= 4096) return launch_skinny<KIND, 2, 2>(p, s);
+  return launch_skinny<KIND, 4, 1>(p, s);
+}
+
 template <int XT>
 static hipError_t launch_gemm_xt(const GemmParams& p, hipStream_t s) {
   const dim3 grid((p.d_out + GT - 1) / GT, (p.n_cols + GT * XT - 1) / (GT * XT)), block(256);
@@ -220,6 +351,23 @@ static hipError_t launch_gemm_xt(const GemmParams& p, hipStream_t s) {
 
 hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s) {
   if (p.d_out == 0 || p.d_in == 0 || (p.d_in & 31) || p.n_cols == 0) return hipErrorInvalidValue;
+  // a handful of columns: a pass over the weights per launch of up to 16 columns (as many as fit the LDS staging),
+  // up to 32 columns in all -- past that the tiled kernel wins (POOLED_ATTN_GEMM_SKINNY=0 keeps it, for measurements)
+  if (p.kind != PA_W_F32 && p.n_cols <= 2 * SK_NC && p.d_in <= 8192 && (p.x_stride & 7) == 0) {
+    const char* k = getenv("POOLED_ATTN_GEMM_SKINNY");
+    const uint32_t fit = (uint32_t)((144 * 1024) / ((size_t)(p.d_in / GK) * GROW));
+    const uint32_t per = fit < SK_NC ? fit : SK_NC;
+    if ((!k || atoi(k) != 0) && per >= 1) {
+      for (uint32_t c0 = 0; c0 < p.n_cols; c0 += per) {
+        GemmParams q = p;
+        q.x = p.x + (size_t)c0 * p.x_stride; q.y = p.y + (size_t)c0 * p.y_stride;
+        q.n_cols = p.n_cols - c0 < per ? p.n_cols - c0 : per;
+        const hipError_t e = p.kind == PA_W_Q4_0 ? launch_skinny_kind<PA_W_Q4_0>(q, s) : launch_skinny_kind<PA_W_Q8_0>(q, s);
+        if (e != hipSuccess) return e;
+      }
+      return hipSuccess;
+    }
+  }
   // 256-column workgroups (two fit a CU) when they still give every CU four: otherwise 128-column ones (three a CU)
   const size_t wgs2 = (size_t)((p.d_out + GT - 1) / GT) * ((p.n_cols + 2 * GT - 1) / (2 * GT));
   const char* e = getenv("POOLED_ATTN_GEMM_XT");

@@ -121,7 +121,8 @@ def test_attn_layer_decode_matches_oracle(shape, dim, kind, pos):
 # ---- column-batched passes: rmsnorm -> f16, GEMM on the matrix cores, the whole attention half of a layer ----
 
 @pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q8_0, PA_W_Q4_0])
-@pytest.mark.parametrize("d_out,d_in,n", [(9216, 2048, 300), (2048, 4096, 129), (37, 96, 5), (130, 8192, 17), (256, 32, 128), (384, 96, 700)])
+@pytest.mark.parametrize("d_out,d_in,n", [(9216, 2048, 300), (2048, 4096, 129), (37, 96, 5), (130, 8192, 40), (256, 32, 128), (384, 96, 700),
+                                          (9216, 2048, 8), (2048, 4096, 16), (130, 8192, 3), (70, 64, 1), (2048, 4096, 31), (130, 8192, 17)])   # from (9216, 2048, 8) on: the skinny-chunk kernel, one or more launches
 @pytest.mark.parametrize("wide", [False, True])
 def test_gemm_matches_oracle(kind, d_out, d_in, n, wide, monkeypatch):
     # wide: force the 256-column workgroups that large chunks get (the library reads the switch at every call)
