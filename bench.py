@@ -282,6 +282,11 @@ def layer_leg(pa, cfg, ctx, steps, warmup, attn_ms):
     b_o = dim * qd // 2 + dim * (qd // 32) * 2
     kv_bytes = 2 * (ctx + 1) * kvd * 2
     log("layer: [q|k|v] GEMV %.2f us, wo GEMV %.2f us, whole attention half %.2f us" % (t_qkv * 1e3, t_o * 1e3, t_layer * 1e3))
+    # a speculative-verify block of 8 tokens through the same half of the layer (column-batched call, engine/qwen35.js:2416-2425)
+    nv = 8
+    d_xv = pa.to_device(rng.standard_normal((nv, dim)).astype(np.float32))
+    t_verify = timed(lambda i: pa.attn_layer_prefill(i % N_LAYERS, wq[i % n_sets], wo[i % n_sets], d_nw, d_hw, d_hw, d_xv, dim, ctx - nv + 1, nv))
+    log("layer, verify block of %d tokens: %.2f us" % (nv, t_verify * 1e3))
     return dict(workload="one token through the attention half of a full-attention layer (engine/qwen35.js:1586-1641): rmsnorm + [q|k|v] "
                          "GEMV %dx%d, pre-step + split-K attention over %d rows + merge/gate, wo GEMV %dx%d accumulated into the residual; "
                          "Q4_0 weights, 4 launches; weights and caches in rotation (cold HBM)" % (rows_qkv, dim, ctx, dim, qd),
@@ -289,7 +294,10 @@ def layer_leg(pa, cfg, ctx, steps, warmup, attn_ms):
                 gemv_qkv_norm=dict(us=round(t_qkv * 1e3, 2), weight_bytes=b_qkv, gbs=round(b_qkv / t_qkv / 1e6, 1)),
                 gemv_o_acc=dict(us=round(t_o * 1e3, 2), weight_bytes=b_o, gbs=round(b_o / t_o / 1e6, 1)),
                 bytes_per_step=kv_bytes + b_qkv + b_o, gbs=round((kv_bytes + b_qkv + b_o) / t_layer / 1e6, 1),
-                pct_hbm_peak=round(100 * (kv_bytes + b_qkv + b_o) / t_layer / 1e6 / HBM_PEAK_GBS, 2))
+                pct_hbm_peak=round(100 * (kv_bytes + b_qkv + b_o) / t_layer / 1e6 / HBM_PEAK_GBS, 2),
+                verify_block=dict(workload="%d tokens at positions %d .. %d through the same half of the layer (pa_attn_layer_prefill: rmsnorm, skinny-chunk "
+                                           "projections, pre-step, split-K attention in column groups, merge/gate)" % (nv, ctx - nv + 1, ctx),
+                                  us_per_step=round(t_verify * 1e3, 2), us_per_token=round(t_verify * 1e3 / nv, 2)))
 
 
 def main():
