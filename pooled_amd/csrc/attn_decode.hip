@@ -32,6 +32,7 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 
 #define TILE 32
 #define NEG_INF (-__builtin_inff())
+#define DEC_RESCALE_TH 8.f   // tile loop: a row maximum may pass the reference maximum by this much before O is rescaled
 
 // Optional per-wave timeline (development builds only): lane 0 of every wave stores the 100 MHz wall clock at
 // up to 12 points into p.trace.  Compiled out unless PA_TRACE is defined.
@@ -672,10 +673,14 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     qk(s);
     PA_TP(4);
     // ---- online softmax; lane holds row nb*16 + ln, positions tp + pb*16 + 4*kg + i ----
+    // m_run is a lazily updated reference maximum: O and l are rescaled only when some row's tile maximum passes it
+    // by more than DEC_RESCALE_TH (natural-log units), so exp(x - m_run) <= e^TH stays far inside the f16 range and
+    // the rescale of the whole accumulator tile is off the common path.
     h8 pfrag[NB];
+    float v[NB][8], mxs[NB];
+    bool grow = false;
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
-      float v[8];
       float mx = NEG_INF;
 #pragma unroll
       for (int pb = 0; pb < 2; pb++)
@@ -683,23 +688,34 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
         for (int i = 0; i < 4; i++) {
           const uint32_t pos = tp + pb * 16 + 4 * kg + i;
           const float x = pos < end_pos[nb] ? s[pb][nb][i] * p.scale : NEG_INF;
-          v[pb * 4 + i] = x;
+          v[nb][pb * 4 + i] = x;
           mx = fmaxf(mx, x);
         }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run[nb], mx);
-      const float m_safe = m_new == NEG_INF ? 0.f : m_new;
-      const float alpha = __expf(m_run[nb] - m_safe);
+      mxs[nb] = mx;
+      grow |= mx > m_run[nb] + DEC_RESCALE_TH;
+    }
+    if (__builtin_expect(__any(grow), 0)) {
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+        const float m_new = fmaxf(m_run[nb], mxs[nb]);
+        const float alpha = m_new == NEG_INF ? 1.f : __expf(m_run[nb] - m_new);
+        l_run[nb] *= alpha;
+        m_run[nb] = m_new;
+#pragma unroll
+        for (int db = 0; db < S::DB; db++) acc[db][nb] *= alpha;
+      }
+    }
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+      const float m_safe = m_run[nb] == NEG_INF ? 0.f : m_run[nb];
       float ps = 0.f;
       h8 pf;
 #pragma unroll
-      for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - m_safe); ps += e; pf[j] = (_Float16)e; }
+      for (int j = 0; j < 8; j++) { const float e = __expf(v[nb][j] - m_safe); ps += e; pf[j] = (_Float16)e; }
       pfrag[nb] = pf;
-      l_run[nb] = l_run[nb] * alpha + ps;
-      m_run[nb] = m_new;
-#pragma unroll
-      for (int db = 0; db < S::DB; db++) acc[db][nb] *= alpha;
+      l_run[nb] += ps;
     }
     // V after the softmax, so that the wait for the V loads comes as late as possible
     stage_v(tp, more, tp + W * TILE);
