@@ -703,8 +703,15 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
         const float alpha = m_new == NEG_INF ? 1.f : __expf(m_run[nb] - m_new);
         l_run[nb] *= alpha;
         m_run[nb] = m_new;
+        // With two or more row blocks the accumulators live in AGPRs.  The empty statements pin them there on both
+        // sides of the multiply, so that the VGPR round trip stays inside this rare block instead of being hoisted
+        // into the hot loop (128 register moves a tile).
 #pragma unroll
-        for (int db = 0; db < S::DB; db++) acc[db][nb] *= alpha;
+        for (int db = 0; db < S::DB; db++) {
+          if constexpr (NB > 1) asm volatile("" : "+a"(acc[db][nb]));
+          acc[db][nb] *= alpha;
+          if constexpr (NB > 1) asm volatile("" : "+a"(acc[db][nb]));
+        }
       }
     }
 #pragma unroll

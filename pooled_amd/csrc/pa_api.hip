@@ -285,9 +285,17 @@ static bool plan_self_row(const pa_plan& pl) { return pl.kernel == 0 && pl.slots
 static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, bool self_ok = true, uint32_t* wgs = nullptr) {
   const pa_config& c = ctx->cfg;
   const uint32_t G = c.n_heads / c.n_kv_heads;
-  // rows per workgroup: 16-row blocks whose O^T accumulators still fit the register file next to the
-  // in-flight K/V tile (hd 256: 2 blocks, hd 128: 4 blocks)
-  const uint32_t max_rows = c.head_dim == 256 ? 32 : 64;
+  static const uint32_t floor_tiles[5] = {1, 1, 4, 6, 8};     // tiles per wave, by row blocks
+  // rows per workgroup: 16-row blocks whose O^T accumulators fit the register file next to the
+  // in-flight K/V tile (hd 256: 2 blocks, 3 in the case below; hd 128: 4 blocks)
+  // hd 256: three blocks (48 rows) when that saves a column group and the context is long enough to fill the chip
+  // with splits of the three-block tile floor (27B shape, 8 columns at 64K: one group of 48 rows instead of two)
+  uint32_t max_rows = c.head_dim == 256 ? 32 : 64;
+  if (c.head_dim == 256 && n_cols * G > 32 && 48 / G > 0) {
+    const uint32_t g32 = ceil_div(n_cols, 32 / G), g48 = ceil_div(n_cols, 48 / G);
+    const uint32_t splits48 = ceil_div(base_pos + n_cols, 32) / (floor_tiles[3] * 4);
+    if (g48 < g32 && !ctx->decode_splits_override && (uint64_t)splits48 * c.n_kv_heads * g48 >= (uint64_t)ctx->n_cu) max_rows = 48;
+  }
   uint32_t cw = n_cols, groups = 1;
   if (n_cols * G > max_rows) { cw = max_rows / G; if (cw == 0) return PA_ERR_UNSUPPORTED; groups = ceil_div(n_cols, cw); }
   const uint32_t nb = ceil_div(cw * G, 16);
@@ -298,7 +306,6 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   const uint32_t occ = nb == 1 ? 2 : 1;
   uint32_t target = ctx->decode_splits_override ? ctx->decode_splits_override
                                                 : std::max(1u, (occ * (uint32_t)ctx->n_cu) / (c.n_kv_heads * groups));
-  static const uint32_t floor_tiles[5] = {1, 1, 4, 6, 8};     // tiles per wave, by row blocks
   uint32_t tpw = std::max(ceil_div(tiles, target * W), ctx->decode_splits_override ? 1u : floor_tiles[nb]);
   uint32_t sl = 32 * W * tpw, ns = ceil_div(seq_max, sl);
   // A context a little past target x split_len (a 32K context plus the token being decoded) would double the
