@@ -344,9 +344,12 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
   // (Q staging, one partial per split and row, the merge) amount to.  Measured crossover on the MoE and 27B shapes
   // at 32K - 64K rows: about 1.4 GB of L2-level K/V traffic; below 4096 rows both kernels take 25 - 40 us.
   if (n_cols * G <= 512 && base_pos + n_cols >= 4096 && max_rows_sk >= G) {
-    const uint64_t groups_sk = ceil_div(n_cols, max_rows_sk / G);
+    pa_plan sk; uint32_t sk_wgs = 0;
     const uint64_t kv_bytes = 2ull * (base_pos + n_cols) * c.n_kv_heads * c.head_dim * (kv_q8(ctx) ? 1 : 2);
-    if (groups_sk * kv_bytes <= 1400000000ull) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
+    if (plan_decode(ctx, base_pos, n_cols, &sk, true, &sk_wgs) == PA_OK && (uint64_t)sk.col_groups * kv_bytes <= 1400000000ull) {
+      *pl = sk; if (wgs) *wgs = sk_wgs;
+      return PA_OK;
+    }
   }
   const uint32_t rows_wg = 256;
   const uint32_t cw = rows_wg / G;
