@@ -413,7 +413,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     const uint32_t self_slot = min((seq_max + p.split_len - 1) / p.split_len, p.n_splits);
     const bool on = lane < HD / 4;
     const f4 vxf = { (float)vx[0], (float)vx[1], (float)vx[2], (float)vx[3] };
-#pragma unroll 4
     for (uint32_t r = 0; r < G; r++) {                                 // one column: row r is head g * G + r
       const h4 qv = *(const h4*)(q_lds + r * S::QROW + min(lane, (uint32_t)HD / 4 - 1) * 8);
       float d = 0.f;

@@ -54,7 +54,6 @@ template <int HD, int W> struct PfShape {
 template <int HD, int QB, int W, bool PP>
 __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p, uint32_t n_col_blocks) {
   typedef PfShape<HD, W> S;
-  constexpr int RW = W * QB * 32;                  // query rows per workgroup
   // four separate LDS objects (two K, two V buffers): the compiler then orders an LDS read only after the
   // LDS-direct loads into the *same* buffer, and the prefetch into the other buffer stays in flight
   __shared__ __attribute__((aligned(1024))) unsigned char kbuf0[S::TILE];
@@ -78,7 +77,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   const uint32_t G = p.group, nH = p.n_heads;
   const uint32_t c0 = cb * p.cols_per_group;
   const uint32_t ncl = min(p.cols_per_group, p.n_cols - c0);
-  const uint32_t R = ncl * G;                      // live rows (<= RW)
+  const uint32_t R = ncl * G;                      // live rows (<= W * QB * 32)
   const uint32_t seq_max = p.base_pos + c0 + ncl;  // rows visible to the block's last column
   const uint32_t t_begin = sp * p.split_len;
   if (t_begin >= seq_max) return;
@@ -131,7 +130,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 
   // ---- per-lane rows: query row of block qb is wave*QB*32 + qb*32 + ln = (column r / G, head r % G) ----
   uint32_t end_pos[QB], row_id[QB];
-  uint32_t w_min_end = 0xffffffffu, w_max_end = 0;
+  uint32_t w_min_end = 0xffffffffu;
 #pragma unroll
   for (int qb = 0; qb < QB; qb++) {
     const uint32_t r = wave * QB * 32 + qb * 32 + ln;
@@ -139,8 +138,8 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     end_pos[qb] = r < R ? p.base_pos + c0 + r / G + 1 : 0u;
   }
   {
-    const uint32_t r_first = wave * QB * 32, r_last = min(r_first + QB * 32, R) - 1;
-    if (r_first < R) { w_min_end = p.base_pos + c0 + r_first / G + 1; w_max_end = p.base_pos + c0 + r_last / G + 1; }
+    const uint32_t r_first = wave * QB * 32;
+    if (r_first < R) w_min_end = p.base_pos + c0 + r_first / G + 1;
   }
 
   // ---- Q fragments (B operand of S^T = K Q^T): row ln of block qb, dims 16 ks + 8 hb .. + 7, as f16 ----

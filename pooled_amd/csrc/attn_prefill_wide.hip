@@ -80,7 +80,7 @@ template <int HD, int QR_> struct PwShape {
 template <int HD, int QR_>
 __global__ __launch_bounds__(256, 1) void pa_prefill_wide_kernel(AttnParams p, uint32_t n_col_blocks) {
   typedef PwShape<HD, QR_> S;
-  constexpr int W = S::W, QB = S::QB, QR = S::QR;
+  constexpr int QB = S::QB, QR = S::QR;
   __shared__ __attribute__((aligned(1024))) unsigned char kbuf0[S::TILE];
   __shared__ __attribute__((aligned(1024))) unsigned char kbuf1[S::TILE];
   __shared__ __attribute__((aligned(1024))) unsigned char vbuf0[S::TILE];
