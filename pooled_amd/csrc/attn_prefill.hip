@@ -61,12 +61,16 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   __shared__ __attribute__((aligned(1024))) unsigned char vbuf0[S::TILE];
   __shared__ __attribute__((aligned(1024))) unsigned char vbuf1[S::TILE];
 
-  // ---- XCD-aware id -> (kv head, column block) ----
-  const uint32_t total = n_col_blocks * p.n_kv_heads;
+  // ---- XCD-aware id -> (kv head, split, column block) ----
+  // Work items are (kv head, split, column block), column block fastest: the workgroups of one (kv head, split) read
+  // the same K/V rows.  The grid is one-dimensional; dispatch id i runs on XCD i % 8, and XCD k owns the contiguous
+  // item range [k per_xcd, (k + 1) per_xcd): every XCD gets the same number of workgroups whatever the split count,
+  // and the workgroups that share a K/V stream share an L2.
+  const uint32_t total = n_col_blocks * p.n_kv_heads * p.n_splits;
   const uint32_t per_xcd = (total + 7) / 8;
   const uint32_t lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (lid >= total) return;
-  const uint32_t g = lid / n_col_blocks, cb = lid % n_col_blocks, sp = blockIdx.y;
+  const uint32_t cb = lid % n_col_blocks, sp = (lid / n_col_blocks) % p.n_splits, g = lid / (n_col_blocks * p.n_splits);
 
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform (scalar) so per-wave branches are scalar branches
@@ -456,9 +460,9 @@ static hipError_t launch_prefill_t(const AttnParams& p, uint32_t col_groups, hip
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  const uint32_t total = col_groups * p.n_kv_heads;
+  const uint32_t total = col_groups * p.n_kv_heads * p.n_splits;
   const uint32_t gx = ((total + 7) / 8) * 8;       // whole rounds of the 8 XCDs
-  PA_LAUNCH((pa_prefill_kernel<HD, QB, W, PP>), dim3(gx, p.n_splits), dim3(W * 64), lds, s, t, p, col_groups);
+  PA_LAUNCH((pa_prefill_kernel<HD, QB, W, PP>), dim3(gx), dim3(W * 64), lds, s, t, p, col_groups);
   return hipGetLastError();
 }
 
