@@ -157,7 +157,18 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     if (lin < nf * gridDim.y) { g = lin / nf; sp = lin % nf; }
     else { const uint32_t e = lin - nf * gridDim.y; g = e % gridDim.y; sp = nf + e / gridDim.y; }
   }
-  const uint32_t cg = blockIdx.z;
+  uint32_t cg = blockIdx.z;
+  if constexpr (!SR) {
+    // Tile loop: a one-dimensional grid over (kv head, split, column group) items, column group fastest.  Dispatch
+    // id i runs on XCD i % 8 and XCD k owns the contiguous item range [k per, (k + 1) per): the column groups of a
+    // (kv head, split) read the same K/V rows, so they sit on one XCD, side by side, and share the rows in its L2
+    // whatever the number of splits.
+    const uint32_t ncg = (p.n_cols + p.cols_per_group - 1) / p.cols_per_group;
+    const uint32_t total = p.n_splits * p.n_kv_heads * ncg, per = (total + 7) / 8;
+    const uint32_t item = (blockIdx.x % 8) * per + blockIdx.x / 8;
+    if (item >= total) return;
+    cg = item % ncg; sp = (item / ncg) % p.n_splits; g = item / (ncg * p.n_splits);
+  }
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t ln = lane & 15, kg = lane >> 4;
   const uint32_t G = p.group, nH = p.n_heads;
@@ -980,7 +991,9 @@ static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipS
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), dim3(p.n_splits, p.n_kv_heads, col_groups), dim3(W * 64), lds, s, t, p);
+  if (!SR && col_groups != (p.n_cols + p.cols_per_group - 1) / p.cols_per_group) return hipErrorInvalidValue;
+  const dim3 grid = SR ? dim3(p.n_splits, p.n_kv_heads, col_groups) : dim3((p.n_splits * p.n_kv_heads * col_groups + 7) / 8 * 8);
+  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), grid, dim3(W * 64), lds, s, t, p);
   return hipGetLastError();
 }
 
