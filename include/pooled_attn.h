@@ -66,8 +66,8 @@ typedef struct pa_ctx pa_ctx;
 typedef struct pa_plan {
   uint32_t kernel;       /* 0 = split-K decode/verify kernel, 1 = MFMA prefill kernel */
   uint32_t split_len;    /* cache rows per split */
-  uint32_t n_splits;     /* splits over the streamed rows (grid x); a one-column decode streams rows 0 .. base_pos - 1 */
-  uint32_t col_groups;   /* column groups (grid z) */
+  uint32_t n_splits;     /* splits over the streamed rows; a one-column decode streams rows 0 .. base_pos - 1 */
+  uint32_t col_groups;   /* column groups (workgroups = n_splits x kv heads x col_groups) */
   uint32_t cols_per_group;
   uint32_t waves;        /* wavefronts per workgroup */
   uint32_t row_blocks;   /* 16-row (decode) or 32-row (prefill) query blocks per workgroup */
