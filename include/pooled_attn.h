@@ -276,6 +276,13 @@ int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, c
  * be read against. */
 int pa_mfma_probe(pa_ctx* ctx, int random_operands, uint32_t iters, float* tflops, float* shader_mhz);
 
+/* Device probe (measurement infrastructure, no counterpart in the reference): one workgroup of waves_per_cu (1 .. 8)
+ * wavefronts per CU reads LDS back to back, conflict-free, with ds_read_b128 (transpose_reads = 0) or with the
+ * transpose read ds_read_b64_tr_b16 the V^T fragments use (1), iters x 8 KB per wavefront, and returns the bytes per
+ * shader clock and CU it sustained.  Blocks until done.  It tells how far an attention kernel's fragment traffic is
+ * from what the LDS delivers. */
+int pa_lds_probe(pa_ctx* ctx, int transpose_reads, uint32_t waves_per_cu, uint32_t iters, float* bytes_per_clk);
+
 /* library / device description, e.g. "pooled_attn 0.1 gfx950 256CU" (static storage) */
 const char* pa_version(void);
 

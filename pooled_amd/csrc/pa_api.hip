@@ -915,6 +915,11 @@ extern "C" int pa_mfma_probe(pa_ctx* ctx, int random_operands, uint32_t iters, f
   HIPCHK(ctx, pa_run_mfma_probe(ctx->n_cu, random_operands != 0, iters, ctx->stream, tflops, shader_mhz));
   return PA_OK;
 }
+extern "C" int pa_lds_probe(pa_ctx* ctx, int transpose_reads, uint32_t waves_per_cu, uint32_t iters, float* bytes_per_clk) {
+  if (!ctx || !bytes_per_clk || iters == 0 || waves_per_cu == 0 || waves_per_cu > 8) return PA_ERR_INVALID;
+  HIPCHK(ctx, pa_run_lds_probe(ctx->n_cu, transpose_reads != 0, waves_per_cu, iters, ctx->stream, bytes_per_clk));
+  return PA_OK;
+}
 extern "C" int pa_profile_enable(pa_ctx* ctx, int on) {
   if (!ctx) return PA_ERR_INVALID;
   ctx->profiling = on != 0;
