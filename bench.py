@@ -333,7 +333,7 @@ def main():
         # warm-up long enough for the clock to settle
         pa = PooledAttn(C3, 64, n_layers=1, max_cols=1)
         res = {}
-        for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        for name, rnd in (("constant_operands", 0), ("random_operands", 1), ("random_operands_16x16x32", 2)):
             for _ in range(3):
                 pa.mfma_probe(rnd, 20000)
             tf, mhz = pa.mfma_probe(rnd, 60000)

@@ -270,7 +270,8 @@ int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, c
 
 /* Device probe (measurement infrastructure, no counterpart in the reference): runs back-to-back
  * v_mfma_f32_32x32x16_f16 on every CU for iters x 64 instructions per wavefront, with constant operands
- * (random_operands = 0) or random f16 fragments, and returns the achieved TFLOP/s and the mean shader clock during
+ * (random_operands = 0) or random f16 fragments (1; 2 = the same flops as twice as many v_mfma_f32_16x16x32_f16),
+ * and returns the achieved TFLOP/s and the mean shader clock during
  * the kernel (shader clock counter against the 100 MHz wall clock).  Blocks until done.  It tells what the matrix
  * pipe of this part sustains under its power limit, which is what an MFMA-bound kernel's roofline fraction has to
  * be read against. */

@@ -345,7 +345,7 @@ class PooledAttn:
     def mfma_probe(self, random_operands, iters):
         """(TFLOP/s, shader MHz) of back-to-back f16 MFMAs on every CU with constant or random operands."""
         tf, mhz = ctypes.c_float(), ctypes.c_float()
-        self._chk(self.L.pa_mfma_probe(self.ctx, int(bool(random_operands)), iters, ctypes.byref(tf), ctypes.byref(mhz)))
+        self._chk(self.L.pa_mfma_probe(self.ctx, int(random_operands), iters, ctypes.byref(tf), ctypes.byref(mhz)))
         return tf.value, mhz.value
 
     def lds_probe(self, transpose_reads, waves_per_cu, iters):

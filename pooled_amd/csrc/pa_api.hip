@@ -912,7 +912,7 @@ extern "C" int pa_timer_stop(pa_ctx* ctx, float* ms) {
 }
 extern "C" int pa_mfma_probe(pa_ctx* ctx, int random_operands, uint32_t iters, float* tflops, float* shader_mhz) {
   if (!ctx || !tflops || !shader_mhz || iters == 0) return PA_ERR_INVALID;
-  HIPCHK(ctx, pa_run_mfma_probe(ctx->n_cu, random_operands != 0, iters, ctx->stream, tflops, shader_mhz));
+  HIPCHK(ctx, pa_run_mfma_probe(ctx->n_cu, random_operands != 0, random_operands == 2, iters, ctx->stream, tflops, shader_mhz));
   return PA_OK;
 }
 extern "C" int pa_lds_probe(pa_ctx* ctx, int transpose_reads, uint32_t waves_per_cu, uint32_t iters, float* bytes_per_clk) {

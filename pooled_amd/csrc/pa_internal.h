@@ -114,7 +114,7 @@ hipError_t pa_launch_widen_q8(const void* k8, const void* v8, const float* ks, c
                               uint32_t n_kv_heads, uint32_t hd, uint32_t head_rows, uint32_t n_live, uint32_t n_rows, hipStream_t s);
 
 // device probe (probe.hip): sustained f16 MFMA rate and shader clock, constant or random operands
-hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, uint32_t iters, hipStream_t st, float* tflops, float* shader_mhz);
+hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, bool small_tiles, uint32_t iters, hipStream_t st, float* tflops, float* shader_mhz);
 hipError_t pa_run_lds_probe(int n_cu, bool transpose_reads, uint32_t waves, uint32_t iters, hipStream_t st, float* bytes_per_clk);
 
 // ---- context -----------------------------------------------------------------------------------

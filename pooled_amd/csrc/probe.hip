@@ -15,33 +15,54 @@ typedef __fp16 probe_hh4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
+typedef float probe_f4 __attribute__((ext_vector_type(4)));
+
+// SMALL = false: v_mfma_f32_32x32x16_f16 on 8 accumulators; true: v_mfma_f32_16x16x32_f16 on 16 accumulators.  Both issue
+// 64 x 32768 flops per wavefront and iteration.
+template <bool SMALL>
 __global__ __launch_bounds__(256) void pa_mfma_probe_kernel(const h8* frag, float* sink, unsigned long long* clk, uint32_t iters) {
   const long long c0 = clock64(), w0 = wall_clock64();
   h8 a[8], b[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) { a[i] = frag[i * 256 + threadIdx.x]; b[i] = frag[(8 + i) * 256 + threadIdx.x]; }
-  f16v acc[8];
-#pragma unroll
-  for (int k = 0; k < 8; k++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) acc[k][i] = 0.f;
-  for (uint32_t it = 0; it < iters; it++) {
-#pragma unroll
-    for (int u = 0; u < 8; u++)
-#pragma unroll
-      for (int k = 0; k < 8; k++) acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[(u + k) & 7], b[k], acc[k], 0, 0, 0);
-  }
   float s = 0.f;
+  if constexpr (!SMALL) {
+    f16v acc[8];
 #pragma unroll
-  for (int k = 0; k < 8; k++)
+    for (int k = 0; k < 8; k++)
 #pragma unroll
-    for (int i = 0; i < 16; i++) s += acc[k][i];
+      for (int i = 0; i < 16; i++) acc[k][i] = 0.f;
+    for (uint32_t it = 0; it < iters; it++) {
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+#pragma unroll
+        for (int k = 0; k < 8; k++) acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[(u + k) & 7], b[k], acc[k], 0, 0, 0);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; k++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) s += acc[k][i];
+  } else {
+    probe_f4 acc[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) acc[k] = (probe_f4){0.f, 0.f, 0.f, 0.f};
+    for (uint32_t it = 0; it < iters; it++) {
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+#pragma unroll
+        for (int k = 0; k < 16; k++) acc[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(u + k) & 7], b[k & 7], acc[k], 0, 0, 0);
+    }
+#pragma unroll
+    for (int k = 0; k < 16; k++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) s += acc[k][i];
+  }
   sink[blockIdx.x * 256 + threadIdx.x] = s;
   if (threadIdx.x == 0) { clk[blockIdx.x * 2] = clock64() - c0; clk[blockIdx.x * 2 + 1] = wall_clock64() - w0; }
 }
 
 // blocks = 2 per CU (8 wavefronts per CU); 64 MFMAs of 32768 flops per wavefront and iteration
-hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, uint32_t iters, hipStream_t st, float* tflops, float* shader_mhz) {
+hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, bool small_tiles, uint32_t iters, hipStream_t st, float* tflops, float* shader_mhz) {
   const uint32_t blocks = 2 * (uint32_t)n_cu;
   std::vector<_Float16> h(16 * 256 * 8);
   uint32_t lcg = 12345u;
@@ -55,7 +76,8 @@ hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, uint32_t iters, hip
   if ((e = hipMalloc((void**)&clk, (size_t)blocks * 16)) != hipSuccess) return done(e);
   if ((e = hipMemcpy(frag, h.data(), h.size() * 2, hipMemcpyHostToDevice)) != hipSuccess) return done(e);
   if ((e = hipEventCreate(&e0)) != hipSuccess || (e = hipEventCreate(&e1)) != hipSuccess) return done(e);
-  hipExtLaunchKernelGGL(pa_mfma_probe_kernel, dim3(blocks), dim3(256), 0, st, e0, e1, 0, (const h8*)frag, sink, clk, iters);
+  if (small_tiles) hipExtLaunchKernelGGL(pa_mfma_probe_kernel<true>, dim3(blocks), dim3(256), 0, st, e0, e1, 0, (const h8*)frag, sink, clk, iters);
+  else hipExtLaunchKernelGGL(pa_mfma_probe_kernel<false>, dim3(blocks), dim3(256), 0, st, e0, e1, 0, (const h8*)frag, sink, clk, iters);
   if ((e = hipGetLastError()) != hipSuccess) return done(e);
   if ((e = hipEventSynchronize(e1)) != hipSuccess) return done(e);
   float ms = 0.f;

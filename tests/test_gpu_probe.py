@@ -8,8 +8,9 @@ pytestmark = pytest.mark.gpu
 
 def test_mfma_and_lds_probe():
     with PooledAttn(SHAPES["qwen36_moe"], 64, n_layers=1, max_cols=1) as pa:
-        tf, mhz = pa.mfma_probe(1, 2000)
-        assert 500.0 < tf < 2600.0 and 500.0 < mhz < 3000.0, (tf, mhz)
+        for mode in (1, 2):                                             # random operands: 32x32x16 tiles, 16x16x32 tiles
+            tf, mhz = pa.mfma_probe(mode, 2000)
+            assert 500.0 < tf < 2600.0 and 500.0 < mhz < 3000.0, (mode, tf, mhz)
         for tr in (0, 1):
             for waves in (4, 8):
                 bpc = pa.lds_probe(tr, waves, 2000)
