@@ -83,6 +83,7 @@ hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);
 hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
 // the 4-wave, 64-rows-per-wave software-pipelined variant (same contract)
 hipError_t pa_launch_prefill_wide(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
+hipError_t pa_launch_prefill_small(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
 
 // one-token projection y = W x (proj_gemv.hip): kind PA_W_*, w = f32 [d_out][d_in] / int8 [d_out][d_in] / nibbles
 // [d_out][d_in / 2], scales = f16 bits [d_out][d_in / 32] (quantised kinds); norm_w != nullptr: x is the raw vector and

@@ -99,6 +99,20 @@ def test_prefill_wide_variant(shape, base, n, k_scale, monkeypatch):
     assert_parity(got, ref, "wide %s base %d n %d" % (shape, base, n))
 
 
+@pytest.mark.parametrize("shape,base,n,k_scale", [
+    ("qwen36_moe", 301, 16, 1.0), ("qwen36_moe", 1000, 200, 1.0), ("qwen3_1p7b", 219, 257, 1.0),
+    ("qwen38_27b", 500, 96, 3.0), ("qwen36_moe", 20000, 80, 1.0),
+])
+def test_prefill_small_tile_variant(shape, base, n, k_scale, monkeypatch):
+    """The variant of the prefill kernel on the 16 x 16 x 32 matrix instruction (the default only for wide chunks of
+    hd 256 over long contexts; forced here by the environment variable read at each call): same parity bar, including
+    the rescale path (peaked scores), the split path and hd 128."""
+    monkeypatch.setenv("POOLED_ATTN_PREFILL_SMALL", "1")
+    got, ref, plan = _prefill(SHAPES[shape], base, n, seed=base + n + 2, k_scale=k_scale)
+    assert plan["kernel"] == 1
+    assert_parity(got, ref, "small tile %s base %d n %d" % (shape, base, n))
+
+
 def test_c2_prefill_full():
     """Config 2: 512-token chunk at positions 1536-2047 over a 1536-token prefix, Qwen3-1.7B shape, pre-step on
     the GPU (QK-RMSNorm + full RoPE theta 1e6 + KV write for the chunk), f16 output."""
