@@ -4,8 +4,9 @@
 // and outputs as pa_prefill_kernel (attn_prefill.hip; it replaces the same reference kernels:
 // engine/wgsl/attn_tile.js:108-193, engine/wgsl/qwen35.js:877-887).  What differs is the matrix instruction: the
 // products run on v_mfma_f32_16x16x32_f16 instead of v_mfma_f32_32x32x16_f16.  Under the power limit of the part the
-// small shape sustains 7-8 % more flops (it spends less energy per flop; see the device probe in probe.hip), and the
-// prefill kernel is bound by exactly that limit.
+// small shape sustains 7-8 % more flops in a kernel of nothing but MFMAs (see the device probe in probe.hip); in this
+// kernel that does not show -- it runs level with pa_prefill_kernel on the MoE shape at 128K rows and behind it on
+// the other shapes -- so it is a measured alternative, selected by POOLED_ATTN_PREFILL_SMALL=1, not a default.
 //
 // A wavefront still owns 32 query rows, now as two 16-row blocks, and a step still covers 32 positions, as two
 // 16-position blocks:

@@ -411,12 +411,12 @@ static int prof_pair(pa_ctx* ctx, PaTiming* t) {
 // POOLED_ATTN_PREFILL_WIDE selects the 4-wave prefill kernel for measurements; read at every call (a getenv is
 // nothing next to a kernel launch) so that a test can switch it inside one process
 static bool prefill_wide_selected() { return getenv("POOLED_ATTN_PREFILL_WIDE") != nullptr; }
-// The small-MFMA-tile prefill kernel (attn_prefill_small.hip) spends less energy per flop and wins where the chip sits
-// at its power limit for the length of the launch: wide, unsplit chunks of hd 256 over long contexts (C5: 2.5 % faster;
-// 4096 columns at 12K rows, a 1 ms launch: 3.5 % slower).  POOLED_ATTN_PREFILL_SMALL=1 / =0 forces either kernel.
-static bool prefill_small_selected(const pa_config& c, const pa_plan& pl, uint32_t base_pos, uint32_t n_cols) {
-  if (const char* e = getenv("POOLED_ATTN_PREFILL_SMALL")) return atoi(e) != 0;
-  return c.head_dim == 256 && pl.n_splits == 1 && (uint64_t)base_pos + n_cols >= 65536;
+// POOLED_ATTN_PREFILL_SMALL=1 selects the prefill kernel on the 16 x 16 x 32 matrix instruction (attn_prefill_small.hip)
+// for measurements.  Interleaved A/B runs put it level with the 32 x 32 x 16 kernel on C5 and behind it on the other
+// shapes, so the plan never picks it by itself.
+static bool prefill_small_selected() {
+  const char* e = getenv("POOLED_ATTN_PREFILL_SMALL");
+  return e != nullptr && atoi(e) != 0;
 }
 
 static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, const float* d_q, uint32_t q_stride,
@@ -477,7 +477,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   if ((rc = prof_pair(ctx, &tm))) return rc;
   if (pl.kernel == 0) HIPCHK(ctx, pa_launch_decode(p, c.head_dim, pl.row_blocks, pl.waves, pl.col_groups, ctx->stream, &tm));
   else if (prefill_wide_selected()) HIPCHK(ctx, pa_launch_prefill_wide(p, c.head_dim, pl.col_groups, ctx->stream, &tm));
-  else if (prefill_small_selected(c, pl, base_pos, n_cols)) HIPCHK(ctx, pa_launch_prefill_small(p, c.head_dim, pl.col_groups, ctx->stream, &tm));
+  else if (prefill_small_selected()) HIPCHK(ctx, pa_launch_prefill_small(p, c.head_dim, pl.col_groups, ctx->stream, &tm));
   else HIPCHK(ctx, pa_launch_prefill(p, c.head_dim, pl.row_blocks, pl.col_groups, ctx->stream, &tm));
   if (!direct) HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;

@@ -104,9 +104,8 @@ def test_prefill_wide_variant(shape, base, n, k_scale, monkeypatch):
     ("qwen38_27b", 500, 96, 3.0), ("qwen36_moe", 20000, 80, 1.0),
 ])
 def test_prefill_small_tile_variant(shape, base, n, k_scale, monkeypatch):
-    """The variant of the prefill kernel on the 16 x 16 x 32 matrix instruction (the default only for wide chunks of
-    hd 256 over long contexts; forced here by the environment variable read at each call): same parity bar, including
-    the rescale path (peaked scores), the split path and hd 128."""
+    """The variant of the prefill kernel on the 16 x 16 x 32 matrix instruction (selected by an environment variable
+    read at each call): same parity bar, including the rescale path (peaked scores), the split path and hd 128."""
     monkeypatch.setenv("POOLED_ATTN_PREFILL_SMALL", "1")
     got, ref, plan = _prefill(SHAPES[shape], base, n, seed=base + n + 2, k_scale=k_scale)
     assert plan["kernel"] == 1
