@@ -39,6 +39,13 @@ extern "C" {
                                  context allocates on first use (one layer's f16 cache in size) and runs the
                                  matrix-core prefill kernel on it. */
 
+#define PA_FLAG_VERIFY_EXACT 8u /* pa_attn_decode with n_cols > 1 runs every column as the one-column decode at its own position
+                                 (its own splits, its own row block): column c then has the bits of pa_attn_decode(base_pos + c,
+                                 n_cols = 1), the invariant the reference states for its pair (engine/wgsl/attn_dec.js:12-16,
+                                 tests/test_attn_dec.js:89-97) and its speculative decoding leans on (spec greedy == plain
+                                 greedy).  Cost: the K/V stream is read once per column, as the reference does, instead of
+                                 once per block.  Off by default: see the note at pa_attn_decode. */
+
 /* output element types */
 #define PA_OUT_F32 0          /* the engine's attnOut feeding wo (engine/qwen35.js:881) */
 #define PA_OUT_F16 1
@@ -132,6 +139,12 @@ float* pa_gate_buffer(pa_ctx* ctx);
  * engine/wgsl/qwen35.js:406-416, :877-887) and the v1 pair attn_flash + attn_combine(_g)
  * (engine/wgsl/qwen35.js:99-197, :1059-1080, engine/wgsl/layer_fuse.js:148-181).
  * Call sites: engine/qwen35.js:1618-1640 (one token), :2494-2516 (verify columns).
+ * A verify column is NOT bit-identical to the one-column decode at the same position unless PA_FLAG_VERIFY_EXACT is set:
+ * the columns of a block are stacked into shared matrix-core tiles and the block's splits are chosen from the block,
+ * while a one-column decode streams whole 128-row splits and keeps its own row as a separate partial, so the two sum
+ * in different orders.  They agree to rounding (the tests bound |block - sequential| by 1e-3; measured 3e-4), which
+ * is inside the path's tolerance but weaker than the reference's own guarantee (engine/wgsl/attn_dec.js:12-16): an
+ * engine that needs speculative greedy decoding to reproduce plain greedy decoding token for token sets the flag.
  *   d_q   : f32 [n_cols][q_stride], a column holds roped q [nH][hd]; NULL = pa_q_buffer
  *   d_gate: f32 [n_cols][gate_stride] gate pre-activations [nH][hd]; NULL = no gate
  *   d_out : [n_cols][out_stride] of out_dtype, a column holds [nH][hd]
@@ -158,12 +171,25 @@ int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_st
  * pa_q_buffer / pa_gate_buffer are not written by this call. */
 int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
                         const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype);
+/* pa_attn_decode_step_noalloc: pa_attn_decode_step for callers that cannot allocate.  No counterpart in the reference;
+ * it exists for callers under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same
+ * arguments, same kernels and the same bits as pa_attn_decode_step, but the split partials go to a file-scope device
+ * array of the library (8 MiB per GPU, held until the process ends; its device address is looked up at pa_create) and
+ * the call makes no hipMalloc / hipFree and creates no events (pa_profile_enable does not see it).  A shape whose
+ * partials -- n_heads x (splits + 1) x (head_dim + 2) floats -- do not fit returns PA_ERR_UNSUPPORTED (the MoE shape
+ * at 32K uses 4.3 MB).  All calls on one GPU share the array, contexts included: calls that overlap on one GPU (two
+ * streams, two contexts) race; calls queued on one stream do not.  Nothing in the array needs clearing between calls:
+ * every partial the merge reads is written by the same call. */
+int pa_attn_decode_step_noalloc(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
+                                const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype);
 /* pa_attn_decode_gather: decode / verify attention where every column attends to a list of cache rows instead of
  * rows [0, base_pos + c] -- the gather mode of the reference's split-K kernel used by its sparse-attention layers:
  * attn_dec_qsa + attn_dec_qsa_combine(_g) (engine/wgsl/attn_dec.js:33-38, :105, :170-183, :246; dispatch
  * engine/qsa.js:41-56).  Same q / gate / out contract as pa_attn_decode.
- *   d_sel: u32 [n_cols][sel_stride]; column c's list is d_sel[c * sel_stride] = n (1 <= n <= max_rows), then n row
- *          indices < max_seq at d_sel[c * sel_stride + 1 ..], ascending (the reference's QSA_SEL_STRIDE layout)
+ *   d_sel: u32 [n_cols][sel_stride]; column c's list is d_sel[c * sel_stride] = n (0 <= n <= max_rows), then n row
+ *          indices < max_seq at d_sel[c * sel_stride + 1 ..], ascending (the reference's QSA_SEL_STRIDE layout).  The
+ *          device-side length word is not trusted: n > max_rows is read as max_rows (a list never runs into the next
+ *          column's), row indices are clamped to the cache, and n == 0 gives a column of zeros.
  *   max_rows: the longest list of the pass (engine/qsa.js:34 qsaMaxRows); sizes the splits
  * List position t stands where position t stands in pa_attn_decode: with the list 0 .. pos a single column gives
  * pa_attn_decode's result at base_pos = pos to rounding (2e-5; the dense call keeps the column's own row out of the
@@ -184,6 +210,10 @@ int pa_set_decode_splits(pa_ctx* ctx, uint32_t splits);
  *      (the reference's kCache / vCache / kScale / vScale parts, engine/qwen35.js:121-131) */
 int pa_kv_read(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, void* h_dst);
 int pa_kv_write(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, const void* h_src);
+/* bytes of one row of the host view of cache tensor `which` (nKV * hd f16 / int8 values, or nKV * hd / 32 f32 scales):
+ * what pa_kv_read / pa_kv_write move per row and pa_slot_export / pa_slot_import per saved position -- the part sizes of
+ * the reference's saved states (engine/qwen35.js:121-131).  0 for a tensor the context does not have. */
+size_t pa_kv_row_bytes(const pa_ctx* ctx, int which);
 /* device address of a cache (read-only use; the head-major device layout described at pa_layer_alloc) */
 const void* pa_kv_device_ptr(pa_ctx* ctx, uint32_t layer, int which);
 
@@ -284,7 +314,8 @@ int pa_mfma_probe(pa_ctx* ctx, int random_operands, uint32_t iters, float* tflop
  * from what the LDS delivers. */
 int pa_lds_probe(pa_ctx* ctx, int transpose_reads, uint32_t waves_per_cu, uint32_t iters, float* bytes_per_clk);
 
-/* library / device description, e.g. "pooled_attn 0.1 gfx950 256CU" (static storage) */
+/* library / device description, e.g. "pooled_attn 0.1 gfx950 256CU" (storage owned by the library, one buffer per
+ * calling thread) */
 const char* pa_version(void);
 
 #ifdef __cplusplus

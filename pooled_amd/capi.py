@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libpooled_attn.so")
 
 PA_OK, PA_ERR_INVALID, PA_ERR_UNSUPPORTED, PA_ERR_HIP, PA_ERR_NOMEM = 0, 1, 2, 3, 4
-PA_FLAG_QK_NORM, PA_FLAG_GATE, PA_FLAG_KV_Q8 = 1, 2, 4
+PA_FLAG_QK_NORM, PA_FLAG_GATE, PA_FLAG_KV_Q8, PA_FLAG_VERIFY_EXACT = 1, 2, 4, 8
 PA_W_F32, PA_W_Q8_0, PA_W_Q4_0 = 0, 1, 2
 PA_OUT_F32, PA_OUT_F16 = 0, 1
 
@@ -52,10 +52,12 @@ SYMBOLS = {
     "pa_attn_prefill": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32, vp, u32, c_int]),
     "pa_attn_decode_gather": (c_int, [vp, u32, f32p, u32, f32p, u32, vp, u32, u32, u32, vp, u32, c_int]),
     "pa_attn_decode_step": (c_int, [vp, u32, f32p, f32p, f32p, f32p, f32p, u32, vp, c_int]),
+    "pa_attn_decode_step_noalloc": (c_int, [vp, u32, f32p, f32p, f32p, f32p, f32p, u32, vp, c_int]),
     "pa_plan_query": (c_int, [vp, c_int, u32, u32, ctypes.POINTER(PaPlan)]),
     "pa_set_decode_splits": (c_int, [vp, u32]),
     "pa_kv_read": (c_int, [vp, u32, c_int, u32, u32, vp]),
     "pa_kv_write": (c_int, [vp, u32, c_int, u32, u32, vp]),
+    "pa_kv_row_bytes": (ctypes.c_size_t, [vp, c_int]),
     "pa_kv_device_ptr": (vp, [vp, u32, c_int]),
     "pa_timer_start": (c_int, [vp]),
     "pa_timer_stop": (c_int, [vp, ctypes.POINTER(ctypes.c_float)]),
@@ -132,13 +134,13 @@ class DeviceBuffer:
 
 
 class PooledAttn:
-    """One pa_ctx.  cfg keys: n_heads, n_kv_heads, head_dim, n_rot, rope_theta, eps, qk_norm, gate, kv_q8."""
+    """One pa_ctx.  cfg keys: n_heads, n_kv_heads, head_dim, n_rot, rope_theta, eps, qk_norm, gate, kv_q8, verify_exact."""
 
     def __init__(self, cfg, max_seq, n_layers=1, max_cols=16):
         self.L = load()
         self.cfg = dict(cfg)
         flags = ((PA_FLAG_QK_NORM if cfg.get("qk_norm", True) else 0) | (PA_FLAG_GATE if cfg.get("gate", False) else 0)
-                 | (PA_FLAG_KV_Q8 if cfg.get("kv_q8", False) else 0))
+                 | (PA_FLAG_KV_Q8 if cfg.get("kv_q8", False) else 0) | (PA_FLAG_VERIFY_EXACT if cfg.get("verify_exact", False) else 0))
         c = PaConfig(cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["n_rot"], cfg["rope_theta"], cfg["eps"],
                      max_seq, n_layers, max_cols, flags)
         h = vp()
@@ -231,8 +233,9 @@ class PooledAttn:
         gp = d_gate if isinstance(d_gate, (int, type(None))) else d_gate.ptr
         self._chk(fn(self.ctx, layer, qp, q_stride, gp, gate_stride, base_pos, n_cols, d_out.ptr, out_stride, out_dtype))
 
-    def attn_decode_step(self, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype=PA_OUT_F32):
-        self._chk(self.L.pa_attn_decode_step(self.ctx, layer, d_q_in.ptr, d_k.ptr, d_v.ptr, d_qw.ptr if d_qw else None,
+    def attn_decode_step(self, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype=PA_OUT_F32, noalloc=False):
+        fn = self.L.pa_attn_decode_step_noalloc if noalloc else self.L.pa_attn_decode_step
+        self._chk(fn(self.ctx, layer, d_q_in.ptr, d_k.ptr, d_v.ptr, d_qw.ptr if d_qw else None,
                                              d_kw.ptr if d_kw else None, pos, d_out.ptr, out_dtype))
 
     def q_buffer_ptr(self):

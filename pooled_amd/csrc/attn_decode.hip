@@ -178,7 +178,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   const uint32_t sel_base = GATHER ? c0 * p.sel_stride + 1 : 0;      // gather: first list entry of this column
   // rows visible to the group's last column (gather: the column's list length)
   // self_row (one-column decode): the column's own row base_pos is not streamed with the others -- see below
-  const uint32_t seq_max = GATHER ? p.sel[c0 * p.sel_stride] : p.base_pos + c0 + ncl - p.self_row;
+  const uint32_t seq_max = GATHER ? min(p.sel[c0 * p.sel_stride], p.sel_max) : p.base_pos + c0 + ncl - p.self_row;
   const uint32_t t_begin = sp * p.split_len;
   // The workgroup of split 0 turns the column's own row into a partial of its own (wave 0, while the tile loads are
   // in flight), so it runs even when no other row exists (base_pos == 0).
@@ -863,7 +863,7 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
   __shared__ float red[256];
   __shared__ f4 ored[256];
   const uint32_t h = blockIdx.x / CQ, dq = blockIdx.x % CQ, col = blockIdx.y, tid = threadIdx.x;
-  const uint32_t col_end = p.sel ? p.sel[col * p.sel_stride] : p.base_pos + col + 1 - p.self_row;   // gather: the column's list length
+  const uint32_t col_end = p.sel ? min(p.sel[col * p.sel_stride], p.sel_max) : p.base_pos + col + 1 - p.self_row;   // gather: the column's list length
   // the last split is open-ended; a one-column decode's own row is one more partial after the splits that hold rows
   const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
@@ -928,7 +928,7 @@ __global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
     f4 t = ored[tid];
 #pragma unroll
     for (int i = 1; i < 16; i++) t += ored[i * 16 + tid];
-    f4 r = t / L;
+    f4 r = ns ? t / L : zero;                      // an empty gather list: a column of zeros
     const uint32_t d = d_out;
     if (p.gate) {
 #pragma unroll
@@ -953,7 +953,7 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
   const size_t ch = e / (HD / 4);
   if (ch >= (size_t)p.n_cols * p.n_heads) return;
   const uint32_t col = (uint32_t)(ch / p.n_heads), h = (uint32_t)(ch % p.n_heads);
-  const uint32_t col_end = p.sel ? p.sel[col * p.sel_stride] : p.base_pos + col + 1 - p.self_row;
+  const uint32_t col_end = p.sel ? min(p.sel[col * p.sel_stride], p.sel_max) : p.base_pos + col + 1 - p.self_row;
   const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
   const size_t base = ch * p.slots;
   const float* po = p.part_o + base * HD + 4 * d4;
@@ -966,7 +966,7 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
     L += p.part_ml[(base + s) * 2 + 1] * w;
     o += *(const f4*)(po + (size_t)s * HD) * w;
   }
-  f4 r = o / L;
+  f4 r = ns ? o / L : (f4){0.f, 0.f, 0.f, 0.f};
   const uint32_t d = 4 * d4;
   if (p.gate) {
     const f4 gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d);
@@ -981,16 +981,31 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
   }
 }
 
-template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
-static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
+template <int HD, int NB, int W>
+static constexpr size_t decode_lds_bytes() {
   typedef DecShape<HD> S;
-  const size_t lds = 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float);
+  return 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float);
+}
+// the kernel's dynamic LDS limit, raised once per instantiation (at its first launch, or ahead of it by
+// pa_prepare_decode_step)
+template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
+static hipError_t decode_lds_attr() {
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)decode_lds_bytes<HD, NB, W>());
     if (e != hipSuccess) return e;
     attr_set = true;
   }
+  return hipSuccess;
+}
+
+template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
+static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
+  typedef DecShape<HD> S;
+  const size_t lds = decode_lds_bytes<HD, NB, W>();
+  hipError_t e = decode_lds_attr<HD, NB, W, FUSED, GATHER, Q8, SR>();
+  if (e != hipSuccess) return e;
   if (!SR && col_groups != (p.n_cols + p.cols_per_group - 1) / p.cols_per_group) return hipErrorInvalidValue;
   const dim3 grid = SR ? dim3(p.n_splits, p.n_kv_heads, col_groups) : dim3((p.n_splits * p.n_kv_heads * col_groups + 7) / 8 * 8);
   PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), grid, dim3(W * 64), lds, s, t, p);
@@ -1043,6 +1058,19 @@ hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s
   if (hd == 256) return launch_decode_t<256, 1, 4, true>(p, 1, s, t);
   if (hd == 128) return launch_decode_t<128, 1, 4, true>(p, 1, s, t);
   return hipErrorInvalidValue;
+}
+
+// one-time set-up of the fused step's kernels (both split shapes), so that a later launch makes no other runtime call
+hipError_t pa_prepare_decode_step(uint32_t hd, bool q8) {
+  hipError_t e = hipErrorInvalidValue;
+  if (hd == 256) {
+    e = q8 ? decode_lds_attr<256, 1, 4, true, false, true, true>() : decode_lds_attr<256, 1, 4, true, false, false, true>();
+    if (e == hipSuccess) e = q8 ? decode_lds_attr<256, 1, 4, true, false, true, false>() : decode_lds_attr<256, 1, 4, true, false, false, false>();
+  } else if (hd == 128) {
+    e = q8 ? decode_lds_attr<128, 1, 4, true, false, true, true>() : decode_lds_attr<128, 1, 4, true, false, false, true>();
+    if (e == hipSuccess) e = q8 ? decode_lds_attr<128, 1, 4, true, false, true, false>() : decode_lds_attr<128, 1, 4, true, false, false, false>();
+  }
+  return e;
 }
 
 hipError_t pa_launch_decode_gather(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t) {

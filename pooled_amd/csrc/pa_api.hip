@@ -4,9 +4,21 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 static thread_local std::string g_create_err;
+
+// Scratch of the allocation-free entry point pa_attn_decode_step_noalloc: the split partials of one decode token live
+// in this file-scope device array instead of a buffer the context allocates.  Every GPU the library runs on holds
+// its own copy until the process ends.  Host code never uses the array's name as an address: pa_create looks the
+// device address up once per device (hipGetSymbolAddress with that device current) and everything -- kernel
+// arguments included -- goes through that pointer.
+#define PA_STATIC_SCRATCH_BYTES (8u << 20)
+#define PA_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[PA_STATIC_SCRATCH_BYTES];
+static void* g_scratch_ptr[PA_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
 
 static int fail(pa_ctx* ctx, int code, const std::string& msg) {
   if (ctx) ctx->err = msg; else g_create_err = msg;
@@ -18,9 +30,10 @@ static int fail_hip(pa_ctx* ctx, hipError_t e, const char* what) {
 #define HIPCHK(ctx, call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return fail_hip(ctx, e_, #call); } while (0)
 
 static inline uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+static int ensure_partials(pa_ctx* ctx, uint32_t n_cols, uint32_t slots);
 
 extern "C" const char* pa_version(void) {
-  static char buf[128];
+  static thread_local char buf[128];
   int dev = 0, cus = 0;
   hipDeviceProp_t pr;
   if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&pr, dev) == hipSuccess) {
@@ -66,6 +79,18 @@ extern "C" int pa_create(const pa_config* cfg, pa_ctx** out) {
     delete ctx; return fail(nullptr, PA_ERR_UNSUPPORTED, m);
   }
   ctx->n_cu = pr.multiProcessorCount;
+  if (ctx->device < 0 || ctx->device >= PA_MAX_DEVICES) { delete ctx; return fail(nullptr, PA_ERR_UNSUPPORTED, "pa_create: device ordinal beyond the library's table"); }
+  {
+    // this device's address of the static scratch array (the device is current: hipGetDevice above)
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[ctx->device]) {
+      void* ptr = nullptr;
+      if ((e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) != hipSuccess || !ptr) { delete ctx; return fail_hip(nullptr, e, "pa_create: hipGetSymbolAddress(scratch)"); }
+      g_scratch_ptr[ctx->device] = ptr;
+    }
+    ctx->static_scratch = g_scratch_ptr[ctx->device];
+  }
+  if ((e = pa_prepare_decode_step(c.head_dim, (c.flags & PA_FLAG_KV_Q8) != 0)) != hipSuccess) { delete ctx; return fail_hip(nullptr, e, "pa_create: kernel set-up"); }
   const size_t qbytes = (size_t)c.max_cols * c.n_heads * c.head_dim * sizeof(float);
   std::vector<float> freq(c.n_rot / 2);
   for (uint32_t i = 0; i < c.n_rot / 2; i++) freq[i] = (float)std::pow((double)c.rope_theta, -(2.0 * i) / (double)c.n_rot);
@@ -85,6 +110,13 @@ extern "C" int pa_create(const pa_config* cfg, pa_ctx** out) {
       && (e = pa_launch_rope_table(ctx->rope_tab, ctx->inv_freq, c.n_rot / 2, c.max_seq, ctx->stream)) == hipSuccess
       && (e = hipStreamSynchronize(ctx->stream)) == hipSuccess;
     if (!ok) { int rc = fail_hip(nullptr, e, "pa_create: rope table"); pa_destroy(ctx); return rc; }
+  }
+  // split partials for a one-column decode at any position: at most two workgroup slots a CU, an eighth more for the
+  // remainder splits, the column's own row (wider passes and split overrides grow the buffers on first use)
+  {
+    const uint32_t slots = (2u * (uint32_t)ctx->n_cu / c.n_kv_heads + 1) * 9 / 8 + 2;
+    int rc = ensure_partials(ctx, 1, slots);
+    if (rc) { g_create_err = ctx->err; pa_destroy(ctx); return rc; }
   }
   *out = ctx;
   return PA_OK;
@@ -116,6 +148,7 @@ extern "C" int pa_destroy(pa_ctx* ctx) {
   if (ctx->chunk_buf) (void)hipFree(ctx->chunk_buf);
   if (ctx->wide_k) (void)hipFree(ctx->wide_k);
   if (ctx->wide_v) (void)hipFree(ctx->wide_v);
+  for (void* r : ctx->retired) (void)hipFree(r);
   for (auto ev : ctx->prof_events) (void)hipEventDestroy(ev);
   if (ctx->t0) (void)hipEventDestroy(ctx->t0);
   if (ctx->t1) (void)hipEventDestroy(ctx->t1);
@@ -377,23 +410,27 @@ extern "C" int pa_set_decode_splits(pa_ctx* ctx, uint32_t splits) {
 
 // ---- attention ----------------------------------------------------------------------------------
 
+// Context scratch (split partials, projection and chunk buffers, the int8 staging cache) grows on demand and is never
+// freed or moved while the context lives: launches recorded into a HIP graph by the caller carry the address they
+// were recorded with, and a later, larger pass must not pull that memory from under a replay.  The outgrown block is
+// kept until pa_destroy.  (Growth itself allocates, so a pass that grows a buffer cannot be captured; one eager call
+// of the same or a larger shape before the capture is enough.)
+static int grow_scratch(pa_ctx* ctx, void** buf, size_t* have, size_t need) {
+  if (need <= *have) return PA_OK;
+  void* mem = nullptr;
+  HIPCHK(ctx, hipMalloc(&mem, need));
+  if (*buf) ctx->retired.push_back(*buf);
+  *buf = mem; *have = need;
+  return PA_OK;
+}
+
 static int ensure_partials(pa_ctx* ctx, uint32_t n_cols, uint32_t slots) {
   const pa_config& c = ctx->cfg;
   const size_t need_o = (size_t)n_cols * c.n_heads * slots * c.head_dim * sizeof(float);
   const size_t need_ml = (size_t)n_cols * c.n_heads * slots * 2 * sizeof(float);
-  if (need_o > ctx->part_o_bytes) {
-    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->part_o) { HIPCHK(ctx, hipFree(ctx->part_o)); ctx->part_o = nullptr; ctx->part_o_bytes = 0; }
-    HIPCHK(ctx, hipMalloc((void**)&ctx->part_o, need_o));
-    ctx->part_o_bytes = need_o;
-  }
-  if (need_ml > ctx->part_ml_bytes) {
-    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->part_ml) { HIPCHK(ctx, hipFree(ctx->part_ml)); ctx->part_ml = nullptr; ctx->part_ml_bytes = 0; }
-    HIPCHK(ctx, hipMalloc((void**)&ctx->part_ml, need_ml));
-    ctx->part_ml_bytes = need_ml;
-  }
-  return PA_OK;
+  int rc = grow_scratch(ctx, (void**)&ctx->part_o, &ctx->part_o_bytes, need_o);
+  if (rc) return rc;
+  return grow_scratch(ctx, (void**)&ctx->part_ml, &ctx->part_ml_bytes, need_ml);
 }
 
 // an event pair for a kernel-exact timing of the next main-kernel launch (profiling on), else an empty PaTiming
@@ -434,6 +471,17 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
     return fail(ctx, PA_ERR_INVALID, std::string(who) + ": column stride shorter than a column");
   if ((q_stride & 3) || (out_stride & 3) || (d_gate && (gate_stride & 3)) || ((uintptr_t)d_q & 15) || ((uintptr_t)d_out & 15) || ((uintptr_t)d_gate & 15))
     return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned with strides a multiple of 4 elements");
+  if (kind == 0 && n_cols > 1 && (c.flags & PA_FLAG_VERIFY_EXACT)) {
+    // column-exact verify: every column is the one-column decode at its own position (its own splits, its own row
+    // block), so its bits are those of a sequential decode; the K/V stream is read once per column
+    const size_t osz = out_dtype == PA_OUT_F16 ? 2 : 4;
+    for (uint32_t col = 0; col < n_cols; col++) {
+      rc = attn_common(ctx, who, 0, layer, d_q + (size_t)col * q_stride, q_stride, d_gate ? d_gate + (size_t)col * gate_stride : nullptr, gate_stride,
+                       base_pos + col, 1, (unsigned char*)d_out + (size_t)col * out_stride * osz, out_stride, out_dtype);
+      if (rc) return rc;
+    }
+    return PA_OK;
+  }
   pa_plan pl;
   uint32_t n_wgs = 0;
   rc = kind == 0 ? plan_decode(ctx, base_pos, n_cols, &pl, true, &n_wgs) : plan_prefill(ctx, base_pos, n_cols, &pl, &n_wgs);
@@ -494,9 +542,9 @@ extern "C" int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, ui
   return attn_common(ctx, "pa_attn_prefill", 1, layer, d_q, q_stride, d_gate, gate_stride, base_pos, n_cols, d_out, out_stride, out_dtype);
 }
 
-extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
-                                   const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
-  const char* who = "pa_attn_decode_step";
+// static_scratch: the partials go to the library's file-scope device array and the call allocates nothing
+static int decode_step_common(pa_ctx* ctx, const char* who, bool static_scratch, uint32_t layer, const float* d_q_in, const float* d_k,
+                              const float* d_v, const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
   if (!ctx) return PA_ERR_INVALID;
   int rc = check_cols(ctx, who, layer, true, pos, 1);
   if (rc) return rc;
@@ -514,11 +562,22 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
   if (pl.row_blocks != 1 || pl.waves != 4 || pl.col_groups != 1 || !plan_self_row(pl)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": plan is not a one-block decode");
-  if ((rc = ensure_partials(ctx, 1, pl.slots))) return rc;
+  float* part_o = nullptr; float* part_ml = nullptr;
+  if (static_scratch) {
+    const size_t need_o = ((size_t)c.n_heads * pl.slots * c.head_dim * sizeof(float) + 255) & ~(size_t)255;
+    const size_t need_ml = (size_t)c.n_heads * pl.slots * 2 * sizeof(float);
+    if (need_o + need_ml > PA_STATIC_SCRATCH_BYTES)
+      return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": the split partials of this shape (" + std::to_string(need_o + need_ml) +
+                  " bytes) exceed the library's static scratch (" + std::to_string(PA_STATIC_SCRATCH_BYTES) + " bytes); use pa_attn_decode_step");
+    part_o = (float*)ctx->static_scratch; part_ml = (float*)((unsigned char*)ctx->static_scratch + need_o);
+  } else {
+    if ((rc = ensure_partials(ctx, 1, pl.slots))) return rc;
+    part_o = ctx->part_o; part_ml = ctx->part_ml;
+  }
   AttnParams p; memset(&p, 0, sizeof p);
   p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
   p.k_scale = ctx->layers[layer].ks; p.v_scale = ctx->layers[layer].vs;
-  p.part_o = ctx->part_o; p.part_ml = ctx->part_ml; p.out = d_out;
+  p.part_o = part_o; p.part_ml = part_ml; p.out = d_out;
   p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
   p.base_pos = pos; p.n_cols = 1;
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
@@ -532,11 +591,20 @@ extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q
   p.f_q_head_stride = c.head_dim * (gated ? 2 : 1); p.n_rot = c.n_rot; p.eps = c.eps;
   p.gate = gated ? d_q_in + c.head_dim : nullptr;
   p.gate_head_stride = p.f_q_head_stride;
-  PaTiming tm;
-  if ((rc = prof_pair(ctx, &tm))) return rc;
+  PaTiming tm;                                        // profiling may create events: not on the allocation-free path
+  if (!static_scratch && (rc = prof_pair(ctx, &tm))) return rc;
   HIPCHK(ctx, pa_launch_decode_step(p, c.head_dim, ctx->stream, &tm));
   HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;
+}
+
+extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
+                                   const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
+  return decode_step_common(ctx, "pa_attn_decode_step", false, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype);
+}
+extern "C" int pa_attn_decode_step_noalloc(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
+                                           const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
+  return decode_step_common(ctx, "pa_attn_decode_step_noalloc", true, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype);
 }
 
 // ---- projections (one-token passes) -------------------------------------------------------------
@@ -609,17 +677,12 @@ extern "C" int pa_attn_layer_decode(pa_ctx* ctx, uint32_t layer, const pa_weight
   const uint32_t q_rows = qd * ((c.flags & PA_FLAG_GATE) ? 2 : 1);
   if (w_qkv->d_out != q_rows + 2 * kvd) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": w_qkv must have q (+ gate), k and v rows");
   if (w_o->d_in != qd || w_o->d_out != w_qkv->d_in) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": w_o must map n_heads x head_dim back to the model width");
-  const size_t need = (size_t)w_qkv->d_out + qd;
-  if (need > ctx->proj_buf_floats) {
-    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->proj_buf) { HIPCHK(ctx, hipFree(ctx->proj_buf)); ctx->proj_buf = nullptr; ctx->proj_buf_floats = 0; }
-    HIPCHK(ctx, hipMalloc((void**)&ctx->proj_buf, need * sizeof(float)));
-    ctx->proj_buf_floats = need;
-  }
+  const size_t need = ((size_t)w_qkv->d_out + qd) * sizeof(float);
+  int rc = grow_scratch(ctx, (void**)&ctx->proj_buf, &ctx->proj_buf_bytes, need);
+  if (rc) return rc;
   float* qkv = ctx->proj_buf;
   float* attn_out = ctx->proj_buf + w_qkv->d_out;
-  int rc = gemv_common(ctx, who, w_qkv, d_x, d_attn_norm_w, nullptr, qkv, 0);
-  if (rc) return rc;
+  if ((rc = gemv_common(ctx, who, w_qkv, d_x, d_attn_norm_w, nullptr, qkv, 0))) return rc;
   if ((rc = pa_attn_decode_step(ctx, layer, qkv, qkv + q_rows, qkv + q_rows + kvd, d_qw, d_kw, pos, attn_out, PA_OUT_F32))) return rc;
   return gemv_common(ctx, who, w_o, attn_out, nullptr, nullptr, d_x, 1);
 }
@@ -667,12 +730,7 @@ extern "C" int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weigh
   // chunk scratch: xn f16 [cols][dim] | qkv f32 [cols][rows] | attnOut f16 [cols][qd], each 256-byte aligned
   auto up256 = [](size_t b) { return (b + 255) & ~(size_t)255; };
   const size_t b_xn = up256((size_t)n_cols * dim * 2), b_qkv = up256((size_t)n_cols * rows * 4), b_at = up256((size_t)n_cols * qd * 2);
-  if (b_xn + b_qkv + b_at > ctx->chunk_buf_bytes) {
-    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->chunk_buf) { HIPCHK(ctx, hipFree(ctx->chunk_buf)); ctx->chunk_buf = nullptr; ctx->chunk_buf_bytes = 0; }
-    HIPCHK(ctx, hipMalloc(&ctx->chunk_buf, b_xn + b_qkv + b_at));
-    ctx->chunk_buf_bytes = b_xn + b_qkv + b_at;
-  }
+  if ((rc = grow_scratch(ctx, &ctx->chunk_buf, &ctx->chunk_buf_bytes, b_xn + b_qkv + b_at))) return rc;
   uint16_t* xn = (uint16_t*)ctx->chunk_buf;
   float* qkv = (float*)((unsigned char*)ctx->chunk_buf + b_xn);
   uint16_t* at = (uint16_t*)((unsigned char*)ctx->chunk_buf + b_xn + b_qkv);
@@ -712,6 +770,10 @@ static int kv_copy(pa_ctx* ctx, const char* who, uint32_t layer, int which, uint
     }
   }
   return PA_OK;
+}
+extern "C" size_t pa_kv_row_bytes(const pa_ctx* ctx, int which) {
+  if (!ctx || which < 0 || which >= n_tensors(ctx)) return 0;
+  return head_row_bytes(ctx, which) * ctx->cfg.n_kv_heads;
 }
 extern "C" int pa_kv_read(pa_ctx* ctx, uint32_t layer, int which, uint32_t row0, uint32_t n_rows, void* h_dst) {
   if (!ctx) return PA_ERR_INVALID;
@@ -765,7 +827,7 @@ extern "C" int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   p.gate_head_stride = c.head_dim;
-  p.sel = d_sel; p.sel_stride = sel_stride; p.n_wgs = n_wgs;
+  p.sel = d_sel; p.sel_stride = sel_stride; p.sel_max = std::min(max_rows, sel_stride - 1); p.n_wgs = n_wgs;
   PaTiming tm;
   if ((rc = prof_pair(ctx, &tm))) return rc;
   HIPCHK(ctx, pa_launch_decode_gather(p, c.head_dim, ctx->stream, &tm));

@@ -55,7 +55,9 @@ struct AttnParams {
   uint32_t f_q_head_stride, n_rot;
   float eps;
   // gather mode (pa_attn_decode_gather): per column sel[col * sel_stride] = n, then n cache rows; nullptr otherwise
-  const uint32_t* sel; uint32_t sel_stride;
+  // sel_max: the longest list the pass was sized for; a longer length word is read as sel_max (the list cannot run
+  // into the next column's), a length of 0 gives a column of zeros
+  const uint32_t* sel; uint32_t sel_stride, sel_max;
 };
 
 // ---- kernel launchers (defined next to their kernels) ------------------------------------------
@@ -78,6 +80,7 @@ hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint3
 hipError_t pa_launch_decode_gather(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t = nullptr);
 // the same with the pre-step of the one column fused in (p.f_* set; one 16-row block, n_cols == 1)
 hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t = nullptr);
+hipError_t pa_prepare_decode_step(uint32_t hd, bool q8);
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);
 // MFMA prefill; returns hipErrorNotSupported for shapes it does not cover
 hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
@@ -155,10 +158,12 @@ struct pa_ctx {
   float* part_o = nullptr; float* part_ml = nullptr;
   size_t part_o_bytes = 0, part_ml_bytes = 0;
   float* proj_buf = nullptr;    // pa_attn_layer_decode: [q(+gate) | k | v] projections, then attnOut [nH*hd]
-  size_t proj_buf_floats = 0;
+  size_t proj_buf_bytes = 0;
   void* chunk_buf = nullptr;    // pa_attn_layer_prefill: xn f16 [cols][dim], qkv f32 [cols][rows], attnOut f16 [cols][nH*hd]
   size_t chunk_buf_bytes = 0;
   uint16_t* wide_k = nullptr; uint16_t* wide_v = nullptr;   // int8 caches: f16 staging cache of one layer for the prefill kernel
+  void* static_scratch = nullptr;   // this device's copy of the library's file-scope scratch array (pa_attn_decode_step_noalloc)
+  std::vector<void*> retired;   // outgrown scratch blocks, kept until pa_destroy (a recorded launch may still name them)
   uint32_t decode_splits_override = 0;
   // timing
   hipEvent_t t0 = nullptr, t1 = nullptr;

@@ -23,6 +23,11 @@ static napi_value throw_pa(napi_env env, pa_ctx* ctx, int rc, const char* who) {
   return nullptr;
 }
 
+// What the JS handle points at.  destroy() clears ctx, so a stale handle is refused instead of reaching freed memory;
+// the box itself lives until the handle is garbage collected.
+struct CtxBox { pa_ctx* ctx; };
+static void box_finalize(napi_env, void* data, void*) { CtxBox* b = (CtxBox*)data; if (b) { if (b->ctx) pa_destroy(b->ctx); delete b; } }
+
 struct Args {
   napi_env env; size_t argc; napi_value argv[16]; bool ok;
   Args(napi_env e, napi_callback_info info) : env(e), argc(16), ok(true) { if (napi_get_cb_info(e, info, &argc, argv, nullptr, nullptr) != napi_ok) ok = false; }
@@ -34,7 +39,13 @@ struct Args {
     if (t == napi_null || t == napi_undefined) return nullptr;
     return (void*)(uintptr_t)num(i);
   }
-  pa_ctx* ctx(size_t i) { void* p = nullptr; if (i >= argc || napi_get_value_external(env, argv[i], &p) != napi_ok) ok = false; return (pa_ctx*)p; }
+  // the handle create() returned: an external holding a CtxBox; a destroyed context reads as a bad argument
+  pa_ctx* ctx(size_t i) {
+    void* p = nullptr;
+    if (i >= argc || napi_get_value_external(env, argv[i], &p) != napi_ok || !p || !((CtxBox*)p)->ctx) { ok = false; return nullptr; }
+    return ((CtxBox*)p)->ctx;
+  }
+  CtxBox* box(size_t i) { void* p = nullptr; if (i >= argc || napi_get_value_external(env, argv[i], &p) != napi_ok) ok = false; return (CtxBox*)p; }
   void* host(size_t i, size_t* bytes) {       // TypedArray / ArrayBuffer contents
     void* data = nullptr; *bytes = 0;
     bool is = false;
@@ -81,12 +92,17 @@ static napi_value Create(napi_env env, napi_callback_info info) {
   pa_ctx* ctx = nullptr;
   int rc = pa_create(&c, &ctx);
   if (rc) return throw_pa(env, nullptr, rc, "pa_create");
+  CtxBox* box = new CtxBox{ctx};
   napi_value ext;
-  NAPI_OK(napi_create_external(env, ctx, nullptr, nullptr, &ext));
+  if (napi_create_external(env, box, box_finalize, nullptr, &ext) != napi_ok) { pa_destroy(ctx); delete box; napi_throw_error(env, nullptr, "pooled_attn addon: napi_create_external failed"); return nullptr; }
   return ext;
 }
-static napi_value Destroy(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); CHECK_ARGS("destroy"); pa_destroy(c); return undefined(env); }
-static napi_value LastError(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.argc ? a.ctx(0) : nullptr; napi_value v; napi_create_string_utf8(env, pa_last_error(c), NAPI_AUTO_LENGTH, &v); return v; }
+static napi_value Destroy(napi_env env, napi_callback_info info) {
+  ARGS; CtxBox* b = a.box(0); CHECK_ARGS("destroy");
+  if (b && b->ctx) { pa_destroy(b->ctx); b->ctx = nullptr; }
+  return undefined(env);
+}
+static napi_value LastError(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.argc ? a.ctx(0) : nullptr; a.ok = true; napi_value v; napi_create_string_utf8(env, pa_last_error(c), NAPI_AUTO_LENGTH, &v); return v; }
 static napi_value Version(napi_env env, napi_callback_info) { napi_value v; napi_create_string_utf8(env, pa_version(), NAPI_AUTO_LENGTH, &v); return v; }
 
 static napi_value LayerAlloc(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); uint32_t l = a.u32(1); CHECK_ARGS("layerAlloc"); int rc = pa_layer_alloc(c, l); if (rc) return throw_pa(env, c, rc, "pa_layer_alloc"); return undefined(env); }
@@ -176,10 +192,12 @@ static napi_value SetDecodeSplits(napi_env env, napi_callback_info info) { ARGS;
 // kvRead(ctx, layer, which, row0, nRows, Uint16Array) / kvWrite(ctx, layer, which, row0, nRows, Uint16Array)
 static napi_value KvRead(napi_env env, napi_callback_info info) {
   ARGS; pa_ctx* c = a.ctx(0); uint32_t layer = a.u32(1); int which = (int)a.u32(2); uint32_t r0 = a.u32(3), nr = a.u32(4); size_t n; void* h = a.host(5, &n); CHECK_ARGS("kvRead");
+  if (n < (size_t)nr * pa_kv_row_bytes(c, which)) { napi_throw_range_error(env, nullptr, "kvRead: array shorter than nRows rows of this cache tensor"); return nullptr; }
   int rc = pa_kv_read(c, layer, which, r0, nr, h); if (rc) return throw_pa(env, c, rc, "pa_kv_read"); return undefined(env);
 }
 static napi_value KvWrite(napi_env env, napi_callback_info info) {
   ARGS; pa_ctx* c = a.ctx(0); uint32_t layer = a.u32(1); int which = (int)a.u32(2); uint32_t r0 = a.u32(3), nr = a.u32(4); size_t n; void* h = a.host(5, &n); CHECK_ARGS("kvWrite");
+  if (n < (size_t)nr * pa_kv_row_bytes(c, which)) { napi_throw_range_error(env, nullptr, "kvWrite: array shorter than nRows rows of this cache tensor"); return nullptr; }
   int rc = pa_kv_write(c, layer, which, r0, nr, h); if (rc) return throw_pa(env, c, rc, "pa_kv_write"); return undefined(env);
 }
 static napi_value KvDevicePtr(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); uint32_t layer = a.u32(1); int which = (int)a.u32(2); CHECK_ARGS("kvDevicePtr"); return num_value(env, (double)(uintptr_t)pa_kv_device_ptr(c, layer, which)); }
@@ -200,10 +218,14 @@ static napi_value SlotPos(napi_env env, napi_callback_info info) { ARGS; pa_ctx*
 static napi_value SlotCreate(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1), pos = a.u32(2); CHECK_ARGS("slotCreate"); int rc = pa_slot_create(c, id, pos); if (rc) return throw_pa(env, c, rc, "pa_slot_create"); return undefined(env); }
 static napi_value SlotExport(napi_env env, napi_callback_info info) {
   ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1), layer = a.u32(2); int which = (int)a.u32(3); size_t n; void* h = a.host(4, &n); CHECK_ARGS("slotExport");
+  { uint32_t pos = 0; int rc0 = pa_slot_pos(c, id, &pos); if (rc0) return throw_pa(env, c, rc0, "pa_slot_pos");
+    if (n < (size_t)pos * pa_kv_row_bytes(c, which)) { napi_throw_range_error(env, nullptr, "slotExport: array shorter than the slot's rows of this cache tensor"); return nullptr; } }
   int rc = pa_slot_export(c, id, layer, which, h); if (rc) return throw_pa(env, c, rc, "pa_slot_export"); return undefined(env);
 }
 static napi_value SlotImport(napi_env env, napi_callback_info info) {
   ARGS; pa_ctx* c = a.ctx(0); uint32_t id = a.u32(1), layer = a.u32(2); int which = (int)a.u32(3); size_t n; void* h = a.host(4, &n); CHECK_ARGS("slotImport");
+  { uint32_t pos = 0; int rc0 = pa_slot_pos(c, id, &pos); if (rc0) return throw_pa(env, c, rc0, "pa_slot_pos");
+    if (n < (size_t)pos * pa_kv_row_bytes(c, which)) { napi_throw_range_error(env, nullptr, "slotImport: array shorter than the slot's rows of this cache tensor"); return nullptr; } }
   int rc = pa_slot_import(c, id, layer, which, h); if (rc) return throw_pa(env, c, rc, "pa_slot_import"); return undefined(env);
 }
 

@@ -17,43 +17,12 @@
 const path = require("path");
 const addon = require(path.join(__dirname, "..", "lib", "pooled_attn.node"));
 
-const PA_FLAG_QK_NORM = 1, PA_FLAG_GATE = 2, PA_FLAG_KV_Q8 = 4, PA_OUT_F32 = 0, PA_OUT_F16 = 1;
+const PA_FLAG_QK_NORM = 1, PA_FLAG_GATE = 2, PA_FLAG_KV_Q8 = 4, PA_FLAG_VERIFY_EXACT = 8, PA_OUT_F32 = 0, PA_OUT_F16 = 1;
 const PA_W_F32 = 0, PA_W_Q8_0 = 1, PA_W_Q4_0 = 2;             // weight kinds of the projections (include/pooled_attn.h)
 
-// ---- the reference's sizing formulas, kept for callers that still size grids or slot buffers with them.
-//      The HIP kernels take their splits from the gfx950 table instead (HipAttention.plan). ----
-// engine/wgsl/attn_dec.js:40-51
-function attnDecConfig(o) {
-  const hd = o.hd, G = o.G, nKV = o.nKV, splits = o.splits || 0, R = o.R || 1;
-  if (o.kvQ8 || hd !== 256 || !(G >= 1 && G <= 8) || !(R >= 1)) return null;
-  const S = splits > 0 ? splits | 0 : Math.max(16, Math.floor(256 / nKV));
-  return { HD: hd, G: G, S: S, R: R };
-}
-const decSplitLen = (s, S) => Math.max(64, Math.ceil(Math.ceil(s / S) / 64) * 64);
-const decSplits = (s, S) => Math.ceil(s / decSplitLen(s, S));
-const DEC_CQ = 4;
-// engine/wgsl/attn_tile.js:43-56
-function attnTileConfig(o) {
-  const hd = o.hd, G = o.G, wgMem = o.wgMem || 16384;
-  if (!(hd % 16 === 0 && hd >= 16 && hd <= 256 && G >= 1 && G <= 64)) return null;
-  if (o.faSplit % 64 !== 0 || o.faSplits < 1) return null;
-  const bytes = (TK) => TK * hd * 4 + TK * 256 * 4;
-  const TK = o.tk || [16, 8, 4].find((t) => bytes(t) <= wgMem);
-  if (!TK || bytes(TK) > wgMem) return null;
-  return { HD: hd, G: G, CW: Math.floor(64 / G), TK: TK, FASPLIT: o.faSplit, FASPLITS: o.faSplits, TARGET: Math.max(1, (o.target === undefined ? 32 : o.target) | 0) };
-}
-function tileSplitLen(seqEnd, c) {
-  const up64 = (x) => Math.ceil(x / 64) * 64;
-  return Math.min(c.FASPLIT, Math.max(64, up64(Math.ceil(seqEnd / c.TARGET)), up64(Math.ceil(seqEnd / c.FASPLITS))));
-}
-// engine/qwen35.js:367-368
-function faSizing(maxSeq) {
-  const faSplit = Math.max(256, Math.ceil(maxSeq / 128 / 64) * 64);
-  return { faSplit: faSplit, faSplits: Math.ceil(maxSeq / faSplit) };
-}
-
 class HipAttention {
-  // opts: { nH, nKV, hd, nRot, ropeTheta, eps, maxSeq, nLayers, batchCols, qkNorm = true, gate = false, outF16 = false }
+  // opts: { nH, nKV, hd, nRot, ropeTheta, eps, maxSeq, nLayers, batchCols, qkNorm = true, gate = false, outF16 = false,
+  //         kvQ8 = false, fusedStep = true, verifyExact = false }
   constructor(opts) {
     const nH = opts.nH, nKV = opts.nKV, hd = opts.hd;
     if (!(nH > 0 && nKV > 0 && nH % nKV === 0)) throw new Error("HipAttention: nH must be a positive multiple of nKV");
@@ -69,7 +38,11 @@ class HipAttention {
     this._snapNow = null;                                          // set by a verify pass (engine/qwen35.js:2960-2965)
     this.pos = 0;
     this.kvQ8 = !!opts.kvQ8;                                       // int8 caches (engine option kvQ8)
-    const flags = (this.qkNorm ? PA_FLAG_QK_NORM : 0) | (this.gate ? PA_FLAG_GATE : 0) | (this.kvQ8 ? PA_FLAG_KV_Q8 : 0);
+    // verifyExact: every column of a verify block is run as the one-column decode at its position, so it has the bits
+    // of a sequential decode (the reference's invariant, engine/wgsl/attn_dec.js:12-16); the K/V stream is then read
+    // once per column.  Off by default: a block's columns then agree with sequential decodes to rounding only.
+    this.verifyExact = !!opts.verifyExact;
+    const flags = (this.qkNorm ? PA_FLAG_QK_NORM : 0) | (this.gate ? PA_FLAG_GATE : 0) | (this.kvQ8 ? PA_FLAG_KV_Q8 : 0) | (this.verifyExact ? PA_FLAG_VERIFY_EXACT : 0);
     // a readable throw at create, like the engine's KV binding check (engine/qwen35.js:378-383)
     this.ctx = addon.create({ nH: nH, nKV: nKV, hd: hd, nRot: this.dims.nRot, ropeTheta: opts.ropeTheta, eps: opts.eps,
       maxSeq: opts.maxSeq, nLayers: opts.nLayers || 1, maxCols: this.NC, flags: flags });
@@ -129,7 +102,11 @@ class HipAttention {
     return which < 2 ? new Int8Array(nRows * this.dims.kvDim) : new Float32Array(nRows * this.dims.kvDim / 32);
   }
   kvRead(layer, which, row0, nRows) { const a = this._kvPart(which, nRows); addon.kvRead(this.ctx, layer, which, row0, nRows, a); return a; }
-  kvWrite(layer, which, row0, rows) { addon.kvWrite(this.ctx, layer, which, row0, rows.length / this._kvPart(which, 1).length, rows); }
+  kvWrite(layer, which, row0, rows) {
+    const per = this._kvPart(which, 1).length;
+    if (rows.length % per !== 0) throw new RangeError("kvWrite: " + rows.length + " elements is not a whole number of rows of " + per);
+    addon.kvWrite(this.ctx, layer, which, row0, rows.length / per, rows);
+  }
   sync() { addon.sync(this.ctx); }
   plan(kind, basePos, nCols) { return addon.planQuery(this.ctx, kind === "prefill" ? 1 : 0, basePos, nCols); }
 
@@ -191,8 +168,11 @@ class HipAttention {
     addon.glue(this.ctx, this.B.qFull.ptr, this._strideF(this.B.qFull), this.B.k.ptr, this._strideF(this.B.k), n[0], n[1], M.basePos, nCols);
   }
   // kv_store + attention + sigmoid gate: B.q / B.k / B.v / gate -> B.attnOut.  Kernel selection as the reference's:
-  // a full-width pass that is not a verify runs the tiled prefill kernel, everything else the split-K decode kernel
-  // (so a verify column is a decode at the same position).
+  // a full-width pass that is not a verify runs the tiled prefill kernel, everything else the split-K decode kernel.
+  // Unlike the reference's pair (engine/wgsl/attn_dec.js:12-16) a verify column here equals the one-column decode at
+  // the same position to rounding only (|difference| <= 1e-3 by test, 3e-4 measured): the block's columns share
+  // matrix-core tiles and splits.  Constructing with { verifyExact: true } restores the bit identity at the cost of
+  // one K/V read per column.
   _encAttnCore(p, LB, M, basePos, nCols) {
     const B = this.B, layer = LB.layer;
     addon.kvStore(this.ctx, layer, B.k.ptr, this._strideF(B.k), B.v.ptr, this._strideF(B.v), basePos, nCols);
@@ -297,5 +277,4 @@ class HipAttention {
   }
 }
 
-module.exports = { HipAttention, addon, attnDecConfig, decSplitLen, decSplits, DEC_CQ, attnTileConfig, tileSplitLen, faSizing,
-  PA_FLAG_QK_NORM, PA_FLAG_GATE, PA_FLAG_KV_Q8, PA_OUT_F32, PA_OUT_F16 };
+module.exports = { HipAttention, addon, PA_FLAG_QK_NORM, PA_FLAG_GATE, PA_FLAG_KV_Q8, PA_FLAG_VERIFY_EXACT, PA_OUT_F32, PA_OUT_F16 };

@@ -4,10 +4,12 @@
 //   2. the same columns as a verify pass (decode kernel, snapshot set)
 //   3. one token at a time                            encodeLayerAttn
 //   4. session state                                  saveSlot / loadSlot / dropSlot / exportSlot / importState
-// against the expected values (max-abs 2e-3, rel 1e-2) and the written KV rows bit for bit.
+// against the expected values (max-abs 2e-3, rel 1e-2) and the written KV rows bit for bit; and the verify pass
+// against the token-by-token outputs: within 1e-3 by default, bit for bit on a context made with verifyExact
+// (the reference's verify column == decode invariant, engine/wgsl/attn_dec.js:12-16, tests/test_attn_dec.js:89-97).
 "use strict";
 const fs = require("fs"), path = require("path");
-const { HipAttention, decSplits, decSplitLen, faSizing } = require(path.join(__dirname, "..", "..", "pooled_amd", "js", "hip_attention.js"));
+const { HipAttention } = require(path.join(__dirname, "..", "..", "pooled_amd", "js", "hip_attention.js"));
 const dir = process.argv[2];
 const C = JSON.parse(fs.readFileSync(path.join(dir, "case.json"), "utf8"));
 const f32 = (n) => { const b = fs.readFileSync(path.join(dir, n)); return new Float32Array(b.buffer.slice(b.byteOffset, b.byteOffset + b.byteLength)); };
@@ -20,9 +22,6 @@ const check = (what, got, ref) => {
   console.log(what + ": max-abs " + md.toExponential(2) + " rel " + (md / mr).toExponential(2) + (ok ? " ok" : " FAIL"));
   if (!ok) fails++;
 };
-// the reference's sizing mirrors (engine/wgsl/attn_dec.js:47-48, engine/qwen35.js:367-368)
-if (decSplitLen(32769, 128) !== 320 || decSplits(32769, 128) !== 103 || faSizing(131072).faSplit !== 1024) { console.log("sizing mirrors FAIL"); fails++; }
-
 const cfg = C.cfg, n = C.nCols, base = C.basePos;
 const A = new HipAttention({ nH: cfg.n_heads, nKV: cfg.n_kv_heads, hd: cfg.head_dim, nRot: cfg.n_rot, ropeTheta: cfg.rope_theta, eps: cfg.eps,
   maxSeq: base + n, nLayers: 1, batchCols: n, qkNorm: true, gate: !!cfg.gate });
@@ -49,11 +48,48 @@ if (!eqBits(A.kvRead(0, 0, base, n), kNew) || !eqBits(A.kvRead(0, 1, base, n), v
 loadCols(0, n);
 A.encodeLayerBatchAttn(null, 0, base, n, true);
 A.sync();
-check("verify pass (decode kernel)", flat(A.readAttnOut(n)), expect);
+const verifyOut = flat(A.readAttnOut(n));
+check("verify pass (decode kernel)", verifyOut, expect);
 // 3. token by token
 const outs = [];
 for (let c = 0; c < n; c++) { loadCols(c, 1); A.encodeLayerAttn(null, 0, base + c); A.sync(); outs.push(A.readAttnOut(1)[0]); }
-check("token by token (fused glue + decode)", flat(outs), expect);
+const seqOut = flat(outs);
+check("token by token (fused glue + decode)", seqOut, expect);
+// verify block vs sequential decodes: to rounding by default ...
+{
+  let md = 0; for (let i = 0; i < seqOut.length; i++) md = Math.max(md, Math.abs(seqOut[i] - verifyOut[i]));
+  console.log("verify block vs sequential decodes: max-abs " + md.toExponential(2) + (md <= 1e-3 ? " ok" : " FAIL"));
+  if (!(md <= 1e-3)) fails++;
+}
+// ... and bit for bit on a context constructed with verifyExact
+{
+  const E = new HipAttention({ nH: cfg.n_heads, nKV: cfg.n_kv_heads, hd: cfg.head_dim, nRot: cfg.n_rot, ropeTheta: cfg.rope_theta, eps: cfg.eps,
+    maxSeq: base + n, nLayers: 1, batchCols: n, qkNorm: true, gate: !!cfg.gate, verifyExact: true });
+  E.setLayerNorms(0, f32("qw.bin"), f32("kw.bin"));
+  E.kvWrite(0, 0, 0, K0); E.kvWrite(0, 1, 0, V0);
+  const m = Math.min(n, 16);                                      // a verify block is a few columns wide
+  for (let c = 0; c < m; c++) {
+    E.writeColumn(E.B.qFull, c, qraw.subarray(c * qIn, (c + 1) * qIn));
+    E.writeColumn(E.B.k, c, kraw.subarray(c * D.kvDim, (c + 1) * D.kvDim));
+    E.writeColumn(E.B.v, c, vraw.subarray(c * D.kvDim, (c + 1) * D.kvDim));
+  }
+  E._snapNow = 1;
+  E._encAttnGlue(null, { layer: 0, basePos: base }, m);
+  E._encAttnCore(null, { layer: 0 }, { layer: 0, basePos: base }, base, m);
+  E._snapNow = null;
+  E.sync();
+  const ex = flat(E.readAttnOut(m));
+  const same = eqBits(new Uint32Array(ex.buffer), new Uint32Array(seqOut.buffer, 0, m * D.qDim));
+  console.log("verifyExact block == sequential encodeLayerAttn bit for bit: " + (same ? "ok" : "FAIL"));
+  if (!same) fails++;
+  // a short array is refused before anything is copied (RangeError), and a destroyed context is a bad argument
+  try { E.kvRead(0, 0, 0, 4).length; require(path.join(__dirname, "..", "..", "pooled_amd", "lib", "pooled_attn.node")).kvRead(E.ctx, 0, 0, 0, 4, new Uint16Array(8)); console.log("short kvRead array did not throw FAIL"); fails++; }
+  catch (e) { if (!(e instanceof RangeError)) { console.log("short kvRead array: unexpected error " + e.message + " FAIL"); fails++; } }
+  const stale = E.ctx;
+  E.destroy();
+  try { require(path.join(__dirname, "..", "..", "pooled_amd", "lib", "pooled_attn.node")).sync(stale); console.log("call on a destroyed context did not throw FAIL"); fails++; }
+  catch (e) { if (!(e instanceof TypeError)) { console.log("destroyed context: unexpected error " + e.message + " FAIL"); fails++; } }
+}
 if (!eqBits(A.kvRead(0, 0, base, n), kNew)) { console.log("KV rows written token by token differ FAIL"); fails++; }
 // error path: a readable throw, not an abort
 try { A.encodeLayerAttn(null, 0, base + n); console.log("out-of-range position did not throw FAIL"); fails++; } catch (e) { if (!/max_seq/.test(e.message)) { console.log("unexpected error text: " + e.message + " FAIL"); fails++; } }

@@ -106,6 +106,26 @@ def test_verify_equals_sequential_decodes(shape, n_cols, base):
             assert np.abs(single[0] - multi[c]).max() <= 1e-3
 
 
+@pytest.mark.parametrize("shape,n_cols,base", [("qwen36_moe", 4, 996), ("qwen38_27b", 8, 2040), ("qwen3_1p7b", 5, 510), ("qwen36_moe", 3, 32767)])
+def test_verify_exact_flag_gives_the_sequential_decodes_bits(shape, n_cols, base):
+    """PA_FLAG_VERIFY_EXACT: every column of a verify block has the bits of the one-column decode at its position
+    (the reference's invariant, engine/wgsl/attn_dec.js:12-16; tests/test_attn_dec.js:89-97 checks it with Object.is);
+    the plan a plan query reports is unchanged."""
+    cfg = dict(SHAPES[shape], verify_exact=True)
+    rng = np.random.default_rng(base + n_cols)
+    L = base + n_cols
+    k16, v16 = random_cache(cfg, L + 5, seed=14)
+    q = rng.standard_normal((n_cols, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    gate = rng.standard_normal(q.shape, dtype=np.float32) if cfg["gate"] else None
+    ref = C.attention(q, k16, v16, base, gate=gate)
+    with _ctx_with_cache(cfg, k16, v16, L + 5, poison_from=L) as pa:
+        multi = pa.run_attn("decode", 0, q, base, gate=gate)
+        assert_parity(multi, ref, "column-exact verify block")
+        for c in range(n_cols):
+            single = pa.run_attn("decode", 0, q[c:c + 1], base + c, gate=None if gate is None else gate[c:c + 1])
+            assert np.array_equal(single[0].view(np.uint32), multi[c].view(np.uint32)), "column %d differs from its decode" % c
+
+
 def test_decode_f16_output_and_strides():
     cfg = SHAPES["qwen36_moe"]
     rng = np.random.default_rng(14)

@@ -78,3 +78,32 @@ def test_gather_f16_out_and_bad_arguments():
         assert e.value.code == PA_ERR_INVALID
         with pytest.raises(PaError):                                         # more rows than the cache holds
             pa._chk(pa.L.pa_attn_decode_gather(pa.ctx, 0, dq.ptr, pa.q_dim, None, 0, dsel.ptr, 1000, 501, 2, dout.ptr, pa.q_dim, 0))
+
+
+def test_gather_does_not_trust_the_length_word():
+    """The length word of a list lives in device memory the caller's selection kernel wrote: a length past max_rows is
+    read as max_rows (the list cannot run into the next column's), a length of 0 gives a column of zeros, and the
+    other columns of the pass are unaffected."""
+    cfg = SHAPES["qwen36_moe"]
+    rng = np.random.default_rng(23)
+    rows_total, max_rows = 3000, 300
+    k16, v16 = random_cache(cfg, rows_total, seed=24)
+    lists = [np.sort(rng.choice(rows_total, size=max_rows, replace=False)) for _ in range(3)]
+    q = rng.standard_normal((3, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    ref = _oracle(q, k16, v16, lists, None)
+    stride = max_rows + 1
+    sel = np.zeros((3, stride), np.uint32)
+    for c, l in enumerate(lists):
+        sel[c, 0] = len(l); sel[c, 1:] = l
+    sel[0, 0] = 100000                      # far past max_rows and the stride: must read as max_rows
+    sel[1, 0] = 0                           # an empty list
+    with PooledAttn(cfg, rows_total, n_layers=1, max_cols=4) as pa:
+        pa.layer_alloc(0); pa.kv_write(0, 0, 0, k16); pa.kv_write(0, 1, 0, v16)
+        dq = pa.to_device(q.reshape(3, -1)); dsel = pa.to_device(sel)
+        dout = pa.to_device(np.full((3, pa.q_dim), np.nan, np.float32))
+        pa._chk(pa.L.pa_attn_decode_gather(pa.ctx, 0, dq.ptr, pa.q_dim, None, 0, dsel.ptr, stride, max_rows, 3, dout.ptr, pa.q_dim, 0))
+        pa.sync()
+        got = dout.download(np.float32, 3 * pa.q_dim).reshape(ref.shape)
+    assert_parity(got[0:1], ref[0:1], "over-long length word")
+    assert np.all(got[1] == 0.0), "empty list must give zeros"
+    assert_parity(got[2:3], ref[2:3], "neighbour of the bad lists")
