@@ -399,15 +399,25 @@ def main():
     for i in range(args.warmup):
         step(i)
     pa.sync()
-    t0 = time.perf_counter()
-    pa.timer_start()
-    for i in range(args.steps):
-        step(i)
-    gpu_ms = pa.timer_stop()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    ms_per_step = max(gpu_ms, wall_ms) / args.steps
+
+    def window():
+        """EXACTLY args.steps steps between two synchronisations; the larger of the event and the host clock."""
+        pa.sync()
+        t0 = time.perf_counter()
+        pa.timer_start()
+        for i in range(args.steps):
+            step(i)
+        gpu_ms = pa.timer_stop()                       # blocks until the last step has finished
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        return max(gpu_ms, wall_ms) / args.steps
+
+    # A window of a few hundred 20-microsecond steps is short against the box's noise (clock ramps, the host thread
+    # being descheduled): the window is repeated and the median window is the reported ms_per_step.
+    n_windows = max(5, min(25, -(-3000 // max(args.steps, 1))))
+    windows = sorted(window() for _ in range(n_windows))
+    ms_per_step = windows[len(windows) // 2]
     value = kv_bytes / (ms_per_step * 1e-3) / 1e9
-    log("timed %d steps: %.2f us/step (events %.2f ms, wall %.2f ms) -> %.0f GB/s" % (args.steps, ms_per_step * 1e3, gpu_ms, wall_ms, value))
+    log("timed %d windows of %d steps: median %.2f us/step (min %.2f, max %.2f) -> %.0f GB/s" % (n_windows, args.steps, ms_per_step * 1e3, windows[0] * 1e3, windows[-1] * 1e3, value))
 
     # the dominant kernel alone: one HIP event pair around every split-K launch, on the launch stream
     pa.profile_enable(True)
@@ -417,16 +427,20 @@ def main():
     pa.profile_enable(False)
     k_ms = ksum / max(kcount, 1)
     achieved = kv_bytes / (k_ms * 1e-3) / 1e9
-    traffic = None
+    # HBM bytes per launch are not measured in this run: they come from two rocprofv3 --pmc runs of this same command
+    # (FETCH_SIZE, WRITE_SIZE) whose summary is committed; the line names the file and the commit it was taken at
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", "decode_c3_traffic.json")
     if os.path.exists(tpath) and not args.kv_q8 and not args.unfused:      # measured for the default (fused, f16) kernel
-        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        tj = json.load(open(tpath))
+        traffic = tj.get("hbm_bytes_per_launch")
+        traffic_source = "profiles/decode_c3_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, measured at commit %s; not re-measured by this run)" % tj.get("head", "unknown")
     plan = pa.plan("decode", ctx, 1)
     # template arguments: head_dim, row blocks, waves, fused pre-step, gather, int8 caches, single-round splits
     kname = "pa_decode_kernel<256, 1, 4, %s, false, %s, %s>" % ("false" if args.unfused else "true", "true" if args.kv_q8 else "false",
                                                                "true" if plan["split_len"] == 128 and plan["row_blocks"] == 1 else "false")
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
-                    traffic=traffic, kernel=kname, kernel_us=round(k_ms * 1e3, 3),
+                    traffic=traffic, traffic_source=traffic_source, kernel=kname, kernel_us=round(k_ms * 1e3, 3),
                     algorithmic_bytes_per_launch=kv_bytes, launches=kcount)
     log("split-K kernel: %.2f us/launch -> %.0f GB/s (%.1f%% of 8 TB/s)" % (k_ms * 1e3, achieved, 100 * achieved / HBM_PEAK_GBS))
 
@@ -449,7 +463,8 @@ def main():
     line = dict(
         metric="decode attn KV-read GB/s (% HBM peak) @32K ctx; prefill attn TFLOP/s (% MFMA)",
         value=round(value, 1), unit="GB/s", n_gpus=1, steps=args.steps, warmup=args.warmup,
-        ms_per_step=round(ms_per_step, 6), higher_is_better=True, scaling="weak", vs_baseline=None,
+        ms_per_step=round(ms_per_step, 6), windows=dict(count=n_windows, steps_each=args.steps, reported="median", min_ms_per_step=round(windows[0], 6), max_ms_per_step=round(windows[-1], 6)),
+        higher_is_better=True, scaling="weak", vs_baseline=None,
         dtype="f16 (int8 cache widened to f16)" if args.kv_q8 else "f16", data="synthetic",
         config=dict(workload="C3 gated decode: 16q/2kv heads, head_dim 256, ctx 32768, 1 token, %s KV," % ("int8 (f32 scale per 32)" if args.kv_q8 else "f16") + " partial RoPE 64 dims theta 1e7, sigmoid gate, f16 out",
                     step="%s on one layer; %d layers' caches in rotation (cold HBM)" % ("pa_glue_kv + pa_attn_decode (pre-step, split-K decode, LSE merge/gate: 3 launches)" if args.unfused else "pa_attn_decode_step (pre-step fused into the split-K decode kernel + LSE merge/gate: 2 launches)", N_LAYERS),

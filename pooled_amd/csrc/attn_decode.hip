@@ -772,6 +772,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   }
 
   // ---- merge the W waves of the workgroup ----
+  const bool direct = p.direct_out != 0;       // one split and no own-row partial: this workgroup holds the whole result
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     l_run[nb] += __shfl_xor(l_run[nb], 16, 64);
@@ -826,11 +827,33 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
 #pragma unroll
         for (int w = 1; w < W; w++) o += part[j][w];
         const uint32_t col = c0 + r / G, hq = g * G + r % G;
-        const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
-        *(f4*)(p.part_o + slot * HD + 4 * d4) = o;
+        if (direct) {
+          // the only split of the pass: normalise, gate, convert and store here -- no partial, no merge launch
+          float Mr = NEG_INF, L = 0.f;
+#pragma unroll
+          for (int w = 0; w < W; w++) Mr = fmaxf(Mr, mex[w * 16 * NB + r]);
+          const float ms = Mr == NEG_INF ? 0.f : Mr;
+#pragma unroll
+          for (int w = 0; w < W; w++) L += lex[w * 16 * NB + r] * __expf(mex[w * 16 * NB + r] - ms);
+          o = o / L;
+          if (p.gate) {
+            const f4 gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)hq * p.gate_head_stride + 4 * d4);
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] *= 1.f / (1.f + __expf(-gt[i]));
+          }
+          if (p.out_f16) {
+            const h4 hv = { (_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3] };
+            *(h4*)((_Float16*)p.out + (size_t)col * p.out_stride + (size_t)hq * HD + 4 * d4) = hv;
+          } else {
+            *(f4*)((float*)p.out + (size_t)col * p.out_stride + (size_t)hq * HD + 4 * d4) = o;
+          }
+        } else {
+          const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
+          *(f4*)(p.part_o + slot * HD + 4 * d4) = o;
+        }
       }
     }
-    if (ml_thread) {
+    if (ml_thread && !direct) {
       const uint32_t r = nb * 16 + tid;
       float Mr = NEG_INF;
 #pragma unroll
@@ -849,96 +872,91 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
 }
 
 // ---- second pass: log-sum-exp merge over a column's splits, sigmoid gate, output conversion ----
-// One workgroup per (head, 64-dim slice, column) -- the reference's layout (engine/wgsl/attn_dec.js:215-287,
-// DEC_CQ slices per head) -- so the merge of a decode token runs on nH * HD/64 workgroups instead of nH.
-// 256 threads = 16 split groups x 16 float4 lanes.  The kernel is latency-bound (a few KB per workgroup, read
-// once, from the memory side), so it is written as one round trip: a thread issues all 17 output-partial loads of
-// its first 272-split chunk and its (m, l) loads before anything waits; the maximum and the weighted sum of l are
-// fixed-order tree reductions, a group's splits are accumulated in split order and the 16 groups in group order.
-template <int HD>
-__global__ __launch_bounds__(256) void pa_combine_kernel(AttnParams p) {
-  constexpr int CQ = HD / 64, CH = 17;      // CH loads in flight per thread = 272 splits per chunk (256 + the own-row partial)
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  float* wl = (float*)smem;                 // [slots] split weights exp(m_s - M)
-  __shared__ float red[256];
-  __shared__ f4 ored[256];
-  const uint32_t h = blockIdx.x / CQ, dq = blockIdx.x % CQ, col = blockIdx.y, tid = threadIdx.x;
-  const uint32_t col_end = p.sel ? min(p.sel[col * p.sel_stride], p.sel_max) : p.base_pos + col + 1 - p.self_row;   // gather: the column's list length
-  // the last split is open-ended; a one-column decode's own row is one more partial after the splits that hold rows
+// (the reference's attn_dec_combine(_g), engine/wgsl/attn_dec.js:215-287: M = max m_s, w_s = exp(m_s - M),
+// out = sum O_s w_s / sum l_s w_s, times sigmoid(gate))
+// The kernel is latency-bound (a few KB per output slice, read once from the memory side, after a dependent launch),
+// so it has no barrier and no LDS: one wavefront per (head, 16-dim slice, column) -- nH x HD/16 single-wave
+// workgroups, spread over the whole chip -- as 16 split groups x 4 float4 lanes.  A lane loads the (m, l) pairs and
+// the output partials of its group's splits (group + 16 k) in one round trip, the maximum and the sums over the 16
+// groups are xor-shuffle trees (fixed order), lanes 0 .. 3 finish and store.  The four lanes of a group hold the same
+// (m, l), so each computes its splits' weights itself instead of fetching them from a neighbour.
+#ifndef PA_COMBINE_XCD
+#define PA_COMBINE_XCD 1
+#endif
+#ifndef PA_COMBINE_DS
+#define PA_COMBINE_DS 16
+#endif
+template <int HD, int DS>
+__global__ __launch_bounds__(64) void pa_combine_wave_kernel(AttnParams p) {
+  constexpr int SL = HD / DS, LPG = DS / 4, NG = 64 / LPG, CH = (272 + NG - 1) / NG;     // CH splits per lane and chunk: NG x CH >= 272 (256 + the own-row partial)
+  // dispatch id i runs on XCD i % 8: XCD k takes the contiguous slice range [k n / 8, (k + 1) n / 8), so the slices that
+  // share the 128-byte lines of a partial row (two 16-dim slices a line) read them through one L2
+  uint32_t wg = blockIdx.x;
+  if (PA_COMBINE_XCD && gridDim.x % 8 == 0) wg = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+  const uint32_t h = wg / SL, dq = wg % SL, col = blockIdx.y, lane = threadIdx.x;
+  const uint32_t col_end = p.sel ? min(p.sel[col * p.sel_stride], p.sel_max) : p.base_pos + col + 1 - p.self_row;
   const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
-  const uint32_t grp = tid >> 4, l4 = tid & 15;
-  const float* po = p.part_o + base * HD + dq * 64 + 4 * l4;
+  const uint32_t grp = lane / LPG, l4 = lane % LPG;
+  const float* po = p.part_o + base * HD + dq * DS + 4 * l4;
+  const float2* pml = (const float2*)p.part_ml + base;
   const f4 zero = {0.f, 0.f, 0.f, 0.f};
   f4 ov[CH];
+  float2 mlv[CH];
 #pragma unroll
   for (int k = 0; k < CH; k++) {
-    const uint32_t s = grp + 16 * k;
+    const uint32_t s = grp + NG * k;
+    mlv[k] = s < ns ? pml[s] : make_float2(NEG_INF, 0.f);
     ov[k] = s < ns ? *(const f4*)(po + (size_t)s * HD) : zero;
   }
-  // the gate of this thread's output dims (only the 16 writer threads need it) goes out with the first loads
-  const uint32_t d_out = dq * 64 + 4 * (tid & 15);
+  const uint32_t d_out = dq * DS + 4 * l4;
   f4 gt = zero;
-  if (p.gate && tid < 16) gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d_out);
-  // (m, l) of this thread's first two splits; further ones (more than 512 splits) in the loops below
-  const float2 ml0 = tid < ns ? *(const float2*)(p.part_ml + (base + tid) * 2) : make_float2(NEG_INF, 0.f);
-  const float2 ml1 = tid + 256 < ns ? *(const float2*)(p.part_ml + (base + tid + 256) * 2) : make_float2(NEG_INF, 0.f);
-  float lm = fmaxf(ml0.x, ml1.x);
-  for (uint32_t s = tid + 512; s < ns; s += 256) lm = fmaxf(lm, p.part_ml[(base + s) * 2]);
-  // maximum: xor-shuffle tree inside each wave, then the 4 waves' values in wave order
+  if (p.gate && lane < LPG) gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d_out);
+  float M = NEG_INF;
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) lm = fmaxf(lm, __shfl_xor(lm, o, 64));
-  if ((tid & 63) == 0) red[tid >> 6] = lm;
-  __syncthreads();
-  const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-  float ll = 0.f;
-  if (tid < ns) { const float w = __expf(ml0.x - M); wl[tid] = w; ll = ml0.y * w; }
-  if (tid + 256 < ns) { const float w = __expf(ml1.x - M); wl[tid + 256] = w; ll += ml1.y * w; }
-  for (uint32_t s = tid + 512; s < ns; s += 256) {
-    const float w = __expf(p.part_ml[(base + s) * 2] - M);
-    wl[s] = w;
-    ll += p.part_ml[(base + s) * 2 + 1] * w;
-  }
+  for (int k = 0; k < CH; k++) M = fmaxf(M, mlv[k].x);
+  for (uint32_t s = grp + NG * CH; s < ns; s += NG) M = fmaxf(M, pml[s].x);        // more than 272 splits
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) ll += __shfl_xor(ll, o, 64);
-  if ((tid & 63) == 0) red[4 + (tid >> 6)] = ll;
-  __syncthreads();
-  const float L = (red[4] + red[5]) + (red[6] + red[7]);
+  for (int o = LPG; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+  float L = 0.f;
   f4 o = zero;
 #pragma unroll
   for (int k = 0; k < CH; k++) {
-    const uint32_t s = grp + 16 * k;
-    if (s < ns) o += ov[k] * wl[s];
+    const float w = __expf(mlv[k].x - M);        // -inf for a split past the column's end: weight 0
+    L += mlv[k].y * w;
+    o += ov[k] * w;
   }
-  for (uint32_t s0 = 16 * CH; s0 < ns; s0 += 16 * CH) {          // contexts with more than 272 splits
+  for (uint32_t s0 = NG * CH; s0 < ns; s0 += NG * CH) {
 #pragma unroll
     for (int k = 0; k < CH; k++) {
-      const uint32_t s = s0 + grp + 16 * k;
+      const uint32_t s = s0 + grp + NG * k;
+      mlv[k] = s < ns ? pml[s] : make_float2(NEG_INF, 0.f);
       ov[k] = s < ns ? *(const f4*)(po + (size_t)s * HD) : zero;
     }
 #pragma unroll
     for (int k = 0; k < CH; k++) {
-      const uint32_t s = s0 + grp + 16 * k;
-      if (s < ns) o += ov[k] * wl[s];
+      const float w = __expf(mlv[k].x - M);
+      L += mlv[k].y * w;
+      o += ov[k] * w;
     }
   }
-  ored[tid] = o;
-  __syncthreads();
-  if (tid < 16) {
-    f4 t = ored[tid];
 #pragma unroll
-    for (int i = 1; i < 16; i++) t += ored[i * 16 + tid];
-    f4 r = ns ? t / L : zero;                      // an empty gather list: a column of zeros
-    const uint32_t d = d_out;
+  for (int x = LPG; x < 64; x <<= 1) {
+    L += __shfl_xor(L, x, 64);
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] += __shfl_xor(o[i], x, 64);
+  }
+  if (lane < LPG) {
+    f4 r = ns ? o / L : zero;                      // an empty gather list: a column of zeros
     if (p.gate) {
 #pragma unroll
       for (int i = 0; i < 4; i++) r[i] *= 1.f / (1.f + __expf(-gt[i]));
     }
     if (p.out_f16) {
       const h4 hv = { (_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3] };
-      *(h4*)((_Float16*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + d) = hv;
+      *(h4*)((_Float16*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + d_out) = hv;
     } else {
-      *(f4*)((float*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + d) = r;
+      *(f4*)((float*)p.out + (size_t)col * p.out_stride + (size_t)h * HD + d_out) = r;
     }
   }
 }
@@ -1022,7 +1040,18 @@ static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipS
 }
 
 template <int HD>
-static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
+static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
+#ifdef PA_DEV
+  if (waves == 8 && !p.k_scale) {
+    switch (nb) {
+      case 1: return launch_decode_t<HD, 1, 8, false>(p, col_groups, s, t);
+      case 2: return launch_decode_t<HD, 2, 8, false>(p, col_groups, s, t);
+      case 4: if constexpr (HD == 128) return launch_decode_t<HD, 4, 8, false>(p, col_groups, s, t);
+      default: return hipErrorInvalidValue;
+    }
+  }
+#endif
+  if (waves != 4) return hipErrorInvalidValue;
   if (p.k_scale) {                                // int8 caches
     switch (nb) {
       case 1: return launch_decode_t<HD, 1, 4, false, false, true>(p, col_groups, s, t);
@@ -1042,9 +1071,8 @@ static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t co
 }
 
 hipError_t pa_launch_decode(const AttnParams& p, uint32_t hd, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
-  if (waves != 4) return hipErrorInvalidValue;
-  if (hd == 256) return launch_decode_hd<256>(p, nb, col_groups, s, t);
-  if (hd == 128) return launch_decode_hd<128>(p, nb, col_groups, s, t);
+  if (hd == 256) return launch_decode_hd<256>(p, nb, waves, col_groups, s, t);
+  if (hd == 128) return launch_decode_hd<128>(p, nb, waves, col_groups, s, t);
   return hipErrorInvalidValue;
 }
 
@@ -1089,9 +1117,8 @@ hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s) {
     else hipLaunchKernelGGL(pa_combine_wide_kernel<128>, grid, dim3(256), 0, s, p);
     return hipGetLastError();
   }
-  const size_t lds = (size_t)p.slots * sizeof(float);
-  if (hd == 256) hipLaunchKernelGGL(pa_combine_kernel<256>, dim3(p.n_heads * 4, p.n_cols), dim3(256), lds, s, p);
-  else if (hd == 128) hipLaunchKernelGGL(pa_combine_kernel<128>, dim3(p.n_heads * 2, p.n_cols), dim3(256), lds, s, p);
+  if (hd == 256) hipLaunchKernelGGL((pa_combine_wave_kernel<256, PA_COMBINE_DS>), dim3(p.n_heads * (256 / PA_COMBINE_DS), p.n_cols), dim3(64), 0, s, p);
+  else if (hd == 128) hipLaunchKernelGGL((pa_combine_wave_kernel<128, PA_COMBINE_DS>), dim3(p.n_heads * (128 / PA_COMBINE_DS), p.n_cols), dim3(64), 0, s, p);
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }

@@ -4,21 +4,9 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
-#include <mutex>
 #include <new>
 
 static thread_local std::string g_create_err;
-
-// Scratch of the allocation-free entry point pa_attn_decode_step_noalloc: the split partials of one decode token live
-// in this file-scope device array instead of a buffer the context allocates.  Every GPU the library runs on holds
-// its own copy until the process ends.  Host code never uses the array's name as an address: pa_create looks the
-// device address up once per device (hipGetSymbolAddress with that device current) and everything -- kernel
-// arguments included -- goes through that pointer.
-#define PA_STATIC_SCRATCH_BYTES (8u << 20)
-#define PA_MAX_DEVICES 64
-static __device__ __align__(256) unsigned char scratch[PA_STATIC_SCRATCH_BYTES];
-static void* g_scratch_ptr[PA_MAX_DEVICES];
-static std::mutex g_scratch_mutex;
 
 static int fail(pa_ctx* ctx, int code, const std::string& msg) {
   if (ctx) ctx->err = msg; else g_create_err = msg;
@@ -79,17 +67,6 @@ extern "C" int pa_create(const pa_config* cfg, pa_ctx** out) {
     delete ctx; return fail(nullptr, PA_ERR_UNSUPPORTED, m);
   }
   ctx->n_cu = pr.multiProcessorCount;
-  if (ctx->device < 0 || ctx->device >= PA_MAX_DEVICES) { delete ctx; return fail(nullptr, PA_ERR_UNSUPPORTED, "pa_create: device ordinal beyond the library's table"); }
-  {
-    // this device's address of the static scratch array (the device is current: hipGetDevice above)
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (!g_scratch_ptr[ctx->device]) {
-      void* ptr = nullptr;
-      if ((e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) != hipSuccess || !ptr) { delete ctx; return fail_hip(nullptr, e, "pa_create: hipGetSymbolAddress(scratch)"); }
-      g_scratch_ptr[ctx->device] = ptr;
-    }
-    ctx->static_scratch = g_scratch_ptr[ctx->device];
-  }
   if ((e = pa_prepare_decode_step(c.head_dim, (c.flags & PA_FLAG_KV_Q8) != 0)) != hipSuccess) { delete ctx; return fail_hip(nullptr, e, "pa_create: kernel set-up"); }
   const size_t qbytes = (size_t)c.max_cols * c.n_heads * c.head_dim * sizeof(float);
   std::vector<float> freq(c.n_rot / 2);
@@ -315,7 +292,11 @@ extern "C" int pa_kv_store(pa_ctx* ctx, uint32_t layer, const float* d_k, uint32
 static bool plan_self_row(const pa_plan& pl) { return pl.kernel == 0 && pl.slots == pl.n_splits + 1; }
 // wgs (optional): splits per kv head and column group that fit the chip at once; the single-round kernel dispatches
 // the workgroups of further splits (a short remainder) last.
-static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, bool self_ok = true, uint32_t* wgs = nullptr) {
+// rows_cap (optional): at most this many stacked rows per workgroup (16 or 32) instead of the table's choice;
+// one_split: the whole context as one split per workgroup -- with no own-row partial the kernel then writes the
+// output itself (no partials, no merge launch).  Both are what plan_prefill asks for on small chunks.
+static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, bool self_ok = true, uint32_t* wgs = nullptr,
+                       uint32_t rows_cap = 0, bool one_split = false) {
   const pa_config& c = ctx->cfg;
   const uint32_t G = c.n_heads / c.n_kv_heads;
   static const uint32_t floor_tiles[5] = {1, 1, 4, 6, 8};     // tiles per wave, by row blocks
@@ -329,10 +310,15 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
     const uint32_t splits48 = ceil_div(base_pos + n_cols, 32) / (floor_tiles[3] * 4);
     if (g48 < g32 && !ctx->decode_splits_override && (uint64_t)splits48 * c.n_kv_heads * g48 >= (uint64_t)ctx->n_cu) max_rows = 48;
   }
+  if (rows_cap) max_rows = rows_cap;
   uint32_t cw = n_cols, groups = 1;
   if (n_cols * G > max_rows) { cw = max_rows / G; if (cw == 0) return PA_ERR_UNSUPPORTED; groups = ceil_div(n_cols, cw); }
-  const uint32_t nb = ceil_div(cw * G, 16);
-  const uint32_t W = 4;
+  uint32_t nb = ceil_div(cw * G, 16);
+  uint32_t W = 4;
+#ifdef PA_DEV
+  if (getenv("POOLED_DEV_W") && n_cols > 1) W = 8;
+  if (getenv("POOLED_DEV_NB") && n_cols > 1) { max_rows = 16 * atoi(getenv("POOLED_DEV_NB")); cw = n_cols; groups = 1; if (n_cols * G > max_rows) { cw = max_rows / G; groups = ceil_div(n_cols, cw); } nb = ceil_div(cw * G, 16); }
+#endif
   const uint32_t self = self_ok && n_cols == 1 ? 1 : 0;
   const uint32_t seq_max = std::max(base_pos + n_cols - self, 1u);   // streamed rows (position 0 alone: one empty split)
   const uint32_t tiles = ceil_div(seq_max, 32);
@@ -340,12 +326,13 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   uint32_t target = ctx->decode_splits_override ? ctx->decode_splits_override
                                                 : std::max(1u, (occ * (uint32_t)ctx->n_cu) / (c.n_kv_heads * groups));
   uint32_t tpw = std::max(ceil_div(tiles, target * W), ctx->decode_splits_override ? 1u : floor_tiles[nb]);
+  if (one_split) tpw = std::max(ceil_div(tiles, W), 1u);
   uint32_t sl = 32 * W * tpw, ns = ceil_div(seq_max, sl);
   // A context a little past target x split_len (a 32K context plus the token being decoded) would double the
   // split length and leave half the workgroup slots empty, or spill a near-empty split into a second round of
   // workgroups.  The last split takes the remainder instead (the kernels treat split n_splits - 1 as open-ended),
   // as long as that is less than one more split.
-  if (!ctx->decode_splits_override && tpw > floor_tiles[nb]) {
+  if (!ctx->decode_splits_override && !one_split && tpw > floor_tiles[nb]) {
     const uint32_t tpw_lo = std::max(tiles / (target * W), floor_tiles[nb]), sl_lo = 32 * W * tpw_lo;
     if ((uint64_t)seq_max < (uint64_t)(target + 1) * sl_lo) { sl = sl_lo; ns = std::max(1u, std::min(target, seq_max / sl_lo)); }
     // one tile per wave: up to an eighth more splits than slots stay single-round splits (their workgroups start as
@@ -371,12 +358,34 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
   const uint32_t G = c.n_heads / c.n_kv_heads;
   const uint32_t max_rows_sk = c.head_dim == 256 ? 32u : 64u;
   if (n_cols * G <= max_rows_sk) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
+  // pa_set_prefill_tile: 2 = never the matrix-core kernel (where the split-K kernel can hold a column's heads),
+  // 1 = always (the two table rules below are skipped), 0 = the table
+  if (ctx->prefill_tile_mode == 2 && max_rows_sk >= G) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
+  const bool table = ctx->prefill_tile_mode == 0;
   // A chunk of a few column groups over a long context (the reference's own prefill passes are 16 columns wide) is
   // bound by the K/V stream, not by the matrix cores: the split-K kernel serves it in column groups, whose workgroups
   // share the stream through L2, for as long as groups x K/V bytes stays below what the MFMA kernel's fixed costs
   // (Q staging, one partial per split and row, the merge) amount to.  Measured crossover on the MoE and 27B shapes
   // at 32K - 64K rows: about 1.4 GB of L2-level K/V traffic; below 4096 rows both kernels take 25 - 40 us.
-  if (n_cols * G <= 512 && base_pos + n_cols >= 4096 && max_rows_sk >= G) {
+#ifdef PA_DEV
+  if (getenv("POOLED_DEV_SK") && max_rows_sk >= G) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
+#endif
+  // A small chunk (the first chunks of a prompt, a 512-column chunk over a 2K context): the matrix-core kernel's
+  // 256-row workgroups leave most CUs idle unless the chunk is also split over the context, and then the partials
+  // (a row of head_dim floats per split and stacked row) and the merge launch cost more than the attention itself.
+  // Below about 8 GFLOP of causal work the split-K kernel serves the chunk in one launch instead: 16- or 32-row
+  // workgroups (the larger that still gives every CU a workgroup), each over the whole context of its columns,
+  // writing the normalised, gated output itself.  Measured crossover (us per call, this path vs the matrix-core
+  // kernel): dense shape 256 columns from position 0: 6.3 vs 16.8, 512 columns at 1536: 25 vs 32, 2048 from 0: 48 vs
+  // 47; MoE shape 256 from 0: 11 vs 33, 512 from 0: 21 vs 36, 1024 from 0: 52 vs 44.
+  {
+    const double flops = 4.0 * c.n_heads * c.head_dim * ((double)n_cols * base_pos + 0.5 * (double)n_cols * (n_cols + 1));
+    if (table && flops <= 8.0e9 && G <= 16 && !ctx->decode_splits_override) {
+      const uint32_t rows = G <= 32 && (uint64_t)ceil_div(n_cols, 32 / G) * c.n_kv_heads >= (uint64_t)ctx->n_cu ? 32u : 16u;
+      return plan_decode(ctx, base_pos, n_cols, pl, true, wgs, rows, true);
+    }
+  }
+  if (table && n_cols * G <= 512 && base_pos + n_cols >= 4096 && max_rows_sk >= G) {
     pa_plan sk; uint32_t sk_wgs = 0;
     const uint64_t kv_bytes = 2ull * (base_pos + n_cols) * c.n_kv_heads * c.head_dim * (kv_q8(ctx) ? 1 : 2);
     if (plan_decode(ctx, base_pos, n_cols, &sk, true, &sk_wgs) == PA_OK && (uint64_t)sk.col_groups * kv_bytes <= 1400000000ull) {
@@ -401,6 +410,12 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
 extern "C" int pa_plan_query(const pa_ctx* ctx, int kind, uint32_t base_pos, uint32_t n_cols, pa_plan* out) {
   if (!ctx || !out || n_cols == 0) return PA_ERR_INVALID;
   return kind == 0 ? plan_decode(ctx, base_pos, n_cols, out) : plan_prefill(ctx, base_pos, n_cols, out);
+}
+extern "C" int pa_set_prefill_tile(pa_ctx* ctx, int mode) {
+  if (!ctx) return PA_ERR_INVALID;
+  if (mode < 0 || mode > 2) return fail(ctx, PA_ERR_INVALID, "pa_set_prefill_tile: mode must be 0 (table), 1 (always) or 2 (never)");
+  ctx->prefill_tile_mode = mode;
+  return PA_OK;
 }
 extern "C" int pa_set_decode_splits(pa_ctx* ctx, uint32_t splits) {
   if (!ctx) return PA_ERR_INVALID;
@@ -487,7 +502,9 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   rc = kind == 0 ? plan_decode(ctx, base_pos, n_cols, &pl, true, &n_wgs) : plan_prefill(ctx, base_pos, n_cols, &pl, &n_wgs);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
-  const bool direct = pl.kernel == 1 && pl.n_splits == 1;     // the prefill kernel writes the output itself
+  // one split and no own-row partial: the kernel writes the output itself (the prefill kernel, or the split-K kernel's
+  // tile loop: its single-round form always leaves a partial)
+  const bool direct = pl.n_splits == 1 && !plan_self_row(pl) && (pl.kernel == 1 || pl.split_len != 32 * pl.waves || pl.row_blocks > 1);
   if (!direct && (rc = ensure_partials(ctx, n_cols, pl.slots))) return rc;
   AttnParams p; memset(&p, 0, sizeof p);
   p.q = d_q; p.gate = d_gate; p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
@@ -517,6 +534,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   }
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
   p.self_row = plan_self_row(pl) ? 1 : 0;
+  p.direct_out = direct && pl.kernel == 0 ? 1 : 0;
   p.n_wgs = pl.kernel == 0 ? n_wgs : 0;
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
@@ -542,8 +560,7 @@ extern "C" int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, ui
   return attn_common(ctx, "pa_attn_prefill", 1, layer, d_q, q_stride, d_gate, gate_stride, base_pos, n_cols, d_out, out_stride, out_dtype);
 }
 
-// static_scratch: the partials go to the library's file-scope device array and the call allocates nothing
-static int decode_step_common(pa_ctx* ctx, const char* who, bool static_scratch, uint32_t layer, const float* d_q_in, const float* d_k,
+static int decode_step_common(pa_ctx* ctx, const char* who, uint32_t layer, const float* d_q_in, const float* d_k,
                               const float* d_v, const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
   if (!ctx) return PA_ERR_INVALID;
   int rc = check_cols(ctx, who, layer, true, pos, 1);
@@ -562,18 +579,8 @@ static int decode_step_common(pa_ctx* ctx, const char* who, bool static_scratch,
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
   if (pl.row_blocks != 1 || pl.waves != 4 || pl.col_groups != 1 || !plan_self_row(pl)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": plan is not a one-block decode");
-  float* part_o = nullptr; float* part_ml = nullptr;
-  if (static_scratch) {
-    const size_t need_o = ((size_t)c.n_heads * pl.slots * c.head_dim * sizeof(float) + 255) & ~(size_t)255;
-    const size_t need_ml = (size_t)c.n_heads * pl.slots * 2 * sizeof(float);
-    if (need_o + need_ml > PA_STATIC_SCRATCH_BYTES)
-      return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": the split partials of this shape (" + std::to_string(need_o + need_ml) +
-                  " bytes) exceed the library's static scratch (" + std::to_string(PA_STATIC_SCRATCH_BYTES) + " bytes); use pa_attn_decode_step");
-    part_o = (float*)ctx->static_scratch; part_ml = (float*)((unsigned char*)ctx->static_scratch + need_o);
-  } else {
-    if ((rc = ensure_partials(ctx, 1, pl.slots))) return rc;
-    part_o = ctx->part_o; part_ml = ctx->part_ml;
-  }
+  if ((rc = ensure_partials(ctx, 1, pl.slots))) return rc;
+  float* part_o = ctx->part_o; float* part_ml = ctx->part_ml;
   AttnParams p; memset(&p, 0, sizeof p);
   p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
   p.k_scale = ctx->layers[layer].ks; p.v_scale = ctx->layers[layer].vs;
@@ -591,8 +598,8 @@ static int decode_step_common(pa_ctx* ctx, const char* who, bool static_scratch,
   p.f_q_head_stride = c.head_dim * (gated ? 2 : 1); p.n_rot = c.n_rot; p.eps = c.eps;
   p.gate = gated ? d_q_in + c.head_dim : nullptr;
   p.gate_head_stride = p.f_q_head_stride;
-  PaTiming tm;                                        // profiling may create events: not on the allocation-free path
-  if (!static_scratch && (rc = prof_pair(ctx, &tm))) return rc;
+  PaTiming tm;
+  if ((rc = prof_pair(ctx, &tm))) return rc;
   HIPCHK(ctx, pa_launch_decode_step(p, c.head_dim, ctx->stream, &tm));
   HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;
@@ -600,11 +607,7 @@ static int decode_step_common(pa_ctx* ctx, const char* who, bool static_scratch,
 
 extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
                                    const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
-  return decode_step_common(ctx, "pa_attn_decode_step", false, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype);
-}
-extern "C" int pa_attn_decode_step_noalloc(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
-                                           const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
-  return decode_step_common(ctx, "pa_attn_decode_step_noalloc", true, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype);
+  return decode_step_common(ctx, "pa_attn_decode_step", layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype);
 }
 
 // ---- projections (one-token passes) -------------------------------------------------------------

@@ -44,6 +44,8 @@ struct AttnParams {
   uint32_t self_row;                          // 1: one-column decode whose own row base_pos is a partial of its own (slot
                                               // = number of splits that hold rows) instead of a streamed row; else 0
   int out_f16;
+  uint32_t direct_out;                        // tile-loop split-K kernel with one split and no own-row partial: the workgroup
+                                              // normalises, gates and stores the output itself (no partials, no merge launch)
   float scale;                                // 1 / sqrt(hd)
   unsigned long long* trace;                  // per-wave timestamps when built with PA_TRACE (else unused, nullptr)
   uint32_t gate_head_stride;                  // floats between consecutive heads in gate (head_dim, or 2*head_dim
@@ -162,9 +164,9 @@ struct pa_ctx {
   void* chunk_buf = nullptr;    // pa_attn_layer_prefill: xn f16 [cols][dim], qkv f32 [cols][rows], attnOut f16 [cols][nH*hd]
   size_t chunk_buf_bytes = 0;
   uint16_t* wide_k = nullptr; uint16_t* wide_v = nullptr;   // int8 caches: f16 staging cache of one layer for the prefill kernel
-  void* static_scratch = nullptr;   // this device's copy of the library's file-scope scratch array (pa_attn_decode_step_noalloc)
   std::vector<void*> retired;   // outgrown scratch blocks, kept until pa_destroy (a recorded launch may still name them)
   uint32_t decode_splits_override = 0;
+  int prefill_tile_mode = 0;    // pa_set_prefill_tile: 0 table, 1 always the matrix-core kernel, 2 never
   // timing
   hipEvent_t t0 = nullptr, t1 = nullptr;
   bool profiling = false;

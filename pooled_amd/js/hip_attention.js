@@ -22,7 +22,7 @@ const PA_W_F32 = 0, PA_W_Q8_0 = 1, PA_W_Q4_0 = 2;             // weight kinds of
 
 class HipAttention {
   // opts: { nH, nKV, hd, nRot, ropeTheta, eps, maxSeq, nLayers, batchCols, qkNorm = true, gate = false, outF16 = false,
-  //         kvQ8 = false, fusedStep = true, verifyExact = false }
+  //         kvQ8 = false, fusedStep = true, verifyExact = false, attnPrefillTile = "auto" }
   constructor(opts) {
     const nH = opts.nH, nKV = opts.nKV, hd = opts.hd;
     if (!(nH > 0 && nKV > 0 && nH % nKV === 0)) throw new Error("HipAttention: nH must be a positive multiple of nKV");
@@ -34,7 +34,7 @@ class HipAttention {
     this.outDtype = opts.outF16 ? PA_OUT_F16 : PA_OUT_F32;
     this.fusedStep = opts.fusedStep !== false;
     // engine fields the attention dispatch reads (engine/qwen35.js:366, :416-419): always the f16-KV split-K path here
-    this.flash = true; this.attnDecode = "v2"; this.attnPrefillTile = true;
+    this.flash = true; this.attnDecode = "v2"; this.attnPrefillTile = opts.attnPrefillTile !== false;
     this._snapNow = null;                                          // set by a verify pass (engine/qwen35.js:2960-2965)
     this.pos = 0;
     this.kvQ8 = !!opts.kvQ8;                                       // int8 caches (engine option kvQ8)
@@ -46,6 +46,10 @@ class HipAttention {
     // a readable throw at create, like the engine's KV binding check (engine/qwen35.js:378-383)
     this.ctx = addon.create({ nH: nH, nKV: nKV, hd: hd, nRot: this.dims.nRot, ropeTheta: opts.ropeTheta, eps: opts.eps,
       maxSeq: opts.maxSeq, nLayers: opts.nLayers || 1, maxCols: this.NC, flags: flags });
+    // the engine's attnPrefillTile option (engine/qwen35.js:389-401): undefined / "auto" = the library's table picks the
+    // kernel of a prefill chunk, true = always the matrix-core kernel, false = full-width passes go through the decode
+    // entry point like every other pass
+    if (opts.attnPrefillTile === true) addon.setPrefillTile(this.ctx, 1);
     this.kvBufBytes = opts.maxSeq * this.dims.kvDim * 2;
     this.layers = [];
     for (let i = 0; i < (opts.nLayers || 1); i++) { addon.layerAlloc(this.ctx, i); this.layers.push({ index: i, qNorm: null, kNorm: null }); }

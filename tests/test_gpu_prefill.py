@@ -11,7 +11,9 @@ pytestmark = pytest.mark.gpu
 NAN16 = 0x7E00
 
 
-def _prefill(cfg, base, n, seed, max_seq=None, gate=True, out_dtype=0, check_rows=None, k_scale=1.0):
+def _prefill(cfg, base, n, seed, max_seq=None, gate=True, out_dtype=0, check_rows=None, k_scale=1.0, tile=1):
+    """tile: pa_set_prefill_tile mode -- 1 (default here) forces the matrix-core kernel, which the table would not pick
+    for the small chunks most of these cases are; 0 = the table's choice."""
     rng = np.random.default_rng(seed)
     max_seq = max_seq or base + n + 7
     k16, v16 = random_cache(cfg, max_seq, seed=seed + 1, k_scale=k_scale)
@@ -25,6 +27,7 @@ def _prefill(cfg, base, n, seed, max_seq=None, gate=True, out_dtype=0, check_row
         K, V = k16.copy(), v16.copy()
         K[base + n:] = NAN16; V[base + n:] = NAN16        # rows past the chunk's end must never be used
         pa.kv_write(0, 0, 0, K); pa.kv_write(0, 1, 0, V)
+        pa.set_prefill_tile(tile)
         plan = pa.plan("prefill", base, n)
         got = pa.run_attn("prefill", 0, q, base, gate=gt, out_dtype=out_dtype)
     finally:
@@ -72,9 +75,39 @@ def test_prefill_split_path_and_f16_out():
 def test_prefill_narrow_chunk_on_a_long_context_takes_the_stream_kernel(shape, base, n):
     """Chunks of at most 512 stacked rows over 4096 or more cache rows (the reference's own passes are 16 columns wide)
     are bound by the K/V stream: the plan hands them to the split-K kernel in column groups."""
-    got, ref, plan = _prefill(SHAPES[shape], base, n, seed=base + n)
+    got, ref, plan = _prefill(SHAPES[shape], base, n, seed=base + n, tile=0)
     assert plan["kernel"] == 0 and plan["col_groups"] > 1
     assert_parity(got, ref, "narrow chunk")
+
+
+@pytest.mark.parametrize("shape,base,n,rows", [
+    ("qwen3_1p7b", 0, 256, 16), ("qwen3_1p7b", 0, 512, 32), ("qwen3_1p7b", 1536, 512, 32), ("qwen36_moe", 0, 256, 16), ("qwen36_moe", 0, 512, 32),
+    ("qwen38_27b", 0, 300, 12), ("qwen36_moe", 77, 129, 16), ("qwen3_1p7b", 5, 40, 16),
+])
+def test_prefill_small_chunk_takes_the_stream_kernel_in_one_launch(shape, base, n, rows):
+    """Chunks of little causal work (the first chunks of a prompt, configuration 2's 512 columns over 2K rows): the table
+    hands them to the split-K kernel as one split per workgroup -- 16- or 32-row workgroups over the whole context of
+    their columns -- which writes the gated output itself: no partials, no merge launch.  Rows past the chunk are NaN;
+    f16 and f32 output."""
+    cfg = SHAPES[shape]
+    G = cfg["n_heads"] // cfg["n_kv_heads"]
+    for out_dtype in (0, PA_OUT_F16):
+        got, ref, plan = _prefill(cfg, base, n, seed=base + n + 7, tile=0, out_dtype=out_dtype)
+        assert plan["kernel"] == 0 and plan["n_splits"] == 1 and plan["slots"] == 1 and plan["cols_per_group"] * G == rows, plan
+        assert_parity(got, ref, "small chunk %s base %d n %d" % (shape, base, n))
+
+
+def test_prefill_tile_override():
+    """pa_set_prefill_tile (the reference's attnPrefillTile option, engine/qwen35.js:389-401): 1 forces the matrix-core
+    kernel, 2 the split-K kernel, 0 is the table; all three give the same result within tolerance."""
+    cfg = SHAPES["qwen36_moe"]
+    outs = {}
+    for mode, kernel in ((0, 0), (1, 1), (2, 0)):
+        got, ref, plan = _prefill(cfg, 900, 120, seed=3, tile=mode)
+        assert plan["kernel"] == kernel, (mode, plan)
+        assert_parity(got, ref, "tile mode %d" % mode)
+        outs[mode] = got
+    assert np.abs(outs[1] - outs[2]).max() <= 1e-3
 
 
 def test_prefill_peaked_softmax():

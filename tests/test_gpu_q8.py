@@ -83,7 +83,9 @@ def test_q8_verify_block_prefill_chunk_and_slots():
         for w, a in enumerate((kq, vq, ks, vs)):
             pa.kv_write(0, w, 0, a)
         assert_parity(pa.run_attn("decode", 0, q[:8], base, gate=gate[:8]), ref[:8], "q8 verify block")
-        # a narrow chunk runs on the split-K kernel, a wide one on the MFMA prefill kernel over rows widened to f16
+        # a narrow chunk runs on the split-K kernel, a wide one on the MFMA prefill kernel over rows widened to f16 (forced:
+        # the table would serve a chunk this small on the split-K kernel too)
+        pa.set_prefill_tile(1)
         assert pa.plan("prefill", base, 4)["kernel"] == 0 and pa.plan("prefill", base, n)["kernel"] == 1
         assert_parity(pa.run_attn("prefill", 0, q[:4], base, gate=gate[:4]), ref[:4], "q8 narrow prefill chunk")
         assert_parity(pa.run_attn("prefill", 0, q, base, gate=gate, out_dtype=PA_OUT_F16).astype(np.float32), ref, "q8 prefill chunk")
@@ -153,6 +155,7 @@ def test_q8_prefill_on_the_matrix_cores(shape, base, n):
             pa.kv_write(0, w, 0, a)
         bad = np.full((64, nKV, hd // 32), np.nan, np.float32)
         pa.kv_write(0, 2, L, bad); pa.kv_write(0, 3, L, bad)
+        pa.set_prefill_tile(1)                       # the matrix-core kernel, whatever the table would pick for the size
         assert pa.plan("prefill", base, n)["kernel"] == 1
         ref = O.attention_values(q, kf, vf, base, gate=gate)
         assert_parity(pa.run_attn("prefill", 0, q, base, gate=gate), ref, "q8 wide prefill %s base %d n %d" % (shape, base, n))

@@ -309,3 +309,37 @@ def test_rmsnorm_closed_forms():
     y = O.rmsnorm(x, np.ones(n, np.float32), 0.0)
     assert abs(np.mean(y.astype(np.float64) ** 2) - 1.0) < 1e-6                      # unit RMS
     assert np.allclose(O.rmsnorm(4.0 * x, w, 0.0), O.rmsnorm(x, w, 0.0), rtol=1e-6)  # scale invariance at eps = 0
+
+
+def test_gemm_f16_pins():
+    """gemm_f16 (the reference's "f16" prefill math, engine/wgsl/gemm.js:31-36) pinned without restating it:
+    unit-vector columns pick the f16-rounded columns of w_dequant (known answers for hand-made blocks whose scales
+    make the products inexact in f16); f16-representable inputs over weights whose dequantised values are already
+    f16 reproduce gemv exactly; the result is linear in x over f16-representable inputs; and an activation that is
+    not f16-representable is rounded before the product (closed form on a one-hot weight row)."""
+    rng = np.random.default_rng(31)
+    d_out, d_in = 5, 64
+    for kind in (O.W_Q8_0, O.W_Q4_0):
+        w = rng.integers(-127, 128, (d_out, d_in)).astype(np.int8) if kind == O.W_Q8_0 else rng.integers(0, 256, (d_out, d_in // 2), dtype=np.uint8)
+        sc = rng.uniform(0.01, 0.3, (d_out, d_in // 32)).astype(np.float16).view(np.uint16)
+        W = O.w_dequant(kind, w, sc)                                   # exact products int x f16 scale (f64)
+        W16 = W.astype(np.float32).astype(np.float16).astype(np.float64)
+        assert np.any(W16 != W), "the case is meant to include weights that f16 rounds"
+        # unit vectors pick the rounded columns
+        Y = O.gemm_f16(kind, w, sc, np.eye(d_in, dtype=np.float32))    # [d_in, d_out]
+        assert np.array_equal(Y, W16.T)
+        # linearity over f16-representable inputs (small integers: every product and sum is exact in f64)
+        xa = rng.integers(-8, 9, (3, d_in)).astype(np.float32); xb = rng.integers(-8, 9, (3, d_in)).astype(np.float32)
+        assert np.array_equal(O.gemm_f16(kind, w, sc, xa + xb), O.gemm_f16(kind, w, sc, xa) + O.gemm_f16(kind, w, sc, xb))
+    # weights whose dequantised values are f16-representable (power-of-two scales): gemm_f16 == gemv on f16 inputs
+    w8 = rng.integers(-127, 128, (d_out, d_in)).astype(np.int8)
+    sc2 = np.full((d_out, d_in // 32), 0.125, np.float16).view(np.uint16)
+    x16 = rng.standard_normal((4, d_in)).astype(np.float16).astype(np.float32)
+    want = np.stack([O.gemv(O.W_Q8_0, w8, sc2, x16[c]) for c in range(4)])
+    assert np.array_equal(O.gemm_f16(O.W_Q8_0, w8, sc2, x16), want)
+    # f32 weights: a one-hot row times x returns f16(w) * f16(x)
+    wf = np.zeros((2, 32), np.float32); wf[0, 3] = 1.0 + 2.0 ** -12; wf[1, 7] = 3.0       # 1 + 2^-12 rounds to 1 in f16
+    x = np.zeros((1, 32), np.float32); x[0, 3] = 1.0 + 2.0 ** -11 + 2.0 ** -12; x[0, 7] = 0.1   # rounds up to 1 + 2^-10
+    y = O.gemm_f16(O.W_F32, wf, None, x)
+    assert y[0, 0] == 1.0 + 2.0 ** -10
+    assert y[0, 1] == 3.0 * float(np.float16(0.1))
