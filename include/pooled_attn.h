@@ -171,6 +171,17 @@ int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, uint32_t q_st
  * pa_q_buffer / pa_gate_buffer are not written by this call. */
 int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
                         const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype);
+/* pa_attn_decode_step_noalloc: pa_attn_decode_step for callers that cannot allocate.  No counterpart in the reference;
+ * it exists for callers under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same
+ * arguments, same kernels and the same bits as pa_attn_decode_step, but the split partials go to a file-scope device
+ * array of the library (8 MiB per GPU, held until the process ends; its device address is looked up at pa_create) and
+ * the call makes no hipMalloc / hipFree and creates no events (pa_profile_enable does not see it).  A shape whose
+ * partials -- n_heads x (splits + 1) x (head_dim + 2) floats -- do not fit returns PA_ERR_UNSUPPORTED (the MoE shape
+ * at 32K uses 4.3 MB).  All calls on one GPU share the array, contexts included: calls that overlap on one GPU (two
+ * streams, two contexts) race; calls queued on one stream do not.  Nothing in the array needs clearing between calls:
+ * every partial the merge reads is written by the same call. */
+int pa_attn_decode_step_noalloc(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
+                                const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype);
 /* pa_attn_decode_gather: decode / verify attention where every column attends to a list of cache rows instead of
  * rows [0, base_pos + c] -- the gather mode of the reference's split-K kernel used by its sparse-attention layers:
  * attn_dec_qsa + attn_dec_qsa_combine(_g) (engine/wgsl/attn_dec.js:33-38, :105, :170-183, :246; dispatch

@@ -52,6 +52,7 @@ SYMBOLS = {
     "pa_attn_prefill": (c_int, [vp, u32, f32p, u32, f32p, u32, u32, u32, vp, u32, c_int]),
     "pa_attn_decode_gather": (c_int, [vp, u32, f32p, u32, f32p, u32, vp, u32, u32, u32, vp, u32, c_int]),
     "pa_attn_decode_step": (c_int, [vp, u32, f32p, f32p, f32p, f32p, f32p, u32, vp, c_int]),
+    "pa_attn_decode_step_noalloc": (c_int, [vp, u32, f32p, f32p, f32p, f32p, f32p, u32, vp, c_int]),
     "pa_plan_query": (c_int, [vp, c_int, u32, u32, ctypes.POINTER(PaPlan)]),
     "pa_set_decode_splits": (c_int, [vp, u32]),
     "pa_set_prefill_tile": (c_int, [vp, c_int]),
@@ -233,8 +234,9 @@ class PooledAttn:
         gp = d_gate if isinstance(d_gate, (int, type(None))) else d_gate.ptr
         self._chk(fn(self.ctx, layer, qp, q_stride, gp, gate_stride, base_pos, n_cols, d_out.ptr, out_stride, out_dtype))
 
-    def attn_decode_step(self, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype=PA_OUT_F32):
-        self._chk(self.L.pa_attn_decode_step(self.ctx, layer, d_q_in.ptr, d_k.ptr, d_v.ptr, d_qw.ptr if d_qw else None,
+    def attn_decode_step(self, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype=PA_OUT_F32, noalloc=False):
+        fn = self.L.pa_attn_decode_step_noalloc if noalloc else self.L.pa_attn_decode_step
+        self._chk(fn(self.ctx, layer, d_q_in.ptr, d_k.ptr, d_v.ptr, d_qw.ptr if d_qw else None,
                                              d_kw.ptr if d_kw else None, pos, d_out.ptr, out_dtype))
 
     def q_buffer_ptr(self):

@@ -4,9 +4,21 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 static thread_local std::string g_create_err;
+
+// Scratch of the allocation-free entry point pa_attn_decode_step_noalloc: the split partials of one decode token live
+// in this file-scope device array instead of a buffer the context allocates.  Every GPU the library runs on holds
+// its own copy until the process ends.  Host code never uses the array's name as an address: pa_create looks the
+// device address up once per device (hipGetSymbolAddress with that device current) and everything -- kernel
+// arguments included -- goes through that pointer.
+#define PA_STATIC_SCRATCH_BYTES (8u << 20)
+#define PA_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[PA_STATIC_SCRATCH_BYTES];
+static void* g_scratch_ptr[PA_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
 
 static int fail(pa_ctx* ctx, int code, const std::string& msg) {
   if (ctx) ctx->err = msg; else g_create_err = msg;
@@ -67,6 +79,17 @@ extern "C" int pa_create(const pa_config* cfg, pa_ctx** out) {
     delete ctx; return fail(nullptr, PA_ERR_UNSUPPORTED, m);
   }
   ctx->n_cu = pr.multiProcessorCount;
+  if (ctx->device < 0 || ctx->device >= PA_MAX_DEVICES) { delete ctx; return fail(nullptr, PA_ERR_UNSUPPORTED, "pa_create: device ordinal beyond the library's table"); }
+  {
+    // this device's address of the static scratch array (the device is current: hipGetDevice above)
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[ctx->device]) {
+      void* ptr = nullptr;
+      if ((e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) != hipSuccess || !ptr) { delete ctx; return fail_hip(nullptr, e, "pa_create: hipGetSymbolAddress(scratch)"); }
+      g_scratch_ptr[ctx->device] = ptr;
+    }
+    ctx->static_scratch = g_scratch_ptr[ctx->device];
+  }
   if ((e = pa_prepare_decode_step(c.head_dim, (c.flags & PA_FLAG_KV_Q8) != 0)) != hipSuccess) { delete ctx; return fail_hip(nullptr, e, "pa_create: kernel set-up"); }
   const size_t qbytes = (size_t)c.max_cols * c.n_heads * c.head_dim * sizeof(float);
   std::vector<float> freq(c.n_rot / 2);
@@ -560,7 +583,8 @@ extern "C" int pa_attn_prefill(pa_ctx* ctx, uint32_t layer, const float* d_q, ui
   return attn_common(ctx, "pa_attn_prefill", 1, layer, d_q, q_stride, d_gate, gate_stride, base_pos, n_cols, d_out, out_stride, out_dtype);
 }
 
-static int decode_step_common(pa_ctx* ctx, const char* who, uint32_t layer, const float* d_q_in, const float* d_k,
+// static_scratch: the partials go to the library's file-scope device array and the call allocates nothing
+static int decode_step_common(pa_ctx* ctx, const char* who, bool static_scratch, uint32_t layer, const float* d_q_in, const float* d_k,
                               const float* d_v, const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
   if (!ctx) return PA_ERR_INVALID;
   int rc = check_cols(ctx, who, layer, true, pos, 1);
@@ -579,8 +603,18 @@ static int decode_step_common(pa_ctx* ctx, const char* who, uint32_t layer, cons
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
   if (pl.row_blocks != 1 || pl.waves != 4 || pl.col_groups != 1 || !plan_self_row(pl)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": plan is not a one-block decode");
-  if ((rc = ensure_partials(ctx, 1, pl.slots))) return rc;
-  float* part_o = ctx->part_o; float* part_ml = ctx->part_ml;
+  float* part_o = nullptr; float* part_ml = nullptr;
+  if (static_scratch) {
+    const size_t need_o = ((size_t)c.n_heads * pl.slots * c.head_dim * sizeof(float) + 255) & ~(size_t)255;
+    const size_t need_ml = (size_t)c.n_heads * pl.slots * 2 * sizeof(float);
+    if (need_o + need_ml > PA_STATIC_SCRATCH_BYTES)
+      return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": the split partials of this shape (" + std::to_string(need_o + need_ml) +
+                  " bytes) exceed the library's static scratch (" + std::to_string(PA_STATIC_SCRATCH_BYTES) + " bytes); use pa_attn_decode_step");
+    part_o = (float*)ctx->static_scratch; part_ml = (float*)((unsigned char*)ctx->static_scratch + need_o);
+  } else {
+    if ((rc = ensure_partials(ctx, 1, pl.slots))) return rc;
+    part_o = ctx->part_o; part_ml = ctx->part_ml;
+  }
   AttnParams p; memset(&p, 0, sizeof p);
   p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
   p.k_scale = ctx->layers[layer].ks; p.v_scale = ctx->layers[layer].vs;
@@ -598,8 +632,8 @@ static int decode_step_common(pa_ctx* ctx, const char* who, uint32_t layer, cons
   p.f_q_head_stride = c.head_dim * (gated ? 2 : 1); p.n_rot = c.n_rot; p.eps = c.eps;
   p.gate = gated ? d_q_in + c.head_dim : nullptr;
   p.gate_head_stride = p.f_q_head_stride;
-  PaTiming tm;
-  if ((rc = prof_pair(ctx, &tm))) return rc;
+  PaTiming tm;                                        // profiling may create events: not on the allocation-free path
+  if (!static_scratch && (rc = prof_pair(ctx, &tm))) return rc;
   HIPCHK(ctx, pa_launch_decode_step(p, c.head_dim, ctx->stream, &tm));
   HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;
@@ -607,7 +641,11 @@ static int decode_step_common(pa_ctx* ctx, const char* who, uint32_t layer, cons
 
 extern "C" int pa_attn_decode_step(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
                                    const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
-  return decode_step_common(ctx, "pa_attn_decode_step", layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype);
+  return decode_step_common(ctx, "pa_attn_decode_step", false, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype);
+}
+extern "C" int pa_attn_decode_step_noalloc(pa_ctx* ctx, uint32_t layer, const float* d_q_in, const float* d_k, const float* d_v,
+                                           const float* d_qw, const float* d_kw, uint32_t pos, void* d_out, int out_dtype) {
+  return decode_step_common(ctx, "pa_attn_decode_step_noalloc", true, layer, d_q_in, d_k, d_v, d_qw, d_kw, pos, d_out, out_dtype);
 }
 
 // ---- projections (one-token passes) -------------------------------------------------------------

@@ -164,6 +164,7 @@ struct pa_ctx {
   void* chunk_buf = nullptr;    // pa_attn_layer_prefill: xn f16 [cols][dim], qkv f32 [cols][rows], attnOut f16 [cols][nH*hd]
   size_t chunk_buf_bytes = 0;
   uint16_t* wide_k = nullptr; uint16_t* wide_v = nullptr;   // int8 caches: f16 staging cache of one layer for the prefill kernel
+  void* static_scratch = nullptr;   // this device's copy of the library's file-scope scratch array (pa_attn_decode_step_noalloc)
   std::vector<void*> retired;   // outgrown scratch blocks, kept until pa_destroy (a recorded launch may still name them)
   uint32_t decode_splits_override = 0;
   int prefill_tile_mode = 0;    // pa_set_prefill_tile: 0 table, 1 always the matrix-core kernel, 2 never
