@@ -312,9 +312,6 @@ def main():
     ap.add_argument("--kv-q8", action="store_true", help="run the C3 decode step on int8 caches (one f32 scale per 32 values) instead of f16")
     ap.add_argument("--no-layer", action="store_true", help="skip the whole-layer leg (projections + attention, pa_attn_layer_decode)")
     ap.add_argument("--other-configs", action="store_true", help="only time configurations 1, 2 and 4 (attention call alone, caches in rotation)")
-    ap.add_argument("--mfma-probe", action="store_true",
-                    help="only run the device probe: sustained f16 MFMA TFLOP/s and shader clock with constant and with random operands")
-    ap.add_argument("--lds-probe", action="store_true", help="only run the device probe of the LDS read rate (bytes per clock and CU)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 10 device-to-device copies of 256 MiB (the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -327,32 +324,6 @@ def main():
     log("library:", L.pa_version().decode())
     if args.other_configs:
         print(json.dumps({"other_configs": other_configs()}))
-        return
-    if args.mfma_probe:
-        # what the f16 matrix pipe sustains on this part, and at which clock: constant vs random operands, after a
-        # warm-up long enough for the clock to settle
-        pa = PooledAttn(C3, 64, n_layers=1, max_cols=1)
-        res = {}
-        for name, rnd in (("constant_operands", 0), ("random_operands", 1), ("random_operands_16x16x32", 2)):
-            for _ in range(3):
-                pa.mfma_probe(rnd, 20000)
-            tf, mhz = pa.mfma_probe(rnd, 60000)
-            res[name] = dict(tflops=round(tf, 1), shader_mhz=round(mhz), frac_of_nominal_peak=round(tf / MFMA_F16_PEAK_TFLOPS, 3))
-            log("mfma probe, %s: %.0f TFLOP/s at %.0f MHz" % (name, tf, mhz))
-        pa.close()
-        print(json.dumps({"mfma_probe": res}))
-        return
-    if args.lds_probe:
-        # what the LDS of a CU delivers to fragment reads, with one and with two wavefronts a SIMD
-        pa = PooledAttn(C3, 64, n_layers=1, max_cols=1)
-        res = {}
-        for name, tr in (("ds_read_b128", 0), ("ds_read_b64_tr_b16", 1)):
-            for waves in (4, 8):
-                bpc = pa.lds_probe(tr, waves, 20000)
-                res["%s_%dwaves" % (name, waves)] = round(bpc, 1)
-                log("lds probe, %s, %d wavefronts a CU: %.1f bytes per clock and CU" % (name, waves, bpc))
-        pa.close()
-        print(json.dumps({"lds_probe_bytes_per_clk_per_cu": res}))
         return
     if args.copy_calibration:
         pa = PooledAttn(C3, 64, n_layers=1, max_cols=1)

@@ -304,22 +304,6 @@ int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uint32_t x_str
 int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
                           const float* d_qw, const float* d_kw, float* d_x, uint32_t x_stride, uint32_t base_pos, uint32_t n_cols);
 
-/* Device probe (measurement infrastructure, no counterpart in the reference): runs back-to-back
- * v_mfma_f32_32x32x16_f16 on every CU for iters x 64 instructions per wavefront, with constant operands
- * (random_operands = 0) or random f16 fragments (1; 2 = the same flops as twice as many v_mfma_f32_16x16x32_f16),
- * and returns the achieved TFLOP/s and the mean shader clock during
- * the kernel (shader clock counter against the 100 MHz wall clock).  Blocks until done.  It tells what the matrix
- * pipe of this part sustains under its power limit, which is what an MFMA-bound kernel's roofline fraction has to
- * be read against. */
-int pa_mfma_probe(pa_ctx* ctx, int random_operands, uint32_t iters, float* tflops, float* shader_mhz);
-
-/* Device probe (measurement infrastructure, no counterpart in the reference): one workgroup of waves_per_cu (1 .. 8)
- * wavefronts per CU reads LDS back to back, conflict-free, with ds_read_b128 (transpose_reads = 0) or with the
- * transpose read ds_read_b64_tr_b16 the V^T fragments use (1), iters x 8 KB per wavefront, and returns the bytes per
- * shader clock and CU it sustained.  Blocks until done.  It tells how far an attention kernel's fragment traffic is
- * from what the LDS delivers. */
-int pa_lds_probe(pa_ctx* ctx, int transpose_reads, uint32_t waves_per_cu, uint32_t iters, float* bytes_per_clk);
-
 /* library / device description, e.g. "pooled_attn 0.1 gfx950 256CU" (storage owned by the library, one buffer per
  * calling thread) */
 const char* pa_version(void);

@@ -13,7 +13,7 @@ LIBDIR = os.path.join(ROOT, "pooled_amd", "lib")
 LIB = os.path.join(LIBDIR, "libpooled_attn.so")
 ADDON = os.path.join(LIBDIR, "pooled_attn.node")
 
-HIP_SOURCES = ["pa_api.hip", "glue_kv.hip", "attn_decode.hip", "attn_prefill.hip", "attn_prefill_wide.hip", "attn_prefill_small.hip", "probe.hip", "proj_gemv.hip", "proj_gemm.hip"]
+HIP_SOURCES = ["pa_api.hip", "glue_kv.hip", "attn_decode.hip", "attn_prefill.hip", "proj_gemv.hip", "proj_gemm.hip"]
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
                # packed-FP32 VALU forms are kept off for all device code
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -21,35 +21,6 @@ HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "
 
 def _hipcc():
     return shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-
-
-def check_hand_allocated_agprs(verbose=False):
-    """attn_prefill_wide.hip keeps its O accumulators in AGPRs that only its inline assembly touches.  The kernel is
-    only correct if the compiler never uses an AGPR of its own (e.g. as a spill slot), so the generated code is
-    scanned: every AGPR reference has to sit inside an assembly block."""
-    asm = os.path.join(LIBDIR, "attn_prefill_wide.s")
-    cmd = [_hipcc()] + HIPCC_FLAGS + ["-I", os.path.join(ROOT, "include"), "-S", "--cuda-device-only",
-                                      os.path.join(CSRC, "attn_prefill_wide.hip"), "-o", asm]
-    if verbose:
-        print(" ".join(cmd))
-    subprocess.run(cmd, check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
-    import re
-    agpr = re.compile(r"(?<![\w.])a(\[\d+(:\d+)?\]|\d+)(?![\w])")
-    inside, bad = False, []
-    with open(asm) as f:
-        for n, line in enumerate(f, 1):
-            if "#ASMSTART" in line:
-                inside = True
-            elif "#ASMEND" in line:
-                inside = False
-            elif not inside:
-                code = line.split(";", 1)[0]
-                if code.strip() and not code.lstrip().startswith(".") and agpr.search(code):
-                    bad.append("%d: %s" % (n, line.rstrip()))
-    os.remove(asm)
-    if bad:
-        raise RuntimeError("compiler-generated AGPR use in attn_prefill_wide.hip (would corrupt the hand-allocated "
-                           "accumulators):\n" + "\n".join(bad[:20]))
 
 
 def build_lib(verbose=False, extra=()):
@@ -70,7 +41,6 @@ def build_lib(verbose=False, extra=()):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
         if out.strip():
             print(out)
-    check_hand_allocated_agprs(verbose)
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     subprocess.check_call(cmd)
     return LIB

@@ -71,8 +71,6 @@ SYMBOLS = {
     "pa_slot_create": (c_int, [vp, u32, u32]),
     "pa_slot_export": (c_int, [vp, u32, u32, c_int, vp]),
     "pa_slot_import": (c_int, [vp, u32, u32, c_int, vp]),
-    "pa_mfma_probe": (c_int, [vp, c_int, u32, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]),
-    "pa_lds_probe": (c_int, [vp, c_int, u32, u32, ctypes.POINTER(ctypes.c_float)]),
     "pa_weight_create": (c_int, [vp, c_int, u32, u32, vp, vp, ctypes.POINTER(vp)]),
     "pa_weight_destroy": (c_int, [vp, vp]),
     "pa_gemv": (c_int, [vp, vp, f32p, f32p, c_int]),
@@ -349,18 +347,6 @@ class PooledAttn:
     def attn_layer_prefill(self, layer, w_qkv, w_o, d_attn_norm_w, d_qw, d_kw, d_x, x_stride, base_pos, n_cols):
         self._chk(self.L.pa_attn_layer_prefill(self.ctx, layer, w_qkv, w_o, d_attn_norm_w.ptr, d_qw.ptr if d_qw else None,
                                                d_kw.ptr if d_kw else None, d_x.ptr, x_stride, base_pos, n_cols))
-
-    def mfma_probe(self, random_operands, iters):
-        """(TFLOP/s, shader MHz) of back-to-back f16 MFMAs on every CU with constant or random operands."""
-        tf, mhz = ctypes.c_float(), ctypes.c_float()
-        self._chk(self.L.pa_mfma_probe(self.ctx, int(random_operands), iters, ctypes.byref(tf), ctypes.byref(mhz)))
-        return tf.value, mhz.value
-
-    def lds_probe(self, transpose_reads, waves_per_cu, iters):
-        """Bytes per shader clock and CU of back-to-back conflict-free LDS reads (ds_read_b128, or the transpose read)."""
-        bpc = ctypes.c_float()
-        self._chk(self.L.pa_lds_probe(self.ctx, int(bool(transpose_reads)), waves_per_cu, iters, ctypes.byref(bpc)))
-        return bpc.value
 
     # ---- numpy convenience used by tests / smoke: whole passes from host arrays ----
     def run_glue_kv(self, layer, q_in, k_in, v_in, qw, kw, base_pos):

@@ -34,14 +34,6 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 #define NEG_INF (-__builtin_inff())
 #define DEC_RESCALE_TH 8.f   // tile loop: a row maximum may pass the reference maximum by this much before O is rescaled
 
-// Optional per-wave timeline (development builds only): lane 0 of every wave stores the 100 MHz wall clock at
-// up to 12 points into p.trace.  Compiled out unless PA_TRACE is defined.
-#ifdef PA_TRACE
-#define PA_TP(k) do { if (p.trace && lane == 0) p.trace[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * W * 12 + wave * 12 + (k)] = wall_clock64(); } while (0)
-#else
-#define PA_TP(k) do { } while (0)
-#endif
-
 static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
   hh4 t = __builtin_amdgcn_ds_read_tr16_b64_v4f16((hh4 __attribute__((address_space(3)))*)p);
   h4 r; __builtin_memcpy(&r, &t, 8); return r;
@@ -188,7 +180,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   // the last split is open-ended: the plan may hand it up to one split length of remainder
   const uint32_t t_end = !SR && sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
   const size_t head_rows = (size_t)p.max_seq + TILE;              // rows of one kv head's plane, padding included
-  PA_TP(0);
   // SR: the whole splits of a kv head are interleaved.  With nw = (whole splits) x W waves, wave v of
   // them takes rows [(c nw + v) 8, + 8), c = 0 .. 3, instead of 32 consecutive ones: at any moment the loads in
   // flight on the chip then sweep a compact range of the cache (4 KB pieces, neighbouring waves on neighbouring
@@ -343,7 +334,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
   // microseconds (the memory pipeline is full), so arithmetic placed after all of them starts that much later, while
   // the K requests already queued keep the pipeline fed during the arithmetic.
   if constexpr (!FUSED) first_v_loads();
-  PA_TP(1);
   __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the load issue
   // ---- q -> f16 rows in LDS; waits only for the q loads, which were issued first ----
   if constexpr (FUSED) {
@@ -415,7 +405,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     end_pos[nb] = r < R ? (GATHER ? seq_max : p.base_pos + c0 + r / G + 1 - p.self_row) : 0u;
   }
   __syncthreads();
-  PA_TP(2);
   // ---- the column's own row as a partial of its own (slot = number of splits that hold rows): m = its score,
   // l = 1, O = its value row.  The scores run on the VALU over the f16 operands the MFMA path would see, f32 sums in a
   // fixed order; the work hides under the latency of the tile loads.  Decoding a token at a position that is a
@@ -574,10 +563,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       const bool has_tile = wave < n_tiles;
       const uint32_t tp = t_begin + min(wave, n_tiles - 1) * TILE;      // the tile this wave holds in registers
       stage_k(tp, false, 0);
-      PA_TP(3);
       f4 s[2][NB];
       qk(s);
-      PA_TP(4);
       const uint32_t row_end = has_tile ? end_pos[0] : 0u;              // a wave without a tile contributes nothing
       float v[8], mx = NEG_INF;
 #pragma unroll
@@ -601,9 +588,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       stage_v(ILV && ilv ? 0u : tp, false, 0);                          // interleaved splits are whole: no row past the end to zero
       *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pf;
       if (kg == 0) { mex[wave * 16 + ln] = mx; lex[wave * 16 + ln] = ps; }
-      PA_TP(5);
       __syncthreads();
-      PA_TP(6);
       {
         // V^T fragments (two transpose reads each) and the tile's P are fetched VD steps ahead of their MFMA
         constexpr int NS = W * DBW, VD = 4;
@@ -652,7 +637,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
 #pragma unroll
           for (int j = 0; j < DBW; j++) o[j] += (dead ? (f4){0.f, 0.f, 0.f, 0.f} : pr[w2][j]) * c;
         }
-        PA_TP(7); PA_TP(8); PA_TP(10);
         if (ln < R) {
           const uint32_t col = c0 + ln / G, hq = g * G + ln % G;
           const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
@@ -662,7 +646,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
         }
       }
     }
-    PA_TP(9);
     return;
   }
   // ---- tile loop: every wave streams its own tiles and keeps its own (m, l, O) ----
@@ -678,10 +661,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     const uint32_t tp = t_begin + tile * TILE;
     const bool more = tile + W < n_tiles;
     stage_k(tp, more, tp + W * TILE);
-    PA_TP(3);
     f4 s[2][NB];
     qk(s);
-    PA_TP(4);
     // ---- online softmax; lane holds row nb*16 + ln, positions tp + pb*16 + 4*kg + i ----
     // m_run is a lazily updated reference maximum: O and l are rescaled only when some row's tile maximum passes it
     // by more than DEC_RESCALE_TH (natural-log units), so exp(x - m_run) <= e^TH stays far inside the f16 range and
@@ -736,9 +717,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     }
     // V after the softmax, so that the wait for the V loads comes as late as possible
     stage_v(tp, more, tp + W * TILE);
-    PA_TP(5);
     wave_lds_fence();
-    PA_TP(6);
     // ---- O^T += V^T P^T ----
     {
       // the same for the V^T fragments (two transpose reads each), VD blocks ahead
@@ -768,7 +747,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       }
     }
     wave_lds_fence();
-    PA_TP(7);
   }
 
   // ---- merge the W waves of the workgroup ----
@@ -780,7 +758,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     if (kg == 0) { mex[wave * 16 * NB + nb * 16 + ln] = m_run[nb]; lex[wave * 16 * NB + nb * 16 + ln] = l_run[nb]; }
   }
   __syncthreads();
-  PA_TP(8);
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     float M = NEG_INF;
@@ -796,7 +773,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
       }
     }
     __syncthreads();
-    PA_TP(10);
     // rows nb*16 .. nb*16+15, HD/4 float4 each, summed over waves in wave order.  Every thread first issues all
     // its LDS reads (the accumulators are dead, registers are free), then adds and stores: one LDS latency, not one
     // per element.  The (m, l) of a row is merged by one of the first 16 threads.
@@ -868,7 +844,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     }
     if (nb + 1 < NB) __syncthreads();                                  // the regions are rewritten by the next row block
   }
-  PA_TP(9);
 }
 
 // ---- second pass: log-sum-exp merge over a column's splits, sigmoid gate, output conversion ----
@@ -1020,7 +995,6 @@ static hipError_t decode_lds_attr() {
 
 template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
 static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
-  typedef DecShape<HD> S;
   const size_t lds = decode_lds_bytes<HD, NB, W>();
   hipError_t e = decode_lds_attr<HD, NB, W, FUSED, GATHER, Q8, SR>();
   if (e != hipSuccess) return e;
@@ -1041,16 +1015,6 @@ static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipS
 
 template <int HD>
 static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
-#ifdef PA_DEV
-  if (waves == 8 && !p.k_scale) {
-    switch (nb) {
-      case 1: return launch_decode_t<HD, 1, 8, false>(p, col_groups, s, t);
-      case 2: return launch_decode_t<HD, 2, 8, false>(p, col_groups, s, t);
-      case 4: if constexpr (HD == 128) return launch_decode_t<HD, 4, 8, false>(p, col_groups, s, t);
-      default: return hipErrorInvalidValue;
-    }
-  }
-#endif
   if (waves != 4) return hipErrorInvalidValue;
   if (p.k_scale) {                                // int8 caches
     switch (nb) {

@@ -29,29 +29,32 @@
 //   * Optional split over the context (short chunks on long contexts would otherwise leave CUs idle): partial
 //     (m, l, O) go to the same buffers the decode kernel uses and the same merge kernel finishes them.
 #include "pf_common.h"
-#include <cstdlib>
 
+#ifndef PF_PRIO
+#define PF_PRIO 0
+#endif
+#ifndef PF_KD
+#define PF_KD 4
+#endif
+#ifndef PF_QR
+#define PF_QR 8
+#endif
+#ifndef PF_VD
+#define PF_VD 3
+#endif
 template <int HD, int W> struct PfShape {
   static constexpr int ROWB = HD * 2;             // bytes of one kv head's row
   static constexpr int TILE = PF_TN * ROWB;       // bytes of one staged tile (K or V)
   static constexpr int KS = HD / 16;              // k-steps of QK^T
   static constexpr int DB = HD / 32;              // 32-dim blocks of the output
-  static constexpr int QR = HD == 256 ? 8 : KS;   // k-steps whose Q fragments stay in registers
+  static constexpr int QR = HD == 256 ? PF_QR : KS;   // k-steps whose Q fragments stay in registers
   static constexpr int CPR = HD / 8;              // 16-byte chunks per row
   static constexpr int RPB = 64 / CPR;            // rows per 1 KB LDS-direct load
   static constexpr int NLD = PF_TN / RPB / W;     // LDS-direct loads per wave, tensor and step
   static_assert(NLD >= 1 && NLD * W * RPB == PF_TN, "tile must divide evenly over the waves");
 };
 
-// Optional per-wave timeline (development builds only, -DPA_TRACE): lane 0 stores the 100 MHz wall clock at 6
-// points of 8 consecutive steps starting at step 1000 into p.trace.
-#ifdef PA_TRACE
-#define PF_TP(k) do { if (p.trace && lane == 0 && blockIdx.y == 0) { const uint32_t st_ = (tp - t_begin) / PF_TN; if (st_ >= 1000 && st_ < 1008) p.trace[(((size_t)blockIdx.x * W + wave) * 8 + (st_ - 1000)) * 6 + (k)] = wall_clock64(); } } while (0)
-#else
-#define PF_TP(k) do { } while (0)
-#endif
-
-template <int HD, int QB, int W, bool PP>
+template <int HD, int QB, int W>
 __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p, uint32_t n_col_blocks) {
   typedef PfShape<HD, W> S;
   // four separate LDS objects (two K, two V buffers): the compiler then orders an LDS read only after the
@@ -75,9 +78,6 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform (scalar) so per-wave branches are scalar branches
   const uint32_t ln = lane & 31, hb = lane >> 5;   // MFMA row / column index, k half
-#ifdef PF_CLK   // development builds: shader clock vs 100 MHz wall clock over the kernel
-  long long clk0 = clock64(), wc0 = wall_clock64();
-#endif
   const uint32_t G = p.group, nH = p.n_heads;
   const uint32_t c0 = cb * p.cols_per_group;
   const uint32_t ncl = min(p.cols_per_group, p.n_cols - c0);
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     }
   };
   issue_k(kbuf0, t_begin);
-  if (!PP) issue_v(vbuf0, t_begin);
+  issue_v(vbuf0, t_begin);
 
   // ---- per-lane rows: query row of block qb is wave*QB*32 + qb*32 + ln = (column r / G, head r % G) ----
   uint32_t end_pos[QB], row_id[QB];
@@ -193,13 +193,12 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   h8 pf[QB][2];
   // ---- S^T = K Q^T : rows = 32 positions, columns = 32 query rows per block ----
   auto qk = [&](const unsigned char* kb, const uint32_t tp) {
-    PF_TP(0);
 #pragma unroll
     for (int qb = 0; qb < QB; qb++)
 #pragma unroll
       for (int i = 0; i < 16; i++) s[qb][i] = 0.f;
     // K fragments (and the Q fragments parked in LDS) are fetched KD k-steps ahead of the MFMA that consumes them
-    constexpr int KD = 4;
+    constexpr int KD = PF_KD;
     h8 ka[KD], qa[QB][KD];
 #pragma unroll
     for (int i = 0; i < KD; i++) {
@@ -233,14 +232,12 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
       __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
       if (ks + KD < S::KS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); if (ks + KD >= QR) __builtin_amdgcn_sched_group_barrier(0x100, QB, 0); }
     }
-    PF_TP(1);
   };
   // ---- online softmax; lane holds query row ln of each block, positions tp + 8 (i / 4) + 4 hb + i % 4 ----
   // Raw scores stay unscaled: the scale rides in the exp2 argument (one fma per element), the row sum is a
   // v_dot2 over the f16-rounded probabilities (the values PV really uses), and the mask is a separate pass
   // that only tiles straddling a row end execute.
   auto sm = [&](const uint32_t tp) {
-    PF_TP(2);
     if (tp + PF_TN > w_min_end) {
       asm volatile("; causal tile" ::: "memory");   // keeps this a branch: most tiles skip the 3 ops per element
 #pragma unroll
@@ -289,13 +286,12 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
       }
       l_run[qb] = ps;
     }
-    PF_TP(3);
   };
   // ---- O^T += V^T P^T : rows = 32 dims, contraction over 2 x 16 positions ----
   auto pv = [&](const unsigned char* vb, const uint32_t tp) {
     // fragment f = j DB + db: positions 16 j .., dims 32 db .. (consecutive MFMAs hit different accumulators);
     // fetched VD fragments ahead
-    constexpr int VD = 3, NF = 2 * S::DB;
+    constexpr int VD = PF_VD, NF = 2 * S::DB;
     h4 vlo[VD], vhi[VD];
 #pragma unroll
     for (int f = 0; f < VD; f++) {
@@ -323,56 +319,23 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
       __builtin_amdgcn_sched_group_barrier(0x008, QB, 1);
       if (f + VD < NF) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
     }
-    PF_TP(4);
   };
 
-  // ---- main loop: two wave groups in anti-phase ----
-  // Waves w and w + W/2 share a SIMD.  Group 0 runs [PV(i-1) QK(i)] | SM(i) in the two halves of step i, group 1
-  // runs SM(i-1) | [PV(i-1) QK(i)], so in each half one wave of a SIMD owns the MFMA pipe while the other does its
-  // softmax on the VALU.  The mid-step barrier only keeps the phases aligned (no memory is exchanged across it, so
-  // it is a bare s_barrier that does not wait for the loads in flight); the end-of-step barrier publishes the tiles
-  // the LDS-direct loads of this step brought in: K(i+1) into the K buffer not in use, V(i) into the V buffer
-  // that tile i-2 has left.  V(i) is consumed during step i + 1 by both groups.
-  const bool grp1 = W >= 8 && wave >= W / 2;
-  auto issue_next = [&](auto PAR, const uint32_t i, const uint32_t tp) {
-    constexpr int par = decltype(PAR)::value;
-    if (i + 1 < n_steps) issue_k(par ? kbuf0 : kbuf1, tp + PF_TN);
-    issue_v(par ? vbuf1 : vbuf0, tp);
-  };
-  auto step_a = [&](auto PAR, const uint32_t i) {          // group 0
-    constexpr int par = decltype(PAR)::value;
-    const uint32_t tp = t_begin + i * PF_TN;
-    issue_next(PAR, i, tp);
-    if (i > 0) pv(par ? vbuf0 : vbuf1, tp - PF_TN);
-    qk(par ? kbuf1 : kbuf0, tp);
-    __builtin_amdgcn_s_barrier();
-    sm(tp);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this wave's LDS-direct loads have landed
-    __syncthreads();
-  };
-  auto step_b = [&](auto PAR, const uint32_t i) {          // group 1
-    constexpr int par = decltype(PAR)::value;
-    const uint32_t tp = t_begin + i * PF_TN;
-    issue_next(PAR, i, tp);
-    if (i > 0) sm(tp - PF_TN);
-    __builtin_amdgcn_s_barrier();
-    if (i > 0) pv(par ? vbuf0 : vbuf1, tp - PF_TN);
-    qk(par ? kbuf1 : kbuf0, tp);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-  };
-  const uint32_t tl = t_begin + (n_steps - 1) * PF_TN;
-  const unsigned char* v_last = ((n_steps - 1) & 1) ? vbuf1 : vbuf0;
+  // ---- main loop ----
   const uint32_t n_even = n_steps & ~1u;
-  if (!PP) {
+  {
     // all waves in phase: QK, softmax, PV of a tile between two barriers (tile i + 1 of both K and V in flight)
     auto step_s = [&](auto PAR, const uint32_t i) {
       constexpr int par = decltype(PAR)::value;
       const uint32_t tp = t_begin + i * PF_TN;
       if (i + 1 < n_steps) { issue_k(par ? kbuf0 : kbuf1, tp + PF_TN); issue_v(par ? vbuf0 : vbuf1, tp + PF_TN); }
+      if (PF_PRIO) __builtin_amdgcn_s_setprio(PF_PRIO);
       qk(par ? kbuf1 : kbuf0, tp);
+      if (PF_PRIO) __builtin_amdgcn_s_setprio(0);
       sm(tp);
+      if (PF_PRIO) __builtin_amdgcn_s_setprio(PF_PRIO);
       pv(par ? vbuf1 : vbuf0, tp);
+      if (PF_PRIO) __builtin_amdgcn_s_setprio(0);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
     };
@@ -381,26 +344,8 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
       step_s(std::integral_constant<int, 1>{}, i + 1);
     }
     if (n_steps & 1) step_s(std::integral_constant<int, 0>{}, n_even);
-  } else if (!grp1) {
-    for (uint32_t i = 0; i < n_even; i += 2) {
-      step_a(std::integral_constant<int, 0>{}, i);
-      step_a(std::integral_constant<int, 1>{}, i + 1);
-    }
-    if (n_steps & 1) step_a(std::integral_constant<int, 0>{}, n_even);
-    pv(v_last, tl);                                         // drain: the last tile's V landed before the last barrier
-  } else {
-    for (uint32_t i = 0; i < n_even; i += 2) {
-      step_b(std::integral_constant<int, 0>{}, i);
-      step_b(std::integral_constant<int, 1>{}, i + 1);
-    }
-    if (n_steps & 1) step_b(std::integral_constant<int, 0>{}, n_even);
-    sm(tl);
-    pv(v_last, tl);
   }
 
-#ifdef PF_CLK
-  if (p.trace && tid == 0) { p.trace[blockIdx.x * 2] = clock64() - clk0; p.trace[blockIdx.x * 2 + 1] = wall_clock64() - wc0; }
-#endif
   // ---- epilogue ----
 #pragma unroll
   for (int qb = 0; qb < QB; qb++) {
@@ -450,30 +395,26 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   }
 }
 
-template <int HD, int QB, int W, bool PP>
+template <int HD, int QB, int W>
 static hipError_t launch_prefill_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   typedef PfShape<HD, W> S;
   const size_t lds = (size_t)W * QB * (S::KS - S::QR) * 1024;     // Q fragments parked in LDS (dynamic part)
   static bool attr_set = false;
   if (!attr_set && lds > 0) {
-    hipError_t e = hipFuncSetAttribute((const void*)pa_prefill_kernel<HD, QB, W, PP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)pa_prefill_kernel<HD, QB, W>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
   const uint32_t total = col_groups * p.n_kv_heads * p.n_splits;
   const uint32_t gx = ((total + 7) / 8) * 8;       // whole rounds of the 8 XCDs
-  PA_LAUNCH((pa_prefill_kernel<HD, QB, W, PP>), dim3(gx), dim3(W * 64), lds, s, t, p, col_groups);
+  PA_LAUNCH((pa_prefill_kernel<HD, QB, W>), dim3(gx), dim3(W * 64), lds, s, t, p, col_groups);
   return hipGetLastError();
 }
 
 // row_blocks = 32-row query blocks per workgroup (8: one per wavefront)
 hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   if (row_blocks != 8) return hipErrorNotSupported;
-  // In-phase waves measure faster than the anti-phase schedule on MI355X (C5: 7.27 ms vs 7.77 ms): with one wave
-  // of a SIMD alone on the MFMA pipe, every LDS fragment wait is exposed.  The anti-phase variant stays selectable
-  // for measurements.
-  static const bool anti_phase = getenv("POOLED_ATTN_PREFILL_ANTI_PHASE") != nullptr;
-  if (hd == 256) return anti_phase ? launch_prefill_t<256, 1, 8, true>(p, col_groups, s, t) : launch_prefill_t<256, 1, 8, false>(p, col_groups, s, t);
-  if (hd == 128) return anti_phase ? launch_prefill_t<128, 1, 8, true>(p, col_groups, s, t) : launch_prefill_t<128, 1, 8, false>(p, col_groups, s, t);
+  if (hd == 256) return launch_prefill_t<256, 1, 8>(p, col_groups, s, t);
+  if (hd == 128) return launch_prefill_t<128, 1, 8>(p, col_groups, s, t);
   return hipErrorNotSupported;
 }

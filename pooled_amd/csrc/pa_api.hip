@@ -338,10 +338,6 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   if (n_cols * G > max_rows) { cw = max_rows / G; if (cw == 0) return PA_ERR_UNSUPPORTED; groups = ceil_div(n_cols, cw); }
   uint32_t nb = ceil_div(cw * G, 16);
   uint32_t W = 4;
-#ifdef PA_DEV
-  if (getenv("POOLED_DEV_W") && n_cols > 1) W = 8;
-  if (getenv("POOLED_DEV_NB") && n_cols > 1) { max_rows = 16 * atoi(getenv("POOLED_DEV_NB")); cw = n_cols; groups = 1; if (n_cols * G > max_rows) { cw = max_rows / G; groups = ceil_div(n_cols, cw); } nb = ceil_div(cw * G, 16); }
-#endif
   const uint32_t self = self_ok && n_cols == 1 ? 1 : 0;
   const uint32_t seq_max = std::max(base_pos + n_cols - self, 1u);   // streamed rows (position 0 alone: one empty split)
   const uint32_t tiles = ceil_div(seq_max, 32);
@@ -390,30 +386,22 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
   // share the stream through L2, for as long as groups x K/V bytes stays below what the MFMA kernel's fixed costs
   // (Q staging, one partial per split and row, the merge) amount to.  Measured crossover on the MoE and 27B shapes
   // at 32K - 64K rows: about 1.4 GB of L2-level K/V traffic; below 4096 rows both kernels take 25 - 40 us.
-#ifdef PA_DEV
-  if (getenv("POOLED_DEV_SK") && max_rows_sk >= G) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
-#endif
   // A small chunk (the first chunks of a prompt, a 512-column chunk over a 2K context): the matrix-core kernel's
   // 256-row workgroups leave most CUs idle unless the chunk is also split over the context, and then the partials
   // (a row of head_dim floats per split and stacked row) and the merge launch cost more than the attention itself.
   // Below about 8 GFLOP of causal work the split-K kernel serves the chunk in one launch instead: 16- or 32-row
   // workgroups (the larger that still gives every CU a workgroup), each over the whole context of its columns,
-  // writing the normalised, gated output itself.  Measured crossover (us per call, this path vs the matrix-core
+  // writing the normalised, gated output itself -- for contexts below 4096 rows (longer ones are the rule above) and
+  // chunks whose column groups fill at least half the chip.  Measured crossover (us per call, this path vs the matrix-core
   // kernel): dense shape 256 columns from position 0: 6.3 vs 16.8, 512 columns at 1536: 25 vs 32, 2048 from 0: 48 vs
   // 47; MoE shape 256 from 0: 11 vs 33, 512 from 0: 21 vs 36, 1024 from 0: 52 vs 44.
   {
     const double flops = 4.0 * c.n_heads * c.head_dim * ((double)n_cols * base_pos + 0.5 * (double)n_cols * (n_cols + 1));
-    if (table && flops <= 8.0e9 && G <= 16 && !ctx->decode_splits_override) {
-      const uint32_t rows = G <= 32 && (uint64_t)ceil_div(n_cols, 32 / G) * c.n_kv_heads >= (uint64_t)ctx->n_cu ? 32u : 16u;
-      return plan_decode(ctx, base_pos, n_cols, pl, true, wgs, rows, true);
-    }
-  }
-  if (table && n_cols * G <= 512 && base_pos + n_cols >= 4096 && max_rows_sk >= G) {
-    pa_plan sk; uint32_t sk_wgs = 0;
-    const uint64_t kv_bytes = 2ull * (base_pos + n_cols) * c.n_kv_heads * c.head_dim * (kv_q8(ctx) ? 1 : 2);
-    if (plan_decode(ctx, base_pos, n_cols, &sk, true, &sk_wgs) == PA_OK && (uint64_t)sk.col_groups * kv_bytes <= 1400000000ull) {
-      *pl = sk; if (wgs) *wgs = sk_wgs;
-      return PA_OK;
+    if (table && flops <= 8.0e9 && G <= 16 && base_pos + n_cols < 4096 && !ctx->decode_splits_override) {
+      const uint32_t rows = (uint64_t)ceil_div(n_cols, 32 / G) * c.n_kv_heads >= (uint64_t)ctx->n_cu ? 32u : 16u;
+      // one split per workgroup only pays when the column groups alone occupy the chip (or the context is a few tiles)
+      if ((uint64_t)ceil_div(n_cols, rows / G) * c.n_kv_heads * 2 >= (uint64_t)ctx->n_cu || base_pos + n_cols <= 256)
+        return plan_decode(ctx, base_pos, n_cols, pl, true, wgs, rows, true);
     }
   }
   const uint32_t rows_wg = 256;
@@ -481,17 +469,6 @@ static int prof_pair(pa_ctx* ctx, PaTiming* t) {
   t->start = ctx->prof_events[ctx->prof_used]; t->stop = ctx->prof_events[ctx->prof_used + 1];
   ctx->prof_used += 2;
   return PA_OK;
-}
-
-// POOLED_ATTN_PREFILL_WIDE selects the 4-wave prefill kernel for measurements; read at every call (a getenv is
-// nothing next to a kernel launch) so that a test can switch it inside one process
-static bool prefill_wide_selected() { return getenv("POOLED_ATTN_PREFILL_WIDE") != nullptr; }
-// POOLED_ATTN_PREFILL_SMALL=1 selects the prefill kernel on the 16 x 16 x 32 matrix instruction (attn_prefill_small.hip)
-// for measurements.  Interleaved A/B runs put it level with the 32 x 32 x 16 kernel on C5 and behind it on the other
-// shapes, so the plan never picks it by itself.
-static bool prefill_small_selected() {
-  const char* e = getenv("POOLED_ATTN_PREFILL_SMALL");
-  return e != nullptr && atoi(e) != 0;
 }
 
 static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, const float* d_q, uint32_t q_stride,
@@ -565,8 +542,6 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   PaTiming tm;
   if ((rc = prof_pair(ctx, &tm))) return rc;
   if (pl.kernel == 0) HIPCHK(ctx, pa_launch_decode(p, c.head_dim, pl.row_blocks, pl.waves, pl.col_groups, ctx->stream, &tm));
-  else if (prefill_wide_selected()) HIPCHK(ctx, pa_launch_prefill_wide(p, c.head_dim, pl.col_groups, ctx->stream, &tm));
-  else if (prefill_small_selected()) HIPCHK(ctx, pa_launch_prefill_small(p, c.head_dim, pl.col_groups, ctx->stream, &tm));
   else HIPCHK(ctx, pa_launch_prefill(p, c.head_dim, pl.row_blocks, pl.col_groups, ctx->stream, &tm));
   if (!direct) HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream));
   return PA_OK;
@@ -1019,16 +994,6 @@ extern "C" int pa_timer_stop(pa_ctx* ctx, float* ms) {
   HIPCHK(ctx, hipEventRecord(ctx->t1, ctx->stream));
   HIPCHK(ctx, hipEventSynchronize(ctx->t1));
   HIPCHK(ctx, hipEventElapsedTime(ms, ctx->t0, ctx->t1));
-  return PA_OK;
-}
-extern "C" int pa_mfma_probe(pa_ctx* ctx, int random_operands, uint32_t iters, float* tflops, float* shader_mhz) {
-  if (!ctx || !tflops || !shader_mhz || iters == 0) return PA_ERR_INVALID;
-  HIPCHK(ctx, pa_run_mfma_probe(ctx->n_cu, random_operands != 0, random_operands == 2, iters, ctx->stream, tflops, shader_mhz));
-  return PA_OK;
-}
-extern "C" int pa_lds_probe(pa_ctx* ctx, int transpose_reads, uint32_t waves_per_cu, uint32_t iters, float* bytes_per_clk) {
-  if (!ctx || !bytes_per_clk || iters == 0 || waves_per_cu == 0 || waves_per_cu > 8) return PA_ERR_INVALID;
-  HIPCHK(ctx, pa_run_lds_probe(ctx->n_cu, transpose_reads != 0, waves_per_cu, iters, ctx->stream, bytes_per_clk));
   return PA_OK;
 }
 extern "C" int pa_profile_enable(pa_ctx* ctx, int on) {

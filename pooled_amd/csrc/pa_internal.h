@@ -47,7 +47,6 @@ struct AttnParams {
   uint32_t direct_out;                        // tile-loop split-K kernel with one split and no own-row partial: the workgroup
                                               // normalises, gates and stores the output itself (no partials, no merge launch)
   float scale;                                // 1 / sqrt(hd)
-  unsigned long long* trace;                  // per-wave timestamps when built with PA_TRACE (else unused, nullptr)
   uint32_t gate_head_stride;                  // floats between consecutive heads in gate (head_dim, or 2*head_dim
                                               // when gate is read in place from an interleaved [q | gate] column)
   // fused pre-step of pa_attn_decode_step (one column at base_pos; f_q_in == nullptr otherwise): raw projections
@@ -86,9 +85,6 @@ hipError_t pa_prepare_decode_step(uint32_t hd, bool q8);
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);
 // MFMA prefill; returns hipErrorNotSupported for shapes it does not cover
 hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
-// the 4-wave, 64-rows-per-wave software-pipelined variant (same contract)
-hipError_t pa_launch_prefill_wide(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
-hipError_t pa_launch_prefill_small(const AttnParams& p, uint32_t hd, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
 
 // one-token projection y = W x (proj_gemv.hip): kind PA_W_*, w = f32 [d_out][d_in] / int8 [d_out][d_in] / nibbles
 // [d_out][d_in / 2], scales = f16 bits [d_out][d_in / 32] (quantised kinds); norm_w != nullptr: x is the raw vector and
@@ -118,10 +114,6 @@ hipError_t pa_launch_rmsnorm_f16(const float* x, uint32_t x_stride, const float*
 // int8 caches -> f16 staging cache of the same geometry (glue_kv.hip): rows [0, n_live) widened, [n_live, n_rows) zeroed
 hipError_t pa_launch_widen_q8(const void* k8, const void* v8, const float* ks, const float* vs, uint16_t* ko, uint16_t* vo,
                               uint32_t n_kv_heads, uint32_t hd, uint32_t head_rows, uint32_t n_live, uint32_t n_rows, hipStream_t s);
-
-// device probe (probe.hip): sustained f16 MFMA rate and shader clock, constant or random operands
-hipError_t pa_run_mfma_probe(int n_cu, bool random_operands, bool small_tiles, uint32_t iters, hipStream_t st, float* tflops, float* shader_mhz);
-hipError_t pa_run_lds_probe(int n_cu, bool transpose_reads, uint32_t waves, uint32_t iters, hipStream_t st, float* bytes_per_clk);
 
 // ---- context -----------------------------------------------------------------------------------
 

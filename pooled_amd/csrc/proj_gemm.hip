@@ -352,12 +352,11 @@ static hipError_t launch_gemm_xt(const GemmParams& p, hipStream_t s) {
 hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s) {
   if (p.d_out == 0 || p.d_in == 0 || (p.d_in & 31) || p.n_cols == 0) return hipErrorInvalidValue;
   // a handful of columns: a pass over the weights per launch of up to 16 columns (as many as fit the LDS staging),
-  // up to 32 columns in all -- past that the tiled kernel wins (POOLED_ATTN_GEMM_SKINNY=0 keeps it, for measurements)
+  // up to 32 columns in all -- past that the tiled kernel wins
   if (p.kind != PA_W_F32 && p.n_cols <= 2 * SK_NC && p.d_in <= 8192 && (p.x_stride & 7) == 0) {
-    const char* k = getenv("POOLED_ATTN_GEMM_SKINNY");
     const uint32_t fit = (uint32_t)((144 * 1024) / ((size_t)(p.d_in / GK) * GROW));
     const uint32_t per = fit < SK_NC ? fit : SK_NC;
-    if ((!k || atoi(k) != 0) && per >= 1) {
+    if (per >= 1) {
       for (uint32_t c0 = 0; c0 < p.n_cols; c0 += per) {
         GemmParams q = p;
         q.x = p.x + (size_t)c0 * p.x_stride; q.y = p.y + (size_t)c0 * p.y_stride;
@@ -370,8 +369,7 @@ hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s) {
   }
   // 256-column workgroups (two fit a CU) when they still give every CU four: otherwise 128-column ones (three a CU)
   const size_t wgs2 = (size_t)((p.d_out + GT - 1) / GT) * ((p.n_cols + 2 * GT - 1) / (2 * GT));
-  const char* e = getenv("POOLED_ATTN_GEMM_XT");
-  const bool xt2 = e ? atoi(e) == 2 : wgs2 >= (size_t)4 * (n_cu > 0 ? n_cu : 256);
+  const bool xt2 = wgs2 >= (size_t)4 * (n_cu > 0 ? n_cu : 256);
   return xt2 ? launch_gemm_xt<2>(p, s) : launch_gemm_xt<1>(p, s);
 }
 

@@ -103,7 +103,7 @@ def test_prefill_tile_override():
     cfg = SHAPES["qwen36_moe"]
     outs = {}
     for mode, kernel in ((0, 0), (1, 1), (2, 0)):
-        got, ref, plan = _prefill(cfg, 900, 120, seed=3, tile=mode)
+        got, ref, plan = _prefill(cfg, 900, 200, seed=3, tile=mode)
         assert plan["kernel"] == kernel, (mode, plan)
         assert_parity(got, ref, "tile mode %d" % mode)
         outs[mode] = got
@@ -117,32 +117,6 @@ def test_prefill_peaked_softmax():
     cfg = SHAPES["qwen38_27b"]
     got, ref, _ = _prefill(cfg, 500, 96, seed=9, k_scale=3.0)
     assert_parity(got, ref, "peaked")
-
-
-@pytest.mark.parametrize("shape,base,n,k_scale", [
-    ("qwen36_moe", 301, 16, 1.0), ("qwen36_moe", 1000, 200, 1.0), ("qwen3_1p7b", 219, 257, 1.0),
-    ("qwen38_27b", 500, 96, 3.0), ("qwen36_moe", 20000, 80, 1.0),
-])
-def test_prefill_wide_variant(shape, base, n, k_scale, monkeypatch):
-    """The 4-wave, 64-rows-per-wave variant of the prefill kernel (selected by an environment variable read at
-    each call): same parity bar, including the rescale path (peaked scores) and the split path."""
-    monkeypatch.setenv("POOLED_ATTN_PREFILL_WIDE", "1")
-    got, ref, plan = _prefill(SHAPES[shape], base, n, seed=base + n + 1, k_scale=k_scale)
-    assert plan["kernel"] == 1
-    assert_parity(got, ref, "wide %s base %d n %d" % (shape, base, n))
-
-
-@pytest.mark.parametrize("shape,base,n,k_scale", [
-    ("qwen36_moe", 301, 16, 1.0), ("qwen36_moe", 1000, 200, 1.0), ("qwen3_1p7b", 219, 257, 1.0),
-    ("qwen38_27b", 500, 96, 3.0), ("qwen36_moe", 20000, 80, 1.0),
-])
-def test_prefill_small_tile_variant(shape, base, n, k_scale, monkeypatch):
-    """The variant of the prefill kernel on the 16 x 16 x 32 matrix instruction (selected by an environment variable
-    read at each call): same parity bar, including the rescale path (peaked scores), the split path and hd 128."""
-    monkeypatch.setenv("POOLED_ATTN_PREFILL_SMALL", "1")
-    got, ref, plan = _prefill(SHAPES[shape], base, n, seed=base + n + 2, k_scale=k_scale)
-    assert plan["kernel"] == 1
-    assert_parity(got, ref, "small tile %s base %d n %d" % (shape, base, n))
 
 
 def test_c2_prefill_full():

@@ -123,10 +123,7 @@ def test_attn_layer_decode_matches_oracle(shape, dim, kind, pos):
 @pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q8_0, PA_W_Q4_0])
 @pytest.mark.parametrize("d_out,d_in,n", [(9216, 2048, 300), (2048, 4096, 129), (37, 96, 5), (130, 8192, 40), (256, 32, 128), (384, 96, 700),
                                           (9216, 2048, 8), (2048, 4096, 16), (130, 8192, 3), (70, 64, 1), (2048, 4096, 31), (130, 8192, 17)])   # from (9216, 2048, 8) on: the skinny-chunk kernel, one or more launches
-@pytest.mark.parametrize("wide", [False, True])
-def test_gemm_matches_oracle(kind, d_out, d_in, n, wide, monkeypatch):
-    # wide: force the 256-column workgroups that large chunks get (the library reads the switch at every call)
-    monkeypatch.setenv("POOLED_ATTN_GEMM_XT", "2" if wide else "1")
+def test_gemm_matches_oracle(kind, d_out, d_in, n):
     if kind == PA_W_F32 and d_in > 4096:
         pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
     rng = np.random.default_rng(d_out + 3 * d_in + n + kind)
@@ -145,6 +142,23 @@ def test_gemm_matches_oracle(kind, d_out, d_in, n, wide, monkeypatch):
         assert np.array_equal(got[:, d_out:], y0[:, d_out:]), "the stride padding of y must stay untouched"
         pa.gemm(wh, dx, xs, n, dy, ys, acc=True); pa.sync()
         assert _rel(dy.download(np.float32, n * ys).reshape(n, ys)[:, :d_out], 2.0 * ref) < 2e-5, "accumulate"
+
+
+@pytest.mark.parametrize("kind", [PA_W_Q8_0, PA_W_Q4_0])
+def test_gemm_large_chunk_takes_the_256_column_workgroups(kind):
+    """A chunk large enough to give every CU four 256-column workgroups (the [q | k | v] projection of a 4096-column
+    chunk) runs the kernel's wide form; ragged edges on both axes."""
+    d_out, d_in, n = 9216 - 40, 2048, 4096 - 3
+    rng = np.random.default_rng(kind)
+    w, sc = _weights(kind, d_out, d_in, rng)
+    x16 = rng.standard_normal((n, d_in)).astype(np.float16)
+    ref = O.gemm_f16(kind, w, sc, x16.astype(np.float32))
+    with PooledAttn(SHAPES["qwen36_moe"], 64, n_layers=1, max_cols=1) as pa:
+        wh = pa.weight(kind, w, sc)
+        dx = pa.to_device(x16.view(np.uint16)); dy = pa.alloc(n * d_out * 4)
+        pa.gemm(wh, dx, d_in, n, dy, d_out); pa.sync()
+        got = dy.download(np.float32, n * d_out).reshape(n, d_out)
+    assert _rel(got, ref) < 2e-5
 
 
 def test_rmsnorm_f16_columns():
