@@ -33,6 +33,9 @@
 #ifndef PF_PRIO
 #define PF_PRIO 0
 #endif
+#ifndef PF_ABL
+#define PF_ABL 0        // development ablations (wrong results, timing only): bit 0 no exp, 1 one K fragment, 2 one V fragment, 3 no softmax, 4 no tile loads in the loop
+#endif
 #ifndef PF_KD
 #define PF_KD 4
 #endif
@@ -202,7 +205,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     h8 ka[KD], qa[QB][KD];
 #pragma unroll
     for (int i = 0; i < KD; i++) {
-      ka[i] = *(const h8*)(kb + (k_rd ^ (i * 32)));
+      ka[i] = *(const h8*)(kb + (k_rd ^ ((PF_ABL & 2) ? 0 : i * 32)));
       if (i >= QR) {
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) qa[qb][i] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (i - QR)) * 1024);
@@ -215,7 +218,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 #pragma unroll
       for (int qb = 0; qb < QB; qb++) b[qb] = ks < QR ? qf[qb][ks < QR ? ks : 0] : qa[qb][ks % KD];
       if (ks + KD < S::KS) {
-        ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
+        if (!(PF_ABL & 2)) ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
         if (ks + KD >= QR) {
 #pragma unroll
           for (int qb = 0; qb < QB; qb++) qa[qb][ks % KD] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (ks + KD - QR)) * 1024);
@@ -238,6 +241,13 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   // v_dot2 over the f16-rounded probabilities (the values PV really uses), and the mask is a separate pass
   // that only tiles straddling a row end execute.
   auto sm = [&](const uint32_t tp) {
+    if (PF_ABL & 8) {
+#pragma unroll
+      for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) { pf[qb][i >> 3][i & 7] = (_Float16)s[qb][i]; pf[qb][i >> 3][(i & 7) + 1] = (_Float16)s[qb][i + 1]; }
+      return;
+    }
     if (tp + PF_TN > w_min_end) {
       asm volatile("; causal tile" ::: "memory");   // keeps this a branch: most tiles skip the 3 ops per element
 #pragma unroll
@@ -278,8 +288,8 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
       float ps = l_run[qb];
 #pragma unroll
       for (int i = 0; i < 16; i += 2) {
-        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], c1, nmr));
-        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], c1, nmr));
+        const float e0 = (PF_ABL & 1) ? __builtin_fmaf(s[qb][i], c1, nmr) : __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], c1, nmr));
+        const float e1 = (PF_ABL & 1) ? __builtin_fmaf(s[qb][i + 1], c1, nmr) : __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], c1, nmr));
         const h2 pp = { (_Float16)e0, (_Float16)e1 };
         ps = __builtin_amdgcn_fdot2(pp, ones, ps, false);
         pf[qb][i >> 3][i & 7] = pp[0]; pf[qb][i >> 3][(i & 7) + 1] = pp[1];
@@ -302,7 +312,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 #pragma unroll
     for (int f = 0; f < NF; f++) {
       const h4 lo = vlo[f % VD], hi = vhi[f % VD];
-      if (f + VD < NF) {
+      if (f + VD < NF && !(PF_ABL & 4)) {
         const int fn = f + VD;
         const unsigned char* vp = vb + (v_rd ^ ((fn % S::DB) * 64)) + (fn / S::DB) * 16 * S::ROWB;
         vlo[f % VD] = lds_read_tr16(vp);
@@ -328,7 +338,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     auto step_s = [&](auto PAR, const uint32_t i) {
       constexpr int par = decltype(PAR)::value;
       const uint32_t tp = t_begin + i * PF_TN;
-      if (i + 1 < n_steps) { issue_k(par ? kbuf0 : kbuf1, tp + PF_TN); issue_v(par ? vbuf0 : vbuf1, tp + PF_TN); }
+      if (i + 1 < n_steps && !((PF_ABL & 16) && i > 0)) { issue_k(par ? kbuf0 : kbuf1, tp + PF_TN); issue_v(par ? vbuf0 : vbuf1, tp + PF_TN); }
       if (PF_PRIO) __builtin_amdgcn_s_setprio(PF_PRIO);
       qk(par ? kbuf1 : kbuf0, tp);
       if (PF_PRIO) __builtin_amdgcn_s_setprio(0);

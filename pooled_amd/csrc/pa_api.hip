@@ -146,6 +146,7 @@ extern "C" int pa_destroy(pa_ctx* ctx) {
   if (ctx->part_ml) (void)hipFree(ctx->part_ml);
   if (ctx->proj_buf) (void)hipFree(ctx->proj_buf);
   if (ctx->chunk_buf) (void)hipFree(ctx->chunk_buf);
+  if (ctx->w16_buf) (void)hipFree(ctx->w16_buf);
   if (ctx->wide_k) (void)hipFree(ctx->wide_k);
   if (ctx->wide_v) (void)hipFree(ctx->wide_v);
   for (void* r : ctx->retired) (void)hipFree(r);
@@ -386,6 +387,14 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
   // share the stream through L2, for as long as groups x K/V bytes stays below what the MFMA kernel's fixed costs
   // (Q staging, one partial per split and row, the merge) amount to.  Measured crossover on the MoE and 27B shapes
   // at 32K - 64K rows: about 1.4 GB of L2-level K/V traffic; below 4096 rows both kernels take 25 - 40 us.
+  if (table && n_cols * G <= 512 && base_pos + n_cols >= 4096 && max_rows_sk >= G) {
+    pa_plan sk; uint32_t sk_wgs = 0;
+    const uint64_t kv_bytes = 2ull * (base_pos + n_cols) * c.n_kv_heads * c.head_dim * (kv_q8(ctx) ? 1 : 2);
+    if (plan_decode(ctx, base_pos, n_cols, &sk, true, &sk_wgs) == PA_OK && (uint64_t)sk.col_groups * kv_bytes <= 1400000000ull) {
+      *pl = sk; if (wgs) *wgs = sk_wgs;
+      return PA_OK;
+    }
+  }
   // A small chunk (the first chunks of a prompt, a 512-column chunk over a 2K context): the matrix-core kernel's
   // 256-row workgroups leave most CUs idle unless the chunk is also split over the context, and then the partials
   // (a row of head_dim floats per split and stacked row) and the merge launch cost more than the attention itself.
@@ -725,6 +734,12 @@ extern "C" int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uin
   GemmParams p; memset(&p, 0, sizeof p);
   p.w = w->w; p.scales = w->scales; p.x = (const uint16_t*)d_x_f16; p.y = d_y; p.x_stride = x_stride; p.y_stride = y_stride;
   p.d_out = w->d_out; p.d_in = w->d_in; p.n_cols = n_cols; p.acc = acc; p.kind = w->kind;
+  if (pa_gemm_wide_serves(p, ctx->n_cu)) {
+    int rc = grow_scratch(ctx, &ctx->w16_buf, &ctx->w16_buf_bytes, (size_t)w->d_out * w->d_in * sizeof(uint16_t));
+    if (rc) return rc;
+    HIPCHK(ctx, pa_launch_gemm_wide(p, (uint16_t*)ctx->w16_buf, ctx->n_cu, ctx->stream));
+    return PA_OK;
+  }
   HIPCHK(ctx, pa_launch_gemm(p, ctx->n_cu, ctx->stream));
   return PA_OK;
 }

@@ -107,6 +107,10 @@ struct GemmParams {
   int acc; int kind;
 };
 hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s);
+// large chunks (proj_gemm_wide.hip): the weights widened once into w16 (f16 [d_out][d_in], the caller's staging), then a
+// GEMM over two f16 operands; pa_gemm_wide_serves tells whether a call qualifies
+bool pa_gemm_wide_serves(const GemmParams& p, int n_cu);
+hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, int n_cu, hipStream_t s);
 // rmsnorm of n_cols f32 columns, written as f16 (the GEMM's activation operand)
 hipError_t pa_launch_rmsnorm_f16(const float* x, uint32_t x_stride, const float* w, uint32_t dim, float eps, uint32_t n_cols,
                                  uint16_t* out, uint32_t out_stride, hipStream_t s);
@@ -153,6 +157,8 @@ struct pa_ctx {
   size_t part_o_bytes = 0, part_ml_bytes = 0;
   float* proj_buf = nullptr;    // pa_attn_layer_decode: [q(+gate) | k | v] projections, then attnOut [nH*hd]
   size_t proj_buf_bytes = 0;
+  void* w16_buf = nullptr;      // pa_gemm on large chunks: the call's weights widened to f16 [d_out][d_in]
+  size_t w16_buf_bytes = 0;
   void* chunk_buf = nullptr;    // pa_attn_layer_prefill: xn f16 [cols][dim], qkv f32 [cols][rows], attnOut f16 [cols][nH*hd]
   size_t chunk_buf_bytes = 0;
   uint16_t* wide_k = nullptr; uint16_t* wide_v = nullptr;   // int8 caches: f16 staging cache of one layer for the prefill kernel

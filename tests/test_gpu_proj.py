@@ -144,21 +144,34 @@ def test_gemm_matches_oracle(kind, d_out, d_in, n):
         assert _rel(dy.download(np.float32, n * ys).reshape(n, ys)[:, :d_out], 2.0 * ref) < 2e-5, "accumulate"
 
 
-@pytest.mark.parametrize("kind", [PA_W_Q8_0, PA_W_Q4_0])
-def test_gemm_large_chunk_takes_the_256_column_workgroups(kind):
-    """A chunk large enough to give every CU four 256-column workgroups (the [q | k | v] projection of a 4096-column
-    chunk) runs the kernel's wide form; ragged edges on both axes."""
-    d_out, d_in, n = 9216 - 40, 2048, 4096 - 3
-    rng = np.random.default_rng(kind)
+@pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q8_0, PA_W_Q4_0])
+@pytest.mark.parametrize("d_out,d_in,n", [(9216 - 40, 2048, 4096 - 3), (2048, 4096, 600), (300, 128, 520), (130, 8192, 513), (1000, 64, 1100)])
+def test_gemm_large_chunks(kind, d_out, d_in, n):
+    """Chunks of 512 columns and more over d_in a multiple of 64: the weights are widened once into the context's f16
+    staging matrix and the GEMM runs over two f16 operands (128-column wave tiles, 128 to 256 weight rows a workgroup).
+    Ragged edges on both axes, padded strides that must stay untouched, the accumulating form, and a second call with
+    other weights through the same staging matrix."""
+    if kind == PA_W_F32 and d_in > 4096:
+        pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
+    rng = np.random.default_rng(d_out + d_in + n + kind)
     w, sc = _weights(kind, d_out, d_in, rng)
     x16 = rng.standard_normal((n, d_in)).astype(np.float16)
     ref = O.gemm_f16(kind, w, sc, x16.astype(np.float32))
+    xs, ys = d_in + 8, d_out + 5
+    xpad = np.zeros((n, xs), np.float16); xpad[:, :d_in] = x16
+    y0 = rng.standard_normal((n, ys)).astype(np.float32)
     with PooledAttn(SHAPES["qwen36_moe"], 64, n_layers=1, max_cols=1) as pa:
         wh = pa.weight(kind, w, sc)
-        dx = pa.to_device(x16.view(np.uint16)); dy = pa.alloc(n * d_out * 4)
-        pa.gemm(wh, dx, d_in, n, dy, d_out); pa.sync()
-        got = dy.download(np.float32, n * d_out).reshape(n, d_out)
-    assert _rel(got, ref) < 2e-5
+        dx = pa.to_device(xpad.view(np.uint16)); dy = pa.to_device(y0)
+        pa.gemm(wh, dx, xs, n, dy, ys); pa.sync()
+        got = dy.download(np.float32, n * ys).reshape(n, ys)
+        assert _rel(got[:, :d_out], ref) < 2e-5, "plain"
+        assert np.array_equal(got[:, d_out:], y0[:, d_out:]), "the stride padding of y must stay untouched"
+        pa.gemm(wh, dx, xs, n, dy, ys, acc=True); pa.sync()
+        assert _rel(dy.download(np.float32, n * ys).reshape(n, ys)[:, :d_out], 2.0 * ref) < 2e-5, "accumulate"
+        w2, sc2 = _weights(kind, d_out, d_in, rng)
+        pa.gemm(pa.weight(kind, w2, sc2), dx, xs, n, dy, ys); pa.sync()
+        assert _rel(dy.download(np.float32, n * ys).reshape(n, ys)[:, :d_out], O.gemm_f16(kind, w2, sc2, x16.astype(np.float32))) < 2e-5, "second weight"
 
 
 def test_rmsnorm_f16_columns():
