@@ -142,7 +142,7 @@ def prefill_leg(steps, with_cpu, kv_q8=False):
                         % ("int8 (widened once per chunk into an f16 staging cache, inside the step)" if kv_q8 else "f16"),
                value=round(tf_step, 1), unit="TFLOP/s", ms_per_step=round(ms_step, 4), steps=steps, flops_per_step=flops, plan=pa.plan("prefill", base, n),
                roofline=dict(bound="mfma", achieved=round(tf_kernel, 1), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s", frac=round(tf_kernel / MFMA_F16_PEAK_TFLOPS, 4),
-                             traffic=None, kernel="pa_prefill_kernel<256, 1, 8, false>", kernel_ms=round(k_ms, 4), algorithmic_flops_per_launch=flops, launches=kcount))
+                             traffic=None, kernel="pa_prefill_kernel<256, 1, 8>", kernel_ms=round(k_ms, 4), algorithmic_flops_per_launch=flops, launches=kcount))
     if with_cpu:
         # CPU leg: the reference loops on a fixed subsample (head group of kv head 0 is irrelevant to the loops: all
         # 16 heads of 4 evenly spaced columns), scaled by columns; labelled extrapolated

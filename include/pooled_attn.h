@@ -295,6 +295,14 @@ int pa_rmsnorm_f16(pa_ctx* ctx, const float* d_x, uint32_t x_stride, const float
  * passes through its batched matvec, engine/wgsl/coop.js) are served by a kernel that streams the weights once per
  * 16 columns instead of the tiled one; same operand precision either way. */
 int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uint32_t x_stride, uint32_t n_cols, float* d_y, uint32_t y_stride, int acc);
+/* Chunks of 512 columns and more run on a GEMM over two f16 operands: the weight handle's values widened to f16
+ * ((nibble - 8) * scale, int8 * scale, f32 rounded -- the arithmetic of the tiled kernel's staging, so results do not
+ * depend on which way a call goes) in matrix-core fragment order.  That copy (2 bytes a weight) is made on the first
+ * such call on a handle (which therefore allocates: not under stream capture) and kept until pa_weight_destroy, while
+ * the copies kept by this context stay within max_bytes (default 8 GiB; 0: keep none); past the budget a call widens
+ * into per-context staging every time (+8 % on a 4096 x 9216 x 2048 chunk).  Changing the budget keeps what is
+ * already held.  No counterpart in the reference, whose WGSL GEMMs dequantise in the inner loop. */
+int pa_set_weight_cache(pa_ctx* ctx, size_t max_bytes);
 /* n_cols tokens at positions base_pos .. through the attention half of a full-attention layer, as
  * _encodeLayerBatch / _encodeLayerWide record it (engine/qwen35.js:2416-2425, :2827): rmsnorm -> [q | k | v] GEMM ->
  * pre-step + cache write -> causal attention -> gate -> wo GEMM accumulated into the residual columns d_x

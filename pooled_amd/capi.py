@@ -56,6 +56,7 @@ SYMBOLS = {
     "pa_plan_query": (c_int, [vp, c_int, u32, u32, ctypes.POINTER(PaPlan)]),
     "pa_set_decode_splits": (c_int, [vp, u32]),
     "pa_set_prefill_tile": (c_int, [vp, c_int]),
+    "pa_set_weight_cache": (c_int, [vp, ctypes.c_size_t]),
     "pa_kv_read": (c_int, [vp, u32, c_int, u32, u32, vp]),
     "pa_kv_write": (c_int, [vp, u32, c_int, u32, u32, vp]),
     "pa_kv_row_bytes": (ctypes.c_size_t, [vp, c_int]),
@@ -264,6 +265,10 @@ class PooledAttn:
     def set_prefill_tile(self, mode):
         """0: the table picks the kernel of a prefill chunk, 1: always the matrix-core kernel, 2: never."""
         self._chk(self.L.pa_set_prefill_tile(self.ctx, mode))
+
+    def set_weight_cache(self, max_bytes):
+        """Budget of the f16 weight copies that large-chunk gemm calls keep with their weight handles (0: keep none)."""
+        self._chk(self.L.pa_set_weight_cache(self.ctx, max_bytes))
 
     # ---- timing ----
     def timer_start(self):

@@ -855,19 +855,13 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
 // the output partials of its group's splits (group + 16 k) in one round trip, the maximum and the sums over the 16
 // groups are xor-shuffle trees (fixed order), lanes 0 .. 3 finish and store.  The four lanes of a group hold the same
 // (m, l), so each computes its splits' weights itself instead of fetching them from a neighbour.
-#ifndef PA_COMBINE_XCD
-#define PA_COMBINE_XCD 1
-#endif
-#ifndef PA_COMBINE_DS
-#define PA_COMBINE_DS 16
-#endif
 template <int HD, int DS>
 __global__ __launch_bounds__(64) void pa_combine_wave_kernel(AttnParams p) {
   constexpr int SL = HD / DS, LPG = DS / 4, NG = 64 / LPG, CH = (272 + NG - 1) / NG;     // CH splits per lane and chunk: NG x CH >= 272 (256 + the own-row partial)
   // dispatch id i runs on XCD i % 8: XCD k takes the contiguous slice range [k n / 8, (k + 1) n / 8), so the slices that
   // share the 128-byte lines of a partial row (two 16-dim slices a line) read them through one L2
   uint32_t wg = blockIdx.x;
-  if (PA_COMBINE_XCD && gridDim.x % 8 == 0) wg = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+  if (gridDim.x % 8 == 0) wg = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
   const uint32_t h = wg / SL, dq = wg % SL, col = blockIdx.y, lane = threadIdx.x;
   const uint32_t col_end = p.sel ? min(p.sel[col * p.sel_stride], p.sel_max) : p.base_pos + col + 1 - p.self_row;
   const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
@@ -1081,8 +1075,8 @@ hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s) {
     else hipLaunchKernelGGL(pa_combine_wide_kernel<128>, grid, dim3(256), 0, s, p);
     return hipGetLastError();
   }
-  if (hd == 256) hipLaunchKernelGGL((pa_combine_wave_kernel<256, PA_COMBINE_DS>), dim3(p.n_heads * (256 / PA_COMBINE_DS), p.n_cols), dim3(64), 0, s, p);
-  else if (hd == 128) hipLaunchKernelGGL((pa_combine_wave_kernel<128, PA_COMBINE_DS>), dim3(p.n_heads * (128 / PA_COMBINE_DS), p.n_cols), dim3(64), 0, s, p);
+  if (hd == 256) hipLaunchKernelGGL((pa_combine_wave_kernel<256, 16>), dim3(p.n_heads * (256 / 16), p.n_cols), dim3(64), 0, s, p);
+  else if (hd == 128) hipLaunchKernelGGL((pa_combine_wave_kernel<128, 16>), dim3(p.n_heads * (128 / 16), p.n_cols), dim3(64), 0, s, p);
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }

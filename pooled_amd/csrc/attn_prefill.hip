@@ -30,27 +30,12 @@
 //     (m, l, O) go to the same buffers the decode kernel uses and the same merge kernel finishes them.
 #include "pf_common.h"
 
-#ifndef PF_PRIO
-#define PF_PRIO 0
-#endif
-#ifndef PF_ABL
-#define PF_ABL 0        // development ablations (wrong results, timing only): bit 0 no exp, 1 one K fragment, 2 one V fragment, 3 no softmax, 4 no tile loads in the loop
-#endif
-#ifndef PF_KD
-#define PF_KD 4
-#endif
-#ifndef PF_QR
-#define PF_QR 8
-#endif
-#ifndef PF_VD
-#define PF_VD 3
-#endif
 template <int HD, int W> struct PfShape {
   static constexpr int ROWB = HD * 2;             // bytes of one kv head's row
   static constexpr int TILE = PF_TN * ROWB;       // bytes of one staged tile (K or V)
   static constexpr int KS = HD / 16;              // k-steps of QK^T
   static constexpr int DB = HD / 32;              // 32-dim blocks of the output
-  static constexpr int QR = HD == 256 ? PF_QR : KS;   // k-steps whose Q fragments stay in registers
+  static constexpr int QR = HD == 256 ? 8 : KS;   // k-steps whose Q fragments stay in registers
   static constexpr int CPR = HD / 8;              // 16-byte chunks per row
   static constexpr int RPB = 64 / CPR;            // rows per 1 KB LDS-direct load
   static constexpr int NLD = PF_TN / RPB / W;     // LDS-direct loads per wave, tensor and step
@@ -201,11 +186,11 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 #pragma unroll
       for (int i = 0; i < 16; i++) s[qb][i] = 0.f;
     // K fragments (and the Q fragments parked in LDS) are fetched KD k-steps ahead of the MFMA that consumes them
-    constexpr int KD = PF_KD;
+    constexpr int KD = 4;
     h8 ka[KD], qa[QB][KD];
 #pragma unroll
     for (int i = 0; i < KD; i++) {
-      ka[i] = *(const h8*)(kb + (k_rd ^ ((PF_ABL & 2) ? 0 : i * 32)));
+      ka[i] = *(const h8*)(kb + (k_rd ^ (i * 32)));
       if (i >= QR) {
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) qa[qb][i] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (i - QR)) * 1024);
@@ -218,7 +203,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 #pragma unroll
       for (int qb = 0; qb < QB; qb++) b[qb] = ks < QR ? qf[qb][ks < QR ? ks : 0] : qa[qb][ks % KD];
       if (ks + KD < S::KS) {
-        if (!(PF_ABL & 2)) ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
+        ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
         if (ks + KD >= QR) {
 #pragma unroll
           for (int qb = 0; qb < QB; qb++) qa[qb][ks % KD] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (ks + KD - QR)) * 1024);
@@ -241,13 +226,6 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   // v_dot2 over the f16-rounded probabilities (the values PV really uses), and the mask is a separate pass
   // that only tiles straddling a row end execute.
   auto sm = [&](const uint32_t tp) {
-    if (PF_ABL & 8) {
-#pragma unroll
-      for (int qb = 0; qb < QB; qb++)
-#pragma unroll
-        for (int i = 0; i < 16; i += 2) { pf[qb][i >> 3][i & 7] = (_Float16)s[qb][i]; pf[qb][i >> 3][(i & 7) + 1] = (_Float16)s[qb][i + 1]; }
-      return;
-    }
     if (tp + PF_TN > w_min_end) {
       asm volatile("; causal tile" ::: "memory");   // keeps this a branch: most tiles skip the 3 ops per element
 #pragma unroll
@@ -288,8 +266,8 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
       float ps = l_run[qb];
 #pragma unroll
       for (int i = 0; i < 16; i += 2) {
-        const float e0 = (PF_ABL & 1) ? __builtin_fmaf(s[qb][i], c1, nmr) : __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], c1, nmr));
-        const float e1 = (PF_ABL & 1) ? __builtin_fmaf(s[qb][i + 1], c1, nmr) : __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], c1, nmr));
+        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], c1, nmr));
+        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], c1, nmr));
         const h2 pp = { (_Float16)e0, (_Float16)e1 };
         ps = __builtin_amdgcn_fdot2(pp, ones, ps, false);
         pf[qb][i >> 3][i & 7] = pp[0]; pf[qb][i >> 3][(i & 7) + 1] = pp[1];
@@ -301,7 +279,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   auto pv = [&](const unsigned char* vb, const uint32_t tp) {
     // fragment f = j DB + db: positions 16 j .., dims 32 db .. (consecutive MFMAs hit different accumulators);
     // fetched VD fragments ahead
-    constexpr int VD = PF_VD, NF = 2 * S::DB;
+    constexpr int VD = 3, NF = 2 * S::DB;
     h4 vlo[VD], vhi[VD];
 #pragma unroll
     for (int f = 0; f < VD; f++) {
@@ -312,7 +290,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 #pragma unroll
     for (int f = 0; f < NF; f++) {
       const h4 lo = vlo[f % VD], hi = vhi[f % VD];
-      if (f + VD < NF && !(PF_ABL & 4)) {
+      if (f + VD < NF) {
         const int fn = f + VD;
         const unsigned char* vp = vb + (v_rd ^ ((fn % S::DB) * 64)) + (fn / S::DB) * 16 * S::ROWB;
         vlo[f % VD] = lds_read_tr16(vp);
@@ -338,14 +316,10 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     auto step_s = [&](auto PAR, const uint32_t i) {
       constexpr int par = decltype(PAR)::value;
       const uint32_t tp = t_begin + i * PF_TN;
-      if (i + 1 < n_steps && !((PF_ABL & 16) && i > 0)) { issue_k(par ? kbuf0 : kbuf1, tp + PF_TN); issue_v(par ? vbuf0 : vbuf1, tp + PF_TN); }
-      if (PF_PRIO) __builtin_amdgcn_s_setprio(PF_PRIO);
+      if (i + 1 < n_steps) { issue_k(par ? kbuf0 : kbuf1, tp + PF_TN); issue_v(par ? vbuf0 : vbuf1, tp + PF_TN); }
       qk(par ? kbuf1 : kbuf0, tp);
-      if (PF_PRIO) __builtin_amdgcn_s_setprio(0);
       sm(tp);
-      if (PF_PRIO) __builtin_amdgcn_s_setprio(PF_PRIO);
       pv(par ? vbuf1 : vbuf0, tp);
-      if (PF_PRIO) __builtin_amdgcn_s_setprio(0);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
     };

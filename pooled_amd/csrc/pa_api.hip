@@ -668,7 +668,14 @@ extern "C" int pa_weight_destroy(pa_ctx* ctx, pa_weight* w) {
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   if (w->w) (void)hipFree(w->w);
   if (w->scales) (void)hipFree(w->scales);
+  if (w->w16) { (void)hipFree(w->w16); ctx->weight_cache_used -= std::min(ctx->weight_cache_used, w->w16_bytes); }
   delete w;
+  return PA_OK;
+}
+
+extern "C" int pa_set_weight_cache(pa_ctx* ctx, size_t max_bytes) {
+  if (!ctx) return PA_ERR_INVALID;
+  ctx->weight_cache_limit = max_bytes;
   return PA_OK;
 }
 
@@ -735,9 +742,24 @@ extern "C" int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uin
   p.w = w->w; p.scales = w->scales; p.x = (const uint16_t*)d_x_f16; p.y = d_y; p.x_stride = x_stride; p.y_stride = y_stride;
   p.d_out = w->d_out; p.d_in = w->d_in; p.n_cols = n_cols; p.acc = acc; p.kind = w->kind;
   if (pa_gemm_wide_serves(p, ctx->n_cu)) {
-    int rc = grow_scratch(ctx, &ctx->w16_buf, &ctx->w16_buf_bytes, (size_t)w->d_out * w->d_in * sizeof(uint16_t));
-    if (rc) return rc;
-    HIPCHK(ctx, pa_launch_gemm_wide(p, (uint16_t*)ctx->w16_buf, ctx->n_cu, ctx->stream));
+    // the weights as f16 in fragment order: a copy kept with the weight from its first large chunk on, while the
+    // context's budget lasts (the handle's contents never change); past the budget, or where the allocation fails,
+    // widened per call into the context's staging
+    const size_t need = pa_gemm_wide_staging_bytes(w->d_out, w->d_in);
+    pa_weight* wm = const_cast<pa_weight*>(w);
+    bool widen = false;
+    if (!wm->w16 && ctx->weight_cache_used + need <= ctx->weight_cache_limit) {
+      void* buf = nullptr;
+      if (hipMalloc(&buf, need) == hipSuccess) { wm->w16 = (uint16_t*)buf; wm->w16_bytes = need; ctx->weight_cache_used += need; widen = true; }
+      else (void)hipGetLastError();
+    }
+    uint16_t* w16 = wm->w16;
+    if (!w16) {
+      int rc = grow_scratch(ctx, &ctx->w16_buf, &ctx->w16_buf_bytes, need);
+      if (rc) return rc;
+      w16 = (uint16_t*)ctx->w16_buf; widen = true;
+    }
+    HIPCHK(ctx, pa_launch_gemm_wide(p, w16, widen, ctx->n_cu, ctx->stream));
     return PA_OK;
   }
   HIPCHK(ctx, pa_launch_gemm(p, ctx->n_cu, ctx->stream));

@@ -107,10 +107,11 @@ struct GemmParams {
   int acc; int kind;
 };
 hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s);
-// large chunks (proj_gemm_wide.hip): the weights widened once into w16 (f16 [d_out][d_in], the caller's staging), then a
+// large chunks (proj_gemm_wide.hip): the weights widened once into w16 (f16 in fragment order, the caller's staging), then a
 // GEMM over two f16 operands; pa_gemm_wide_serves tells whether a call qualifies
 bool pa_gemm_wide_serves(const GemmParams& p, int n_cu);
-hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, int n_cu, hipStream_t s);
+size_t pa_gemm_wide_staging_bytes(uint32_t d_out, uint32_t d_in);
+hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, bool widen, int n_cu, hipStream_t s);
 // rmsnorm of n_cols f32 columns, written as f16 (the GEMM's activation operand)
 hipError_t pa_launch_rmsnorm_f16(const float* x, uint32_t x_stride, const float* w, uint32_t dim, float eps, uint32_t n_cols,
                                  uint16_t* out, uint32_t out_stride, hipStream_t s);
@@ -139,6 +140,8 @@ struct pa_weight {
   uint32_t d_out = 0, d_in = 0;
   void* w = nullptr;              // values plane on the device
   uint16_t* scales = nullptr;     // f16 bits [d_out][d_in / 32]; nullptr for f32 weights
+  uint16_t* w16 = nullptr;        // the weights widened to f16 in fragment order, kept from the first large-chunk pa_gemm on
+  size_t w16_bytes = 0;           // (while the context's budget lasts); nullptr: widened per call into the context's staging
 };
 
 struct pa_ctx {
@@ -159,6 +162,7 @@ struct pa_ctx {
   size_t proj_buf_bytes = 0;
   void* w16_buf = nullptr;      // pa_gemm on large chunks: the call's weights widened to f16 [d_out][d_in]
   size_t w16_buf_bytes = 0;
+  size_t weight_cache_limit = (size_t)8 << 30, weight_cache_used = 0;   // pa_set_weight_cache: budget of the kept f16 copies
   void* chunk_buf = nullptr;    // pa_attn_layer_prefill: xn f16 [cols][dim], qkv f32 [cols][rows], attnOut f16 [cols][nH*hd]
   size_t chunk_buf_bytes = 0;
   uint16_t* wide_k = nullptr; uint16_t* wide_v = nullptr;   // int8 caches: f16 staging cache of one layer for the prefill kernel

@@ -189,6 +189,7 @@ static napi_value PlanQuery(napi_env env, napi_callback_info info) {
   return o;
 }
 static napi_value SetPrefillTile(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); int m = (int)a.u32(1); CHECK_ARGS("setPrefillTile"); int rc = pa_set_prefill_tile(c, m); if (rc) return throw_pa(env, c, rc, "pa_set_prefill_tile"); return undefined(env); }
+static napi_value SetWeightCache(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); double b = a.num(1); CHECK_ARGS("setWeightCache"); int rc = pa_set_weight_cache(c, b <= 0 ? 0 : (size_t)b); if (rc) return throw_pa(env, c, rc, "pa_set_weight_cache"); return undefined(env); }
 static napi_value SetDecodeSplits(napi_env env, napi_callback_info info) { ARGS; pa_ctx* c = a.ctx(0); uint32_t s = a.u32(1); CHECK_ARGS("setDecodeSplits"); int rc = pa_set_decode_splits(c, s); if (rc) return throw_pa(env, c, rc, "pa_set_decode_splits"); return undefined(env); }
 // kvRead(ctx, layer, which, row0, nRows, Uint16Array) / kvWrite(ctx, layer, which, row0, nRows, Uint16Array)
 static napi_value KvRead(napi_env env, napi_callback_info info) {
@@ -295,7 +296,7 @@ static napi_value Init(napi_env env, napi_value exports) {
     {"create", Create}, {"destroy", Destroy}, {"lastError", LastError}, {"version", Version}, {"layerAlloc", LayerAlloc}, {"sync", Sync},
     {"setStream", SetStream}, {"malloc", Malloc}, {"free", Free}, {"upload", Upload}, {"download", Download}, {"glueKv", GlueKv}, {"glue", Glue},
     {"kvStore", KvStore}, {"qBuffer", QBuffer}, {"gateBuffer", GateBuffer}, {"attn", Attn}, {"planQuery", PlanQuery},
-    {"setDecodeSplits", SetDecodeSplits}, {"setPrefillTile", SetPrefillTile}, {"kvRead", KvRead}, {"kvWrite", KvWrite}, {"kvDevicePtr", KvDevicePtr}, {"timerStart", TimerStart},
+    {"setDecodeSplits", SetDecodeSplits}, {"setPrefillTile", SetPrefillTile}, {"setWeightCache", SetWeightCache}, {"kvRead", KvRead}, {"kvWrite", KvWrite}, {"kvDevicePtr", KvDevicePtr}, {"timerStart", TimerStart},
     {"timerStop", TimerStop}, {"profileEnable", ProfileEnable}, {"profileRead", ProfileRead}, {"attnDecodeStep", AttnDecodeStep},
     {"copyD2d", CopyD2d}, {"attnGather", AttnGather}, {"slotSave", SlotSave}, {"slotLoad", SlotLoad}, {"slotDrop", SlotDrop}, {"slotPos", SlotPos},
     {"slotCreate", SlotCreate}, {"slotExport", SlotExport}, {"slotImport", SlotImport}, {"weightCreate", WeightCreate},

@@ -1,5 +1,5 @@
 // Column-batched projections for large chunks on gfx950: Y[c][r] = sum_k W[r][k] X[c][k] with the weights widened
-// to f16 once per call and a matrix-core GEMM over two f16 operands.
+// to f16 once and a matrix-core GEMM over two f16 operands.
 //
 // Same contract and the same operand precision as pa_gemm_kernel (proj_gemm.hip) -- the reference's "f16" prefill
 // math, engine/wgsl/gemm.js:31-36: every dequantised weight and every activation rounded to f16, products and sums
@@ -7,30 +7,41 @@
 // engine/qwen35.js:2142-2170, :2600-2620).  What differs is where the widening happens.  The tiled kernel of
 // proj_gemm.hip widens packed weights on their way into LDS inside its main loop; at 64 x 64 wave tiles that loop is
 // bound by LDS traffic and by the widening arithmetic in front of every barrier.  For a chunk of hundreds of columns
-// the weights are re-read by every column block anyway, so here they are widened once into a context-owned f16
-// staging matrix [d_out][d_in] (pa_widen_w_kernel: one pass over the packed planes, HBM-bound), and the GEMM proper
-// has nothing but loads and MFMAs in its loop:
+// the weights are re-read by every column block anyway, so here they are widened once into an f16 staging matrix
+// (pa_widen_w_kernel: one pass over the packed planes, HBM-bound; the caller keeps the matrix with the weight or
+// widens per call), and the GEMM proper has nothing but loads and MFMAs in its loop:
 //
-//   * workgroup = 2 x 2 wavefronts, one per SIMD; a wavefront owns 128 columns x 32 TN rows (TN = 2, 3 or 4) as
-//     4 x TN v_mfma_f32_32x32x16_f16 tiles whose accumulators (up to 256 registers) live in the accumulation
-//     registers; every A (activation) fragment read from LDS feeds TN MFMAs and every B (weight) fragment four:
-//     0.5 KB of LDS reads per MFMA at TN = 4 against 1 KB at 64 x 64 wave tiles;
-//   * both operands go global -> LDS with global_load_lds_dwordx4 (no staging registers, no arithmetic), K in
-//     stages of 64 (128-byte rows), two stages in LDS, one barrier a stage; rows cannot be padded (an LDS-direct
-//     load writes 64 x 16 bytes contiguously), so the 16-byte chunk c of row r is fetched into slot
-//     c ^ ((r >> 1) & 7): the ds_read_b128 fragment reads of any 16 consecutive rows then hit 64 distinct banks;
-//   * one wave a SIMD means nothing hides an LDS round trip, so the fragments are double buffered in registers by
-//     hand: the reads of k-step i + 1 (and, across the barrier, of the next stage's first k-step) are issued among
-//     the MFMAs of k-step i;
+//   * a wavefront owns 128 columns x 32 TN weight rows (TN = 2, 3 or 4) as 4 x TN v_mfma_f32_32x32x16_f16 tiles whose
+//     accumulators (up to 256 registers) live in the accumulation registers, one wave a SIMD; a workgroup is four
+//     such waves side by side along the weight rows: 128 columns x 128 TN rows;
+//   * the staging matrix is written in MFMA fragment order -- for every block of 32 rows and 16 k the 64 lanes' 16
+//     bytes are contiguous (1 KB) -- so a weight (B) fragment is ONE coalesced wave-wide load straight into the
+//     registers the MFMA reads: the weights never touch LDS.  (With both operands staged through LDS, the fragment
+//     reads and the staging writes together kept the LDS port 75 % busy and the loop ran at 740 - 790 TFLOP/s.)  The
+//     fragments of eight k-steps (four at TN = 4) are in flight per wave, a register ring refilled slot by slot
+//     behind the MFMAs that used it;
+//   * the activations (A), which all four waves share, go through LDS, K in stages of 64 (128-byte rows), two stages
+//     in LDS, one bare barrier a stage; a stage is fetched into registers a stage ahead and written with ds_write
+//     (16 registers), rows unpadded with the 16-byte chunk c of row r at slot c ^ ((r >> 1) & 7): the ds_read_b128
+//     fragment reads of any 16 consecutive rows then hit 64 distinct banks.  One wave a SIMD means nothing hides an
+//     LDS round trip, so the A fragments are double buffered in registers by hand: the reads of k-step i + 1 (across
+//     the barrier: of the next stage's first k-step) are issued among the MFMAs of k-step i;
+//   * every load is a plain load the compiler sees, and the issue order is pinned (scheduling barriers per k-step,
+//     the prologue's ring loads in ring order): its vmcnt waits then let a whole ring of fragments stay in flight.
+//     An LDS-direct load issued from inline assembly shares the in-order counter without the compiler knowing, and
+//     a ring slot loaded late in the prologue makes the wait at the head of the loop drain the ring every iteration
+//     (both measured: 0.21 ms instead of 0.18 on a 4096 x 9216 x 2048 chunk);
+//   * workgroup ids are dealt so that the 32 workgroups an XCD runs side by side form a block of 8 column blocks x 4
+//     row blocks, which share 8 activation tiles and 4 weight panels in that XCD's L2 (3 % over row-major order);
 //   * TN is picked per call so that the workgroups fill whole rounds of the chip.
+//
+// Measured on a 4096 x 9216 x 2048 Q4_0 chunk (0.178 ms, 869 TFLOP/s with the staging matrix kept): without the
+// output stores 0.163 ms, without the weight loads of the loop 0.163, with neither and no activation loads 0.134.
 #include "pf_common.h"
 
-#ifndef GW_ABL
-#define GW_ABL 0            // development ablations (wrong results, timing only): bit 0 no loads after the prologue, bit 1 no barriers
-#endif
-#define GW_COLS 256          // columns per workgroup (2 waves x 128)
+#define GW_COLS 128          // columns per workgroup
 #define GW_KS 64             // K per stage
-#define GW_ROWB 128          // bytes of a staged row (64 halves)
+#define GW_ROWB 128          // bytes of a staged activation row (64 halves)
 
 struct Gemm16Params {
   const uint16_t* x; const uint16_t* w16; float* y;
@@ -38,43 +49,68 @@ struct Gemm16Params {
   int acc;
 };
 
-template <int TN>
+template <int TN, bool ACC>
 __global__ __launch_bounds__(256, 1) void pa_gemm16_kernel(Gemm16Params p) {
   constexpr int TM = 4;                                  // 32-column blocks per wave
-  constexpr int ROWS = 64 * TN;                          // weight rows per workgroup
-  constexpr int A_BYTES = GW_COLS * GW_ROWB, B_BYTES = ROWS * GW_ROWB, STAGE = A_BYTES + B_BYTES;
-  constexpr int A_LD = GW_COLS / 8 / 4, B_LD = ROWS / 8 / 4;     // 1 KB loads (8 rows) per wave and stage
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];   // [2][A | B]
+  constexpr int ROWS = 128 * TN;                         // weight rows per workgroup (4 waves x 32 TN)
+  constexpr int STAGE = GW_COLS * GW_ROWB;               // bytes of a staged A tile
+  constexpr int A_LD = GW_COLS / 8 / 4;                  // 1 KB loads (8 rows) per wave and stage
+  constexpr int RING = TN == 4 ? 4 : 8;                  // k-steps of weight fragments in flight per wave (what the register file holds next to 4 x TN accumulator tiles)
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * STAGE];
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t wm = wave >> 1, wn = wave & 1;
-  const uint32_t c0 = blockIdx.y * GW_COLS, r0 = blockIdx.x * ROWS;
-  const uint32_t n_stages = p.d_in / GW_KS;
+  // XCD-aware tile order: dispatch id i runs on XCD i % 8 as that XCD's (i / 8)-th workgroup, so XCD k walks the tiles
+  // [k per, (k + 1) per) of a linear order in which 32 neighbours (what an XCD runs at a time) form a block of 8
+  // column blocks x 4 row blocks: they share 8 activation tiles and 4 weight panels in that XCD's L2 instead of 32 + 1
+  const uint32_t n_cb = (p.n_cols + GW_COLS - 1) / GW_COLS, n_rb = (p.d_out + ROWS - 1) / ROWS, total = n_cb * n_rb;
+  const uint32_t per = (total + 7) / 8, tile = (blockIdx.x % 8) * per + blockIdx.x / 8;
+  if (tile >= total) return;
+  uint32_t cb = tile % n_cb, rb_ = tile / n_cb;
+  if (n_cb % 8 == 0) {
+    const uint32_t panel = tile / (4 * n_cb), r = tile % (4 * n_cb), h = min(4u, n_rb - panel * 4);
+    cb = r / (8 * h) * 8 + r % 8; rb_ = panel * 4 + r % (8 * h) / 8;
+  }
+  const uint32_t c0 = cb * GW_COLS, r0 = rb_ * ROWS;
+  const uint32_t n_stages = p.d_in / GW_KS, nk16 = p.d_in / 16;
 
-  // ---- LDS-direct loads: a load covers 8 rows x 128 bytes; lane i lands at (row i / 8, slot i % 8) and fetches chunk
-  //      slot ^ ((row >> 1) & 7) of that row.  Rows past the end of the operand repeat its last row (never stored). ----
+  // ---- A: LDS-direct loads, 8 rows x 128 bytes each; lane i lands at (row i / 8, slot i % 8) and fetches chunk
+  //      slot ^ ((row >> 1) & 7) of that row.  Columns past the end of the chunk repeat its last column (never stored).
   const uint32_t lrow = lane >> 3, lslot = lane & 7;
-  const unsigned char* a_src[A_LD]; const unsigned char* b_src[B_LD];
+  const unsigned char* a_src[A_LD];
 #pragma unroll
   for (int i = 0; i < A_LD; i++) {
-    const uint32_t row = (wave * A_LD + i) * 8 + lrow;                       // row of the A tile = column of the chunk
+    const uint32_t row = (wave * A_LD + i) * 8 + lrow;
     const size_t col = min((size_t)c0 + row, (size_t)p.n_cols - 1);
     a_src[i] = (const unsigned char*)(p.x + col * p.x_stride) + ((lslot ^ ((row >> 1) & 7)) * 16);
   }
-#pragma unroll
-  for (int i = 0; i < B_LD; i++) {
-    const uint32_t row = (wave * B_LD + i) * 8 + lrow;
-    const size_t wr = min((size_t)r0 + row, (size_t)p.d_out - 1);
-    b_src[i] = (const unsigned char*)(p.w16 + wr * p.d_in) + ((lslot ^ ((row >> 1) & 7)) * 16);
-  }
-  const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr_of(smem));
-  auto issue = [&](uint32_t st) __attribute__((always_inline)) {
-    const uint32_t base = lds0 + (st & 1) * STAGE;
+  // the stage's 16 bytes per lane and load go through registers (fetched a stage ahead) and a ds_write: every load of
+  // the loop is then visible to the compiler, whose vmcnt waits count the weight-fragment ring correctly (an LDS-direct
+  // load issued from inline assembly sits in the same in-order counter without the compiler knowing, and its
+  // conservative wait for a ring slot then also waits for the just-issued activation loads)
+  u4 areg[A_LD];
+  auto fetch_a = [&](uint32_t st) __attribute__((always_inline)) {
     const size_t koff = (size_t)st * GW_ROWB;
 #pragma unroll
-    for (int i = 0; i < A_LD; i++) pf_gll(a_src[i] + koff, base + (wave * A_LD + i) * 1024);
+    for (int i = 0; i < A_LD; i++) areg[i] = *(const u4*)(a_src[i] + koff);
+  };
+  auto store_a = [&](uint32_t buf) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < B_LD; i++) pf_gll(b_src[i] + koff, base + A_BYTES + (wave * B_LD + i) * 1024);
+    for (int i = 0; i < A_LD; i++) *(u4*)(smem + buf * STAGE + (wave * A_LD + i) * 1024 + lane * 16) = areg[i];
+  };
+  // ---- B: fragment (row block rb, k block kb) of the staging matrix = 1 KB at ((rb nk16 + kb) 64 + lane) 16; the
+  //      staging matrix is padded to whole 32-row blocks, row blocks past d_out repeat the last one (never stored)
+  const uint32_t n_rb32 = (p.d_out + 31) / 32;
+  const unsigned char* b_src[TN];
+#pragma unroll
+  for (int t = 0; t < TN; t++) {
+    const uint32_t rb = min(r0 / 32 + wave * TN + t, n_rb32 - 1);
+    b_src[t] = (const unsigned char*)p.w16 + ((size_t)rb * nk16 * 64 + lane) * 16;
+  }
+  u4 ring[RING][TN];
+  auto load_b = [&](int slot, uint32_t kb) __attribute__((always_inline)) {
+    const size_t off = (size_t)min(kb, nk16 - 1) * 1024;         // past the last k block: the last one again, never used
+#pragma unroll
+    for (int t = 0; t < TN; t++) ring[slot][t] = *(const u4*)(b_src[t] + off);
   };
 
   f16v acc[TM][TN];
@@ -85,87 +121,121 @@ __global__ __launch_bounds__(256, 1) void pa_gemm16_kernel(Gemm16Params p) {
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
 
-  // fragment addresses: row fl of a 32-row block, 8 halves at k = 16 ks + 8 fk -> chunk 2 ks + fk, swizzled by the row
-  // (the swizzle is an XOR on the chunk index, and 2 ks has no bit in common with fk)
+  // A fragment addresses: row fl of a 32-row block, 8 halves at k = 16 ks + 8 fk -> chunk 2 ks + fk, swizzled by the
+  // row (the swizzle is an XOR on the chunk index, and 2 ks has no bit in common with fk)
   const uint32_t fl = lane & 31, fk = lane >> 5;
-  uint32_t a_rd[TM], b_rd[TN];
+  uint32_t a_rd[TM];
 #pragma unroll
-  for (int t = 0; t < TM; t++) { const uint32_t row = wm * 128 + t * 32 + fl; a_rd[t] = row * GW_ROWB + ((fk ^ ((row >> 1) & 7)) * 16); }
-#pragma unroll
-  for (int t = 0; t < TN; t++) { const uint32_t row = wn * 32 * TN + t * 32 + fl; b_rd[t] = A_BYTES + row * GW_ROWB + ((fk ^ ((row >> 1) & 7)) * 16); }
-  struct Frag { h8 a[TM]; h8 b[TN]; };
+  for (int t = 0; t < TM; t++) { const uint32_t row = t * 32 + fl; a_rd[t] = row * GW_ROWB + ((fk ^ ((row >> 1) & 7)) * 16); }
+  struct Frag { h8 a[TM]; };
   auto rd = [&](Frag& f, const unsigned char* sb, int ks) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < TM; t++) f.a[t] = *(const h8*)(sb + (a_rd[t] ^ (ks * 32)));
-#pragma unroll
-    for (int t = 0; t < TN; t++) f.b[t] = *(const h8*)(sb + (b_rd[t] ^ (ks * 32)));
   };
-  auto mma = [&](const Frag& f) __attribute__((always_inline)) {
+  auto mma = [&](const Frag& f, int slot) __attribute__((always_inline)) {
+#pragma unroll
+    for (int b = 0; b < TN; b++) {
+      h8 bf; __builtin_memcpy(&bf, &ring[slot][b], 16);
+#pragma unroll
+      for (int a = 0; a < TM; a++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[a], bf, acc[a][b], 0, 0, 0);
+    }
+  };
+
+#pragma unroll
+  for (int j = 0; j < RING; j++) {
+    // in ring order and not reordered: the wait the compiler places at the head of the loop counts the loads behind
+    // slot 0 on both ways into it, and a slot loaded late here would make it drain the ring every iteration
+    load_b(j, j);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  fetch_a(0);
+  store_a(0);
+  __syncthreads();
+  Frag f0, f1;
+  rd(f0, smem, 0);
+  // One stage = four k-steps; PAR = st & 1 picks the LDS buffer and (ring of 8) the half of the register ring, so that
+  // every index into the ring is static.  The body has no branch: past the last stage the A loads fetch the last
+  // stage again into the buffer nobody reads, the B loads the last k block, and the fragment reads a tile nobody uses
+  // (d_in is a multiple of 128 here, so stages come in pairs).
+  auto stage = [&](auto PAR, const uint32_t st) __attribute__((always_inline)) {
+    constexpr int par = decltype(PAR)::value;
+    fetch_a(min(st + 1, n_stages - 1));
+    const unsigned char* sb = smem + par * STAGE;
+    constexpr int s0 = RING == 8 ? par * 4 : 0;                  // this stage's slots of the ring
+    const uint32_t kb_next = st * 4 + RING;                      // a slot is refilled RING k-steps ahead, right after its use
+    // source order = issue order (pinned): the next k-step's four A fragment reads first, then this k-step's MFMAs,
+    // then the refill of the ring slot they just used
+    auto pin = [&]() __attribute__((always_inline)) {
+      __builtin_amdgcn_sched_group_barrier(0x100, TM, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, TN, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    rd(f1, sb, 1); mma(f0, s0 + 0); load_b(s0 + 0, kb_next + 0); pin();
+    rd(f0, sb, 2); mma(f1, s0 + 1); load_b(s0 + 1, kb_next + 1); pin();
+    rd(f1, sb, 3); mma(f0, s0 + 2); load_b(s0 + 2, kb_next + 2); pin();
+    // the stage's last A fragments are on their way; the next stage goes into the other buffer (every wave left it
+    // before the last barrier), and behind this barrier nobody reads this one any more.  The barrier is bare (LDS
+    // traffic only crosses it): a workgroup fence would also wait for the ring refills in flight.
+    store_a(par ^ 1);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    rd(f0, smem + (par ^ 1) * STAGE, 0); mma(f1, s0 + 3); load_b(s0 + 3, kb_next + 3); pin();
+  };
+  for (uint32_t st = 0; st < n_stages; st += 2) {
+    stage(std::integral_constant<int, 0>{}, st);
+    stage(std::integral_constant<int, 1>{}, st + 1);
+  }
+  // accumulator i of a tile: column 8 (i / 4) + 4 (lane / 32) + i % 4, row lane % 32
+  auto col_of = [&](int a, int i) { return c0 + a * 32 + 8 * (i / 4) + 4 * fk + (i % 4); };
+  auto row_of = [&](int b) { return r0 + (wave * TN + b) * 32 + fl; };
+  if constexpr (!ACC) {
 #pragma unroll
     for (int a = 0; a < TM; a++)
 #pragma unroll
-      for (int b = 0; b < TN; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[a], f.b[b], acc[a][b], 0, 0, 0);
-  };
-  // the fragment reads of the next k-step are spread among this k-step's MFMAs (one wave a SIMD: nothing else hides
-  // an LDS round trip)
-  auto interleave = [&]() __attribute__((always_inline)) {
+      for (int b = 0; b < TN; b++)
 #pragma unroll
-    for (int i = 0; i < TM + TN; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, (TM * TN) / (TM + TN) > 0 ? (TM * TN) / (TM + TN) : 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        for (int i = 0; i < 16; i++)
+          if (row_of(b) < p.d_out && col_of(a, i) < p.n_cols) p.y[(size_t)col_of(a, i) * p.y_stride + row_of(b)] = acc[a][b][i];
+  } else {
+    // the old values of tile t + D are fetched before tile t is added up and stored (element by element every add
+    // would wait for its own load)
+    constexpr int D = 3, NT = TM * TN;
+    float old[D][16];
+    auto fetch = [&](int t) __attribute__((always_inline)) {
+      const int a = t / TN, b = t % TN;
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        old[t % D][i] = (row_of(b) < p.d_out && col_of(a, i) < p.n_cols) ? p.y[(size_t)col_of(a, i) * p.y_stride + row_of(b)] : 0.f;
+    };
+#pragma unroll
+    for (int t = 0; t < D; t++) fetch(t);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      const int a = t / TN, b = t % TN;
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        if (row_of(b) < p.d_out && col_of(a, i) < p.n_cols) p.y[(size_t)col_of(a, i) * p.y_stride + row_of(b)] = old[t % D][i] + acc[a][b][i];
+      if (t + D < NT) fetch(t + D);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN) * ((TM * TN) / (TM + TN)), 0);
-  };
-
-  Frag f0, f1;
-  issue(0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  rd(f0, smem, 0);
-  for (uint32_t st = 0; st < n_stages; st++) {
-    const bool more = st + 1 < n_stages;
-    if (more && !((GW_ABL & 1) && st > 0)) issue(st + 1);     // into the buffer every wave left before the last barrier
-    const unsigned char* sb = smem + (st & 1) * STAGE;
-    rd(f1, sb, 1); mma(f0); interleave();
-    rd(f0, sb, 2); mma(f1); interleave();
-    rd(f1, sb, 3); mma(f0); interleave();
-    // the stage's last fragments are on their way; behind the barrier the other buffer holds stage st + 1 (every wave
-    // waited for its own loads) and nobody reads this one any more
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    if (!(GW_ABL & 2)) __syncthreads();
-    if (more) rd(f0, smem + ((st + 1) & 1) * STAGE, 0);
-    mma(f1);
-    if (more) interleave();
   }
-
-  // accumulator i of a tile: column 8 (i / 4) + 4 (lane / 32) + i % 4, row lane % 32
-#pragma unroll
-  for (int a = 0; a < TM; a++)
-#pragma unroll
-    for (int b = 0; b < TN; b++) {
-      const uint32_t row = r0 + wn * 32 * TN + b * 32 + fl;
-#pragma unroll
-      for (int i = 0; i < 16; i++) {
-        const uint32_t col = c0 + wm * 128 + a * 32 + 8 * (i / 4) + 4 * fk + (i % 4);
-        if (row < p.d_out && col < p.n_cols) {
-          float* y = p.y + (size_t)col * p.y_stride + row;
-          *y = p.acc ? *y + acc[a][b][i] : acc[a][b][i];
-        }
-      }
-    }
 }
 
-// ---- weights -> f16 [d_out][d_in], the arithmetic of the tiled kernel's staging: (nibble - 8) * scale and
-//      int8 * scale in f16 (exact integer, one rounding), f32 rounded to nearest even ----
+// ---- weights -> f16 in MFMA fragment order: for row block rb (32 rows, the last one padded with copies of the last
+//      row) and k block kb (16 values) the 1 KB at ((rb nk16 + kb) 64 + lane) 16 holds, for lane = 32 fk + fl, the 8
+//      values k = 16 kb + 8 fk .. + 7 of row 32 rb + fl.  The arithmetic is the tiled kernel's staging: (nibble - 8) *
+//      scale and int8 * scale in f16 (exact integer, one rounding), f32 rounded to nearest even ----
 typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 static __device__ inline h2v gw_as_h2(uint32_t u) { h2v r; __builtin_memcpy(&r, &u, 4); return r; }
 static __device__ inline h2v gw_bytes(uint32_t w, uint32_t sel, h2v bias, h2v sc) { return (gw_as_h2(__builtin_amdgcn_perm(0x64646464u, w, sel)) - bias) * sc; }
 
-// one thread per quantisation block of 32 weights
+// one thread per (row, quantisation block of 32 weights), the 32 rows of a row block on consecutive threads
 template <int KIND>
-__global__ __launch_bounds__(256) void pa_widen_w_kernel(const void* w, const uint16_t* scales, uint16_t* out, size_t n_blocks) {
-  const size_t b = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (b >= n_blocks) return;
+__global__ __launch_bounds__(256) void pa_widen_w_kernel(const void* w, const uint16_t* scales, uint16_t* out, uint32_t d_out, uint32_t nb, size_t n_threads) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n_threads) return;
+  const uint32_t fl = (uint32_t)(idx % 32), bq = (uint32_t)((idx / 32) % nb);
+  const size_t rb = idx / ((size_t)32 * nb);
+  const size_t b = (size_t)min((uint32_t)(rb * 32 + fl), d_out - 1) * nb + bq;          // the packed block this thread widens
   h8 o[4];
   if constexpr (KIND == PA_W_Q4_0) {
     const u4 q = *(const u4*)((const unsigned char*)w + b * 16);       // byte j: element j (low nibble), element 16 + j (high)
@@ -205,56 +275,56 @@ __global__ __launch_bounds__(256) void pa_widen_w_kernel(const void* w, const ui
       o[v] = (h8){ (_Float16)x0[0], (_Float16)x0[1], (_Float16)x0[2], (_Float16)x0[3], (_Float16)x1[0], (_Float16)x1[1], (_Float16)x1[2], (_Float16)x1[3] };
     }
   }
-  h8* dst = (h8*)(out + b * 32);
+  // o[v] = values 8 v .. 8 v + 7 of the block: k block 2 bq + v / 2, half fk = v & 1
+  const size_t nk16 = (size_t)nb * 2;
 #pragma unroll
-  for (int v = 0; v < 4; v++) dst[v] = o[v];
+  for (int v = 0; v < 4; v++) *(h8*)(out + (((rb * nk16 + 2 * bq + v / 2) * 64 + (v & 1) * 32 + fl) * 8)) = o[v];
 }
 
 template <int TN>
 static hipError_t launch_gemm16(const Gemm16Params& q, hipStream_t s) {
-  const size_t lds = 2 * (size_t)(GW_COLS * GW_ROWB + 64 * TN * GW_ROWB);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)pa_gemm16_kernel<TN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
-  const dim3 grid((q.d_out + 64 * TN - 1) / (64 * TN), (q.n_cols + GW_COLS - 1) / GW_COLS);
-  hipLaunchKernelGGL((pa_gemm16_kernel<TN>), grid, dim3(256), lds, s, q);
+  const uint32_t total = ((q.n_cols + GW_COLS - 1) / GW_COLS) * ((q.d_out + 128 * TN - 1) / (128 * TN));
+  if (q.acc) hipLaunchKernelGGL((pa_gemm16_kernel<TN, true>), dim3((total + 7) / 8 * 8), dim3(256), 0, s, q);
+  else hipLaunchKernelGGL((pa_gemm16_kernel<TN, false>), dim3((total + 7) / 8 * 8), dim3(256), 0, s, q);
   return hipGetLastError();
 }
 
-// large chunks only: at least 512 columns, and enough 256-column x 128-row workgroups to give every CU one (below that
+// large chunks only: at least 512 columns, and enough 128-column x 256-row workgroups to give every CU one (below that
 // the tiled kernel's 128 x 128 workgroups fill the chip better)
 bool pa_gemm_wide_serves(const GemmParams& p, int n_cu) {
-  if (p.n_cols < 512 || p.d_in < 128 || (p.x_stride & 7) != 0 || ((uintptr_t)p.x & 15) != 0) return false;
-  if (p.d_in % GW_KS != 0) return false;
-  const uint64_t wgs = (uint64_t)((p.n_cols + GW_COLS - 1) / GW_COLS) * ((p.d_out + 127) / 128);
+  if (p.n_cols < 512 || p.d_in % (2 * GW_KS) != 0 || (p.x_stride & 7) != 0 || ((uintptr_t)p.x & 15) != 0) return false;
+  const uint64_t wgs = (uint64_t)((p.n_cols + GW_COLS - 1) / GW_COLS) * ((p.d_out + 255) / 256);
   return wgs >= (uint64_t)(n_cu > 0 ? n_cu : 256);
 }
 
-// w16: staging for d_out x d_in halves (the caller's, 16-byte aligned)
-hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, int n_cu, hipStream_t s) {
-  const size_t n_blocks = (size_t)p.d_out * (p.d_in / 32);
-  const dim3 wgrid((unsigned)((n_blocks + 255) / 256));
-  switch (p.kind) {
-    case PA_W_Q4_0: hipLaunchKernelGGL(pa_widen_w_kernel<PA_W_Q4_0>, wgrid, dim3(256), 0, s, p.w, p.scales, w16, n_blocks); break;
-    case PA_W_Q8_0: hipLaunchKernelGGL(pa_widen_w_kernel<PA_W_Q8_0>, wgrid, dim3(256), 0, s, p.w, p.scales, w16, n_blocks); break;
-    case PA_W_F32: hipLaunchKernelGGL(pa_widen_w_kernel<PA_W_F32>, wgrid, dim3(256), 0, s, p.w, p.scales, w16, n_blocks); break;
-    default: return hipErrorInvalidValue;
+// bytes of the staging matrix of a weight: whole 32-row blocks
+size_t pa_gemm_wide_staging_bytes(uint32_t d_out, uint32_t d_in) { return (size_t)((d_out + 31) / 32) * 32 * d_in * sizeof(uint16_t); }
+
+// w16: staging of pa_gemm_wide_staging_bytes (the caller's, 16-byte aligned); widen = false: it already holds these weights
+hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, bool widen, int n_cu, hipStream_t s) {
+  if (widen) {
+    const uint32_t nb = p.d_in / 32;
+    const size_t n_threads = (size_t)((p.d_out + 31) / 32) * 32 * nb;
+    const dim3 wgrid((unsigned)((n_threads + 255) / 256));
+    switch (p.kind) {
+      case PA_W_Q4_0: hipLaunchKernelGGL(pa_widen_w_kernel<PA_W_Q4_0>, wgrid, dim3(256), 0, s, p.w, p.scales, w16, p.d_out, nb, n_threads); break;
+      case PA_W_Q8_0: hipLaunchKernelGGL(pa_widen_w_kernel<PA_W_Q8_0>, wgrid, dim3(256), 0, s, p.w, p.scales, w16, p.d_out, nb, n_threads); break;
+      case PA_W_F32: hipLaunchKernelGGL(pa_widen_w_kernel<PA_W_F32>, wgrid, dim3(256), 0, s, p.w, p.scales, w16, p.d_out, nb, n_threads); break;
+      default: return hipErrorInvalidValue;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
   }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
   Gemm16Params q;
   q.x = p.x; q.w16 = w16; q.y = p.y; q.x_stride = p.x_stride; q.y_stride = p.y_stride;
   q.d_out = p.d_out; q.d_in = p.d_in; q.n_cols = p.n_cols; q.acc = p.acc;
-  // rows per workgroup (64 TN): the choice that wastes the least of the chip -- rounds of n_cu workgroups, each
-  // round costing its workgroups' rows
+  // rows per workgroup (128 TN): the choice that wastes the least of the chip -- rounds of n_cu workgroups, each
+  // round costing its workgroups' rows (smaller wave tiles pay a little more LDS traffic per MFMA)
   const uint32_t cb = (p.n_cols + GW_COLS - 1) / GW_COLS, cus = n_cu > 0 ? (uint32_t)n_cu : 256u;
   uint32_t best_tn = 4; uint64_t best = ~0ull;
   for (uint32_t tn = 4; tn >= 2; tn--) {
-    const uint64_t wgs = (uint64_t)((p.d_out + 64 * tn - 1) / (64 * tn)) * cb;
-    const uint64_t cost = ((wgs + cus - 1) / cus) * (64 * tn) * (tn == 4 ? 16 : tn == 3 ? 17 : 19);   // smaller tiles pay more LDS traffic per MFMA
+    const uint64_t wgs = (uint64_t)((p.d_out + 128 * tn - 1) / (128 * tn)) * cb;
+    const uint64_t cost = ((wgs + cus - 1) / cus) * (128 * tn) * (tn == 4 ? 16 : tn == 3 ? 17 : 18);
     if (cost < best) { best = cost; best_tn = tn; }
   }
   return best_tn == 4 ? launch_gemm16<4>(q, s) : best_tn == 3 ? launch_gemm16<3>(q, s) : launch_gemm16<2>(q, s);

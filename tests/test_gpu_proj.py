@@ -145,12 +145,15 @@ def test_gemm_matches_oracle(kind, d_out, d_in, n):
 
 
 @pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q8_0, PA_W_Q4_0])
-@pytest.mark.parametrize("d_out,d_in,n", [(9216 - 40, 2048, 4096 - 3), (2048, 4096, 600), (300, 128, 520), (130, 8192, 513), (1000, 64, 1100)])
+@pytest.mark.parametrize("d_out,d_in,n", [(9216 - 40, 2048, 4096 - 3), (2048, 4096, 4000), (4090, 256, 4096), (600, 128, 11000),
+                                          (2048, 4096, 600), (130, 8192, 513), (1000, 64, 1100)])
 def test_gemm_large_chunks(kind, d_out, d_in, n):
-    """Chunks of 512 columns and more over d_in a multiple of 64: the weights are widened once into the context's f16
-    staging matrix and the GEMM runs over two f16 operands (128-column wave tiles, 128 to 256 weight rows a workgroup).
-    Ragged edges on both axes, padded strides that must stay untouched, the accumulating form, and a second call with
-    other weights through the same staging matrix."""
+    """Chunks of 512 columns and more over d_in a multiple of 128: the weights are widened to f16 in fragment order (a
+    copy kept with the weight handle) and the GEMM runs over two f16 operands (128-column wave tiles, 256 to 512 weight
+    rows a workgroup: the first four shapes take 384, 256, 512 and 384 on a 256-CU part; the last three stay on the
+    tiled kernel, too few workgroups or d_in not a multiple of 128).  Ragged edges on both axes, padded strides that
+    must stay untouched, the accumulating form (the second call on a handle, which finds the kept copy), and a second
+    weight."""
     if kind == PA_W_F32 and d_in > 4096:
         pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
     rng = np.random.default_rng(d_out + d_in + n + kind)
@@ -172,6 +175,33 @@ def test_gemm_large_chunks(kind, d_out, d_in, n):
         w2, sc2 = _weights(kind, d_out, d_in, rng)
         pa.gemm(pa.weight(kind, w2, sc2), dx, xs, n, dy, ys); pa.sync()
         assert _rel(dy.download(np.float32, n * ys).reshape(n, ys)[:, :d_out], O.gemm_f16(kind, w2, sc2, x16.astype(np.float32))) < 2e-5, "second weight"
+
+
+@pytest.mark.parametrize("kind", [PA_W_Q8_0, PA_W_Q4_0])
+def test_gemm_weight_cache_budget(kind):
+    """The kept f16 copy and the per-call staging hold the same values: a context with no budget (every call widens into
+    the context's staging), one whose budget holds the first weight only, and the default give the same bits, also
+    when the weights alternate through the one staging matrix."""
+    d_out, d_in, n = 2100, 256, 4000
+    rng = np.random.default_rng(kind)
+    ws = [_weights(kind, d_out, d_in, rng) for _ in range(2)]
+    x16 = rng.standard_normal((n, d_in)).astype(np.float16)
+    outs = []
+    for budget in (None, 0, 2112 * 256 * 2 + 64):
+        with PooledAttn(SHAPES["qwen36_moe"], 64, n_layers=1, max_cols=1) as pa:
+            if budget is not None:
+                pa.set_weight_cache(budget)
+            whs = [pa.weight(kind, w, sc) for w, sc in ws]
+            dx = pa.to_device(x16.view(np.uint16)); dy = pa.alloc(n * d_out * 4)
+            got = []
+            for i in (0, 1, 0, 1):
+                pa.gemm(whs[i], dx, d_in, n, dy, d_out); pa.sync()
+                got.append(dy.download(np.float32, n * d_out))
+            assert np.array_equal(got[0], got[2]) and np.array_equal(got[1], got[3])
+            outs.append(got[:2])
+    for o in outs[1:]:
+        assert np.array_equal(o[0], outs[0][0]) and np.array_equal(o[1], outs[0][1])
+    assert _rel(outs[0][0].reshape(n, d_out), O.gemm_f16(kind, ws[0][0], ws[0][1], x16.astype(np.float32))) < 2e-5
 
 
 def test_rmsnorm_f16_columns():
