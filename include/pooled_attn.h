@@ -291,16 +291,16 @@ int pa_attn_layer_decode(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, co
 int pa_rmsnorm_f16(pa_ctx* ctx, const float* d_x, uint32_t x_stride, const float* d_norm_w, uint32_t dim, uint32_t n_cols,
                    void* d_xn_f16, uint32_t xn_stride);
 /* y[c][0 .. d_out) = W x[c] for n_cols columns; x: f16 bits, stride in f16 elements (>= d_in, multiple of 8);
- * y: f32, stride in floats; acc != 0: y += W x.  Chunks of up to 32 columns (verify blocks, the reference's 16-column
- * passes through its batched matvec, engine/wgsl/coop.js) are served by a kernel that streams the weights once per
- * 16 columns instead of the tiled one; same operand precision either way. */
+ * y: f32, stride in floats; acc != 0: y += W x.  Chunks of up to 16 columns (verify blocks, the reference's 16-column
+ * passes through its batched matvec, engine/wgsl/coop.js) are served by a kernel that streams the packed weights
+ * once per launch; wider chunks run on the matrix cores; same operand precision either way. */
 int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uint32_t x_stride, uint32_t n_cols, float* d_y, uint32_t y_stride, int acc);
-/* Chunks of 512 columns and more run on a GEMM over two f16 operands: the weight handle's values widened to f16
+/* Chunks of more than 16 columns (over d_in a multiple of 128) run on GEMMs over two f16 operands: the weight handle's values widened to f16
  * ((nibble - 8) * scale, int8 * scale, f32 rounded -- the arithmetic of the tiled kernel's staging, so results do not
  * depend on which way a call goes) in matrix-core fragment order.  That copy (2 bytes a weight) is made on the first
  * such call on a handle (which therefore allocates: not under stream capture) and kept until pa_weight_destroy, while
  * the copies kept by this context stay within max_bytes (default 8 GiB; 0: keep none); past the budget a call widens
- * into per-context staging every time (+8 % on a 4096 x 9216 x 2048 chunk).  Changing the budget keeps what is
+ * into per-context staging every time (+8 % on a 4096 x 9216 x 2048 chunk, about +10 us on a 64-column one).  Changing the budget keeps what is
  * already held.  No counterpart in the reference, whose WGSL GEMMs dequantise in the inner loop. */
 int pa_set_weight_cache(pa_ctx* ctx, size_t max_bytes);
 /* n_cols tokens at positions base_pos .. through the attention half of a full-attention layer, as

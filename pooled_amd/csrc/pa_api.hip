@@ -741,7 +741,8 @@ extern "C" int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uin
   GemmParams p; memset(&p, 0, sizeof p);
   p.w = w->w; p.scales = w->scales; p.x = (const uint16_t*)d_x_f16; p.y = d_y; p.x_stride = x_stride; p.y_stride = y_stride;
   p.d_out = w->d_out; p.d_in = w->d_in; p.n_cols = n_cols; p.acc = acc; p.kind = w->kind;
-  if (pa_gemm_wide_serves(p, ctx->n_cu)) {
+  const bool wide = pa_gemm_wide_serves(p, ctx->n_cu);
+  if (wide || pa_gemm_mid_serves(p)) {
     // the weights as f16 in fragment order: a copy kept with the weight from its first large chunk on, while the
     // context's budget lasts (the handle's contents never change); past the budget, or where the allocation fails,
     // widened per call into the context's staging
@@ -759,7 +760,7 @@ extern "C" int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uin
       if (rc) return rc;
       w16 = (uint16_t*)ctx->w16_buf; widen = true;
     }
-    HIPCHK(ctx, pa_launch_gemm_wide(p, w16, widen, ctx->n_cu, ctx->stream));
+    HIPCHK(ctx, pa_launch_gemm_wide(p, w16, widen, !wide, ctx->n_cu, ctx->stream));
     return PA_OK;
   }
   HIPCHK(ctx, pa_launch_gemm(p, ctx->n_cu, ctx->stream));

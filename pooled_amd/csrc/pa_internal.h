@@ -111,7 +111,8 @@ hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s);
 // GEMM over two f16 operands; pa_gemm_wide_serves tells whether a call qualifies
 bool pa_gemm_wide_serves(const GemmParams& p, int n_cu);
 size_t pa_gemm_wide_staging_bytes(uint32_t d_out, uint32_t d_in);
-hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, bool widen, int n_cu, hipStream_t s);
+bool pa_gemm_mid_serves(const GemmParams& p);
+hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, bool widen, bool mid, int n_cu, hipStream_t s);
 // rmsnorm of n_cols f32 columns, written as f16 (the GEMM's activation operand)
 hipError_t pa_launch_rmsnorm_f16(const float* x, uint32_t x_stride, const float* w, uint32_t dim, float eps, uint32_t n_cols,
                                  uint16_t* out, uint32_t out_stride, hipStream_t s);

@@ -281,6 +281,168 @@ __global__ __launch_bounds__(256) void pa_widen_w_kernel(const void* w, const ui
   for (int v = 0; v < 4; v++) *(h8*)(out + (((rb * nk16 + 2 * bq + v / 2) * 64 + (v & 1) * 32 + fl) * 8)) = o[v];
 }
 
+// ---- chunks too small to give every CU one of the tiles above (a few dozen to a few hundred columns, or few weight
+//      rows): 64 columns x 64 weight rows a workgroup, and the workgroup's four waves split K between them instead of
+//      the tile -- of every K stage of 128 wave w takes the k-steps w and w + 4 -- so that all four share the staged
+//      activations (one coalesced fetch per workgroup) while each loads only the weight fragments of its own
+//      k-steps.  Every wave holds the whole 64 x 64 tile (4 MFMA tiles, 64 accumulators: two workgroups a CU); at the
+//      end the four copies meet in LDS and wave w adds up MFMA tile w in a fixed order (((w0 + w1) + w2) + w3) and
+//      stores it.  A workgroup walks all of K, so there are no partial sums in memory and no second launch; what
+//      bounds it is the L2 -> CU traffic of 64 x 64 tiles (K (64 + 64) 2 bytes a tile), about twice its MFMA time.
+#define GM_T 64              // columns per workgroup
+#define GM_KS 128            // K per stage
+#define GM_ROWB 256          // bytes of a staged activation row
+
+template <int TN, int RING, bool ACC>
+__global__ __launch_bounds__(256, 2) void pa_gemm16_mid_kernel(Gemm16Params p) {
+  constexpr int STAGE = GM_T * GM_ROWB;                  // 16 KB
+  constexpr int ROWS = 32 * TN;                          // weight rows per workgroup
+  constexpr int NT = 2 * TN;                             // MFMA tiles per wave: 2 column blocks x TN row blocks
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[(4 * NT * 16 * 64 * 4 > 2 * STAGE) ? 4 * NT * 16 * 64 * 4 : 2 * STAGE];   // two stages; at the end the four waves' tiles
+  const uint32_t tid = threadIdx.x, lane = tid & 63, fl = lane & 31, fk = lane >> 5;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // XCD k owns a contiguous range of tiles, column blocks fastest: neighbours stream the same weight rows through one L2
+  const uint32_t n_cb = (p.n_cols + GM_T - 1) / GM_T, n_rb = (p.d_out + ROWS - 1) / ROWS, total = n_cb * n_rb;
+  const uint32_t per = (total + 7) / 8, tile = (blockIdx.x % 8) * per + blockIdx.x / 8;
+  if (tile >= total) return;
+  const uint32_t c0 = (tile % n_cb) * GM_T, r0 = (tile / n_cb) * ROWS;
+  const uint32_t n_stages = p.d_in / GM_KS, nk16 = p.d_in / 16;
+
+  // A: a load covers 4 rows x 256 bytes; chunk c of row r is staged at slot c ^ (r & 15)
+  const uint32_t lrow = lane >> 4, lchunk = lane & 15;
+  const unsigned char* a_src[4];
+  uint32_t a_dst[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t row = (wave * 4 + i) * 4 + lrow;
+    const size_t col = min((size_t)c0 + row, (size_t)p.n_cols - 1);     // columns past the end repeat the last one (never stored)
+    a_src[i] = (const unsigned char*)(p.x + col * p.x_stride) + lchunk * 16;
+    a_dst[i] = row * GM_ROWB + ((lchunk ^ (row & 15)) * 16);
+  }
+  // a stage's activations are fetched two stages ahead (two register sets), its weight fragments RING stages ahead:
+  // one stage of MFMAs is far less than a round trip to L2, let alone to HBM, and a workgroup's time is its number of
+  // stages x that latency / the stages it keeps in flight
+  u4 areg[2][4];
+  auto fetch_a = [&](int set, uint32_t st) __attribute__((always_inline)) {
+    const size_t off = (size_t)min(st, n_stages - 1) * GM_ROWB;       // past the last stage: the last one again, never used
+#pragma unroll
+    for (int i = 0; i < 4; i++) areg[set][i] = *(const u4*)(a_src[i] + off);
+  };
+  auto store_a = [&](int set, uint32_t buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) *(u4*)(smem + buf * STAGE + a_dst[i]) = areg[set][i];
+  };
+  // fragment of column block t at k-step j of the stage: row 32 t + fl, chunk 2 j + fk
+  uint32_t a_rd[2][2];
+#pragma unroll
+  for (int t = 0; t < 2; t++)
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const uint32_t row = t * 32 + fl, chunk = 2 * (wave + 4 * u) + fk;
+      a_rd[t][u] = row * GM_ROWB + ((chunk ^ (row & 15)) * 16);
+    }
+  // B: this wave's k blocks 8 st + wave and 8 st + wave + 4 of the TN 32-row blocks
+  const uint32_t n_rb32 = (p.d_out + 31) / 32;
+  const unsigned char* b_src[TN];
+#pragma unroll
+  for (int t = 0; t < TN; t++) b_src[t] = (const unsigned char*)p.w16 + ((size_t)min(r0 / 32 + t, n_rb32 - 1) * nk16 * 64 + lane) * 16;
+  u4 bq[RING][2][TN];                                    // [stage % RING][u][row block]
+  auto load_b = [&](int slot, uint32_t st) __attribute__((always_inline)) {
+    const size_t off = (size_t)(min(st, n_stages - 1) * 8 + wave) * 1024;
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+      for (int t = 0; t < TN; t++) bq[slot][u][t] = *(const u4*)(b_src[t] + off + (size_t)u * 4096);
+  };
+  f16v acc[2][TN];
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < TN; b++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
+
+#pragma unroll
+  for (int j = 0; j < RING; j++) load_b(j, j);
+  fetch_a(0, 0);
+  fetch_a(1, 1);
+  store_a(0, 0);
+  fetch_a(0, 2);
+  __syncthreads();
+  // stage st reads LDS buffer st % 2 and ring slot st % RING; register set p holds the stages of parity p: at the
+  // end of stage st the other set (stage st + 1, fetched two stages ago) goes to the other buffer and then receives
+  // stage st + 3
+  auto stage = [&](auto J, uint32_t st) __attribute__((always_inline)) {
+    constexpr int j = decltype(J)::value, par = j & 1;
+    const unsigned char* sb = smem + par * STAGE;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      h8 af[2], bf[TN];
+#pragma unroll
+      for (int t = 0; t < 2; t++) af[t] = *(const h8*)(sb + a_rd[t][u]);
+#pragma unroll
+      for (int t = 0; t < TN; t++) __builtin_memcpy(&bf[t], &bq[j][u][t], 16);
+#pragma unroll
+      for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[a], bf[b], acc[a][b], 0, 0, 0);
+    }
+    load_b(j, st + RING);
+    store_a(par ^ 1, par ^ 1);          // stage st + 1 into the other buffer: every wave left it before the last barrier
+    fetch_a(par ^ 1, st + 3);
+    __syncthreads();
+  };
+  static_assert(RING == 4 || RING == 8, "the loop below is unrolled by the ring");
+  for (uint32_t st = 0; st < n_stages; st += RING) {
+    stage(std::integral_constant<int, 0>{}, st);
+    if (st + 1 < n_stages) stage(std::integral_constant<int, 1>{}, st + 1);
+    if (st + 2 < n_stages) stage(std::integral_constant<int, 2>{}, st + 2);
+    if (st + 3 < n_stages) stage(std::integral_constant<int, 3>{}, st + 3);
+    if constexpr (RING == 8) {
+      if (st + 4 < n_stages) stage(std::integral_constant<int, 4>{}, st + 4);
+      if (st + 5 < n_stages) stage(std::integral_constant<int, 5>{}, st + 5);
+      if (st + 6 < n_stages) stage(std::integral_constant<int, 6>{}, st + 6);
+      if (st + 7 < n_stages) stage(std::integral_constant<int, 7>{}, st + 7);
+    }
+  }
+  // the four partial tiles meet in LDS (the stages are dead behind the loop's last barrier): [wave][slot][lane], slot =
+  // 16 (TN a + b) + i for accumulator i of the MFMA tile of column block a and row block b
+  float* red = (float*)smem;
+#pragma unroll
+  for (int a = 0; a < 2; a++)
+#pragma unroll
+    for (int b = 0; b < TN; b++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) red[((wave * NT + a * TN + b) * 16 + i) * 64 + lane] = acc[a][b][i];
+  __syncthreads();
+  // wave w finishes slots [w SPW, (w + 1) SPW); accumulator i of a tile = column 8 (i / 4) + 4 fk + i % 4, row fl
+  constexpr int SPW = NT * 16 / 4;
+  float sum[SPW];
+#pragma unroll
+  for (int k = 0; k < SPW; k++) {
+    const uint32_t o = (wave * SPW + k) * 64 + lane;
+    sum[k] = ((red[o] + red[o + NT * 16 * 64]) + red[o + 2 * NT * 16 * 64]) + red[o + 3 * NT * 16 * 64];
+  }
+  auto col_of = [&](int k) { const uint32_t sl = wave * SPW + k, a = sl / (16 * TN), i = sl % 16; return c0 + a * 32 + 8 * (i / 4) + 4 * fk + (i % 4); };
+  auto row_of = [&](int k) { const uint32_t sl = wave * SPW + k, b = sl / 16 % TN; return r0 + b * 32 + fl; };
+  float old[SPW];
+  if constexpr (ACC) {
+#pragma unroll
+    for (int k = 0; k < SPW; k++) old[k] = (row_of(k) < p.d_out && col_of(k) < p.n_cols) ? p.y[(size_t)col_of(k) * p.y_stride + row_of(k)] : 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < SPW; k++)
+    if (row_of(k) < p.d_out && col_of(k) < p.n_cols) p.y[(size_t)col_of(k) * p.y_stride + row_of(k)] = ACC ? old[k] + sum[k] : sum[k];
+}
+
+template <int TN, int RING>
+static hipError_t launch_gemm16_mid(const Gemm16Params& q, hipStream_t s) {
+  const uint32_t total = ((q.n_cols + GM_T - 1) / GM_T) * ((q.d_out + 32 * TN - 1) / (32 * TN));
+  if (q.acc) hipLaunchKernelGGL((pa_gemm16_mid_kernel<TN, RING, true>), dim3((total + 7) / 8 * 8), dim3(256), 0, s, q);
+  else hipLaunchKernelGGL((pa_gemm16_mid_kernel<TN, RING, false>), dim3((total + 7) / 8 * 8), dim3(256), 0, s, q);
+  return hipGetLastError();
+}
+
 template <int TN>
 static hipError_t launch_gemm16(const Gemm16Params& q, hipStream_t s) {
   const uint32_t total = ((q.n_cols + GW_COLS - 1) / GW_COLS) * ((q.d_out + 128 * TN - 1) / (128 * TN));
@@ -297,11 +459,19 @@ bool pa_gemm_wide_serves(const GemmParams& p, int n_cu) {
   return wgs >= (uint64_t)(n_cu > 0 ? n_cu : 256);
 }
 
+// chunks of more than 16 columns that the large-chunk kernel does not serve.  Measured with cold weights (Q4_0, 32 to
+// 64 weights in rotation): [q|k|v] 9216 x 2048 13.0 - 13.5 us for 8 to 32 columns against 12.9 / 17.9 / 28 / 34 us at 8 /
+// 16 / 24 / 32 columns on the skinny kernel (which reads the packed weights, a quarter of the bytes, but one launch
+// per 16 columns); wo 2048 x 4096 16.7 us against 8.5 / 15.9 / 19.9 / 27.6
+bool pa_gemm_mid_serves(const GemmParams& p) {
+  return p.n_cols > 16 && p.d_in % GM_KS == 0 && (p.x_stride & 7) == 0 && ((uintptr_t)p.x & 15) == 0;
+}
+
 // bytes of the staging matrix of a weight: whole 32-row blocks
 size_t pa_gemm_wide_staging_bytes(uint32_t d_out, uint32_t d_in) { return (size_t)((d_out + 31) / 32) * 32 * d_in * sizeof(uint16_t); }
 
 // w16: staging of pa_gemm_wide_staging_bytes (the caller's, 16-byte aligned); widen = false: it already holds these weights
-hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, bool widen, int n_cu, hipStream_t s) {
+hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, bool widen, bool mid, int n_cu, hipStream_t s) {
   if (widen) {
     const uint32_t nb = p.d_in / 32;
     const size_t n_threads = (size_t)((p.d_out + 31) / 32) * 32 * nb;
@@ -318,6 +488,12 @@ hipError_t pa_launch_gemm_wide(const GemmParams& p, uint16_t* w16, bool widen, i
   Gemm16Params q;
   q.x = p.x; q.w16 = w16; q.y = p.y; q.x_stride = p.x_stride; q.y_stride = p.y_stride;
   q.d_out = p.d_out; q.d_in = p.d_in; q.n_cols = p.n_cols; q.acc = p.acc;
+  if (mid) {
+    // fewer 64 x 64 tiles than half the CUs: 32-row tiles (twice the workgroups) with twice the stages in flight
+    // (wo 2048 x 4096 on up to 64 columns, cold: 20 -> 16.7 us; with 144 tiles, [q|k|v], it is 2 us slower)
+    const uint64_t tiles64 = (uint64_t)((p.n_cols + GM_T - 1) / GM_T) * ((p.d_out + 63) / 64);
+    return tiles64 * 2 < (uint64_t)(n_cu > 0 ? n_cu : 256) ? launch_gemm16_mid<1, 8>(q, s) : launch_gemm16_mid<2, 4>(q, s);
+  }
   // rows per workgroup (128 TN): the choice that wastes the least of the chip -- rounds of n_cu workgroups, each
   // round costing its workgroups' rows (smaller wave tiles pay a little more LDS traffic per MFMA)
   const uint32_t cb = (p.n_cols + GW_COLS - 1) / GW_COLS, cus = n_cu > 0 ? (uint32_t)n_cu : 256u;

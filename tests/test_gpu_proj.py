@@ -122,7 +122,8 @@ def test_attn_layer_decode_matches_oracle(shape, dim, kind, pos):
 
 @pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q8_0, PA_W_Q4_0])
 @pytest.mark.parametrize("d_out,d_in,n", [(9216, 2048, 300), (2048, 4096, 129), (37, 96, 5), (130, 8192, 40), (256, 32, 128), (384, 96, 700),
-                                          (9216, 2048, 8), (2048, 4096, 16), (130, 8192, 3), (70, 64, 1), (2048, 4096, 31), (130, 8192, 17)])   # from (9216, 2048, 8) on: the skinny-chunk kernel, one or more launches
+                                          (100, 384, 65), (64, 128, 33), (4096, 2048, 512),      # the 64 x 64 kernel with an odd stage count, one stage, a C2-sized chunk (as are the first two and the fourth)
+                                          (9216, 2048, 8), (2048, 4096, 16), (130, 8192, 3), (70, 64, 1), (2048, 4096, 31), (130, 8192, 17)])   # from (9216, 2048, 8) on: up to 16 columns the skinny-chunk kernel, one or more launches; the last two the 64 x 32 tiles of the mid-size kernel
 def test_gemm_matches_oracle(kind, d_out, d_in, n):
     if kind == PA_W_F32 and d_in > 4096:
         pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
