@@ -240,6 +240,26 @@ def other_configs():
         fl = causal_flops(cfg, base, n)
         out[name] = dict(us_per_call=round(ms * 1e3, 2), kv_gb_s=round(kv / ms / 1e6, 1), tflops=round(fl / ms / 1e9, 2), plan=pa.plan(kind, base, n))
         log("%s: %.2f us/call, %.0f GB/s of KV, %.2f TFLOP/s" % (name, ms * 1e3, kv / ms / 1e6, fl / ms / 1e9))
+        if name == "C2":
+            # the same chunk through the attention half of a layer (projections either side), one weight set per layer
+            from pooled_amd.capi import PA_W_Q4_0
+            dim = 2048
+
+            def mk(d_out, d_in):
+                sc = np.asarray(rng.uniform(0.001, 0.003, (d_out, d_in // 32)), np.float16).view(np.uint16)
+                return pa.weight(PA_W_Q4_0, rng.integers(0, 256, (d_out, d_in // 2), dtype=np.uint8), sc)
+            ws = [(mk(qd + 2 * kvd, dim), mk(dim, qd)) for _ in range(layers)]
+            d_x = pa.to_device(rng.standard_normal((n, dim), dtype=np.float32) * 0.1)
+            d_nw = pa.to_device(np.ones(dim, np.float32)); d_hw = pa.to_device(np.ones(hd, np.float32))
+            lcall = lambda i: pa.attn_layer_prefill(i % layers, ws[i % layers][0], ws[i % layers][1], d_nw, d_hw, d_hw, d_x, dim, base, n)
+            for i in range(layers + 2):
+                lcall(i)
+            pa.sync(); pa.timer_start()
+            for i in range(100):
+                lcall(i)
+            lms = pa.timer_stop() / 100
+            out[name]["layer_us_per_call"] = round(lms * 1e3, 2)
+            log("C2 through the attention half of a layer (rmsnorm, [q|k|v] GEMM %dx%dx%d, pre-step, attention, wo GEMM %dx%dx%d): %.2f us/call" % (n, qd + 2 * kvd, dim, n, dim, qd, lms * 1e3))
         pa.close()
     return out
 

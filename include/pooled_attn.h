@@ -265,7 +265,9 @@ int pa_profile_read(pa_ctx* ctx, float* ms_sum, uint32_t* count);
                          nibble - 8; scales as Q8_0 (base.js:81-118) */
 typedef struct pa_weight pa_weight;
 /* copies a weight matrix to the device.  h_w: the values plane (f32 / int8 / packed nibbles), h_scales: f16 bits
- * (NULL for PA_W_F32).  d_in must be a multiple of 32 and at most 8192 (4096 for PA_W_F32). */
+ * (NULL for PA_W_F32).  d_in must be a multiple of 32 and at most 8192 (4096 for PA_W_F32).  A handle belongs to the
+ * context that made it: use and destroy it through that context only (pa_gemm may attach a derived copy to it, see
+ * pa_set_weight_cache, on that context's stream). */
 int pa_weight_create(pa_ctx* ctx, int kind, uint32_t d_out, uint32_t d_in, const void* h_w, const void* h_scales, pa_weight** out);
 int pa_weight_destroy(pa_ctx* ctx, pa_weight* w);
 /* y[d_out] = W x[d_in]; acc != 0: y += W x (matvec*_coop_acc: the residual add folded into the GEMV) */
