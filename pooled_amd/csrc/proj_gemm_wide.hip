@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256, 1) void pa_gemm16_kernel(Gemm16Params p) {
   } else {
     // the old values of tile t + D are fetched before tile t is added up and stored (element by element every add
     // would wait for its own load)
-    constexpr int D = 3, NT = TM * TN;
+    constexpr int D = TN == 4 ? 4 : 6, NT = TM * TN;     // the ring and the fragment registers are dead by now: room for six tiles of old values
     float old[D][16];
     auto fetch = [&](int t) __attribute__((always_inline)) {
       const int a = t / TN, b = t % TN;
