@@ -22,7 +22,7 @@ const PA_W_F32 = 0, PA_W_Q8_0 = 1, PA_W_Q4_0 = 2;             // weight kinds of
 
 class HipAttention {
   // opts: { nH, nKV, hd, nRot, ropeTheta, eps, maxSeq, nLayers, batchCols, qkNorm = true, gate = false, outF16 = false,
-  //         kvQ8 = false, fusedStep = true, verifyExact = false, attnPrefillTile = "auto" }
+  //         kvQ8 = false, fusedStep = true, verifyExact = false, attnPrefillTile = "auto", weightCacheBytes = 8 GiB }
   constructor(opts) {
     const nH = opts.nH, nKV = opts.nKV, hd = opts.hd;
     if (!(nH > 0 && nKV > 0 && nH % nKV === 0)) throw new Error("HipAttention: nH must be a positive multiple of nKV");
@@ -50,6 +50,9 @@ class HipAttention {
     // kernel of a prefill chunk, true = always the matrix-core kernel, false = full-width passes go through the decode
     // entry point like every other pass
     if (opts.attnPrefillTile === true) addon.setPrefillTile(this.ctx, 1);
+    // budget of the f16 weight copies that gemm() keeps with a weight from its first chunk of more than 16 columns on
+    // (0: none, every such call widens into per-context staging)
+    if (opts.weightCacheBytes !== undefined) addon.setWeightCache(this.ctx, opts.weightCacheBytes);
     this.kvBufBytes = opts.maxSeq * this.dims.kvDim * 2;
     this.layers = [];
     for (let i = 0; i < (opts.nLayers || 1); i++) { addon.layerAlloc(this.ctx, i); this.layers.push({ index: i, qNorm: null, kNorm: null }); }

@@ -24,7 +24,7 @@ const check = (what, got, ref) => {
 };
 const cfg = C.cfg, n = C.nCols, base = C.basePos;
 const A = new HipAttention({ nH: cfg.n_heads, nKV: cfg.n_kv_heads, hd: cfg.head_dim, nRot: cfg.n_rot, ropeTheta: cfg.rope_theta, eps: cfg.eps,
-  maxSeq: base + n, nLayers: 1, batchCols: n, qkNorm: true, gate: !!cfg.gate, attnPrefillTile: true });   // the matrix-core kernel whatever the chunk's size
+  maxSeq: base + n, nLayers: 1, batchCols: n, qkNorm: true, gate: !!cfg.gate, attnPrefillTile: true, weightCacheBytes: 64 * 1024 * 1024 });   // the matrix-core kernel whatever the chunk's size
 const D = A.dims, qIn = cfg.gate ? 2 * D.qDim : D.qDim;
 A.setLayerNorms(0, f32("qw.bin"), f32("kw.bin"));
 const K0 = u16("k16.bin"), V0 = u16("v16.bin"), qraw = f32("qraw.bin"), kraw = f32("kraw.bin"), vraw = f32("vraw.bin"), expect = f32("expect.bin");
