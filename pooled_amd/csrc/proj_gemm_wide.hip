@@ -113,17 +113,48 @@ __global__ __launch_bounds__(256, 1) void pa_gemm16_kernel(Gemm16Params p) {
     for (int t = 0; t < TN; t++) ring[slot][t] = *(const u4*)(b_src[t] + off);
   };
 
+  const uint32_t fl = lane & 31, fk = lane >> 5;
+  auto col_of = [&](int a, int i) { return c0 + a * 32 + 8 * (i / 4) + 4 * fk + (i % 4); };
+  auto row_of = [&](int b) { return r0 + (wave * TN + b) * 32 + fl; };
+  // Accumulating calls.  Loads and stores share one counter on this part, and with both kinds pending the compiler's
+  // wait for a loaded value waits for every store in flight as well: old values fetched in the epilogue tile by tile,
+  // between the stores, cost a memory round trip per tile (0.097 ms against 0.072 plain on a 4096 x 2048 x 4096 chunk,
+  // however many tiles ahead they are fetched).  With 8 tiles a wave (TN = 2) the accumulators therefore START from
+  // the old values -- requested first, they arrive under the prologue's loads -- and the epilogue is the plain store;
+  // with 12 or 16 tiles there is no room to stage them all before the loop, and the epilogue works in phases of
+  // several tiles: all of a phase's loads, then all of its stores.
+  constexpr bool INIT = ACC && TN == 2;
   f16v acc[TM][TN];
+  if constexpr (INIT) {
+    // every load goes out before the first value is moved into an accumulation register (left alone, the compiler
+    // stages them a few at a time: a round trip per batch)
+    float old[TM * TN][16];
 #pragma unroll
-  for (int a = 0; a < TM; a++)
+    for (int a = 0; a < TM; a++)
 #pragma unroll
-    for (int b = 0; b < TN; b++)
+      for (int b = 0; b < TN; b++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
+        for (int i = 0; i < 16; i++)
+          old[a * TN + b][i] = p.y[(size_t)min(col_of(a, i), p.n_cols - 1) * p.y_stride + min(row_of(b), p.d_out - 1)];   // unconditional (clamped): a guarded load is a branch, and one load a basic block is one round trip a load
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+      for (int b = 0; b < TN; b++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[a][b][i] = old[a * TN + b][i];
+    __builtin_amdgcn_sched_barrier(0);
+  } else {
+#pragma unroll
+    for (int a = 0; a < TM; a++)
+#pragma unroll
+      for (int b = 0; b < TN; b++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[a][b][i] = 0.f;
+  }
 
   // A fragment addresses: row fl of a 32-row block, 8 halves at k = 16 ks + 8 fk -> chunk 2 ks + fk, swizzled by the
   // row (the swizzle is an XOR on the chunk index, and 2 ks has no bit in common with fk)
-  const uint32_t fl = lane & 31, fk = lane >> 5;
   uint32_t a_rd[TM];
 #pragma unroll
   for (int t = 0; t < TM; t++) { const uint32_t row = t * 32 + fl; a_rd[t] = row * GW_ROWB + ((fk ^ ((row >> 1) & 7)) * 16); }
@@ -186,9 +217,7 @@ __global__ __launch_bounds__(256, 1) void pa_gemm16_kernel(Gemm16Params p) {
     stage(std::integral_constant<int, 1>{}, st + 1);
   }
   // accumulator i of a tile: column 8 (i / 4) + 4 (lane / 32) + i % 4, row lane % 32
-  auto col_of = [&](int a, int i) { return c0 + a * 32 + 8 * (i / 4) + 4 * fk + (i % 4); };
-  auto row_of = [&](int b) { return r0 + (wave * TN + b) * 32 + fl; };
-  if constexpr (!ACC) {
+  if constexpr (!ACC || INIT) {
 #pragma unroll
     for (int a = 0; a < TM; a++)
 #pragma unroll
@@ -197,25 +226,27 @@ __global__ __launch_bounds__(256, 1) void pa_gemm16_kernel(Gemm16Params p) {
         for (int i = 0; i < 16; i++)
           if (row_of(b) < p.d_out && col_of(a, i) < p.n_cols) p.y[(size_t)col_of(a, i) * p.y_stride + row_of(b)] = acc[a][b][i];
   } else {
-    // the old values of tile t + D are fetched before tile t is added up and stored (element by element every add
-    // would wait for its own load)
-    constexpr int D = TN == 4 ? 4 : 6, NT = TM * TN;     // the ring and the fragment registers are dead by now: room for six tiles of old values
-    float old[D][16];
-    auto fetch = [&](int t) __attribute__((always_inline)) {
-      const int a = t / TN, b = t % TN;
+    constexpr int D = TN == 3 ? 6 : 4, NT = TM * TN;       // tiles per phase (the ring and the fragment registers are dead by now)
+    static_assert(NT % D == 0, "whole phases");
 #pragma unroll
-      for (int i = 0; i < 16; i++)
-        old[t % D][i] = (row_of(b) < p.d_out && col_of(a, i) < p.n_cols) ? p.y[(size_t)col_of(a, i) * p.y_stride + row_of(b)] : 0.f;
-    };
+    for (int t0 = 0; t0 < NT; t0 += D) {
+      float old[D][16];
 #pragma unroll
-    for (int t = 0; t < D; t++) fetch(t);
+      for (int t = 0; t < D; t++)
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-      const int a = t / TN, b = t % TN;
+        for (int i = 0; i < 16; i++) {
+          const int a = (t0 + t) / TN, b = (t0 + t) % TN;
+          old[t][i] = p.y[(size_t)min(col_of(a, i), p.n_cols - 1) * p.y_stride + min(row_of(b), p.d_out - 1)];      // unconditional (clamped), see above
+        }
+      __builtin_amdgcn_sched_barrier(0);                   // every load of the phase before its first store
 #pragma unroll
-      for (int i = 0; i < 16; i++)
-        if (row_of(b) < p.d_out && col_of(a, i) < p.n_cols) p.y[(size_t)col_of(a, i) * p.y_stride + row_of(b)] = old[t % D][i] + acc[a][b][i];
-      if (t + D < NT) fetch(t + D);
+      for (int t = 0; t < D; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          const int a = (t0 + t) / TN, b = (t0 + t) % TN;
+          if (row_of(b) < p.d_out && col_of(a, i) < p.n_cols) p.y[(size_t)col_of(a, i) * p.y_stride + row_of(b)] = old[t][i] + acc[a][b][i];
+        }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 }
@@ -428,7 +459,7 @@ __global__ __launch_bounds__(256, 2) void pa_gemm16_mid_kernel(Gemm16Params p) {
   float old[SPW];
   if constexpr (ACC) {
 #pragma unroll
-    for (int k = 0; k < SPW; k++) old[k] = (row_of(k) < p.d_out && col_of(k) < p.n_cols) ? p.y[(size_t)col_of(k) * p.y_stride + row_of(k)] : 0.f;
+    for (int k = 0; k < SPW; k++) old[k] = p.y[(size_t)min(col_of(k), p.n_cols - 1) * p.y_stride + min(row_of(k), p.d_out - 1)];   // unconditional (clamped): guarded loads would go out one round trip at a time
   }
 #pragma unroll
   for (int k = 0; k < SPW; k++)
