@@ -96,6 +96,11 @@ __global__ __launch_bounds__(256) void pa_gemv_kernel(GemvParams p) {
       if constexpr (KIND != PA_W_F32) sc[r][i] = p.scales[row * nb + b];
     }
   }
+  // accumulating calls: the old values of the wave's rows are requested here, with everything else, instead of in a
+  // round trip of their own behind the reduction
+  float yold[RW];
+#pragma unroll
+  for (int r = 0; r < RW; r++) yold[r] = p.acc ? p.y[min(row0 + r, (size_t)p.d_out - 1)] : 0.f;
   // x -> LDS through coalesced loads (a lane's own slice is 32 consecutive floats: loaded directly, a wave-wide
   // load would touch 64 cache lines for 1 KB), normed on the way when asked; block b sits at xs[b * 36]: the 4-float
   // pad makes the 8 lanes of a 128-bit LDS read phase hit distinct banks
@@ -103,24 +108,23 @@ __global__ __launch_bounds__(256) void pa_gemv_kernel(GemvParams p) {
   __shared__ float red[4];
   constexpr int XPT = 2 * BPL;                                         // float4 of x per thread (d_in <= 2048 * BPL)
   const uint32_t n4 = p.d_in / 4;
-  f4 xv[XPT];
+  f4 xv[XPT], wv[NORM ? XPT : 1];
   float ss = 0.f;
+  // Loads past the end of x re-read its last float4 instead of being guarded (their values are never stored, and are
+  // masked out of the sum of squares by a factor, not by a select on the loaded value): a guarded load is a branch,
+  // and between guarded blocks the compiler placed a full wait -- the norm weights went out a round trip after the
+  // weights and x.
 #pragma unroll
-  for (int k = 0; k < XPT; k++) {
-    const uint32_t e = threadIdx.x + 256 * k;
-    xv[k] = e < n4 ? ((const f4*)p.x)[e] : (f4){0.f, 0.f, 0.f, 0.f};
-  }
+  for (int k = 0; k < XPT; k++) xv[k] = ((const f4*)p.x)[min(threadIdx.x + 256 * k, n4 - 1)];
   if constexpr (NORM) {
-    f4 wv[XPT];
+#pragma unroll
+    for (int k = 0; k < XPT; k++) wv[k] = ((const f4*)p.norm_w)[min(threadIdx.x + 256 * k, n4 - 1)];
 #pragma unroll
     for (int k = 0; k < XPT; k++) {
-      const uint32_t e = threadIdx.x + 256 * k;
-      wv[k] = e < n4 ? ((const f4*)p.norm_w)[e] : (f4){0.f, 0.f, 0.f, 0.f};
+      const float m = threadIdx.x + 256 * k < n4 ? 1.f : 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; j++) ss = __builtin_fmaf(xv[k][j] * m, xv[k][j], ss);
     }
-#pragma unroll
-    for (int k = 0; k < XPT; k++)
-#pragma unroll
-      for (int j = 0; j < 4; j++) ss = __builtin_fmaf(xv[k][j], xv[k][j], ss);
     ss = wave_sum_f32(ss);
     if (lane == 0) red[wave] = ss;
     __syncthreads();
@@ -185,7 +189,7 @@ __global__ __launch_bounds__(256) void pa_gemv_kernel(GemvParams p) {
 #pragma unroll
     for (int r = 0; r < RW; r++) {
       const size_t row = row0 + r;
-      if (row < p.d_out) p.y[row] = p.acc ? p.y[row] + part[r] : part[r];
+      if (row < p.d_out) p.y[row] = p.acc ? yold[r] + part[r] : part[r];
     }
   }
 }
