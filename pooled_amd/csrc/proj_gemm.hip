@@ -241,9 +241,21 @@ __global__ __launch_bounds__(256) void pa_gemm_skinny_kernel(GemmParams p) {
   }
   // the chunk's columns -> LDS, 16 bytes a thread and turn
   const uint32_t cpc = p.d_in / 8;                                    // 16-byte pieces of a column
-  for (uint32_t e = tid; e < ncol * cpc; e += 256) {
-    const uint32_t c = e / cpc, k8 = e % cpc;
-    *(u4*)(sk_lds + c * xcol + (k8 >> 2) * GROW + (k8 & 3) * 16) = *(const u4*)((const unsigned char*)(p.x + (size_t)c * p.x_stride) + k8 * 16);
+  // (eight loads a thread go out before the first is stored -- unconditional, a turn past the end re-reads the last piece:
+  // one load a loop turn is one round trip a turn, eight of them for 8 columns of 2048)
+  const uint32_t pieces = ncol * cpc;
+  for (uint32_t e0 = tid; e0 < pieces; e0 += 256 * 8) {
+    u4 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const uint32_t e = min(e0 + 256 * j, pieces - 1), c = e / cpc, k8 = e % cpc;
+      v[j] = *(const u4*)((const unsigned char*)(p.x + (size_t)c * p.x_stride) + k8 * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const uint32_t e = e0 + 256 * j, c = e / cpc, k8 = e % cpc;
+      if (e < pieces) *(u4*)(sk_lds + c * xcol + (k8 >> 2) * GROW + (k8 & 3) * 16) = v[j];
+    }
   }
   // widen: pair k of a block = elements 2k, 2k + 1
   h2 wv[RW][BPL][16];
@@ -303,13 +315,12 @@ __global__ __launch_bounds__(256) void pa_gemm_skinny_kernel(GemmParams p) {
       for (int r = 0; r < RW; r++) ps[lane * PS + c * RW + r] = part[c][r];
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   for (uint32_t t = lane; t < ncol * RW; t += 64) {
+    const uint32_t c = t / RW, r = t % RW;
+    float* y = p.y + (size_t)c * p.y_stride + min(row0 + r, (size_t)p.d_out - 1);
+    const float yo = p.acc ? *y : 0.f;                                // on its way while the partials are added up
     float a = 0.f;
     for (int l = 0; l < 64; l++) a += ps[l * PS + t];
-    const uint32_t c = t / RW, r = t % RW;
-    if (row0 + r < p.d_out) {
-      float* y = p.y + (size_t)c * p.y_stride + row0 + r;
-      *y = p.acc ? *y + a : a;
-    }
+    if (row0 + r < p.d_out) *y = p.acc ? yo + a : a;
   }
 }
 
