@@ -391,13 +391,44 @@ __global__ __launch_bounds__(256) void pa_rmsnorm_f16_kernel(const float* x, uin
   __shared__ float red[4];
   const uint32_t col = blockIdx.x, tid = threadIdx.x;
   const f4* xs = (const f4*)(x + (size_t)col * x_stride);
+  const uint32_t n4 = dim / 4;
   float ss = 0.f;
-  for (uint32_t e = tid; e < dim / 4; e += 256) { const f4 v = xs[e]; ss = __builtin_fmaf(v[0], v[0], ss); ss = __builtin_fmaf(v[1], v[1], ss); ss = __builtin_fmaf(v[2], v[2], ss); ss = __builtin_fmaf(v[3], v[3], ss); }
+  // Columns of up to 8192 values: x and the norm weights are held in registers (2, 4 or 8 float4 a thread) and requested
+  // together, unconditionally (a turn past the end re-reads the last float4 and is masked out of the sum by a factor):
+  // one load a loop turn, twice over, was four round trips for 2048 values.
+  auto in_regs = [&](auto XPC) __attribute__((always_inline)) {
+    constexpr int XP = decltype(XPC)::value;
+    f4 xv[XP], wv[XP];
+#pragma unroll
+    for (int k = 0; k < XP; k++) xv[k] = xs[min(tid + 256 * k, n4 - 1)];
+#pragma unroll
+    for (int k = 0; k < XP; k++) wv[k] = ((const f4*)w)[min(tid + 256 * k, n4 - 1)];
+#pragma unroll
+    for (int k = 0; k < XP; k++) {
+      const float m = tid + 256 * k < n4 ? 1.f : 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; j++) ss = __builtin_fmaf(xv[k][j] * m, xv[k][j], ss);
+    }
+    ss = wave_sum_f32(ss);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    const float inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)dim + eps);
+#pragma unroll
+    for (int k = 0; k < XP; k++) {
+      const uint32_t e = tid + 256 * k;
+      const _Float16 o[4] = { (_Float16)((xv[k][0] * inv) * wv[k][0]), (_Float16)((xv[k][1] * inv) * wv[k][1]), (_Float16)((xv[k][2] * inv) * wv[k][2]), (_Float16)((xv[k][3] * inv) * wv[k][3]) };
+      if (e < n4) __builtin_memcpy(out + (size_t)col * out_stride + 4 * e, o, 8);
+    }
+  };
+  if (n4 <= 512) { in_regs(std::integral_constant<int, 2>{}); return; }
+  if (n4 <= 1024) { in_regs(std::integral_constant<int, 4>{}); return; }
+  if (n4 <= 2048) { in_regs(std::integral_constant<int, 8>{}); return; }
+  for (uint32_t e = tid; e < n4; e += 256) { const f4 v = xs[e]; ss = __builtin_fmaf(v[0], v[0], ss); ss = __builtin_fmaf(v[1], v[1], ss); ss = __builtin_fmaf(v[2], v[2], ss); ss = __builtin_fmaf(v[3], v[3], ss); }
   ss = wave_sum_f32(ss);
   if ((tid & 63) == 0) red[tid >> 6] = ss;
   __syncthreads();
   const float inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)dim + eps);
-  for (uint32_t e = tid; e < dim / 4; e += 256) {
+  for (uint32_t e = tid; e < n4; e += 256) {
     const f4 v = xs[e], wv = ((const f4*)w)[e];
     const _Float16 o[4] = { (_Float16)((v[0] * inv) * wv[0]), (_Float16)((v[1] * inv) * wv[1]), (_Float16)((v[2] * inv) * wv[2]), (_Float16)((v[3] * inv) * wv[3]) };
     __builtin_memcpy(out + (size_t)col * out_stride + 4 * e, o, 8);
