@@ -944,19 +944,54 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
   const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
   const size_t base = ch * p.slots;
   const float* po = p.part_o + base * HD + 4 * d4;
-  float M = NEG_INF;
-  for (uint32_t s = 0; s < ns; s++) M = fmaxf(M, p.part_ml[(base + s) * 2]);
+  const float2* pml = (const float2*)p.part_ml + base;
+  f4 gt = {0.f, 0.f, 0.f, 0.f};                   // requested with everything else, used last
+  if (p.gate) gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + 4 * d4);
   float L = 0.f;
   f4 o = {0.f, 0.f, 0.f, 0.f};
-  for (uint32_t s = 0; s < ns; s++) {
-    const float w = __expf(p.part_ml[(base + s) * 2] - M);
-    L += p.part_ml[(base + s) * 2 + 1] * w;
-    o += *(const f4*)(po + (size_t)s * HD) * w;
+  if (ns) {
+    // Eight splits a turn, every load of a turn unconditional and issued together (a turn past the last split re-reads
+    // it: harmless for the maximum, weighted 0 in the sums): one load a loop turn was one round trip a split, twice
+    // over.  Up to eight splits -- the usual case -- everything the thread reads is one round trip.
+    constexpr int B = 8;
+    float2 ml[B];
+    f4 ov[B];
+#pragma unroll
+    for (int k = 0; k < B; k++) ml[k] = pml[min((uint32_t)k, ns - 1)];
+#pragma unroll
+    for (int k = 0; k < B; k++) ov[k] = *(const f4*)(po + (size_t)min((uint32_t)k, ns - 1) * HD);
+    float M = NEG_INF;
+#pragma unroll
+    for (int k = 0; k < B; k++) M = fmaxf(M, ml[k].x);
+    for (uint32_t s0 = B; s0 < ns; s0 += B) {
+      float mx[B];
+#pragma unroll
+      for (int k = 0; k < B; k++) mx[k] = pml[min(s0 + k, ns - 1)].x;
+#pragma unroll
+      for (int k = 0; k < B; k++) M = fmaxf(M, mx[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < B; k++) {
+      const float w = __expf(ml[k].x - M) * ((uint32_t)k < ns ? 1.f : 0.f);
+      L += ml[k].y * w;
+      o += ov[k] * w;
+    }
+    for (uint32_t s0 = B; s0 < ns; s0 += B) {
+#pragma unroll
+      for (int k = 0; k < B; k++) ml[k] = pml[min(s0 + k, ns - 1)];
+#pragma unroll
+      for (int k = 0; k < B; k++) ov[k] = *(const f4*)(po + (size_t)min(s0 + k, ns - 1) * HD);
+#pragma unroll
+      for (int k = 0; k < B; k++) {
+        const float w = __expf(ml[k].x - M) * (s0 + k < ns ? 1.f : 0.f);
+        L += ml[k].y * w;
+        o += ov[k] * w;
+      }
+    }
   }
   f4 r = ns ? o / L : (f4){0.f, 0.f, 0.f, 0.f};
   const uint32_t d = 4 * d4;
   if (p.gate) {
-    const f4 gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d);
 #pragma unroll
     for (int i = 0; i < 4; i++) r[i] *= 1.f / (1.f + __expf(-gt[i]));
   }
