@@ -777,6 +777,17 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     // its LDS reads (the accumulators are dead, registers are free), then adds and stores: one LDS latency, not one
     // per element.  The (m, l) of a row is merged by one of the first 16 threads.
     constexpr int EPT = 16 * (HD / 4) / (W * 64);
+    // direct output: the gate values of this thread's elements are requested before the LDS reads, unconditionally
+    // (rows past the last live one re-read it) -- loaded where they are used, under the row guard, each was a round
+    // trip of its own behind the sums
+    f4 gtv[EPT];
+    if (direct && p.gate) {
+#pragma unroll
+      for (int j = 0; j < EPT; j++) {
+        const uint32_t e = tid + j * W * 64, r = min(nb * 16 + e / (HD / 4), R - 1), d4 = e % (HD / 4);
+        gtv[j] = *(const f4*)(p.gate + (size_t)(c0 + r / G) * p.gate_stride + (size_t)(g * G + r % G) * p.gate_head_stride + 4 * d4);
+      }
+    }
     f4 part[EPT][W];
 #pragma unroll
     for (int j = 0; j < EPT; j++) {
@@ -813,9 +824,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
           for (int w = 0; w < W; w++) L += lex[w * 16 * NB + r] * __expf(mex[w * 16 * NB + r] - ms);
           o = o / L;
           if (p.gate) {
-            const f4 gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)hq * p.gate_head_stride + 4 * d4);
 #pragma unroll
-            for (int i = 0; i < 4; i++) o[i] *= 1.f / (1.f + __expf(-gt[i]));
+            for (int i = 0; i < 4; i++) o[i] *= 1.f / (1.f + __expf(-gtv[j][i]));
           }
           if (p.out_f16) {
             const h4 hv = { (_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3] };
