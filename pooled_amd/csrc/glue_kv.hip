@@ -58,29 +58,43 @@ __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
   const uint32_t qDim = nH * hd;
   const float* src = isQ ? p.q_in + (size_t)col * p.q_stride + (size_t)h * (gated ? 2 * hd : hd)
                          : p.k_in + (size_t)col * p.k_stride + (size_t)h * hd;
-  float x[4];
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const uint32_t i = lane + 64 * j;
-    x[j] = 0.f;
-    if (i < hd) {
-      x[j] = src[i];
-      if (isQ && gated) p.gate_out[(size_t)col * qDim + h * hd + i] = src[hd + i];
-    }
-  }
-  const uint32_t half = math ? p.n_rot / 2 : 0;
+  // Everything the wave reads is requested before anything is stored or computed -- the head's values, the gate half
+  // of a gated query head, the value row of a key head, the rotation's (cos, sin), the norm weights -- and every load
+  // is unconditional: an element past head_dim re-reads the last one and is zeroed afterwards.  (A load and a
+  // dependent store per element, or a register preset to zero and loaded under a branch, is one round trip each:
+  // the kernel was seven of them.)
+  float x[4], gt[4] = {0.f, 0.f, 0.f, 0.f}, w[4] = {0.f, 0.f, 0.f, 0.f};
+  float2 vv[2] = { make_float2(0.f, 0.f), make_float2(0.f, 0.f) };
   float2 cs[2] = { make_float2(1.f, 0.f), make_float2(1.f, 0.f) };
-#pragma unroll
-  for (int j = 0; j < 2; j++) {
-    const uint32_t i = lane + 64 * j;
-    if (i < half) cs[j] = rope_pair(p.rope_tab, p.inv_freq, pos, half, i);
-  }
+  const bool gate_copy = isQ && gated;
+  const bool v_copy = !isQ && p.k_cache && !p.ks_cache;
+  const uint32_t half = math ? p.n_rot / 2 : 0;
   const bool norm = math && (p.flags & PA_FLAG_QK_NORM);
-  float w[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; j++) x[j] = src[min(lane + 64 * j, hd - 1)];
+  if (gate_copy) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) gt[j] = src[hd + min(lane + 64 * j, hd - 1)];
+  }
+  if (v_copy) {
+    const float2* vs2 = (const float2*)(p.v_in + (size_t)col * p.v_stride + (size_t)h * hd);
+#pragma unroll
+    for (int t = 0; t < 2; t++) vv[t] = vs2[min(lane + 64 * t, hd / 2 - 1)];
+  }
+  if (half) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) cs[j] = rope_pair(p.rope_tab, p.inv_freq, pos, half, min(lane + 64 * j, half - 1));
+  }
   if (norm) {
     const float* wp = isQ ? p.qw : p.kw;
 #pragma unroll
-    for (int j = 0; j < 4; j++) { const uint32_t i = lane + 64 * j; if (i < hd) w[j] = wp[i]; }
+    for (int j = 0; j < 4; j++) w[j] = wp[min(lane + 64 * j, hd - 1)];
+  }
+#pragma unroll
+  for (int j = 0; j < 4; j++) if (lane + 64 * j >= hd) { x[j] = 0.f; w[j] = 0.f; }
+  if (gate_copy) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) if (lane + 64 * j < hd) p.gate_out[(size_t)col * qDim + h * hd + lane + 64 * j] = gt[j];
   }
   glue_head_wave(x, w, norm, p.eps, hd, half, cs, xs, lane);
   if (isQ) {
@@ -96,11 +110,17 @@ __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
     const size_t ro = ((size_t)h * p.head_rows + pos) * hd;           // head-major caches
     uint32_t* kc = (uint32_t*)(p.k_cache + ro);
     uint32_t* vc = (uint32_t*)(p.v_cache + ro);
-    const float* vs = p.v_in + (size_t)col * p.v_stride + (size_t)h * hd;
-    for (uint32_t w = lane; w < hd / 2; w += 64) {
-      kc[w] = pack_f16x2(xs[2 * w], xs[2 * w + 1]);
-      vc[w] = pack_f16x2(vs[2 * w], vs[2 * w + 1]);
-    }
+    // (the empty statement pins the conversion of the value row here: hoisted to its load, it would make the wave wait for
+    // that load before the rotation's and the norm's loads have gone out)
+#pragma unroll
+    for (int t = 0; t < 2; t++) asm volatile("" : "+v"(vv[t].x), "+v"(vv[t].y));
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+      if (lane + 64 * t < hd / 2) {
+        const uint32_t w = lane + 64 * t;
+        kc[w] = pack_f16x2(xs[2 * w], xs[2 * w + 1]);
+        vc[w] = pack_f16x2(vv[t].x, vv[t].y);
+      }
   }
 }
 
