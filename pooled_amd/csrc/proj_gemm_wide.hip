@@ -35,8 +35,9 @@
 //     row blocks, which share 8 activation tiles and 4 weight panels in that XCD's L2 (3 % over row-major order);
 //   * TN is picked per call so that the workgroups fill whole rounds of the chip.
 //
-// Measured on a 4096 x 9216 x 2048 Q4_0 chunk (0.178 ms, 869 TFLOP/s with the staging matrix kept): without the
-// output stores 0.163 ms, without the weight loads of the loop 0.163, with neither and no activation loads 0.134.
+// Measured on a 4096 x 9216 x 2048 Q4_0 chunk: 0.160 - 0.168 ms (920 - 970 TFLOP/s) with the staging matrix kept.
+// Ablations on an earlier build that ran 0.178 ms: without the output stores 0.163 ms, without the weight loads of
+// the loop 0.163, with neither and no activation loads 0.134.
 #include "pf_common.h"
 
 #define GW_COLS 128          // columns per workgroup
