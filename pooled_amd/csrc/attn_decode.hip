@@ -127,7 +127,7 @@ template <int HD> struct DecShape {
 // O^T = V^T P^T of a split is divided over the waves by output dims, see the code.  Without SR a split has any length
 // and every wave loops over its own tiles.
 template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
-__global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
+__global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
   static_assert(!SR || NB == 1, "single-round splits: one 16-row block");
   static_assert(!FUSED || NB == 1, "the fused pre-step serves one column");
   static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
@@ -342,8 +342,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER ? 2 : 1)) void pa_decod
     switch ((G + W - 1) / W) {
       case 1: fused_q_rows<1, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
       case 2: fused_q_rows<2, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
-      case 3: fused_q_rows<3, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
-      default: fused_q_rows<4, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
+      case 3: if constexpr (W <= 4) fused_q_rows<3, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
+      default: if constexpr (W <= 4) fused_q_rows<4, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
     }
     for (uint32_t e = tid; e < (16 - G) * (HD / 4); e += W * 64)     // padding rows (masked out later)
       *(h4*)(q_lds + (G + e / (HD / 4)) * S::QROW + (e % (HD / 4)) * 8) = (h4){0, 0, 0, 0};
@@ -1054,6 +1054,12 @@ static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipS
 
 template <int HD>
 static hipError_t launch_decode_hd(const AttnParams& p, uint32_t nb, uint32_t waves, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
+  // eight waves: the one-launch path for small chunks at head_dim 128 with two row blocks (its 250 registers a wave
+  // leave room for two waves a SIMD, and a tile's softmax and LDS work is what the loop waits for)
+  if (waves == 8) {
+    if constexpr (HD == 128) { if (nb == 2 && !p.k_scale) return launch_decode_t<HD, 2, 8, false>(p, col_groups, s, t); }
+    return hipErrorInvalidValue;
+  }
   if (waves != 4) return hipErrorInvalidValue;
   if (p.k_scale) {                                // int8 caches
     switch (nb) {

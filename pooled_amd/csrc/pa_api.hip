@@ -338,7 +338,10 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   uint32_t cw = n_cols, groups = 1;
   if (n_cols * G > max_rows) { cw = max_rows / G; if (cw == 0) return PA_ERR_UNSUPPORTED; groups = ceil_div(n_cols, cw); }
   uint32_t nb = ceil_div(cw * G, 16);
-  uint32_t W = 4;
+  // one-launch small chunks at head_dim 128 and two row blocks, at most one workgroup a CU: eight waves (see
+  // pa_launch_decode).  Measured: 512 columns at 1536 (256 workgroups) 24.5 -> 22.2 us; 1024 columns from 0 (512
+  // workgroups, which four waves run two a CU) 20.3 -> 23.9 us, hence the bound.
+  const uint32_t W = one_split && c.head_dim == 128 && nb == 2 && !kv_q8(ctx) && (uint64_t)groups * c.n_kv_heads <= (uint64_t)ctx->n_cu ? 8u : 4u;
   const uint32_t self = self_ok && n_cols == 1 ? 1 : 0;
   const uint32_t seq_max = std::max(base_pos + n_cols - self, 1u);   // streamed rows (position 0 alone: one empty split)
   const uint32_t tiles = ceil_div(seq_max, 32);
