@@ -248,11 +248,14 @@ int pa_slot_import(pa_ctx* ctx, uint32_t slot, uint32_t layer, int which, const 
  * pa_profile_enable(1) additionally times every attention call's main kernel (the split-K or prefill kernel, not
  * glue / merge) with an event pair stamped by the dispatch itself (the kernel's own begin / end timestamps, the
  * figure a kernel trace reports); pa_profile_read blocks, returns the sum of those durations and their count
- * since the last read, and resets them. */
+ * since the last read, and resets them.  pa_profile_read_each does the same but hands back every launch's own
+ * duration, in launch order (ms[0 .. min(*count, cap))); *count is the number of launches timed since the last read),
+ * so that a caller can report a median instead of a mean. */
 int pa_timer_start(pa_ctx* ctx);
 int pa_timer_stop(pa_ctx* ctx, float* ms);
 int pa_profile_enable(pa_ctx* ctx, int on);
 int pa_profile_read(pa_ctx* ctx, float* ms_sum, uint32_t* count);
+int pa_profile_read_each(pa_ctx* ctx, float* ms, uint32_t cap, uint32_t* count);
 
 /* ---- projections either side of the attention block, one-token passes.  Replace the reference's matvec /
  *      matvec_q8 / matvec_q4 dispatches and their cooperative, accumulating and normed forms
@@ -313,6 +316,14 @@ int pa_set_weight_cache(pa_ctx* ctx, size_t max_bytes);
  * prefill kernel (as pa_attn_prefill on such caches). */
 int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
                           const float* d_qw, const float* d_kw, float* d_x, uint32_t x_stride, uint32_t base_pos, uint32_t n_cols);
+
+/* Measurement stand-ins of the one-column decode kernel's K/V stream (bench.py --stream-ceiling; no counterpart in the
+ * reference): launch stand-in `variant` (0 .. pa_probe_count() - 1, described by pa_probe_name) on the context's stream
+ * over 32 MiB at d_k and 32 MiB at d_v; d_sink is 8 MiB of device scratch.  Timed by pa_profile_enable /
+ * pa_profile_read_each like an attention call's main kernel. */
+int pa_probe_count(void);
+const char* pa_probe_name(int variant);
+int pa_probe_stream(pa_ctx* ctx, int variant, const void* d_k, const void* d_v, void* d_sink);
 
 /* library / device description, e.g. "pooled_attn 0.1 gfx950 256CU" (storage owned by the library, one buffer per
  * calling thread) */

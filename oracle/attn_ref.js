@@ -11,9 +11,13 @@
 // usage: node attn_ref.js <in.bin> <out.bin|-> [reps]
 //   in.bin : int32 header [nCols, nH, nKV, hd, basePos, rows, hasGate, selCount] then selCount int32 column
 //            indices, then q f32 [nCols][nH*hd], K u16 [rows][nKV*hd], V u16 [rows][nKV*hd], gate f32 [nCols][nH*hd]
-//   out.bin: f32 [selCount][nH*hd]; prints one JSON line {"ms": best, "reps": n, "node": version, ...}
+//   out.bin: f32 [selCount][nH*hd]; prints one JSON line {"ms": best, "reps": n, "node": version, "max_weight": largest
+//            softmax weight of any (column, head) -- 1 / sum after the maximum is subtracted: a peaked row shows here --
+//            "cpus": os.cpus().length, "cpu_model": ...}
 "use strict";
 const fs = require("fs");
+const os = require("os");
+let maxWeight = 0;
 
 function h2f(h) {
   const s = h & 0x8000 ? -1 : 1, e = (h >> 10) & 31, m = h & 1023;
@@ -38,6 +42,7 @@ function attention(q, K, V, gate, nH, nKV, hd, seqLen, attn) {
     for (let t = 0; t < seqLen; t++) if (sc[t] > mx) mx = sc[t];
     let sum = 0;
     for (let t = 0; t < seqLen; t++) { sc[t] = Math.exp(sc[t] - mx); sum += sc[t]; }
+    if (1 / sum > maxWeight) maxWeight = 1 / sum;
     for (let t = 0; t < seqLen; t++) {
       const wt = sc[t] / sum, vo = t * kvDim + kvH * hd;
       for (let i = 0; i < hd; i++) attn[h * hd + i] += wt * V[vo + i];
@@ -75,6 +80,6 @@ function main() {
     if (ms < best) best = ms;
   }
   if (outPath && outPath !== "-") fs.writeFileSync(outPath, Buffer.from(out.buffer, out.byteOffset, out.byteLength));
-  console.log(JSON.stringify({ ms: best, reps: reps, node: process.version, threads: 1, cols: selCount, nH: nH, nKV: nKV, hd: hd, basePos: basePos }));
+  console.log(JSON.stringify({ ms: best, reps: reps, node: process.version, threads: 1, max_weight: maxWeight, cpus: os.cpus().length, cpu_model: (os.cpus()[0] || {}).model || "unknown", cols: selCount, nH: nH, nKV: nKV, hd: hd, basePos: basePos }));
 }
 main();

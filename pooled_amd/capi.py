@@ -65,6 +65,7 @@ SYMBOLS = {
     "pa_timer_stop": (c_int, [vp, ctypes.POINTER(ctypes.c_float)]),
     "pa_profile_enable": (c_int, [vp, c_int]),
     "pa_profile_read": (c_int, [vp, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(u32)]),
+    "pa_profile_read_each": (c_int, [vp, ctypes.POINTER(ctypes.c_float), u32, ctypes.POINTER(u32)]),
     "pa_slot_save": (c_int, [vp, u32, u32]),
     "pa_slot_load": (c_int, [vp, u32, ctypes.POINTER(u32)]),
     "pa_slot_drop": (c_int, [vp, u32]),
@@ -80,6 +81,9 @@ SYMBOLS = {
     "pa_rmsnorm_f16": (c_int, [vp, f32p, u32, f32p, u32, u32, vp, u32]),
     "pa_gemm": (c_int, [vp, vp, vp, u32, u32, f32p, u32, c_int]),
     "pa_attn_layer_prefill": (c_int, [vp, u32, vp, vp, f32p, f32p, f32p, f32p, u32, u32, u32]),
+    "pa_probe_count": (c_int, []),
+    "pa_probe_name": (ctypes.c_char_p, [c_int]),
+    "pa_probe_stream": (c_int, [vp, c_int, vp, vp, vp]),
     "pa_version": (ctypes.c_char_p, []),
 }
 
@@ -286,6 +290,12 @@ class PooledAttn:
         ms, n = ctypes.c_float(), u32()
         self._chk(self.L.pa_profile_read(self.ctx, ctypes.byref(ms), ctypes.byref(n)))
         return ms.value, n.value
+
+    def profile_read_each(self, cap=4096):
+        """Durations (ms) of the main-kernel launches timed since the last read, in launch order."""
+        buf, n = (ctypes.c_float * cap)(), u32()
+        self._chk(self.L.pa_profile_read_each(self.ctx, buf, cap, ctypes.byref(n)))
+        return [buf[i] for i in range(min(n.value, cap))]
 
     # ---- checkpoint slots ----
     def slot_save(self, slot, pos):

@@ -671,6 +671,7 @@ extern "C" int pa_weight_destroy(pa_ctx* ctx, pa_weight* w) {
   HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
   if (w->w) (void)hipFree(w->w);
   if (w->scales) (void)hipFree(w->scales);
+  if (w->w16_ready) (void)hipEventDestroy(w->w16_ready);
   if (w->w16) { (void)hipFree(w->w16); ctx->weight_cache_used -= std::min(ctx->weight_cache_used, w->w16_bytes); }
   delete w;
   return PA_OK;
@@ -751,19 +752,39 @@ extern "C" int pa_gemm(pa_ctx* ctx, const pa_weight* w, const void* d_x_f16, uin
     // widened per call into the context's staging
     const size_t need = pa_gemm_wide_staging_bytes(w->d_out, w->d_in);
     pa_weight* wm = const_cast<pa_weight*>(w);
-    bool widen = false;
+    void* fresh = nullptr;                        // a copy to keep, allocated by this call; attached only once its fill is queued
     if (!wm->w16 && ctx->weight_cache_used + need <= ctx->weight_cache_limit) {
-      void* buf = nullptr;
-      if (hipMalloc(&buf, need) == hipSuccess) { wm->w16 = (uint16_t*)buf; wm->w16_bytes = need; ctx->weight_cache_used += need; widen = true; }
-      else (void)hipGetLastError();
+      if (hipMalloc(&fresh, need) != hipSuccess) { fresh = nullptr; (void)hipGetLastError(); }
     }
-    uint16_t* w16 = wm->w16;
+    uint16_t* w16 = wm->w16 ? wm->w16 : (uint16_t*)fresh;
+    bool widen = fresh != nullptr;
     if (!w16) {
       int rc = grow_scratch(ctx, &ctx->w16_buf, &ctx->w16_buf_bytes, need);
       if (rc) return rc;
       w16 = (uint16_t*)ctx->w16_buf; widen = true;
     }
-    HIPCHK(ctx, pa_launch_gemm_wide(p, w16, widen, !wide, ctx->n_cu, ctx->stream));
+    if (wm->w16 && wm->w16_ready && wm->w16_stream != ctx->stream) {
+      // the kept copy was filled on another stream: wait for that fill once, on the host; from then on any stream may read it
+      HIPCHK(ctx, hipEventSynchronize(wm->w16_ready));
+      (void)hipEventDestroy(wm->w16_ready);
+      wm->w16_ready = nullptr; wm->w16_stream = nullptr;
+    }
+    hipError_t e = pa_launch_gemm_wide(p, w16, widen, !wide, ctx->n_cu, ctx->stream);
+    if (fresh) {
+      hipEvent_t ready = nullptr;
+      if (e == hipSuccess) e = hipEventCreateWithFlags(&ready, hipEventDisableTiming);
+      if (e == hipSuccess) e = hipEventRecord(ready, ctx->stream);
+      if (e != hipSuccess) {
+        // the fill did not go out (or cannot be tracked): the handle keeps no copy, so a later call widens again
+        (void)hipStreamSynchronize(ctx->stream);
+        if (ready) (void)hipEventDestroy(ready);
+        (void)hipFree(fresh);
+        return fail_hip(ctx, e, "pa_gemm: widening the weights");
+      }
+      wm->w16 = (uint16_t*)fresh; wm->w16_bytes = need; wm->w16_ready = ready; wm->w16_stream = ctx->stream;
+      ctx->weight_cache_used += need;
+    }
+    HIPCHK(ctx, e);
     return PA_OK;
   }
   HIPCHK(ctx, pa_launch_gemm(p, ctx->n_cu, ctx->stream));
@@ -1053,6 +1074,15 @@ extern "C" int pa_profile_read(pa_ctx* ctx, float* ms_sum, uint32_t* count) {
     sum += ms;
   }
   *ms_sum = sum; *count = (uint32_t)(ctx->prof_used / 2);
+  ctx->prof_used = 0;
+  return PA_OK;
+}
+extern "C" int pa_profile_read_each(pa_ctx* ctx, float* ms, uint32_t cap, uint32_t* count) {
+  if (!ctx || !count || (!ms && cap)) return PA_ERR_INVALID;
+  HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+  const size_t n = ctx->prof_used / 2;
+  for (size_t i = 0; i < n && i < cap; i++) HIPCHK(ctx, hipEventElapsedTime(&ms[i], ctx->prof_events[2 * i], ctx->prof_events[2 * i + 1]));
+  *count = (uint32_t)n;
   ctx->prof_used = 0;
   return PA_OK;
 }

@@ -143,6 +143,8 @@ struct pa_weight {
   uint16_t* scales = nullptr;     // f16 bits [d_out][d_in / 32]; nullptr for f32 weights
   uint16_t* w16 = nullptr;        // the weights widened to f16 in fragment order, kept from the first large-chunk pa_gemm on
   size_t w16_bytes = 0;           // (while the context's budget lasts); nullptr: widened per call into the context's staging
+  hipEvent_t w16_ready = nullptr; // recorded behind the kernel that filled w16, on w16_stream; nullptr once a host wait has seen it
+  hipStream_t w16_stream = nullptr;
 };
 
 struct pa_ctx {

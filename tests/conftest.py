@@ -22,3 +22,16 @@ def pytest_collection_modifyitems(config, items):
     for it in items:
         if "gpu" in it.keywords:
             it.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The margins of every parity check of the run (tests/helpers.py assert_parity), worst first."""
+    try:
+        from helpers import MARGINS
+    except Exception:
+        return
+    if not MARGINS:
+        return
+    terminalreporter.write_sep("-", "parity margins: %d checks, worst 25 by share of the effective budget" % len(MARGINS))
+    for what, d, rel, mx, budget in sorted(MARGINS, key=lambda r: -r[1] / r[4])[:25]:
+        terminalreporter.write_line("%-60s max-abs %.3e  rel %.3e  max|ref| %.5f  %5.1f %% of budget %.2e" % (what, d, rel, mx, 100 * d / budget, budget))

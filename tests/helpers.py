@@ -1,4 +1,5 @@
 """Shared test helpers: the benchmark shapes, cache construction through the oracle, the parity gate."""
+import os
 import numpy as np
 from oracle import attn_oracle as O
 
@@ -13,14 +14,47 @@ SHAPES = {
 MAX_ABS, MAX_REL = 2e-3, 1e-2
 
 
-def assert_parity(got, ref, what=""):
+# every parity check of the session: (what, max-abs, relative, max|ref|, effective budget); printed by conftest at the
+# end of the run and appended to the file PA_PARITY_LOG names (default gpurun_out/parity_margins.tsv when that folder
+# exists)
+MARGINS = []
+# a "tight" check must stay within this fraction of its effective budget
+TIGHT_FRACTION = 0.25
+
+
+def _log_margin(rec):
+    MARGINS.append(rec)
+    path = os.environ.get("PA_PARITY_LOG")
+    if path is None:
+        d = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+        path = os.path.join(d, "parity_margins.tsv") if os.path.isdir(d) else ""
+    if path:
+        try:
+            with open(path, "a") as f:
+                f.write("%s\t%.3e\t%.3e\t%.5f\t%.3e\t%.1f%%\n" % (rec[0], rec[1], rec[2], rec[3], rec[4], 100 * rec[1] / rec[4]))
+        except OSError:
+            pass
+
+
+def assert_parity(got, ref, what="", tight=False):
+    """The north star's gate: max-abs <= 2e-3 and max-abs / max|ref| <= 1e-2.  The binding one of the two is the
+    *effective budget* min(2e-3, 1e-2 * max|ref|): a softmax average over tens of thousands of N(0,1) value rows is a
+    few hundredths, so at the long-context configurations the budget is a few 1e-4, not 2e-3.  Every check prints and
+    records its margin; tight=True (the five benchmark configurations) additionally requires the difference to stay
+    within a quarter of the effective budget, so that a loss of accuracy shows long before the gate itself."""
     got = np.asarray(got, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     assert got.shape == ref.shape, (got.shape, ref.shape)
     assert np.all(np.isfinite(got)), "%s: non-finite output" % what
-    d = np.abs(got - ref).max()
-    rel = d / max(np.abs(ref).max(), 1e-30)
+    d = float(np.abs(got - ref).max())
+    mx = float(max(np.abs(ref).max(), 1e-30))
+    rel = d / mx
+    budget = min(MAX_ABS, MAX_REL * mx)
+    print("parity  %-58s max-abs %.3e  rel %.3e  max|ref| %.5f  = %5.1f %% of the effective budget %.2e" % (what, d, rel, mx, 100 * d / budget, budget))
+    _log_margin((what, d, rel, mx, budget))
     assert d <= MAX_ABS and rel <= MAX_REL, "%s: max-abs %.3e (limit %.0e), rel %.3e (limit %.0e)" % (what, d, MAX_ABS, rel, MAX_REL)
+    if tight:
+        assert d <= TIGHT_FRACTION * budget, "%s: max-abs %.3e is more than %.0f %% of the effective budget %.2e (max|ref| %.5f)" % (what, d, 100 * TIGHT_FRACTION, budget, mx)
     return d, rel
 
 

@@ -163,3 +163,54 @@ def test_q8_prefill_on_the_matrix_cores(shape, base, n):
         if pa.plan("prefill", base, m)["kernel"] == 1:
             got = pa.run_attn("prefill", 0, q[:m], base, gate=None if gate is None else gate[:m])
             assert_parity(got, ref[:m], "q8 wide prefill, shorter chunk after a longer one")
+
+
+@pytest.mark.parametrize("base,n,rows", [(0, 256, 16), (0, 512, 32), (77, 129, 16)])
+def test_q8_small_chunk_in_one_launch_writes_the_output_itself(base, n, rows):
+    """The table's one-launch path for small chunks (one split per workgroup, the tile loop's epilogue normalises, gates,
+    converts and stores; no partials, no merge) on an int8 cache: MoE shape, f32 and f16 output, and everything past
+    the chunk -- values and scales -- poisoned (garbage under NaN scales), so a row past a column's end that reached
+    the output would show."""
+    cfg = _q8cfg("qwen36_moe")
+    nKV, hd = cfg["n_kv_heads"], cfg["head_dim"]
+    G = cfg["n_heads"] // nKV
+    rng = np.random.default_rng(100 + base + n)
+    total, tail = base + n, 40
+    kq, ks, vq, vs, kf, vf = _quantised_cache(cfg, total, seed=200 + n)
+    q = rng.standard_normal((n, cfg["n_heads"], hd), dtype=np.float32)
+    gate = rng.standard_normal(q.shape, dtype=np.float32)
+    ref = O.attention_values(q, kf, vf, base, gate=gate)
+    with PooledAttn(cfg, total + tail, n_layers=1, max_cols=n) as pa:
+        pa.layer_alloc(0)
+        for w, a in enumerate((kq, vq, ks, vs)):
+            pa.kv_write(0, w, 0, a)
+        pa.kv_write(0, 0, total, np.full((tail, nKV, hd), 77, np.int8)); pa.kv_write(0, 1, total, np.full((tail, nKV, hd), -99, np.int8))
+        pa.kv_write(0, 2, total, np.full((tail, nKV, hd // 32), np.nan, np.float32)); pa.kv_write(0, 3, total, np.full((tail, nKV, hd // 32), np.nan, np.float32))
+        plan = pa.plan("prefill", base, n)
+        assert plan["kernel"] == 0 and plan["n_splits"] == 1 and plan["slots"] == 1 and plan["cols_per_group"] * G == rows, plan
+        for out_dtype in (0, PA_OUT_F16):
+            got = pa.run_attn("prefill", 0, q, base, gate=gate, out_dtype=out_dtype).astype(np.float32)
+            assert_parity(got, ref, "q8 small chunk base %d n %d out %d" % (base, n, out_dtype))
+
+
+def test_q8_short_verify_block_is_one_split_with_two_row_blocks():
+    """A verify block over a few tiles on an int8 cache: one split, two row blocks (4 columns x 8 heads), output written
+    by the split-K kernel's own epilogue."""
+    cfg = _q8cfg("qwen36_moe")
+    nKV, hd = cfg["n_kv_heads"], cfg["head_dim"]
+    rng = np.random.default_rng(31)
+    base, n, tail = 100, 4, 40
+    kq, ks, vq, vs, kf, vf = _quantised_cache(cfg, base + n, seed=32)
+    q = rng.standard_normal((n, cfg["n_heads"], hd), dtype=np.float32)
+    gate = rng.standard_normal(q.shape, dtype=np.float32)
+    ref = O.attention_values(q, kf, vf, base, gate=gate)
+    with PooledAttn(cfg, base + n + tail, n_layers=1, max_cols=n) as pa:
+        pa.layer_alloc(0)
+        for w, a in enumerate((kq, vq, ks, vs)):
+            pa.kv_write(0, w, 0, a)
+        pa.kv_write(0, 2, base + n, np.full((tail, nKV, hd // 32), np.nan, np.float32)); pa.kv_write(0, 3, base + n, np.full((tail, nKV, hd // 32), np.nan, np.float32))
+        plan = pa.plan("decode", base, n)
+        assert plan["kernel"] == 0 and plan["n_splits"] == 1 and plan["row_blocks"] == 2 and plan["slots"] == 1, plan
+        for out_dtype in (0, PA_OUT_F16):
+            got = pa.run_attn("decode", 0, q, base, gate=gate, out_dtype=out_dtype).astype(np.float32)
+            assert_parity(got, ref, "q8 short verify block out %d" % out_dtype)
