@@ -387,10 +387,11 @@ def layer_leg(pa, cfg, ctx, steps, warmup, attn_ms, n_rot, rng):
                                   us_per_step=round(t_verify * 1e3, 2), us_per_token=round(t_verify * 1e3 / nv, 2)))
 
 
-def stream_ceiling(pa, rotation, step, reps):
+def stream_ceiling(pa, rotation, step, reps, events=True):
     """What a one-shot 64 MiB read reaches on this part with the decode kernel's launch shape: every read-only stand-in
     of the library (pa_probe_stream), the empty kernel of the same grid and the decode step's own split-K kernel, each
-    timed by dispatch-stamped events over `rotation` layers' caches, launches back to back."""
+    timed by dispatch-stamped events over `rotation` layers' caches, launches back to back.  events=False: plain
+    launches only (for a run under rocprofv3 --kernel-trace, whose own timestamps then time undisturbed launches)."""
     L = pa.L
     sink = pa.alloc(8 << 20)
     ptrs = [(L.pa_kv_device_ptr(pa.ctx, l, 0), L.pa_kv_device_ptr(pa.ctx, l, 1)) for l in range(rotation)]
@@ -399,6 +400,15 @@ def stream_ceiling(pa, rotation, step, reps):
     def stats(ms):
         us = sorted(x * 1e3 for x in ms)
         return dict(launches=len(us), median_us=round(us[len(us) // 2], 2), mean_us=round(sum(us) / len(us), 2), min_us=round(us[0], 2), p90_us=round(us[len(us) * 9 // 10], 2))
+    if not events:
+        for v in range(L.pa_probe_count()):
+            for i in range(reps + 2 * rotation):
+                pa._chk(L.pa_probe_stream(pa.ctx, v, ptrs[i % rotation][0], ptrs[i % rotation][1], sink.ptr))
+            pa.sync()
+        for i in range(reps + 2 * rotation):
+            step(i, rotation)
+        pa.sync()
+        return None
     for v in range(L.pa_probe_count()):
         for i in range(2 * rotation):
             pa._chk(L.pa_probe_stream(pa.ctx, v, ptrs[i % rotation][0], ptrs[i % rotation][1], sink.ptr))
@@ -444,6 +454,7 @@ def main():
     ap.add_argument("--rotation", type=int, default=0, help="time the decode step with this many layers' caches in rotation only (default: sweep %s)" % (ROTATIONS,))
     ap.add_argument("--stream-ceiling", action="store_true",
                     help="only time the read-only stand-ins of the decode kernel's K/V stream, the empty kernel of its grid and the kernel itself (events; run under rocprofv3 --kernel-trace for the trace's clock)")
+    ap.add_argument("--no-events", action="store_true", help="with --stream-ceiling: plain launches, no event pairs (for a run under a kernel trace)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
@@ -500,7 +511,7 @@ def main():
         res = {}
         for r in rotations:
             log("stream ceiling, %d layers' caches in rotation (%.0f MiB):" % (r, r * 2 * ctx * kvd * 2 / 2**20))
-            res[str(r)] = stream_ceiling(pa, r, step, max(args.steps, 240))
+            res[str(r)] = stream_ceiling(pa, r, step, max(args.steps, 240), not args.no_events)
         pa.close()
         print(json.dumps({"stream_ceiling": res, "library": L.pa_version().decode()}))
         return

@@ -41,6 +41,30 @@ static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
 
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 
+// Exchanges between the four 16-lane rows of a wavefront on the VALU (gfx950 lane-swap instructions) instead of the LDS
+// crossbar (ds_bpermute: a dependent round trip of ~100 clocks each, four of them on the critical path of every tile's
+// softmax).  xrow16(v): lane i's own value and the value of lane i ^ 16; xrow32(v): the same for i ^ 32.  Both partners see
+// the same pair, so a commutative combine gives both the same bits.
+static __device__ inline void xrow16(float v, float& a, float& b) {
+  const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  a = __uint_as_float(sw[0]); b = __uint_as_float(sw[1]);
+}
+static __device__ inline void xrow32(float v, float& a, float& b) {
+  const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  a = __uint_as_float(sw[0]); b = __uint_as_float(sw[1]);
+}
+// maximum / sum over the four lanes {i, i ^ 16, i ^ 32, i ^ 48} (the four position groups of a query row), the same bits in all four
+static __device__ inline float rows_max(float v) {
+  float a, b;
+  xrow16(v, a, b); v = fmaxf(a, b);
+  xrow32(v, a, b); return fmaxf(a, b);
+}
+static __device__ inline float rows_sum(float v) {
+  float a, b;
+  xrow16(v, a, b); v = a + b;
+  xrow32(v, a, b); return a + b;
+}
+
 // 16 int8 values x scale -> 16 f16 (see the Q8 note at the kernel)
 static __device__ inline void dq16(const u4 raw, const float sc, h8& lo, h8& hi) {
   const h2 s2 = { (_Float16)sc, (_Float16)sc };
@@ -333,7 +357,14 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   // The fused pre-step computes between the K and the V loads: a wave sits in the issue of its tile loads for
   // microseconds (the memory pipeline is full), so arithmetic placed after all of them starts that much later, while
   // the K requests already queued keep the pipeline fed during the arithmetic.
-  if constexpr (!FUSED) first_v_loads();
+  // V_LATE (single-round splits): the V loads go out only after the K tile has been scored.  A wave cannot compute while
+  // it sits in the issue of its loads (the CU's memory pipeline accepts a load as an older one completes: 1 - 2 us for
+  // 16 loads once the chip is streaming), so with K and V requested back to back the last waves' K tiles -- long since
+  // arrived -- waited for the V issue to end, and staging, scores and softmax of K (1.1 us) came on top of the V work at
+  // the very end of the kernel.  Scored first, that work runs while other waves keep the pipeline full, and what follows
+  // the last V load is the V latency, the staging of V and the PV product.  Measured on the 32K decode step: 18.6 -> 18.15 us.
+  constexpr bool V_LATE = SR && !GATHER;
+  if constexpr (!FUSED && !V_LATE) first_v_loads();
   __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the load issue
   // ---- q -> f16 rows in LDS; waits only for the q loads, which were issued first ----
   if constexpr (FUSED) {
@@ -392,7 +423,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
       *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
     }
   }
-  if constexpr (FUSED) {
+  if constexpr (FUSED && !V_LATE) {
     __builtin_amdgcn_sched_barrier(0);
     first_v_loads();
     __builtin_amdgcn_sched_barrier(0);
@@ -474,7 +505,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
     {
       // fragments are fetched FD k-steps ahead of the MFMAs that use them, and the issue order is pinned: left to
       // itself the compiler waits for each k-step's three LDS reads right before its MFMAs, one LDS latency a step
-      constexpr int FD = HD == 256 ? 1 : 3;
+      constexpr int FD = HD == 256 ? (SR ? 4 : 1) : 3;     // the single-round kernel has the registers for four k-steps of fragments in flight
       h8 a0r[FD], a1r[FD], br[FD][NB];
       auto fetch = [&](int ks, int slot) __attribute__((always_inline)) {
         a0r[slot] = *(const h8*)(stage + ln * S::KROW + ks * 64 + kg * 16);
@@ -576,24 +607,24 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
           v[pb * 4 + i] = x;
           mx = fmaxf(mx, x);
         }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = rows_max(mx);
       const float mw_safe = mx == NEG_INF ? 0.f : mx;
       float ps = 0.f;
       h8 pf;
 #pragma unroll
       for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
-      ps += __shfl_xor(ps, 16, 64);
-      ps += __shfl_xor(ps, 32, 64);
+      ps = rows_sum(ps);
+      if constexpr (V_LATE) { __builtin_amdgcn_sched_barrier(0); first_v_loads(); __builtin_amdgcn_sched_barrier(0); }
       stage_v(ILV && ilv ? 0u : tp, false, 0);                          // interleaved splits are whole: no row past the end to zero
       *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pf;
       if (kg == 0) { mex[wave * 16 + ln] = mx; lex[wave * 16 + ln] = ps; }
       __syncthreads();
       {
         // V^T fragments (two transpose reads each) and the tile's P are fetched VD steps ahead of their MFMA
+        // (a tile's P is read once, not once per 16-dim block: the tail of the kernel is bound by the LDS port)
         constexpr int NS = W * DBW, VD = 4;
         h4 lor[VD], hir[VD];
-        h8 pfr[VD];
+        h8 pfr[W];
         f4 pr[W][DBW];
         auto fetch = [&](int st, int slot) __attribute__((always_inline)) {
           const int w2 = st / DBW, db = wave * DBW + st % DBW;
@@ -601,23 +632,24 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
           const unsigned char* vp = sw + (4 * kg + (ln >> 2)) * S::VROW + (db * 16 + 4 * (ln & 3)) * 2;
           lor[slot] = lds_read_tr16(vp);
           hir[slot] = lds_read_tr16(vp + 16 * S::VROW);
-          pfr[slot] = *(const h8*)(sw + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16);
         };
+#pragma unroll
+        for (int w2 = 0; w2 < W; w2++) pfr[w2] = *(const h8*)(stage_all + w2 * S::STAGE + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16);
 #pragma unroll
         for (int st = 0; st < VD; st++) fetch(st, st);
 #pragma unroll
         for (int st = 0; st < NS; st++) {
           const h4 lo = lor[st % VD], hi = hir[st % VD];
-          const h8 pb = pfr[st % VD];
           if (st + VD < NS) fetch(st + VD, st % VD);
           const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
-          pr[st / DBW][st % DBW] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pb, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+          pr[st / DBW][st % DBW] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pfr[st / DBW], (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
         }
+        __builtin_amdgcn_sched_group_barrier(0x100, W, 1);
 #pragma unroll
-        for (int st = 0; st < VD; st++) __builtin_amdgcn_sched_group_barrier(0x100, 3, 1);
+        for (int st = 0; st < VD; st++) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
 #pragma unroll
         for (int st = 0; st < NS; st++) {
-          if (st + VD < NS) __builtin_amdgcn_sched_group_barrier(0x100, 3, 1);
+          if (st + VD < NS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
         }
         // a wave without a tile staged stale rows: its m is -inf, and its products must not reach O even as 0 x NaN
@@ -682,8 +714,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
           v[nb][pb * 4 + i] = x;
           mx = fmaxf(mx, x);
         }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = rows_max(mx);
       mxs[nb] = mx;
       grow |= mx > m_run[nb] + DEC_RESCALE_TH;
     }
@@ -753,8 +784,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   const bool direct = p.direct_out != 0;       // one split and no own-row partial: this workgroup holds the whole result
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
-    l_run[nb] += __shfl_xor(l_run[nb], 16, 64);
-    l_run[nb] += __shfl_xor(l_run[nb], 32, 64);
+    l_run[nb] = rows_sum(l_run[nb]);
     if (kg == 0) { mex[wave * 16 * NB + nb * 16 + ln] = m_run[nb]; lex[wave * 16 * NB + nb * 16 + ln] = l_run[nb]; }
   }
   __syncthreads();
