@@ -437,6 +437,57 @@ def stream_ceiling(pa, rotation, step, reps, events=True):
     return rows
 
 
+def timeline(pa, step, n_rot, iters=24):
+    """In-kernel timeline of the decode step's split-K kernel (trace build of the library: python -m pooled_amd.build
+    --trace): per phase boundary, when the waves pass it -- relative to the first wave entering on the same XCC (the
+    XCCs start a dispatch up to 1.5 us apart) -- and how long each phase takes a wave.  Launches back to back; every
+    sixth launch is read out."""
+    import ctypes
+    L = pa.L
+    L.pa_trace_set.restype = ctypes.c_int; L.pa_trace_set.argtypes = [ctypes.c_void_p]
+    NW, NST = 512 * 4, 16
+    tr = pa.alloc(NW * NST * 8)
+    for i in range(60):
+        step(i, n_rot)
+    pa.sync()
+    if L.pa_trace_set(tr.ptr) != 0:
+        raise RuntimeError("pa_trace_set failed")
+    names = ["entry", "raw q / weights loads issued", "K tile loads issued", "pre-step done, q rows staged", "barrier 1 passed", "K tile arrived and staged",
+             "scores done", "softmax done", "V tile loads issued", "V tile arrived and staged", "barrier 2 passed", "partial stored"]
+    rel_all, span, span_x, clk = [], [], [], []
+    for it in range(iters):
+        for j in range(6):
+            step(it * 6 + j, n_rot)
+        pa.sync()
+        t = tr.download(np.uint64, NW * NST).reshape(NW, NST)
+        ts = t[:, :12].astype(np.int64)
+        xcc = t[:, 14].astype(np.int64)
+        rel = np.zeros(ts.shape, np.float64)
+        for x in range(8):
+            m = xcc == x
+            rel[m] = (ts[m] - ts[m, 0].min()) / 100.0
+        rel_all.append(rel)
+        span.append((ts[:, 11].max() - ts[:, 0].min()) / 100.0)
+        span_x.append(rel[:, 11].max())
+        clk.append(np.median(t[:, 13].astype(np.float64) / np.maximum((ts[:, 11] - ts[:, 0]) / 100.0, 1e-3)))
+    L.pa_trace_set(None)
+    a = np.stack(rel_all[4:])
+    res = dict(launches_read=len(rel_all) - 4, shader_clock_mhz=round(float(np.median(clk[4:]))), span_first_entry_to_last_store_us=round(float(np.median(span[4:])), 2),
+               span_per_xcc_us=round(float(np.median(span_x[4:])), 2), stamps=[], phases=[])
+    log("shader clock %d MHz; first entry -> last store %.2f us (per XCC %.2f us)" % (res["shader_clock_mhz"], res["span_first_entry_to_last_store_us"], res["span_per_xcc_us"]))
+    log("%-32s %7s %7s %7s %7s %7s" % ("when waves pass (us)", "min", "p10", "p50", "p90", "max"))
+    for s_, n in enumerate(names):
+        q = np.percentile(a[:, :, s_], [0, 10, 50, 90, 100], axis=1).mean(1)
+        res["stamps"].append(dict(stamp=n, min=round(q[0], 2), p10=round(q[1], 2), p50=round(q[2], 2), p90=round(q[3], 2), max=round(q[4], 2)))
+        log("%-32s %7.2f %7.2f %7.2f %7.2f %7.2f" % (n, *q))
+    log("%-66s %7s %7s" % ("phase of a wave (us)", "median", "p90"))
+    for s_ in range(1, len(names)):
+        d = a[:, :, s_] - a[:, :, s_ - 1]
+        res["phases"].append(dict(phase="%s -> %s" % (names[s_ - 1], names[s_]), median=round(float(np.median(d)), 2), p90=round(float(np.percentile(d, 90)), 2)))
+        log("%-66s %7.2f %7.2f" % (res["phases"][-1]["phase"], res["phases"][-1]["median"], res["phases"][-1]["p90"]))
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -454,12 +505,16 @@ def main():
     ap.add_argument("--rotation", type=int, default=0, help="time the decode step with this many layers' caches in rotation only (default: sweep %s)" % (ROTATIONS,))
     ap.add_argument("--stream-ceiling", action="store_true",
                     help="only time the read-only stand-ins of the decode kernel's K/V stream, the empty kernel of its grid and the kernel itself (events; run under rocprofv3 --kernel-trace for the trace's clock)")
+    ap.add_argument("--timeline", action="store_true", help="only print the in-kernel timeline of the decode step's split-K kernel (needs the trace build: python -m pooled_amd.build --trace)")
     ap.add_argument("--no-events", action="store_true", help="with --stream-ceiling: plain launches, no event pairs (for a run under a kernel trace)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
+    if args.timeline:
+        from pooled_amd import capi, build as pa_build
+        capi.LIB_PATH = pa_build.TRACE_LIB
     from pooled_amd.capi import PooledAttn, PA_OUT_F16, load
     L = load()
     log("library:", L.pa_version().decode())
@@ -507,6 +562,11 @@ def main():
         else:
             pa.attn_decode_step(layer, d_qfull, d_k, d_v, d_qw, d_kw, ctx, d_out, PA_OUT_F16)
 
+    if args.timeline:
+        res = timeline(pa, step, rotations[0])
+        pa.close()
+        print(json.dumps({"timeline": res, "layers_in_rotation": rotations[0], "library": L.pa_version().decode()}))
+        return
     if args.stream_ceiling:
         res = {}
         for r in rotations:

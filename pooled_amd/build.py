@@ -23,12 +23,16 @@ def _hipcc():
     return shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
 
-def build_lib(verbose=False, extra=()):
-    os.makedirs(LIBDIR, exist_ok=True)
+TRACE_LIB = os.path.join(LIBDIR, "trace", "libpooled_attn.so")
+
+
+def build_lib(verbose=False, extra=(), lib=LIB):
+    objdir = os.path.dirname(lib)
+    os.makedirs(objdir, exist_ok=True)
     objs = []
     procs = []
     for src in HIP_SOURCES:
-        obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
         cmd = [_hipcc()] + HIPCC_FLAGS + list(extra) + ["-I", os.path.join(ROOT, "include"), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd))
@@ -41,9 +45,15 @@ def build_lib(verbose=False, extra=()):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
         if out.strip():
             print(out)
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs
     subprocess.check_call(cmd)
-    return LIB
+    return lib
+
+
+def build_trace_lib(verbose=False):
+    """The development-timeline build of the same sources (-DPA_TRACE: the single-round decode kernel stamps its phases);
+    used by bench.py --timeline only."""
+    return build_lib(verbose, extra=("-DPA_TRACE",), lib=TRACE_LIB)
 
 
 def build_addon(verbose=False):
@@ -67,4 +77,7 @@ def build_all(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build_all(verbose="-v" in sys.argv))
+    if "--trace" in sys.argv:
+        print(build_trace_lib(verbose="-v" in sys.argv))
+    else:
+        print(build_all(verbose="-v" in sys.argv))

@@ -31,6 +31,26 @@ typedef __fp16 hh4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 
 #define TILE 32
+
+// Development timeline (compiled with -DPA_TRACE only: bench.py --timeline): lane 0 of every wave of the single-round kernel
+// stamps the 100 MHz wall clock at the phase boundaries below and writes the stamps, its XCC id and the shader cycles it
+// ran to the buffer pa_trace_set names.  Without PA_TRACE the macros are empty and the kernels are unchanged.
+#ifdef PA_TRACE
+#define PA_TRACE_STAMPS 16
+__device__ unsigned long long* g_pa_trace = nullptr;
+extern "C" int pa_trace_set(void* d_buf) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_pa_trace), &d_buf, sizeof(d_buf)); }
+#define TR_DECL unsigned long long trs[PA_TRACE_STAMPS] = {0}; const unsigned long long trs_clk0 = clock64()
+#define TR(i) do { if (SR) { __builtin_amdgcn_sched_barrier(0); trs[i] = wall_clock64(); __builtin_amdgcn_sched_barrier(0); } } while (0)
+#define TR_FLUSH(W_) do { if (SR && g_pa_trace && lane == 0) {                                                                \
+    unsigned long long* t_ = g_pa_trace + ((size_t)(blockIdx.x + gridDim.x * blockIdx.y) * (W_) + wave) * PA_TRACE_STAMPS;     \
+    for (int i_ = 0; i_ < 13; i_++) t_[i_] = trs[i_];                                                                         \
+    unsigned xcc_; asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_));                                        \
+    t_[13] = clock64() - trs_clk0; t_[14] = xcc_ & 0xf; t_[15] = wall_clock64(); } } while (0)
+#else
+#define TR_DECL do {} while (0)
+#define TR(i) do {} while (0)
+#define TR_FLUSH(W_) do {} while (0)
+#endif
 #define NEG_INF (-__builtin_inff())
 #define DEC_RESCALE_TH 8.f   // tile loop: a row maximum may pass the reference maximum by this much before O is rescaled
 
@@ -94,6 +114,20 @@ static __device__ inline void fused_q_rows(const float (&xq)[16 / W][4], const f
   for (int n = 0; n < N; n++)
 #pragma unroll
     for (int j = 0; j < 4; j++) x[n][j] = xq[n][j];
+  if (glue_regs_serves(half)) {
+    // the usual pair distances: norm and rotation in registers, the heads written as f16 rows element by element
+    glue_heads_regs<N>(x, wq, norm, eps, HD, half, cs, lane);
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+      const uint32_t r = wave + W * n;
+      if (r < G) {
+#pragma unroll
+        for (int j = 0; j < HD / 64; j++) *(_Float16*)(q_lds + r * QROW + (lane + 64 * j) * 2) = (_Float16)x[n][j];
+      }
+    }
+    wave_lds_fence();
+    return;
+  }
   glue_heads_wave<N>(x, wq, norm, eps, HD, half, cs, xs, HD, lane);
 #pragma unroll
   for (int n = 0; n < N; n++) {
@@ -157,6 +191,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
   static_assert(!Q8 || !GATHER, "int8 caches: no gather mode");
   typedef DecShape<HD> S;
+  TR_DECL;
+  TR(0);                              // entry
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]
   unsigned char* stage_all = smem + 16 * NB * S::QROW;               // [W][STAGE]
@@ -294,7 +330,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
 #pragma unroll
     for (int j = 0; j < 2; j++) {
       const uint32_t i = lane + 64 * j;
-      if (half) cs[j] = rope_pair(p.rope_tab, p.inv_freq, p.base_pos, half, min(i, half - 1));
+      // (half == 32: every lane holds the pair lane & 31 -- the in-register rotation reads it in the upper lanes too)
+      if (half) cs[j] = rope_pair(p.rope_tab, p.inv_freq, p.base_pos, half, half == 32 ? i & 31 : min(i, half - 1));
     }
 #pragma unroll
     for (int t = 0; t < HPW; t++)
@@ -311,6 +348,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
       qv[j] = *(const f4*)(p.q + (size_t)(c0 + rc / G) * p.q_stride + (size_t)(g * G + rc % G) * HD + 4 * d4);
     }
   }
+  TR(1);                              // q / raw projection loads issued
   // Loads are unconditional: the caches carry TILE rows of padding past max_seq, so a tile that straddles the
   // end of the context reads valid memory; rows at or past t_end are zeroed (V) or masked (scores) below.
   // A wave with no tile of its own (short splits) loads the split's last tile and discards it: the prologue
@@ -364,6 +402,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   // the very end of the kernel.  Scored first, that work runs while other waves keep the pipeline full, and what follows
   // the last V load is the V latency, the staging of V and the PV product.  Measured on the 32K decode step: 18.6 -> 18.15 us.
   constexpr bool V_LATE = SR && !GATHER;
+  TR(2);                              // K tile loads issued
   if constexpr (!FUSED && !V_LATE) first_v_loads();
   __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the load issue
   // ---- q -> f16 rows in LDS; waits only for the q loads, which were issued first ----
@@ -423,6 +462,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
       *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
     }
   }
+  TR(3);                              // pre-step done (fused), q rows staged
   if constexpr (FUSED && !V_LATE) {
     __builtin_amdgcn_sched_barrier(0);
     first_v_loads();
@@ -436,6 +476,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
     end_pos[nb] = r < R ? (GATHER ? seq_max : p.base_pos + c0 + r / G + 1 - p.self_row) : 0u;
   }
   __syncthreads();
+  TR(4);                              // barrier 1 passed
   // ---- the column's own row as a partial of its own (slot = number of splits that hold rows): m = its score,
   // l = 1, O = its value row.  The scores run on the VALU over the f16 operands the MFMA path would see, f32 sums in a
   // fixed order; the work hides under the latency of the tile loads.  Decoding a token at a position that is a
@@ -594,8 +635,10 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
       const bool has_tile = wave < n_tiles;
       const uint32_t tp = t_begin + min(wave, n_tiles - 1) * TILE;      // the tile this wave holds in registers
       stage_k(tp, false, 0);
+      TR(5);                          // K tile arrived and staged
       f4 s[2][NB];
       qk(s);
+      TR(6);                          // scores done
       const uint32_t row_end = has_tile ? end_pos[0] : 0u;              // a wave without a tile contributes nothing
       float v[8], mx = NEG_INF;
 #pragma unroll
@@ -614,11 +657,15 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
 #pragma unroll
       for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
       ps = rows_sum(ps);
+      TR(7);                          // softmax done
       if constexpr (V_LATE) { __builtin_amdgcn_sched_barrier(0); first_v_loads(); __builtin_amdgcn_sched_barrier(0); }
+      TR(8);                          // V tile loads issued
       stage_v(ILV && ilv ? 0u : tp, false, 0);                          // interleaved splits are whole: no row past the end to zero
       *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pf;
       if (kg == 0) { mex[wave * 16 + ln] = mx; lex[wave * 16 + ln] = ps; }
+      TR(9);                          // V tile arrived and staged, P published
       __syncthreads();
+      TR(10);                         // barrier 2 passed
       {
         // V^T fragments (two transpose reads each) and the tile's P are fetched VD steps ahead of their MFMA
         // (a tile's P is read once, not once per 16-dim block: the tail of the kernel is bound by the LDS port)
@@ -676,6 +723,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
           for (int j = 0; j < DBW; j++) *(f4*)(p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = o[j];
           if (wave == 0 && kg == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(M, Lr);
         }
+        TR(11);                       // partial stored
+        TR_FLUSH(W);
       }
     }
     return;

@@ -65,6 +65,25 @@ static __device__ inline void rope_cos_sin(uint32_t pos, float inv_freq, float& 
   c = (float)cd; s = (float)sd;
 }
 
+// f32(1 / sqrt(ss / hd + eps)): the RMSNorm factor of a head from its f64 sum of squares.  The f64 value is good to a few
+// units of its last place -- ss / hd by exponent arithmetic where hd is a power of two (exact), the reciprocal root from the
+// hardware estimate and three Newton steps -- and is rounded once to f32: the same f32 as a correctly rounded f64 division
+// and root give, except where their result lies within ~2^-50 of an f32 rounding boundary.  The library-call form
+// (division, root, division) is ~40 dependent f64 instructions on the critical path of every wave of the fused decode
+// step; this is ~12.
+static __device__ inline float rms_inv(double ss, uint32_t hd, float eps) {
+  const double mean = (hd & (hd - 1)) == 0 ? ldexp(ss, -(31 - (int)__builtin_clz(hd))) : ss / (double)hd;
+  const double x = mean + (double)eps;
+  const double h = 0.5 * x;
+  double r = __builtin_amdgcn_rsq(x);
+#pragma unroll
+  for (int it = 0; it < 3; it++) {
+    const double e = __builtin_fma(-h * r, r, 0.5);     // 0.5 - (x / 2) r^2
+    r = __builtin_fma(r, e, r);                          // r (1.5 - (x / 2) r^2)
+  }
+  return (float)r;
+}
+
 // (cos, sin) of rotation pair i at position pos: from the per-context table when there is one
 static __device__ inline float2 rope_pair(const float2* rope_tab, const float* inv_freq, uint32_t pos, uint32_t half, uint32_t i) {
   if (rope_tab) return rope_tab[(size_t)pos * half + i];
@@ -98,7 +117,7 @@ static __device__ inline void glue_heads_wave(const float (&x_in)[N][4], const f
     for (int n = 0; n < N; n++) ss[n] = wave_sum_f64(ss[n]);
     float inv[N];
 #pragma unroll
-    for (int n = 0; n < N; n++) inv[n] = (float)(1.0 / sqrt(ss[n] / (double)hd + (double)eps));
+    for (int n = 0; n < N; n++) inv[n] = rms_inv(ss[n], hd, eps);
 #pragma unroll
     for (int n = 0; n < N; n++)
 #pragma unroll
@@ -133,6 +152,60 @@ static __device__ inline void glue_heads_wave(const float (&x_in)[N][4], const f
         if (i < half) { xs[n][i] = ra[n][j]; xs[n][i + half] = rb[n][j]; }
       }
     wave_lds_fence();
+  }
+}
+
+// The same arithmetic without LDS for the pair distances that the lane + 64 j layout keeps inside a register file: half a
+// multiple of 64 (partners are registers j and j + half / 64 of one lane) and half == 32 (partners are lanes l and l ^ 32 of
+// register 0, exchanged by a lane-swap instruction; cs[0] must then hold the (cos, sin) of pair lane & 31 in every lane).
+// On return x holds the normed and rotated head, element lane + 64 j in x[n][j].  Same operations on the same values as
+// glue_heads_wave, so the same bits; four dependent LDS round trips shorter.
+static __device__ inline bool glue_regs_serves(uint32_t half) { return half == 0 || half == 32 || (half & 63) == 0; }
+template <int N>
+static __device__ inline void glue_heads_regs(float (&x)[N][4], const float (&w)[4], bool norm, float eps, uint32_t hd,
+                                              uint32_t half, const float2 (&cs)[2], uint32_t lane) {
+#pragma clang fp contract(off)
+  if (norm) {
+    double ss[N];
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+      ss[n] = 0.0;
+#pragma unroll
+      for (int j = 0; j < 4; j++) ss[n] += (double)x[n][j] * (double)x[n][j];
+    }
+#pragma unroll
+    for (int n = 0; n < N; n++) ss[n] = wave_sum_f64(ss[n]);
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+      const float inv = rms_inv(ss[n], hd, eps);
+#pragma unroll
+      for (int j = 0; j < 4; j++) { const float sw = inv * w[j]; x[n][j] = x[n][j] * sw; }
+    }
+  }
+  if (half == 32) {
+    const float c = cs[0].x, s = cs[0].y;
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+      const float own = x[n][0];
+      const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(own), __float_as_uint(own), false, false);
+      const float other = __uint_as_float(lane < 32 ? sw[1] : sw[0]);      // element i + 32 for lanes i < 32, element i - 32 above
+      const float pc = own * c, ps = other * s;                               // rounded one by one
+      x[n][0] = lane < 32 ? pc - ps : pc + ps;                                // a' = a c - b s ; b' = b c + a s
+    }
+  } else if (half) {
+    const uint32_t step = half >> 6;              // 1 or 2 at hd <= 256
+#pragma unroll
+    for (int n = 0; n < N; n++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        if ((uint32_t)j < step) {
+          const float c = cs[j].x, s = cs[j].y;
+          const float a = x[n][j], b = step == 1 ? x[n][j + 1] : x[n][j + 2];
+          const float ac = a * c, bs = b * s, bc = b * c, as = a * s;
+          x[n][j] = ac - bs;
+          if (step == 1) x[n][j + 1] = bc + as; else x[n][j + 2] = bc + as;
+        }
+      }
   }
 }
 
