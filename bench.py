@@ -452,7 +452,7 @@ def timeline(pa, step, n_rot, iters=24):
     pa.sync()
     if L.pa_trace_set(tr.ptr) != 0:
         raise RuntimeError("pa_trace_set failed")
-    names = ["entry", "raw q / weights loads issued", "K tile loads issued", "pre-step done, q rows staged", "barrier 1 passed", "K tile arrived and staged",
+    names = ["entry", "kernel arguments read", "raw q / weights loads issued", "K tile loads issued", "pre-step done, q rows staged", "barrier 1 passed", "K tile arrived and staged",
              "scores done", "softmax done", "V tile loads issued", "V tile arrived and staged", "barrier 2 passed", "partial stored"]
     rel_all, span, span_x, clk = [], [], [], []
     for it in range(iters):
@@ -460,16 +460,16 @@ def timeline(pa, step, n_rot, iters=24):
             step(it * 6 + j, n_rot)
         pa.sync()
         t = tr.download(np.uint64, NW * NST).reshape(NW, NST)
-        ts = t[:, :12].astype(np.int64)
+        ts = t[:, [0, 12, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11]].astype(np.int64)
         xcc = t[:, 14].astype(np.int64)
         rel = np.zeros(ts.shape, np.float64)
         for x in range(8):
             m = xcc == x
             rel[m] = (ts[m] - ts[m, 0].min()) / 100.0
         rel_all.append(rel)
-        span.append((ts[:, 11].max() - ts[:, 0].min()) / 100.0)
-        span_x.append(rel[:, 11].max())
-        clk.append(np.median(t[:, 13].astype(np.float64) / np.maximum((ts[:, 11] - ts[:, 0]) / 100.0, 1e-3)))
+        span.append((ts[:, 12].max() - ts[:, 0].min()) / 100.0)
+        span_x.append(rel[:, 12].max())
+        clk.append(np.median(t[:, 13].astype(np.float64) / np.maximum((ts[:, 12] - ts[:, 0]) / 100.0, 1e-3)))
     L.pa_trace_set(None)
     a = np.stack(rel_all[4:])
     res = dict(launches_read=len(rel_all) - 4, shader_clock_mhz=round(float(np.median(clk[4:]))), span_first_entry_to_last_store_us=round(float(np.median(span[4:])), 2),

@@ -193,6 +193,10 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   typedef DecShape<HD> S;
   TR_DECL;
   TR(0);                              // entry
+#ifdef PA_TRACE
+  { const void* ka_ = p.k_cache; const uint32_t kb_ = p.base_pos; asm volatile("s_waitcnt lgkmcnt(0)" :: "s"(ka_), "s"(kb_)); }
+  TR(12);                             // kernel arguments read
+#endif
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]
   unsigned char* stage_all = smem + 16 * NB * S::QROW;               // [W][STAGE]
@@ -205,9 +209,12 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   // the others.
   uint32_t sp = blockIdx.x, g = blockIdx.y;
   if constexpr (SR) {
-    const uint32_t nf = p.n_wgs ? min(p.n_wgs, gridDim.x) : gridDim.x, lin = blockIdx.x + gridDim.x * blockIdx.y;
-    if (lin < nf * gridDim.y) { g = lin / nf; sp = lin % nf; }
-    else { const uint32_t e = lin - nf * gridDim.y; g = e % gridDim.y; sp = nf + e / gridDim.y; }
+    const uint32_t nf = p.n_wgs ? min(p.n_wgs, gridDim.x) : gridDim.x;
+    if (__builtin_expect(nf != gridDim.x, 0)) {                       // (no remainder splits: the grid's own coordinates)
+      const uint32_t lin = blockIdx.x + gridDim.x * blockIdx.y;
+      if (lin < nf * gridDim.y) { g = lin / nf; sp = lin % nf; }
+      else { const uint32_t e = lin - nf * gridDim.y; g = e % gridDim.y; sp = nf + e / gridDim.y; }
+    }
   }
   uint32_t cg = blockIdx.z;
   if constexpr (!SR) {
@@ -231,14 +238,15 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   // rows visible to the group's last column (gather: the column's list length)
   // self_row (one-column decode): the column's own row base_pos is not streamed with the others -- see below
   const uint32_t seq_max = GATHER ? min(p.sel[c0 * p.sel_stride], p.sel_max) : p.base_pos + c0 + ncl - p.self_row;
-  const uint32_t t_begin = sp * p.split_len;
+  const uint32_t split_len = SR ? (uint32_t)(W * TILE) : p.split_len;   // single-round splits: one tile per wave
+  const uint32_t t_begin = sp * split_len;
   // The workgroup of split 0 turns the column's own row into a partial of its own (wave 0, while the tile loads are
   // in flight), so it runs even when no other row exists (base_pos == 0).
   const bool self_wg = !GATHER && p.self_row && sp == 0;
   if (t_begin >= seq_max && !self_wg) return;
   const bool has_rows = t_begin < seq_max;
   // the last split is open-ended: the plan may hand it up to one split length of remainder
-  const uint32_t t_end = !SR && sp + 1 == p.n_splits ? seq_max : min(t_begin + p.split_len, seq_max);
+  const uint32_t t_end = !SR && sp + 1 == p.n_splits ? seq_max : min(t_begin + split_len, seq_max);
   const size_t head_rows = (size_t)p.max_seq + TILE;              // rows of one kv head's plane, padding included
   // SR: the whole splits of a kv head are interleaved.  With nw = (whole splits) x W waves, wave v of
   // them takes rows [(c nw + v) 8, + 8), c = 0 .. 3, instead of 32 consecutive ones: at any moment the loads in
@@ -250,7 +258,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   uint32_t ilv_nw = 0, ilv_wv = 0;
   bool ilv = false;
   if constexpr (ILV) {
-    const uint32_t nfull = min(p.n_wgs ? p.n_wgs : p.n_splits, seq_max / p.split_len);
+    const uint32_t nfull = min(p.n_wgs ? p.n_wgs : p.n_splits, seq_max / split_len);
     ilv = sp < nfull;
     ilv_nw = nfull * W;
     ilv_wv = sp * W + (threadIdx.x >> 6);
@@ -279,6 +287,19 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   const uint32_t n_tiles = has_rows ? (t_end - t_begin + TILE - 1) / TILE : 0;
   u4 kr[S::NLD], vr[S::NLD];
   const u4 zero4 = {0u, 0u, 0u, 0u};
+  uint32_t tile = __builtin_amdgcn_readfirstlane(wave);
+  const uint32_t t0 = t_begin + min(tile, max(n_tiles, 1u) - 1) * TILE;
+  // Fused single-round step: the first three eighths of the K tile loads go out ahead of the raw projection / weight
+  // loads, as soon as the first kernel arguments are in: the K/V stream starts half a microsecond earlier.  The small
+  // rows return behind them (loads of a wave complete in order), which is free as long as they are back before the
+  // wave has pushed the rest of its K loads through the memory pipeline: measured on the 32K step, 6 of 16 loads ahead
+  // 17.81 -> 17.63 us; 8 ahead 17.4 or 17.9 us from one process to the next; 10, 12, 16 ahead 18.1 - 18.8 us.
+  constexpr int KF = SR && FUSED && !GATHER && !Q8 ? 3 * S::NLD / 8 : 0;
+  if constexpr (KF > 0) {
+#pragma unroll
+    for (int i = 0; i < KF; i++) kr[i] = *(const u4*)(kbase + (size_t)row_pos(t0, i * S::RPL) * row_bytes + voff);
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   // the column's own K / V row, 4 dims a lane: loaded here (the pre-step wrote it), or made below by the fused pre-step
   const bool self_wave = self_wg && wave == 0;
@@ -312,26 +333,41 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   float2 cs[2] = { make_float2(1.f, 0.f), make_float2(1.f, 0.f) };
   const uint32_t half = FUSED ? p.n_rot / 2 : 0;
   if constexpr (FUSED) {
-    // every load is unconditional (indices clamped) so that the waits below stay exact
+    // Only what the wave uses is requested (wave-uniform conditions): its own query heads -- not the clamped duplicates of
+    // head G - 1 --, and the new key / value row and the key weights in the one wave that makes the cache row.  Every wave
+    // of the chip asks for these small rows in the same first microsecond, through the same L1s that then carry the K/V
+    // stream; the K tile loads queue behind them.
 #pragma unroll
     for (int t = 0; t < HPW; t++) {
-      const uint32_t h = g * G + min(wave + W * t, G - 1);
 #pragma unroll
-      for (int j = 0; j < 4; j++) xq[t][j] = p.f_q_in[(size_t)h * p.f_q_head_stride + min(lane + 64 * j, (uint32_t)HD - 1)];
+      for (int j = 0; j < 4; j++) xq[t][j] = 0.f;
+      if (wave + W * t < G) {
+        const uint32_t h = g * G + wave + W * t;
+#pragma unroll
+        for (int j = 0; j < 4; j++) xq[t][j] = p.f_q_in[(size_t)h * p.f_q_head_stride + min(lane + 64 * j, (uint32_t)HD - 1)];
+      }
     }
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const uint32_t i = min(lane + 64 * j, (uint32_t)HD - 1);
-      xk[j] = p.f_k_in[(size_t)g * HD + i];
       wq[j] = p.f_qw ? p.f_qw[i] : 1.f;
-      wk[j] = p.f_kw ? p.f_kw[i] : 1.f;
+      xk[j] = 0.f; wk[j] = 1.f;
     }
-    xv4 = *(const f4*)(p.f_v_in + (size_t)g * HD + 4 * min(lane, (uint32_t)HD / 4 - 1));
+    if (self_wave) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const uint32_t i = min(lane + 64 * j, (uint32_t)HD - 1);
+        xk[j] = p.f_k_in[(size_t)g * HD + i];
+        if (p.f_kw) wk[j] = p.f_kw[i];
+      }
+      xv4 = *(const f4*)(p.f_v_in + (size_t)g * HD + 4 * min(lane, (uint32_t)HD / 4 - 1));
+    }
 #pragma unroll
     for (int j = 0; j < 2; j++) {
       const uint32_t i = lane + 64 * j;
-      // (half == 32: every lane holds the pair lane & 31 -- the in-register rotation reads it in the upper lanes too)
-      if (half) cs[j] = rope_pair(p.rope_tab, p.inv_freq, p.base_pos, half, half == 32 ? i & 31 : min(i, half - 1));
+      // (half == 32: every lane holds the pair lane & 31 -- the in-register rotation reads it in the upper lanes too;
+      // pairs 64 .. 127 exist only with more than 64 pairs)
+      if (half > 64u * j) cs[j] = rope_pair(p.rope_tab, p.inv_freq, p.base_pos, half, half == 32 ? i & 31 : min(i, half - 1));
     }
 #pragma unroll
     for (int t = 0; t < HPW; t++)
@@ -353,7 +389,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   // end of the context reads valid memory; rows at or past t_end are zeroed (V) or masked (scores) below.
   // A wave with no tile of its own (short splits) loads the split's last tile and discards it: the prologue
   // stays branch-free, so the q staging below waits for the q loads only.
-  uint32_t tile = __builtin_amdgcn_readfirstlane(wave);
   // gather: byte offsets of this lane's rows of a tile, through the list (positions at or past the list's end take
   // its last row: valid memory, masked or zeroed like any row past t_end)
   uint32_t goff[GATHER ? S::NLD : 1];
@@ -366,7 +401,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
       }
     }
   };
-  const uint32_t t0 = t_begin + min(tile, max(n_tiles, 1u) - 1) * TILE;
   if constexpr (GATHER) {
     gather_offsets(t0);
 #pragma unroll
@@ -377,7 +411,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
     ksr = *(const u4*)(ksbase + (size_t)row_pos(t0, srow) * S::SPR * 4 + (lane % S::LPS) * 16);
   } else {
 #pragma unroll
-    for (int i = 0; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)row_pos(t0, i * S::RPL) * row_bytes + voff);
+    for (int i = KF; i < S::NLD; i++) kr[i] = *(const u4*)(kbase + (size_t)row_pos(t0, i * S::RPL) * row_bytes + voff);
   }
   auto first_v_loads = [&]() __attribute__((always_inline)) {
     if constexpr (GATHER) {
@@ -482,7 +516,7 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   // fixed order; the work hides under the latency of the tile loads.  Decoding a token at a position that is a
   // multiple of the split length therefore streams whole tiles only.
   if (self_wave) {
-    const uint32_t self_slot = min((seq_max + p.split_len - 1) / p.split_len, p.n_splits);
+    const uint32_t self_slot = min((seq_max + split_len - 1) / split_len, p.n_splits);
     const bool on = lane < HD / 4;
     const f4 vxf = { (float)vx[0], (float)vx[1], (float)vx[2], (float)vx[3] };
     for (uint32_t r = 0; r < G; r++) {                                 // one column: row r is head g * G + r
