@@ -84,6 +84,21 @@ static __device__ inline float rows_sum(float v) {
   xrow16(v, a, b); v = a + b;
   xrow32(v, a, b); return a + b;
 }
+// lane i's copy of lane (i + N) % 16 of its row of 16 (DPP row rotation)
+template <int N>
+static __device__ inline float row_ror(float v) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x120 + N, 0xf, 0xf, false));
+}
+// maximum / sum over the 16 lanes {(i & 3) + 4 k}: two rotations inside the row, then the four rows.  The sum's
+// association differs from lane to lane (lane i starts at its own element); lanes 0 .. 3 are the ones that are read.
+static __device__ inline float quads_max(float v) {
+  v = fmaxf(v, row_ror<4>(v)); v = fmaxf(v, row_ror<8>(v));
+  return rows_max(v);
+}
+static __device__ inline float quads_sum(float v) {
+  v += row_ror<4>(v); v += row_ror<8>(v);
+  return rows_sum(v);
+}
 
 // 16 int8 values x scale -> 16 f16 (see the Q8 note at the kernel)
 static __device__ inline void dq16(const u4 raw, const float sc, h8& lo, h8& hi) {
@@ -197,6 +212,13 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   { const void* ka_ = p.k_cache; const uint32_t kb_ = p.base_pos; asm volatile("s_waitcnt lgkmcnt(0)" :: "s"(ka_), "s"(kb_)); }
   TR(12);                             // kernel arguments read
 #endif
+  if constexpr (FUSED && SR) {
+    // Every kernel argument the loads of the first microsecond need, fetched in the first batch of scalar loads: left
+    // alone, the compiler fetches arguments where they are first used, four dependent round trips before the first tile
+    // load (measured on the 32K step: 17.62 -> 17.27 us).
+    asm volatile("" :: "s"(p.k_cache), "s"(p.v_cache), "s"(p.f_q_in), "s"(p.f_qw), "s"(p.rope_tab), "s"(p.f_q_head_stride), "s"(p.n_rot),
+                 "s"(p.base_pos), "s"(p.max_seq), "s"(p.n_wgs), "s"(p.self_row), "s"(p.group), "s"(gridDim.x));
+  }
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]
   unsigned char* stage_all = smem + 16 * NB * S::QROW;               // [W][STAGE]
@@ -983,6 +1005,13 @@ __global__ __launch_bounds__(64) void pa_combine_wave_kernel(AttnParams p) {
   constexpr int SL = HD / DS, LPG = DS / 4, NG = 64 / LPG, CH = (272 + NG - 1) / NG;     // CH splits per lane and chunk: NG x CH >= 272 (256 + the own-row partial)
   // dispatch id i runs on XCD i % 8: XCD k takes the contiguous slice range [k n / 8, (k + 1) n / 8), so the slices that
   // share the 128-byte lines of a partial row (two 16-dim slices a line) read them through one L2
+  // Every kernel argument in the first batch of scalar loads: the kernel is a chain of dependent latencies, and left alone
+  // the compiler fetches arguments where they are first used (four round trips before the first partial load).  Whole
+  // runs of the argument block are named, so that no half-used wide load leaves registers whose reuse would force a wait.
+  asm volatile("" :: "s"(p.gate), "s"(p.part_o), "s"(p.part_ml), "s"(p.out), "s"(p.q_stride), "s"(p.gate_stride), "s"(p.out_stride), "s"(p.n_heads),
+               "s"(p.n_kv_heads), "s"(p.group), "s"(p.base_pos), "s"(p.n_cols), "s"(p.split_len), "s"(p.n_splits), "s"(p.slots), "s"(p.n_wgs),
+               "s"(p.cols_per_group), "s"(p.max_seq), "s"(p.self_row), "s"(p.out_f16), "s"(p.direct_out), "s"(p.scale), "s"(p.gate_head_stride),
+               "s"(p.sel), "s"(p.sel_stride), "s"(p.sel_max), "s"(gridDim.x));
   uint32_t wg = blockIdx.x;
   if (gridDim.x % 8 == 0) wg = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
   const uint32_t h = wg / SL, dq = wg % SL, col = blockIdx.y, lane = threadIdx.x;
@@ -1008,8 +1037,12 @@ __global__ __launch_bounds__(64) void pa_combine_wave_kernel(AttnParams p) {
 #pragma unroll
   for (int k = 0; k < CH; k++) M = fmaxf(M, mlv[k].x);
   for (uint32_t s = grp + NG * CH; s < ns; s += NG) M = fmaxf(M, pml[s].x);        // more than 272 splits
+  // over the 16 split groups: on the VALU (row rotations + lane swaps) with four lanes a group, else through the LDS crossbar
+  if constexpr (LPG == 4) M = quads_max(M);
+  else {
 #pragma unroll
-  for (int o = LPG; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+    for (int o = LPG; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+  }
   float L = 0.f;
   f4 o = zero;
 #pragma unroll
@@ -1032,11 +1065,17 @@ __global__ __launch_bounds__(64) void pa_combine_wave_kernel(AttnParams p) {
       o += ov[k] * w;
     }
   }
+  if constexpr (LPG == 4) {
+    L = quads_sum(L);
 #pragma unroll
-  for (int x = LPG; x < 64; x <<= 1) {
-    L += __shfl_xor(L, x, 64);
+    for (int i = 0; i < 4; i++) o[i] = quads_sum(o[i]);
+  } else {
 #pragma unroll
-    for (int i = 0; i < 4; i++) o[i] += __shfl_xor(o[i], x, 64);
+    for (int x = LPG; x < 64; x <<= 1) {
+      L += __shfl_xor(L, x, 64);
+#pragma unroll
+      for (int i = 0; i < 4; i++) o[i] += __shfl_xor(o[i], x, 64);
+    }
   }
   if (lane < LPG) {
     f4 r = ns ? o / L : zero;                      // an empty gather list: a column of zeros

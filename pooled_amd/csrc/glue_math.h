@@ -86,7 +86,7 @@ static __device__ inline float rms_inv(double ss, uint32_t hd, float eps) {
 
 // (cos, sin) of rotation pair i at position pos: from the per-context table when there is one
 static __device__ inline float2 rope_pair(const float2* rope_tab, const float* inv_freq, uint32_t pos, uint32_t half, uint32_t i) {
-  if (__builtin_expect(rope_tab != nullptr, 1)) return rope_tab[(size_t)pos * half + i];   // (the evaluation below: out of the hot path)
+  if (__builtin_expect(rope_tab != nullptr, 1)) return rope_tab[(size_t)pos * half + i];
   float c, s;
   rope_cos_sin(pos, inv_freq[i], c, s);
   return make_float2(c, s);
