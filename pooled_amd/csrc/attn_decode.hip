@@ -212,12 +212,20 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   { const void* ka_ = p.k_cache; const uint32_t kb_ = p.base_pos; asm volatile("s_waitcnt lgkmcnt(0)" :: "s"(ka_), "s"(kb_)); }
   TR(12);                             // kernel arguments read
 #endif
-  if constexpr (FUSED && SR) {
-    // Every kernel argument the loads of the first microsecond need, fetched in the first batch of scalar loads: left
-    // alone, the compiler fetches arguments where they are first used, four dependent round trips before the first tile
-    // load (measured on the 32K step: 17.62 -> 17.27 us).
+  // Every kernel argument the loads of the first microsecond need, fetched in the first batch of scalar loads: left
+  // alone, the compiler fetches arguments where they are first used, four dependent round trips before the first tile
+  // load (measured on the 32K step: 17.62 -> 17.27 us).
+  if constexpr (FUSED) {
     asm volatile("" :: "s"(p.k_cache), "s"(p.v_cache), "s"(p.f_q_in), "s"(p.f_qw), "s"(p.rope_tab), "s"(p.f_q_head_stride), "s"(p.n_rot),
                  "s"(p.base_pos), "s"(p.max_seq), "s"(p.n_wgs), "s"(p.self_row), "s"(p.group), "s"(gridDim.x));
+  } else if constexpr (GATHER) {
+    asm volatile("" :: "s"(p.q), "s"(p.k_cache), "s"(p.v_cache), "s"(p.q_stride), "s"(p.n_heads), "s"(p.group), "s"(p.base_pos), "s"(p.n_cols),
+                 "s"(p.split_len), "s"(p.n_splits), "s"(p.n_wgs), "s"(p.cols_per_group), "s"(p.max_seq), "s"(p.sel), "s"(p.sel_stride), "s"(p.sel_max),
+                 "s"(gridDim.x));
+  } else {
+    asm volatile("" :: "s"(p.q), "s"(p.k_cache), "s"(p.v_cache), "s"(p.q_stride), "s"(p.n_heads), "s"(p.group), "s"(p.base_pos), "s"(p.n_cols),
+                 "s"(p.split_len), "s"(p.n_splits), "s"(p.n_wgs), "s"(p.cols_per_group), "s"(p.max_seq), "s"(p.self_row), "s"(gridDim.x));
+    if constexpr (Q8) asm volatile("" :: "s"(p.k_scale), "s"(p.v_scale));
   }
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]

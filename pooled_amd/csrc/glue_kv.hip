@@ -47,6 +47,10 @@ hipError_t pa_launch_rope_table(float2* tab, const float* inv_freq, uint32_t hal
 }
 
 __global__ __launch_bounds__(64) void pa_glue_kernel(GlueParams p) {
+  // (every kernel argument in the first batch of scalar loads instead of a dependent round trip at each first use)
+  asm volatile("" :: "s"(p.q_in), "s"(p.k_in), "s"(p.v_in), "s"(p.k_out), "s"(p.qw), "s"(p.kw), "s"(p.inv_freq), "s"(p.rope_tab), "s"(p.q_out),
+               "s"(p.gate_out), "s"(p.k_cache), "s"(p.v_cache), "s"(p.ks_cache), "s"(p.vs_cache), "s"(p.head_rows), "s"(p.q_stride), "s"(p.k_stride),
+               "s"(p.v_stride), "s"(p.n_heads), "s"(p.n_kv_heads), "s"(p.head_dim), "s"(p.n_rot), "s"(p.base_pos), "s"(p.n_cols), "s"(p.flags), "s"(p.eps));
   __shared__ float xs[256];
   const uint32_t hh = blockIdx.x, col = blockIdx.y, lane = threadIdx.x;
   const uint32_t nH = p.n_heads, hd = p.head_dim;

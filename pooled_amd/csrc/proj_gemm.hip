@@ -218,6 +218,8 @@ __global__ __launch_bounds__(256, XT == 2 ? 2 : 1) void pa_gemm_kernel(GemmParam
 template <int KIND, int BPL, int RW>
 __global__ __launch_bounds__(256) void pa_gemm_skinny_kernel(GemmParams p) {
   static_assert(KIND == PA_W_Q4_0 || KIND == PA_W_Q8_0, "quantised weights");
+  // (every kernel argument in the first batch of scalar loads instead of a dependent round trip at each first use)
+  asm volatile("" :: "s"(p.w), "s"(p.scales), "s"(p.x), "s"(p.y), "s"(p.x_stride), "s"(p.y_stride), "s"(p.d_out), "s"(p.d_in), "s"(p.n_cols), "s"(p.acc));
   extern __shared__ __attribute__((aligned(16))) unsigned char sk_lds[];
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t nb = p.d_in / GK, ncol = p.n_cols;
@@ -388,6 +390,8 @@ hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s) {
 // inv = 1 / sqrt(mean(x^2) + eps) (engine/wgsl/base.js:119-152); the sum of squares is a fixed-order tree.
 __global__ __launch_bounds__(256) void pa_rmsnorm_f16_kernel(const float* x, uint32_t x_stride, const float* w, uint32_t dim, float eps,
                                                             uint16_t* out, uint32_t out_stride) {
+  // (every kernel argument in the first batch of scalar loads instead of a dependent round trip at each first use)
+  asm volatile("" :: "s"(x), "s"(x_stride), "s"(w), "s"(dim), "s"(eps), "s"(out), "s"(out_stride));
   __shared__ float red[4];
   const uint32_t col = blockIdx.x, tid = threadIdx.x;
   const f4* xs = (const f4*)(x + (size_t)col * x_stride);

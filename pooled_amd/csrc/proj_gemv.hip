@@ -79,11 +79,33 @@ static __device__ inline float dot_block(const BlockRegs<KIND>& r, const float (
 // BPL: blocks per lane (d_in <= 2048 * BPL); RW: rows per wave
 template <int KIND, int BPL, int RW, bool NORM>
 __global__ __launch_bounds__(256) void pa_gemv_kernel(GemvParams p) {
+  // every kernel argument in the first batch of scalar loads (the compiler fetches them where they are first used: a
+  // dependent round trip each before the loads that need them)
+  asm volatile("" :: "s"(p.w), "s"(p.scales), "s"(p.x), "s"(p.norm_w), "s"(p.xn_out), "s"(p.y), "s"(p.d_out), "s"(p.d_in), "s"(p.eps), "s"(p.acc));
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t nb = p.d_in / 32;
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * RW;
   const unsigned char* wbase = (const unsigned char*)p.w;
-  // this wave's rows first: the weight stream is what the kernel waits for
+  // x (and the norm weights) are requested FIRST, the wave's weight rows right behind them: the loads of a wave complete
+  // in order, x comes from L2 in a fraction of the time the weight stream takes from HBM, and everything that depends
+  // on x alone -- the sum of squares, two barriers, the trip through LDS -- then runs under the latency of the weights
+  // instead of after it.
+  extern __shared__ __attribute__((aligned(16))) float xs[];
+  __shared__ float red[4];
+  constexpr int XPT = 2 * BPL;                                         // float4 of x per thread (d_in <= 2048 * BPL)
+  const uint32_t n4 = p.d_in / 4;
+  f4 xv[XPT], wv[NORM ? XPT : 1];
+  float ss = 0.f;
+  // Loads past the end of x re-read its last float4 instead of being guarded (their values are never stored, and are
+  // masked out of the sum of squares by a factor, not by a select on the loaded value): a guarded load is a branch,
+  // and between guarded blocks the compiler placed a full wait.
+#pragma unroll
+  for (int k = 0; k < XPT; k++) xv[k] = ((const f4*)p.x)[min(threadIdx.x + 256 * k, n4 - 1)];
+  if constexpr (NORM) {
+#pragma unroll
+    for (int k = 0; k < XPT; k++) wv[k] = ((const f4*)p.norm_w)[min(threadIdx.x + 256 * k, n4 - 1)];
+  }
+  __builtin_amdgcn_sched_barrier(0);
   BlockRegs<KIND> wr[RW][BPL];
   uint16_t sc[RW][BPL];
 #pragma unroll
@@ -101,24 +123,11 @@ __global__ __launch_bounds__(256) void pa_gemv_kernel(GemvParams p) {
   float yold[RW];
 #pragma unroll
   for (int r = 0; r < RW; r++) yold[r] = p.acc ? p.y[min(row0 + r, (size_t)p.d_out - 1)] : 0.f;
-  // x -> LDS through coalesced loads (a lane's own slice is 32 consecutive floats: loaded directly, a wave-wide
-  // load would touch 64 cache lines for 1 KB), normed on the way when asked; block b sits at xs[b * 36]: the 4-float
-  // pad makes the 8 lanes of a 128-bit LDS read phase hit distinct banks
-  extern __shared__ __attribute__((aligned(16))) float xs[];
-  __shared__ float red[4];
-  constexpr int XPT = 2 * BPL;                                         // float4 of x per thread (d_in <= 2048 * BPL)
-  const uint32_t n4 = p.d_in / 4;
-  f4 xv[XPT], wv[NORM ? XPT : 1];
-  float ss = 0.f;
-  // Loads past the end of x re-read its last float4 instead of being guarded (their values are never stored, and are
-  // masked out of the sum of squares by a factor, not by a select on the loaded value): a guarded load is a branch,
-  // and between guarded blocks the compiler placed a full wait -- the norm weights went out a round trip after the
-  // weights and x.
-#pragma unroll
-  for (int k = 0; k < XPT; k++) xv[k] = ((const f4*)p.x)[min(threadIdx.x + 256 * k, n4 - 1)];
+  __builtin_amdgcn_sched_barrier(0);
+  // x -> LDS (a lane's own slice is 32 consecutive floats: loaded directly, a wave-wide load would touch 64 cache lines
+  // for 1 KB), normed on the way when asked; block b sits at xs[b * 36]: the 4-float pad makes the 8 lanes of a 128-bit
+  // LDS read phase hit distinct banks
   if constexpr (NORM) {
-#pragma unroll
-    for (int k = 0; k < XPT; k++) wv[k] = ((const f4*)p.norm_w)[min(threadIdx.x + 256 * k, n4 - 1)];
 #pragma unroll
     for (int k = 0; k < XPT; k++) {
       const float m = threadIdx.x + 256 * k < n4 ? 1.f : 0.f;
