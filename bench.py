@@ -163,7 +163,7 @@ def median(xs):
     return xs[len(xs) // 2]
 
 
-def prefill_leg(steps, with_cpu, kv_q8=False):
+def prefill_leg(steps, with_cpu, kv_q8=False, clk=False):
     """Configuration 5: a 4096-token causal chunk at positions 126976-131071 over a 126976-token f16 prefix,
     Qwen3.6-35B-MoE attention shape, sigmoid gate, f16 output.  A step = pre-step for the 4096 columns
     (QK-RMSNorm + partial RoPE + KV write) + the MFMA prefill kernel.  PREFILL_WARMUP untimed steps (the first one's
@@ -192,6 +192,13 @@ def prefill_leg(steps, with_cpu, kv_q8=False):
         pa.timer_start(); step()
         return pa.timer_stop()                       # blocks until the step has finished
 
+    clk_buf = None
+    if clk:                                          # ablation builds: wave 0 of every workgroup reports shader cycles and 100 MHz ticks
+        import ctypes
+        pa.L.pa_pf_clk_set.restype = ctypes.c_int; pa.L.pa_pf_clk_set.argtypes = [ctypes.c_void_p]
+        clk_buf = pa.alloc(4096 * 16)
+        if pa.L.pa_pf_clk_set(clk_buf.ptr) != 0:
+            raise RuntimeError("pa_pf_clk_set failed")
     pa.sync()
     cold_first_ms = timed_step()
     for _ in range(PREFILL_WARMUP - 1):
@@ -202,6 +209,11 @@ def prefill_leg(steps, with_cpu, kv_q8=False):
     pa.profile_enable(False)
     ms_step, k_ms = median(step_ms), median(kern_ms)
     k_mean = sum(kern_ms) / max(len(kern_ms), 1)
+    clk_mhz = None
+    if clk_buf is not None:
+        cw = clk_buf.download(np.uint64, 2 * 256).reshape(256, 2).astype(np.float64)       # the last launch's 256 workgroups
+        clk_mhz = float(np.median(cw[:, 0] / np.maximum(cw[:, 1], 1.0) * 100.0))
+        pa.L.pa_pf_clk_set(None)
     flops = causal_flops(cfg, base, n)
     tf_step, tf_kernel = flops / (ms_step * 1e-3) / 1e12, flops / (k_ms * 1e-3) / 1e12
     log("prefill C5: first launch %.3f ms; median of %d steps %.3f ms (min %.3f, max %.3f) -> %.1f TFLOP/s; kernel median %.3f ms (mean %.3f) -> %.1f TFLOP/s (%.1f%% of f16 MFMA peak)"
@@ -210,7 +222,7 @@ def prefill_leg(steps, with_cpu, kv_q8=False):
                         "every tensor an independent N(0,1) stream" % ("int8 (widened once per chunk into an f16 staging cache, inside the step)" if kv_q8 else "f16"),
                value=round(tf_step, 1), unit="TFLOP/s", ms_per_step=round(ms_step, 4), steps=steps, warmup=PREFILL_WARMUP, reported="median of the timed steps",
                min_ms_per_step=round(min(step_ms), 4), max_ms_per_step=round(max(step_ms), 4), cold_first_ms=round(cold_first_ms, 4),
-               step_ms=[round(x, 3) for x in step_ms], flops_per_step=flops, plan=pa.plan("prefill", base, n),
+               step_ms=[round(x, 3) for x in step_ms], flops_per_step=flops, plan=pa.plan("prefill", base, n), shader_clock_mhz=clk_mhz,
                roofline=dict(bound="mfma", achieved=round(tf_kernel, 1), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s", frac=round(tf_kernel / MFMA_F16_PEAK_TFLOPS, 4),
                              traffic=None, kernel="pa_prefill_kernel<256, 1, 8>", kernel_ms=round(k_ms, 4), kernel_ms_mean=round(k_mean, 4),
                              kernel_ms_min=round(min(kern_ms), 4), kernel_ms_max=round(max(kern_ms), 4), reported="median launch",
@@ -505,6 +517,10 @@ def main():
     ap.add_argument("--rotation", type=int, default=0, help="time the decode step with this many layers' caches in rotation only (default: sweep %s)" % (ROTATIONS,))
     ap.add_argument("--stream-ceiling", action="store_true",
                     help="only time the read-only stand-ins of the decode kernel's K/V stream, the empty kernel of its grid and the kernel itself (events; run under rocprofv3 --kernel-trace for the trace's clock)")
+    ap.add_argument("--prefill-ablation", action="store_true",
+                    help="only time the C5 prefill kernel with parts of its step removed (timing-only builds: python -m pooled_amd.build --prefill-ablation), "
+                         "each build in a process of its own, two interleaved rounds")
+    ap.add_argument("--prefill-ablation-child", type=int, default=-1, help=argparse.SUPPRESS)
     ap.add_argument("--timeline", action="store_true", help="only print the in-kernel timeline of the decode step's split-K kernel (needs the trace build: python -m pooled_amd.build --trace)")
     ap.add_argument("--no-events", action="store_true", help="with --stream-ceiling: plain launches, no event pairs (for a run under a kernel trace)")
     args = ap.parse_args()
@@ -512,6 +528,30 @@ def main():
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
+    if args.prefill_ablation:
+        import subprocess
+        from pooled_amd import build as pa_build
+        rounds = []
+        for rnd in range(2):
+            row = {}
+            for mask, label in pa_build.PREFILL_ABLATIONS:
+                out = subprocess.run([sys.executable, os.path.abspath(__file__), "--prefill-ablation-child", str(mask), "--prefill-steps", str(args.prefill_steps)],
+                                     stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=600, check=True).stdout
+                row[mask] = json.loads(out.strip().splitlines()[-1])
+                log("round %d  removed: %-62s kernel median %.3f ms  shader clock %4.0f MHz" % (rnd + 1, label, row[mask]["kernel_ms"], row[mask]["shader_clock_mhz"]))
+            rounds.append(row)
+        full = [r[0]["kernel_ms"] for r in rounds]
+        table = [dict(mask=mask, removed=label, kernel_ms=[r[mask]["kernel_ms"] for r in rounds], shader_clock_mhz=[round(r[mask]["shader_clock_mhz"]) for r in rounds],
+                      vs_full_pct=[round(100 * (r[mask]["kernel_ms"] / f - 1), 1) for r, f in zip(rounds, full)],
+                      tflops=[round(rounds[0][0]["flops"] / (r[mask]["kernel_ms"] * 1e-3) / 1e12, 1) for r in rounds]) for mask, label in pa_build.PREFILL_ABLATIONS]
+        print(json.dumps({"prefill_ablation": table}))
+        return
+    if args.prefill_ablation_child >= 0:
+        from pooled_amd import capi, build as pa_build
+        capi.LIB_PATH = pa_build.ablation_lib(args.prefill_ablation_child)
+        r = prefill_leg(args.prefill_steps, False, clk=True)
+        print(json.dumps(dict(kernel_ms=r["roofline"]["kernel_ms"], shader_clock_mhz=r["shader_clock_mhz"], flops=r["flops_per_step"])))
+        return
     if args.timeline:
         from pooled_amd import capi, build as pa_build
         capi.LIB_PATH = pa_build.TRACE_LIB

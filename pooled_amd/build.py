@@ -56,6 +56,29 @@ def build_trace_lib(verbose=False):
     return build_lib(verbose, extra=("-DPA_TRACE",), lib=TRACE_LIB)
 
 
+# timing-only ablations of the prefill step (attn_prefill.hip, PF_ABL): what is removed from every step
+PREFILL_ABLATIONS = [(0, "nothing"), (1, "the 16 v_exp_f32 per lane (argument passed through)"), (2, "K fragment reads (one fragment reused)"),
+                     (4, "V^T fragment reads"), (6, "K and V^T fragment reads"), (8, "the whole softmax (scores converted straight to f16)"),
+                     (14, "fragment reads and softmax"), (16, "the LDS-direct tile loads (32 KB a step and CU from L2)"),
+                     (30, "all of the above (MFMAs and the barrier remain)")]
+
+
+def ablation_lib(mask):
+    return os.path.join(LIBDIR, "abl%d" % mask, "libpooled_attn.so")
+
+
+def build_prefill_ablations(verbose=False):
+    """One library per ablation mask (results wrong on purpose; bench.py --prefill-ablation times them)."""
+    out = []
+    for mask, _ in PREFILL_ABLATIONS:
+        lib = build_lib(verbose, extra=("-DPF_ABL=%d" % mask,), lib=ablation_lib(mask))
+        for f in os.listdir(os.path.dirname(lib)):
+            if f.endswith(".o"):
+                os.remove(os.path.join(os.path.dirname(lib), f))
+        out.append(lib)
+    return out
+
+
 def build_addon(verbose=False):
     """The thin Node-API layer over the C ABI (plain g++ against the system node headers; no node-gyp)."""
     src = os.path.join(CSRC, "pa_napi.cc")
@@ -79,5 +102,7 @@ def build_all(verbose=False):
 if __name__ == "__main__":
     if "--trace" in sys.argv:
         print(build_trace_lib(verbose="-v" in sys.argv))
+    elif "--prefill-ablation" in sys.argv:
+        print(build_prefill_ablations(verbose="-v" in sys.argv))
     else:
         print(build_all(verbose="-v" in sys.argv))

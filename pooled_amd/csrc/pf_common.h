@@ -13,7 +13,20 @@ typedef __fp16 hh4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 
 #define NEG_INF (-__builtin_inff())
-#define PF_TN 32                 // positions per step
+#define PF_TN 32                 // positions per MFMA tile
+#ifndef PF_SUB
+#define PF_SUB 1                 // tiles per step (between two barriers)
+#endif
+#define PF_STEP (PF_TN * PF_SUB) // positions per step
+#ifndef PF_QR
+#define PF_QR 16                 // head_dim 256: k-steps of Q kept in registers (any others are parked in LDS)
+#endif
+#ifndef PF_KD
+#define PF_KD 2                  // K (and parked Q) fragments fetched this many k-steps ahead
+#endif
+#ifndef PF_VD
+#define PF_VD 2                  // V^T fragments fetched this many MFMAs ahead
+#endif
 #define PF_RESCALE_TH 8.0f       // log2 units
 
 static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
@@ -32,3 +45,9 @@ static __device__ inline uint32_t lds_addr_of(const unsigned char* p) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)p;
 }
 #define PF_GLL(gptr, lptr) pf_gll((gptr), __builtin_amdgcn_readfirstlane(lds_addr_of(lptr)))
+// the same with the address as a wave-uniform base (scalar registers) + a 32-bit per-lane byte offset: the offset is the
+// same for every tile, so no 64-bit per-lane addresses are kept or rebuilt
+static __device__ inline void pf_gll_s(const unsigned char* sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+#define PF_GLL_S(sbase, voff, lptr) pf_gll_s((sbase), (voff), __builtin_amdgcn_readfirstlane(lds_addr_of(lptr)))
