@@ -93,8 +93,8 @@ def build_addon(verbose=False):
     return ADDON
 
 
-def build_all(verbose=False):
-    lib = build_lib(verbose)
+def build_all(verbose=False, extra=()):
+    lib = build_lib(verbose, extra=extra)
     addon = build_addon(verbose)
     return lib, addon
 
@@ -105,4 +105,5 @@ if __name__ == "__main__":
     elif "--prefill-ablation" in sys.argv:
         print(build_prefill_ablations(verbose="-v" in sys.argv))
     else:
-        print(build_all(verbose="-v" in sys.argv))
+        # -DNAME=VALUE arguments go to hipcc (the prefill kernel's PF_SUB / PF_QR / PF_KD / PF_VD experiments)
+        print(build_all(verbose="-v" in sys.argv, extra=tuple(a for a in sys.argv[1:] if a.startswith("-D"))))
