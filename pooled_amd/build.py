@@ -16,7 +16,9 @@ ADDON = os.path.join(LIBDIR, "pooled_attn.node")
 HIP_SOURCES = ["pa_api.hip", "glue_kv.hip", "attn_decode.hip", "attn_prefill.hip", "proj_gemv.hip", "proj_gemm.hip", "proj_gemm_wide.hip", "stream_probe.hip"]
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
                # packed-FP32 VALU forms are kept off for all device code
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               # the first twelve dwords of a kernel's leading scalar / pointer arguments arrive in scalar registers at wave start
+               "-mllvm", "-amdgpu-kernarg-preload-count=12"]
 
 
 def _hipcc():

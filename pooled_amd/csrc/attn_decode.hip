@@ -200,7 +200,16 @@ template <int HD> struct DecShape {
 // O^T = V^T P^T of a split is divided over the waves by output dims, see the code.  Without SR a split has any length
 // and every wave loops over its own tiles.
 template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
-__global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) void pa_decode_kernel(AttnParams p) {
+__global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1))
+void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a_max_seq, uint32_t a_n_wgs, uint32_t a_n_splits, uint32_t a_self_row,
+                      uint32_t a_grid_x, const float* a_f_q_in, uint32_t a_group, uint32_t a_f_q_head_stride, AttnParams p_in) {
+  // The leading arguments repeat fields of p_in: the first twelve dwords of a kernel's arguments are preloaded into
+  // scalar registers by the dispatcher (-amdgpu-kernarg-preload-count), so what the first tile loads' addresses are made
+  // of is there when the wave starts instead of a scalar-load round trip later.
+  AttnParams p = p_in;
+  p.k_cache = a_k_cache; p.base_pos = a_base_pos; p.max_seq = a_max_seq; p.n_wgs = a_n_wgs; p.n_splits = a_n_splits; p.self_row = a_self_row;
+  p.f_q_in = a_f_q_in; p.group = a_group; p.f_q_head_stride = a_f_q_head_stride;
+  const uint32_t grid_x = a_grid_x;
   static_assert(!SR || NB == 1, "single-round splits: one 16-row block");
   static_assert(!FUSED || NB == 1, "the fused pre-step serves one column");
   static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
@@ -212,21 +221,6 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   { const void* ka_ = p.k_cache; const uint32_t kb_ = p.base_pos; asm volatile("s_waitcnt lgkmcnt(0)" :: "s"(ka_), "s"(kb_)); }
   TR(12);                             // kernel arguments read
 #endif
-  // Every kernel argument the loads of the first microsecond need, fetched in the first batch of scalar loads: left
-  // alone, the compiler fetches arguments where they are first used, four dependent round trips before the first tile
-  // load (measured on the 32K step: 17.62 -> 17.27 us).
-  if constexpr (FUSED) {
-    asm volatile("" :: "s"(p.k_cache), "s"(p.v_cache), "s"(p.f_q_in), "s"(p.f_qw), "s"(p.rope_tab), "s"(p.f_q_head_stride), "s"(p.n_rot),
-                 "s"(p.base_pos), "s"(p.max_seq), "s"(p.n_wgs), "s"(p.self_row), "s"(p.group), "s"(gridDim.x));
-  } else if constexpr (GATHER) {
-    asm volatile("" :: "s"(p.q), "s"(p.k_cache), "s"(p.v_cache), "s"(p.q_stride), "s"(p.n_heads), "s"(p.group), "s"(p.base_pos), "s"(p.n_cols),
-                 "s"(p.split_len), "s"(p.n_splits), "s"(p.n_wgs), "s"(p.cols_per_group), "s"(p.max_seq), "s"(p.sel), "s"(p.sel_stride), "s"(p.sel_max),
-                 "s"(gridDim.x));
-  } else {
-    asm volatile("" :: "s"(p.q), "s"(p.k_cache), "s"(p.v_cache), "s"(p.q_stride), "s"(p.n_heads), "s"(p.group), "s"(p.base_pos), "s"(p.n_cols),
-                 "s"(p.split_len), "s"(p.n_splits), "s"(p.n_wgs), "s"(p.cols_per_group), "s"(p.max_seq), "s"(p.self_row), "s"(gridDim.x));
-    if constexpr (Q8) asm volatile("" :: "s"(p.k_scale), "s"(p.v_scale));
-  }
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]
   unsigned char* stage_all = smem + 16 * NB * S::QROW;               // [W][STAGE]
@@ -239,9 +233,9 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   // the others.
   uint32_t sp = blockIdx.x, g = blockIdx.y;
   if constexpr (SR) {
-    const uint32_t nf = p.n_wgs ? min(p.n_wgs, gridDim.x) : gridDim.x;
-    if (__builtin_expect(nf != gridDim.x, 0)) {                       // (no remainder splits: the grid's own coordinates)
-      const uint32_t lin = blockIdx.x + gridDim.x * blockIdx.y;
+    const uint32_t nf = p.n_wgs ? min(p.n_wgs, grid_x) : grid_x;
+    if (__builtin_expect(nf != grid_x, 0)) {                          // (no remainder splits: the grid's own coordinates)
+      const uint32_t lin = blockIdx.x + grid_x * blockIdx.y;
       if (lin < nf * gridDim.y) { g = lin / nf; sp = lin % nf; }
       else { const uint32_t e = lin - nf * gridDim.y; g = e % gridDim.y; sp = nf + e / gridDim.y; }
     }
@@ -261,8 +255,8 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t ln = lane & 15, kg = lane >> 4;
   const uint32_t G = p.group, nH = p.n_heads;
-  const uint32_t c0 = cg * p.cols_per_group;
-  const uint32_t ncl = min(p.cols_per_group, p.n_cols - c0);
+  const uint32_t c0 = FUSED ? 0u : cg * p.cols_per_group;            // (the fused step serves one column)
+  const uint32_t ncl = FUSED ? 1u : min(p.cols_per_group, p.n_cols - c0);
   const uint32_t R = ncl * G;                                        // live rows (<= 16*NB)
   const uint32_t sel_base = GATHER ? c0 * p.sel_stride + 1 : 0;      // gather: first list entry of this column
   // rows visible to the group's last column (gather: the column's list length)
@@ -329,6 +323,18 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
 #pragma unroll
     for (int i = 0; i < KF; i++) kr[i] = *(const u4*)(kbase + (size_t)row_pos(t0, i * S::RPL) * row_bytes + voff);
     __builtin_amdgcn_sched_barrier(0);
+  }
+  // Every other kernel argument the loads of the first microsecond need, fetched in one batch of scalar loads: left
+  // alone, the compiler fetches arguments where they are first used, four dependent round trips before the first tile
+  // load (measured on the 32K step: 17.62 -> 17.27 us).  (The arguments of the first tile loads are preloaded.)
+  if constexpr (FUSED) {
+    asm volatile("" :: "s"(p.v_cache), "s"(p.f_qw), "s"(p.rope_tab), "s"(p.n_rot));
+  } else if constexpr (GATHER) {
+    asm volatile("" :: "s"(p.q), "s"(p.v_cache), "s"(p.q_stride), "s"(p.n_heads), "s"(p.n_cols),
+                 "s"(p.split_len), "s"(p.cols_per_group), "s"(p.sel), "s"(p.sel_stride), "s"(p.sel_max));
+  } else {
+    asm volatile("" :: "s"(p.q), "s"(p.v_cache), "s"(p.q_stride), "s"(p.n_heads), "s"(p.n_cols), "s"(p.split_len), "s"(p.cols_per_group));
+    if constexpr (Q8) asm volatile("" :: "s"(p.k_scale), "s"(p.v_scale));
   }
 
   // the column's own K / V row, 4 dims a lane: loaded here (the pre-step wrote it), or made below by the fused pre-step
@@ -1009,21 +1015,22 @@ __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1)) voi
 // groups are xor-shuffle trees (fixed order), lanes 0 .. 3 finish and store.  The four lanes of a group hold the same
 // (m, l), so each computes its splits' weights itself instead of fetching them from a neighbour.
 template <int HD, int DS>
-__global__ __launch_bounds__(64) void pa_combine_wave_kernel(AttnParams p) {
+__global__ __launch_bounds__(64)
+void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint32_t a_slots, uint32_t a_n_heads, uint32_t a_base_pos, uint32_t a_self_row,
+                            uint32_t a_split_len, uint32_t a_n_splits, uint32_t a_grid_x, uint32_t a_has_sel, AttnParams p_in) {
+  // The leading arguments repeat fields of p_in (a_has_sel: p_in.sel != nullptr): the first twelve dwords of the arguments
+  // are preloaded into scalar registers, so the partial loads' addresses need no scalar-load round trip.  The other
+  // arguments are fetched in one batch behind those loads (the compiler would fetch each where it is first used).
+  AttnParams p = p_in;
+  p.part_o = const_cast<float*>(a_part_o); p.part_ml = const_cast<float*>(a_part_ml); p.slots = a_slots; p.n_heads = a_n_heads;
+  p.base_pos = a_base_pos; p.self_row = a_self_row; p.split_len = a_split_len; p.n_splits = a_n_splits;
   constexpr int SL = HD / DS, LPG = DS / 4, NG = 64 / LPG, CH = (272 + NG - 1) / NG;     // CH splits per lane and chunk: NG x CH >= 272 (256 + the own-row partial)
   // dispatch id i runs on XCD i % 8: XCD k takes the contiguous slice range [k n / 8, (k + 1) n / 8), so the slices that
   // share the 128-byte lines of a partial row (two 16-dim slices a line) read them through one L2
-  // Every kernel argument in the first batch of scalar loads: the kernel is a chain of dependent latencies, and left alone
-  // the compiler fetches arguments where they are first used (four round trips before the first partial load).  Whole
-  // runs of the argument block are named, so that no half-used wide load leaves registers whose reuse would force a wait.
-  asm volatile("" :: "s"(p.gate), "s"(p.part_o), "s"(p.part_ml), "s"(p.out), "s"(p.q_stride), "s"(p.gate_stride), "s"(p.out_stride), "s"(p.n_heads),
-               "s"(p.n_kv_heads), "s"(p.group), "s"(p.base_pos), "s"(p.n_cols), "s"(p.split_len), "s"(p.n_splits), "s"(p.slots), "s"(p.n_wgs),
-               "s"(p.cols_per_group), "s"(p.max_seq), "s"(p.self_row), "s"(p.out_f16), "s"(p.direct_out), "s"(p.scale), "s"(p.gate_head_stride),
-               "s"(p.sel), "s"(p.sel_stride), "s"(p.sel_max), "s"(gridDim.x));
   uint32_t wg = blockIdx.x;
-  if (gridDim.x % 8 == 0) wg = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+  if (a_grid_x % 8 == 0) wg = (blockIdx.x % 8) * (a_grid_x / 8) + blockIdx.x / 8;
   const uint32_t h = wg / SL, dq = wg % SL, col = blockIdx.y, lane = threadIdx.x;
-  const uint32_t col_end = p.sel ? min(p.sel[col * p.sel_stride], p.sel_max) : p.base_pos + col + 1 - p.self_row;
+  const uint32_t col_end = a_has_sel ? min(p.sel[col * p.sel_stride], p.sel_max) : p.base_pos + col + 1 - p.self_row;
   const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
   const uint32_t grp = lane / LPG, l4 = lane % LPG;
@@ -1038,6 +1045,8 @@ __global__ __launch_bounds__(64) void pa_combine_wave_kernel(AttnParams p) {
     mlv[k] = s < ns ? pml[s] : make_float2(NEG_INF, 0.f);
     ov[k] = s < ns ? *(const f4*)(po + (size_t)s * HD) : zero;
   }
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("" :: "s"(p.gate), "s"(p.out), "s"(p.gate_stride), "s"(p.out_stride), "s"(p.out_f16), "s"(p.gate_head_stride));
   const uint32_t d_out = dq * DS + 4 * l4;
   f4 gt = zero;
   if (p.gate && lane < LPG) gt = *(const f4*)(p.gate + (size_t)col * p.gate_stride + (size_t)h * p.gate_head_stride + d_out);
@@ -1199,7 +1208,8 @@ static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipS
   if (e != hipSuccess) return e;
   if (!SR && col_groups != (p.n_cols + p.cols_per_group - 1) / p.cols_per_group) return hipErrorInvalidValue;
   const dim3 grid = SR ? dim3(p.n_splits, p.n_kv_heads, col_groups) : dim3((p.n_splits * p.n_kv_heads * col_groups + 7) / 8 * 8);
-  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), grid, dim3(W * 64), lds, s, t, p);
+  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), grid, dim3(W * 64), lds, s, t, p.k_cache, p.base_pos, p.max_seq, p.n_wgs, p.n_splits, p.self_row,
+            (uint32_t)grid.x, p.f_q_in, p.group, p.f_q_head_stride, p);
   return hipGetLastError();
 }
 
@@ -1286,8 +1296,11 @@ hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s) {
     else hipLaunchKernelGGL(pa_combine_wide_kernel<128>, grid, dim3(256), 0, s, p);
     return hipGetLastError();
   }
-  if (hd == 256) hipLaunchKernelGGL((pa_combine_wave_kernel<256, 16>), dim3(p.n_heads * (256 / 16), p.n_cols), dim3(64), 0, s, p);
-  else if (hd == 128) hipLaunchKernelGGL((pa_combine_wave_kernel<128, 16>), dim3(p.n_heads * (128 / 16), p.n_cols), dim3(64), 0, s, p);
+  const uint32_t gx = p.n_heads * (hd / 16), has_sel = p.sel != nullptr;
+  if (hd == 256) hipLaunchKernelGGL((pa_combine_wave_kernel<256, 16>), dim3(gx, p.n_cols), dim3(64), 0, s, (const float*)p.part_o, (const float*)p.part_ml,
+                                    p.slots, p.n_heads, p.base_pos, p.self_row, p.split_len, p.n_splits, gx, has_sel, p);
+  else if (hd == 128) hipLaunchKernelGGL((pa_combine_wave_kernel<128, 16>), dim3(gx, p.n_cols), dim3(64), 0, s, (const float*)p.part_o, (const float*)p.part_ml,
+                                         p.slots, p.n_heads, p.base_pos, p.self_row, p.split_len, p.n_splits, gx, has_sel, p);
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }

@@ -78,10 +78,13 @@ static __device__ inline float dot_block(const BlockRegs<KIND>& r, const float (
 
 // BPL: blocks per lane (d_in <= 2048 * BPL); RW: rows per wave
 template <int KIND, int BPL, int RW, bool NORM>
-__global__ __launch_bounds__(256) void pa_gemv_kernel(GemvParams p) {
-  // every kernel argument in the first batch of scalar loads (the compiler fetches them where they are first used: a
-  // dependent round trip each before the loads that need them)
-  asm volatile("" :: "s"(p.w), "s"(p.scales), "s"(p.x), "s"(p.norm_w), "s"(p.xn_out), "s"(p.y), "s"(p.d_out), "s"(p.d_in), "s"(p.eps), "s"(p.acc));
+__global__ __launch_bounds__(256)
+void pa_gemv_kernel(const float* a_x, const float* a_norm_w, const void* a_w, const uint16_t* a_scales, float* a_y, uint32_t a_d_out, uint32_t a_d_in, GemvParams p_in) {
+  // The leading arguments repeat fields of p_in: the first twelve dwords of the arguments are preloaded into scalar
+  // registers, so every load address of the kernel is there when the wave starts; the other arguments are fetched in one
+  // batch of scalar loads (the compiler would fetch each where it is first used, a dependent round trip each).
+  GemvParams p = p_in;
+  p.x = a_x; p.norm_w = a_norm_w; p.w = a_w; p.scales = a_scales; p.y = a_y; p.d_out = a_d_out; p.d_in = a_d_in;
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t nb = p.d_in / 32;
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * RW;
@@ -120,6 +123,7 @@ __global__ __launch_bounds__(256) void pa_gemv_kernel(GemvParams p) {
   }
   // accumulating calls: the old values of the wave's rows are requested here, with everything else, instead of in a
   // round trip of their own behind the reduction
+  asm volatile("" :: "s"(p.xn_out), "s"(p.eps), "s"(p.acc));
   float yold[RW];
 #pragma unroll
   for (int r = 0; r < RW; r++) yold[r] = p.acc ? p.y[min(row0 + r, (size_t)p.d_out - 1)] : 0.f;
@@ -207,7 +211,7 @@ template <int KIND, int BPL, int RW, bool NORM>
 static hipError_t launch_k(const GemvParams& p, hipStream_t s) {
   const uint32_t rows_wg = 4 * RW;
   const size_t lds = (size_t)(p.d_in / 32) * 36 * sizeof(float);
-  hipLaunchKernelGGL((pa_gemv_kernel<KIND, BPL, RW, NORM>), dim3((p.d_out + rows_wg - 1) / rows_wg), dim3(256), lds, s, p);
+  hipLaunchKernelGGL((pa_gemv_kernel<KIND, BPL, RW, NORM>), dim3((p.d_out + rows_wg - 1) / rows_wg), dim3(256), lds, s, p.x, p.norm_w, p.w, p.scales, p.y, p.d_out, p.d_in, p);
   return hipGetLastError();
 }
 
