@@ -563,7 +563,10 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       if (!on) d = 0.f;
       d = wave_sum_f32(d);
       const size_t slot = ((size_t)c0 * nH + g * G + r) * p.slots + self_slot;
-      if (on) *(f4*)(p.part_o + slot * HD + 4 * lane) = vxf;
+      if (on) {
+        if (p.part_f16) *(h4*)((_Float16*)p.part_o + slot * HD + 4 * lane) = vx;
+        else *(f4*)(p.part_o + slot * HD + 4 * lane) = vxf;
+      }
       if (lane == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(d * p.scale, 1.f);
     }
   }
@@ -789,8 +792,16 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
         if (ln < R) {
           const uint32_t col = c0 + ln / G, hq = g * G + ln % G;
           const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
+          // f16 partials (|O| <= 128 rows x |v|: far inside the range; the merge adds them up in f32): half the bytes this
+          // kernel writes at its very end and half of what the merge kernel waits for
+          if (p.part_f16) {
 #pragma unroll
-          for (int j = 0; j < DBW; j++) *(f4*)(p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = o[j];
+            for (int j = 0; j < DBW; j++)
+              *(h4*)((_Float16*)p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = (h4){ (_Float16)o[j][0], (_Float16)o[j][1], (_Float16)o[j][2], (_Float16)o[j][3] };
+          } else {
+#pragma unroll
+            for (int j = 0; j < DBW; j++) *(f4*)(p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = o[j];
+          }
           if (wave == 0 && kg == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(M, Lr);
         }
         TR(11);                       // partial stored
@@ -1014,7 +1025,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 // the output partials of its group's splits (group + 16 k) in one round trip, the maximum and the sums over the 16
 // groups are xor-shuffle trees (fixed order), lanes 0 .. 3 finish and store.  The four lanes of a group hold the same
 // (m, l), so each computes its splits' weights itself instead of fetching them from a neighbour.
-template <int HD, int DS>
+template <int HD, int DS, bool PF16>
 __global__ __launch_bounds__(64)
 void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint32_t a_slots, uint32_t a_n_heads, uint32_t a_base_pos, uint32_t a_self_row,
                             uint32_t a_split_len, uint32_t a_n_splits, uint32_t a_grid_x, uint32_t a_has_sel, AttnParams p_in) {
@@ -1035,15 +1046,25 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
   const uint32_t grp = lane / LPG, l4 = lane % LPG;
   const float* po = p.part_o + base * HD + dq * DS + 4 * l4;
+  const _Float16* po16 = (const _Float16*)p.part_o + base * HD + dq * DS + 4 * l4;       // PF16: f16 partial rows
   const float2* pml = (const float2*)p.part_ml + base;
   const f4 zero = {0.f, 0.f, 0.f, 0.f};
-  f4 ov[CH];
+  // the partial rows stay as loaded (f16 rows as two dwords) until they are used: a conversion at the load would make
+  // every load wait for its own data
+  typedef typename std::conditional<PF16, h4, f4>::type orow;
+  const orow zrow = {0, 0, 0, 0};
+  auto load_o = [&](uint32_t s) __attribute__((always_inline)) -> orow {
+    if constexpr (PF16) return *(const h4*)(po16 + (size_t)s * HD);
+    else return *(const f4*)(po + (size_t)s * HD);
+  };
+  auto wide = [&](const orow v) __attribute__((always_inline)) -> f4 { return (f4){ (float)v[0], (float)v[1], (float)v[2], (float)v[3] }; };
+  orow ov[CH];
   float2 mlv[CH];
 #pragma unroll
   for (int k = 0; k < CH; k++) {
     const uint32_t s = grp + NG * k;
     mlv[k] = s < ns ? pml[s] : make_float2(NEG_INF, 0.f);
-    ov[k] = s < ns ? *(const f4*)(po + (size_t)s * HD) : zero;
+    ov[k] = s < ns ? load_o(s) : zrow;
   }
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("" :: "s"(p.gate), "s"(p.out), "s"(p.gate_stride), "s"(p.out_stride), "s"(p.out_f16), "s"(p.gate_head_stride));
@@ -1066,20 +1087,20 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
   for (int k = 0; k < CH; k++) {
     const float w = __expf(mlv[k].x - M);        // -inf for a split past the column's end: weight 0
     L += mlv[k].y * w;
-    o += ov[k] * w;
+    o += wide(ov[k]) * w;
   }
   for (uint32_t s0 = NG * CH; s0 < ns; s0 += NG * CH) {
 #pragma unroll
     for (int k = 0; k < CH; k++) {
       const uint32_t s = s0 + grp + NG * k;
       mlv[k] = s < ns ? pml[s] : make_float2(NEG_INF, 0.f);
-      ov[k] = s < ns ? *(const f4*)(po + (size_t)s * HD) : zero;
+      ov[k] = s < ns ? load_o(s) : zrow;
     }
 #pragma unroll
     for (int k = 0; k < CH; k++) {
       const float w = __expf(mlv[k].x - M);
       L += mlv[k].y * w;
-      o += ov[k] * w;
+      o += wide(ov[k]) * w;
     }
   }
   if constexpr (LPG == 4) {
@@ -1297,10 +1318,11 @@ hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s) {
     return hipGetLastError();
   }
   const uint32_t gx = p.n_heads * (hd / 16), has_sel = p.sel != nullptr;
-  if (hd == 256) hipLaunchKernelGGL((pa_combine_wave_kernel<256, 16>), dim3(gx, p.n_cols), dim3(64), 0, s, (const float*)p.part_o, (const float*)p.part_ml,
-                                    p.slots, p.n_heads, p.base_pos, p.self_row, p.split_len, p.n_splits, gx, has_sel, p);
-  else if (hd == 128) hipLaunchKernelGGL((pa_combine_wave_kernel<128, 16>), dim3(gx, p.n_cols), dim3(64), 0, s, (const float*)p.part_o, (const float*)p.part_ml,
-                                         p.slots, p.n_heads, p.base_pos, p.self_row, p.split_len, p.n_splits, gx, has_sel, p);
-  else return hipErrorInvalidValue;
+  if (hd != 256 && hd != 128) return hipErrorInvalidValue;
+#define PA_COMBINE_WAVE(HD_, F16_) hipLaunchKernelGGL((pa_combine_wave_kernel<HD_, 16, F16_>), dim3(gx, p.n_cols), dim3(64), 0, s, (const float*)p.part_o, \
+    (const float*)p.part_ml, p.slots, p.n_heads, p.base_pos, p.self_row, p.split_len, p.n_splits, gx, has_sel, p)
+  if (hd == 256) { if (p.part_f16) PA_COMBINE_WAVE(256, true); else PA_COMBINE_WAVE(256, false); }
+  else { if (p.part_f16) PA_COMBINE_WAVE(128, true); else PA_COMBINE_WAVE(128, false); }
+#undef PA_COMBINE_WAVE
   return hipGetLastError();
 }

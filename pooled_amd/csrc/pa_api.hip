@@ -314,6 +314,15 @@ extern "C" int pa_kv_store(pa_ctx* ctx, uint32_t layer, const float* d_k, uint32
 // self_ok: a one-column decode keeps the column's own row out of the streamed rows (the kernel turns it
 // into one more partial: slots = n_splits + 1), so a token at a multiple of the split length streams whole tiles only.
 static bool plan_self_row(const pa_plan& pl) { return pl.kernel == 0 && pl.slots == pl.n_splits + 1; }
+// f16 O partials: the single-round split-K kernel (one row block, one tile per wave) merged by the wavefront kernel
+// (pa_launch_combine takes the other merge kernel from 16 columns on), from 64 splits on: each partial's rounding
+// (2^-12 of a 128-row average of V) then enters the output with a weight of a sixty-fourth or less, an order of
+// magnitude under what the f16 probabilities of the MFMA path already cost; shorter contexts, where a partial IS most
+// of the output, and every other pass keep f32 partials.
+#define PA_F16_PARTIALS_MIN_SPLITS 64u
+static bool plan_f16_partials(const pa_plan& pl, uint32_t n_cols) {
+  return pl.kernel == 0 && pl.row_blocks == 1 && pl.split_len == 32 * pl.waves && n_cols < 16 && pl.n_splits >= PA_F16_PARTIALS_MIN_SPLITS;
+}
 // wgs (optional): splits per kv head and column group that fit the chip at once; the single-round kernel dispatches
 // the workgroups of further splits (a short remainder) last.
 // rows_cap (optional): at most this many stacked rows per workgroup (16 or 32) instead of the table's choice;
@@ -547,6 +556,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
   p.self_row = plan_self_row(pl) ? 1 : 0;
   p.direct_out = direct && pl.kernel == 0 ? 1 : 0;
+  p.part_f16 = !direct && plan_f16_partials(pl, n_cols);
   p.n_wgs = pl.kernel == 0 ? n_wgs : 0;
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
@@ -609,7 +619,7 @@ static int decode_step_common(pa_ctx* ctx, const char* who, bool static_scratch,
   p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
   p.base_pos = pos; p.n_cols = 1;
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
-  p.self_row = 1; p.n_wgs = n_wgs;
+  p.self_row = 1; p.n_wgs = n_wgs; p.part_f16 = plan_f16_partials(pl, 1);
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   // the pre-step inputs; the gate is read in place from the interleaved [q | gate] heads
@@ -906,6 +916,7 @@ extern "C" int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   p.gate_head_stride = c.head_dim;
   p.sel = d_sel; p.sel_stride = sel_stride; p.sel_max = std::min(max_rows, sel_stride - 1); p.n_wgs = n_wgs;
+  p.part_f16 = pl.split_len == 32 * 4 && n_cols < 16 && pl.n_splits >= PA_F16_PARTIALS_MIN_SPLITS;   // (as plan_f16_partials)
   PaTiming tm;
   if ((rc = prof_pair(ctx, &tm))) return rc;
   HIPCHK(ctx, pa_launch_decode_gather(p, c.head_dim, ctx->stream, &tm));

@@ -49,6 +49,8 @@ struct AttnParams {
   float scale;                                // 1 / sqrt(hd)
   uint32_t gate_head_stride;                  // floats between consecutive heads in gate (head_dim, or 2*head_dim
                                               // when gate is read in place from an interleaved [q | gate] column)
+  uint32_t part_f16;                          // 1: the O partials in part_o are f16 rows [slot][hd] (single-round decode splits
+                                              // merged by the wavefront kernel); 0: f32
   // fused pre-step of pa_attn_decode_step (one column at base_pos; f_q_in == nullptr otherwise): raw projections
   const float* f_q_in; const float* f_k_in; const float* f_v_in;   // [nH][q_head_stride], [nKV][hd], [nKV][hd]
   const float* f_qw; const float* f_kw;       // norm weights [hd] or nullptr
