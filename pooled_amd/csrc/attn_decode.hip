@@ -89,14 +89,18 @@ template <int N>
 static __device__ inline float row_ror(float v) {
   return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x120 + N, 0xf, 0xf, false));
 }
-// maximum / sum over the 16 lanes {(i & 3) + 4 k}: two rotations inside the row, then the four rows.  The sum's
+// maximum / sum over the 16 lanes {(i & 3) + 4 k} (LPG == 4; LPG == 8: the 8 lanes {(i & 7) + 8 k}): rotations inside the row, then the four rows.  The sum's
 // association differs from lane to lane (lane i starts at its own element); lanes 0 .. 3 are the ones that are read.
+template <int LPG = 4>
 static __device__ inline float quads_max(float v) {
-  v = fmaxf(v, row_ror<4>(v)); v = fmaxf(v, row_ror<8>(v));
+  if constexpr (LPG == 4) v = fmaxf(v, row_ror<4>(v));
+  v = fmaxf(v, row_ror<8>(v));
   return rows_max(v);
 }
+template <int LPG = 4>
 static __device__ inline float quads_sum(float v) {
-  v += row_ror<4>(v); v += row_ror<8>(v);
+  if constexpr (LPG == 4) v += row_ror<4>(v);
+  v += row_ror<8>(v);
   return rows_sum(v);
 }
 
@@ -1076,7 +1080,7 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
   for (int k = 0; k < CH; k++) M = fmaxf(M, mlv[k].x);
   for (uint32_t s = grp + NG * CH; s < ns; s += NG) M = fmaxf(M, pml[s].x);        // more than 272 splits
   // over the 16 split groups: on the VALU (row rotations + lane swaps) with four lanes a group, else through the LDS crossbar
-  if constexpr (LPG == 4) M = quads_max(M);
+  if constexpr (LPG == 4 || LPG == 8) M = quads_max<LPG>(M);
   else {
 #pragma unroll
     for (int o = LPG; o < 64; o <<= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
@@ -1103,10 +1107,10 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
       o += wide(ov[k]) * w;
     }
   }
-  if constexpr (LPG == 4) {
-    L = quads_sum(L);
+  if constexpr (LPG == 4 || LPG == 8) {
+    L = quads_sum<LPG>(L);
 #pragma unroll
-    for (int i = 0; i < 4; i++) o[i] = quads_sum(o[i]);
+    for (int i = 0; i < 4; i++) o[i] = quads_sum<LPG>(o[i]);
   } else {
 #pragma unroll
     for (int x = LPG; x < 64; x <<= 1) {
