@@ -163,7 +163,7 @@ def median(xs):
     return xs[len(xs) // 2]
 
 
-def prefill_leg(steps, with_cpu, kv_q8=False, clk=False):
+def prefill_leg(steps, with_cpu, kv_q8=False):
     """Configuration 5: a 4096-token causal chunk at positions 126976-131071 over a 126976-token f16 prefix,
     Qwen3.6-35B-MoE attention shape, sigmoid gate, f16 output.  A step = pre-step for the 4096 columns
     (QK-RMSNorm + partial RoPE + KV write) + the MFMA prefill kernel.  PREFILL_WARMUP untimed steps (the first one's
@@ -192,13 +192,6 @@ def prefill_leg(steps, with_cpu, kv_q8=False, clk=False):
         pa.timer_start(); step()
         return pa.timer_stop()                       # blocks until the step has finished
 
-    clk_buf = None
-    if clk:                                          # ablation builds: wave 0 of every workgroup reports shader cycles and 100 MHz ticks
-        import ctypes
-        pa.L.pa_pf_clk_set.restype = ctypes.c_int; pa.L.pa_pf_clk_set.argtypes = [ctypes.c_void_p]
-        clk_buf = pa.alloc(4096 * 16)
-        if pa.L.pa_pf_clk_set(clk_buf.ptr) != 0:
-            raise RuntimeError("pa_pf_clk_set failed")
     pa.sync()
     cold_first_ms = timed_step()
     for _ in range(PREFILL_WARMUP - 1):
@@ -209,11 +202,6 @@ def prefill_leg(steps, with_cpu, kv_q8=False, clk=False):
     pa.profile_enable(False)
     ms_step, k_ms = median(step_ms), median(kern_ms)
     k_mean = sum(kern_ms) / max(len(kern_ms), 1)
-    clk_mhz = None
-    if clk_buf is not None:
-        cw = clk_buf.download(np.uint64, 2 * 256).reshape(256, 2).astype(np.float64)       # the last launch's 256 workgroups
-        clk_mhz = float(np.median(cw[:, 0] / np.maximum(cw[:, 1], 1.0) * 100.0))
-        pa.L.pa_pf_clk_set(None)
     flops = causal_flops(cfg, base, n)
     tf_step, tf_kernel = flops / (ms_step * 1e-3) / 1e12, flops / (k_ms * 1e-3) / 1e12
     log("prefill C5: first launch %.3f ms; median of %d steps %.3f ms (min %.3f, max %.3f) -> %.1f TFLOP/s; kernel median %.3f ms (mean %.3f) -> %.1f TFLOP/s (%.1f%% of f16 MFMA peak)"
@@ -222,7 +210,7 @@ def prefill_leg(steps, with_cpu, kv_q8=False, clk=False):
                         "every tensor an independent N(0,1) stream" % ("int8 (widened once per chunk into an f16 staging cache, inside the step)" if kv_q8 else "f16"),
                value=round(tf_step, 1), unit="TFLOP/s", ms_per_step=round(ms_step, 4), steps=steps, warmup=PREFILL_WARMUP, reported="median of the timed steps",
                min_ms_per_step=round(min(step_ms), 4), max_ms_per_step=round(max(step_ms), 4), cold_first_ms=round(cold_first_ms, 4),
-               step_ms=[round(x, 3) for x in step_ms], flops_per_step=flops, plan=pa.plan("prefill", base, n), shader_clock_mhz=clk_mhz,
+               step_ms=[round(x, 3) for x in step_ms], flops_per_step=flops, plan=pa.plan("prefill", base, n),
                roofline=dict(bound="mfma", achieved=round(tf_kernel, 1), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s", frac=round(tf_kernel / MFMA_F16_PEAK_TFLOPS, 4),
                              traffic=None, kernel="pa_prefill_kernel<256, 1, 8>", kernel_ms=round(k_ms, 4), kernel_ms_mean=round(k_mean, 4),
                              kernel_ms_min=round(min(kern_ms), 4), kernel_ms_max=round(max(kern_ms), 4), reported="median launch",
@@ -399,107 +387,6 @@ def layer_leg(pa, cfg, ctx, steps, warmup, attn_ms, n_rot, rng):
                                   us_per_step=round(t_verify * 1e3, 2), us_per_token=round(t_verify * 1e3 / nv, 2)))
 
 
-def stream_ceiling(pa, rotation, step, reps, events=True):
-    """What a one-shot 64 MiB read reaches on this part with the decode kernel's launch shape: every read-only stand-in
-    of the library (pa_probe_stream), the empty kernel of the same grid and the decode step's own split-K kernel, each
-    timed by dispatch-stamped events over `rotation` layers' caches, launches back to back.  events=False: plain
-    launches only (for a run under rocprofv3 --kernel-trace, whose own timestamps then time undisturbed launches)."""
-    L = pa.L
-    sink = pa.alloc(8 << 20)
-    ptrs = [(L.pa_kv_device_ptr(pa.ctx, l, 0), L.pa_kv_device_ptr(pa.ctx, l, 1)) for l in range(rotation)]
-    rows = []
-
-    def stats(ms):
-        us = sorted(x * 1e3 for x in ms)
-        return dict(launches=len(us), median_us=round(us[len(us) // 2], 2), mean_us=round(sum(us) / len(us), 2), min_us=round(us[0], 2), p90_us=round(us[len(us) * 9 // 10], 2))
-    if not events:
-        for v in range(L.pa_probe_count()):
-            for i in range(reps + 2 * rotation):
-                pa._chk(L.pa_probe_stream(pa.ctx, v, ptrs[i % rotation][0], ptrs[i % rotation][1], sink.ptr))
-            pa.sync()
-        for i in range(reps + 2 * rotation):
-            step(i, rotation)
-        pa.sync()
-        return None
-    for v in range(L.pa_probe_count()):
-        for i in range(2 * rotation):
-            pa._chk(L.pa_probe_stream(pa.ctx, v, ptrs[i % rotation][0], ptrs[i % rotation][1], sink.ptr))
-        pa.sync()
-        pa.profile_enable(True)
-        for i in range(reps):
-            pa._chk(L.pa_probe_stream(pa.ctx, v, ptrs[i % rotation][0], ptrs[i % rotation][1], sink.ptr))
-        st = stats(pa.profile_read_each())
-        pa.profile_enable(False)
-        st["variant"] = L.pa_probe_name(v).decode()
-        st["gbs_at_median"] = None if v == 0 else round((64 << 20) / st["median_us"] / 1e3, 1)
-        rows.append(st)
-        log("  [%2d layers] %-90s median %6.2f us  mean %6.2f  min %6.2f" % (rotation, st["variant"], st["median_us"], st["mean_us"], st["min_us"]))
-    for i in range(2 * rotation):
-        step(i, rotation)
-    pa.sync()
-    pa.profile_enable(True)
-    for i in range(reps):
-        step(i, rotation)
-    st = stats(pa.profile_read_each())
-    pa.profile_enable(False)
-    st["variant"] = "the decode step's split-K kernel itself (pa_decode_kernel, fused pre-step, 67.1 MB of K/V)"
-    st["gbs_at_median"] = round(2 * (C3_CTX + 1) * 512 * 2 / st["median_us"] / 1e3, 1)
-    rows.append(st)
-    log("  [%2d layers] %-90s median %6.2f us  mean %6.2f  min %6.2f" % (rotation, st["variant"], st["median_us"], st["mean_us"], st["min_us"]))
-    return rows
-
-
-def timeline(pa, step, n_rot, iters=24):
-    """In-kernel timeline of the decode step's split-K kernel (trace build of the library: python -m pooled_amd.build
-    --trace): per phase boundary, when the waves pass it -- relative to the first wave entering on the same XCC (the
-    XCCs start a dispatch up to 1.5 us apart) -- and how long each phase takes a wave.  Launches back to back; every
-    sixth launch is read out."""
-    import ctypes
-    L = pa.L
-    L.pa_trace_set.restype = ctypes.c_int; L.pa_trace_set.argtypes = [ctypes.c_void_p]
-    NW, NST = 512 * 4, 16
-    tr = pa.alloc(NW * NST * 8)
-    for i in range(60):
-        step(i, n_rot)
-    pa.sync()
-    if L.pa_trace_set(tr.ptr) != 0:
-        raise RuntimeError("pa_trace_set failed")
-    names = ["entry", "kernel arguments read", "raw q / weights loads issued", "K tile loads issued", "pre-step done, q rows staged", "barrier 1 passed", "K tile arrived and staged",
-             "scores done", "softmax done", "V tile loads issued", "V tile arrived and staged", "barrier 2 passed", "partial stored"]
-    rel_all, span, span_x, clk = [], [], [], []
-    for it in range(iters):
-        for j in range(6):
-            step(it * 6 + j, n_rot)
-        pa.sync()
-        t = tr.download(np.uint64, NW * NST).reshape(NW, NST)
-        ts = t[:, [0, 12, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11]].astype(np.int64)
-        xcc = t[:, 14].astype(np.int64)
-        rel = np.zeros(ts.shape, np.float64)
-        for x in range(8):
-            m = xcc == x
-            rel[m] = (ts[m] - ts[m, 0].min()) / 100.0
-        rel_all.append(rel)
-        span.append((ts[:, 12].max() - ts[:, 0].min()) / 100.0)
-        span_x.append(rel[:, 12].max())
-        clk.append(np.median(t[:, 13].astype(np.float64) / np.maximum((ts[:, 12] - ts[:, 0]) / 100.0, 1e-3)))
-    L.pa_trace_set(None)
-    a = np.stack(rel_all[4:])
-    res = dict(launches_read=len(rel_all) - 4, shader_clock_mhz=round(float(np.median(clk[4:]))), span_first_entry_to_last_store_us=round(float(np.median(span[4:])), 2),
-               span_per_xcc_us=round(float(np.median(span_x[4:])), 2), stamps=[], phases=[])
-    log("shader clock %d MHz; first entry -> last store %.2f us (per XCC %.2f us)" % (res["shader_clock_mhz"], res["span_first_entry_to_last_store_us"], res["span_per_xcc_us"]))
-    log("%-32s %7s %7s %7s %7s %7s" % ("when waves pass (us)", "min", "p10", "p50", "p90", "max"))
-    for s_, n in enumerate(names):
-        q = np.percentile(a[:, :, s_], [0, 10, 50, 90, 100], axis=1).mean(1)
-        res["stamps"].append(dict(stamp=n, min=round(q[0], 2), p10=round(q[1], 2), p50=round(q[2], 2), p90=round(q[3], 2), max=round(q[4], 2)))
-        log("%-32s %7.2f %7.2f %7.2f %7.2f %7.2f" % (n, *q))
-    log("%-66s %7s %7s" % ("phase of a wave (us)", "median", "p90"))
-    for s_ in range(1, len(names)):
-        d = a[:, :, s_] - a[:, :, s_ - 1]
-        res["phases"].append(dict(phase="%s -> %s" % (names[s_ - 1], names[s_]), median=round(float(np.median(d)), 2), p90=round(float(np.percentile(d, 90)), 2)))
-        log("%-66s %7.2f %7.2f" % (res["phases"][-1]["phase"], res["phases"][-1]["median"], res["phases"][-1]["p90"]))
-    return res
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -515,46 +402,11 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 10 device-to-device copies of 256 MiB (the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--rotation", type=int, default=0, help="time the decode step with this many layers' caches in rotation only (default: sweep %s)" % (ROTATIONS,))
-    ap.add_argument("--stream-ceiling", action="store_true",
-                    help="only time the read-only stand-ins of the decode kernel's K/V stream, the empty kernel of its grid and the kernel itself (events; run under rocprofv3 --kernel-trace for the trace's clock)")
-    ap.add_argument("--prefill-ablation", action="store_true",
-                    help="only time the C5 prefill kernel with parts of its step removed (timing-only builds: python -m pooled_amd.build --prefill-ablation), "
-                         "each build in a process of its own, two interleaved rounds")
-    ap.add_argument("--prefill-ablation-child", type=int, default=-1, help=argparse.SUPPRESS)
-    ap.add_argument("--timeline", action="store_true", help="only print the in-kernel timeline of the decode step's split-K kernel (needs the trace build: python -m pooled_amd.build --trace)")
-    ap.add_argument("--no-events", action="store_true", help="with --stream-ceiling: plain launches, no event pairs (for a run under a kernel trace)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
-    if args.prefill_ablation:
-        import subprocess
-        from pooled_amd import build as pa_build
-        rounds = []
-        for rnd in range(2):
-            row = {}
-            for mask, label in pa_build.PREFILL_ABLATIONS:
-                out = subprocess.run([sys.executable, os.path.abspath(__file__), "--prefill-ablation-child", str(mask), "--prefill-steps", str(args.prefill_steps)],
-                                     stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=600, check=True).stdout
-                row[mask] = json.loads(out.strip().splitlines()[-1])
-                log("round %d  removed: %-62s kernel median %.3f ms  shader clock %4.0f MHz" % (rnd + 1, label, row[mask]["kernel_ms"], row[mask]["shader_clock_mhz"]))
-            rounds.append(row)
-        full = [r[0]["kernel_ms"] for r in rounds]
-        table = [dict(mask=mask, removed=label, kernel_ms=[r[mask]["kernel_ms"] for r in rounds], shader_clock_mhz=[round(r[mask]["shader_clock_mhz"]) for r in rounds],
-                      vs_full_pct=[round(100 * (r[mask]["kernel_ms"] / f - 1), 1) for r, f in zip(rounds, full)],
-                      tflops=[round(rounds[0][0]["flops"] / (r[mask]["kernel_ms"] * 1e-3) / 1e12, 1) for r in rounds]) for mask, label in pa_build.PREFILL_ABLATIONS]
-        print(json.dumps({"prefill_ablation": table}))
-        return
-    if args.prefill_ablation_child >= 0:
-        from pooled_amd import capi, build as pa_build
-        capi.LIB_PATH = pa_build.ablation_lib(args.prefill_ablation_child)
-        r = prefill_leg(args.prefill_steps, False, clk=True)
-        print(json.dumps(dict(kernel_ms=r["roofline"]["kernel_ms"], shader_clock_mhz=r["shader_clock_mhz"], flops=r["flops_per_step"])))
-        return
-    if args.timeline:
-        from pooled_amd import capi, build as pa_build
-        capi.LIB_PATH = pa_build.TRACE_LIB
     from pooled_amd.capi import PooledAttn, PA_OUT_F16, load
     L = load()
     log("library:", L.pa_version().decode())
@@ -601,20 +453,6 @@ def main():
             pa.attn("decode", layer, None, 0, gate_ptr, qd, ctx, 1, d_out, qd, PA_OUT_F16)
         else:
             pa.attn_decode_step(layer, d_qfull, d_k, d_v, d_qw, d_kw, ctx, d_out, PA_OUT_F16)
-
-    if args.timeline:
-        res = timeline(pa, step, rotations[0])
-        pa.close()
-        print(json.dumps({"timeline": res, "layers_in_rotation": rotations[0], "library": L.pa_version().decode()}))
-        return
-    if args.stream_ceiling:
-        res = {}
-        for r in rotations:
-            log("stream ceiling, %d layers' caches in rotation (%.0f MiB):" % (r, r * 2 * ctx * kvd * 2 / 2**20))
-            res[str(r)] = stream_ceiling(pa, r, step, max(args.steps, 240), not args.no_events)
-        pa.close()
-        print(json.dumps({"stream_ceiling": res, "library": L.pa_version().decode()}))
-        return
 
     kv_bytes = 2 * (ctx + 1) * kvd * 2            # K and V rows [0, 32768], f16
     if args.kv_q8:

@@ -317,14 +317,6 @@ int pa_set_weight_cache(pa_ctx* ctx, size_t max_bytes);
 int pa_attn_layer_prefill(pa_ctx* ctx, uint32_t layer, const pa_weight* w_qkv, const pa_weight* w_o, const float* d_attn_norm_w,
                           const float* d_qw, const float* d_kw, float* d_x, uint32_t x_stride, uint32_t base_pos, uint32_t n_cols);
 
-/* Measurement stand-ins of the one-column decode kernel's K/V stream (bench.py --stream-ceiling; no counterpart in the
- * reference): launch stand-in `variant` (0 .. pa_probe_count() - 1, described by pa_probe_name) on the context's stream
- * over 32 MiB at d_k and 32 MiB at d_v; d_sink is 8 MiB of device scratch.  Timed by pa_profile_enable /
- * pa_profile_read_each like an attention call's main kernel. */
-int pa_probe_count(void);
-const char* pa_probe_name(int variant);
-int pa_probe_stream(pa_ctx* ctx, int variant, const void* d_k, const void* d_v, void* d_sink);
-
 /* library / device description, e.g. "pooled_attn 0.1 gfx950 256CU" (storage owned by the library, one buffer per
  * calling thread) */
 const char* pa_version(void);

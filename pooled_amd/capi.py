@@ -81,9 +81,6 @@ SYMBOLS = {
     "pa_rmsnorm_f16": (c_int, [vp, f32p, u32, f32p, u32, u32, vp, u32]),
     "pa_gemm": (c_int, [vp, vp, vp, u32, u32, f32p, u32, c_int]),
     "pa_attn_layer_prefill": (c_int, [vp, u32, vp, vp, f32p, f32p, f32p, f32p, u32, u32, u32]),
-    "pa_probe_count": (c_int, []),
-    "pa_probe_name": (ctypes.c_char_p, [c_int]),
-    "pa_probe_stream": (c_int, [vp, c_int, vp, vp, vp]),
     "pa_version": (ctypes.c_char_p, []),
 }
 

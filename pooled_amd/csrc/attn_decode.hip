@@ -32,25 +32,6 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 
 #define TILE 32
 
-// Development timeline (compiled with -DPA_TRACE only: bench.py --timeline): lane 0 of every wave of the single-round kernel
-// stamps the 100 MHz wall clock at the phase boundaries below and writes the stamps, its XCC id and the shader cycles it
-// ran to the buffer pa_trace_set names.  Without PA_TRACE the macros are empty and the kernels are unchanged.
-#ifdef PA_TRACE
-#define PA_TRACE_STAMPS 16
-__device__ unsigned long long* g_pa_trace = nullptr;
-extern "C" int pa_trace_set(void* d_buf) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_pa_trace), &d_buf, sizeof(d_buf)); }
-#define TR_DECL unsigned long long trs[PA_TRACE_STAMPS] = {0}; const unsigned long long trs_clk0 = clock64()
-#define TR(i) do { if (SR) { __builtin_amdgcn_sched_barrier(0); trs[i] = wall_clock64(); __builtin_amdgcn_sched_barrier(0); } } while (0)
-#define TR_FLUSH(W_) do { if (SR && g_pa_trace && lane == 0) {                                                                \
-    unsigned long long* t_ = g_pa_trace + ((size_t)(blockIdx.x + gridDim.x * blockIdx.y) * (W_) + wave) * PA_TRACE_STAMPS;     \
-    for (int i_ = 0; i_ < 13; i_++) t_[i_] = trs[i_];                                                                         \
-    unsigned xcc_; asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_));                                        \
-    t_[13] = clock64() - trs_clk0; t_[14] = xcc_ & 0xf; t_[15] = wall_clock64(); } } while (0)
-#else
-#define TR_DECL do {} while (0)
-#define TR(i) do {} while (0)
-#define TR_FLUSH(W_) do {} while (0)
-#endif
 #define NEG_INF (-__builtin_inff())
 #define DEC_RESCALE_TH 8.f   // tile loop: a row maximum may pass the reference maximum by this much before O is rescaled
 
@@ -219,12 +200,6 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
   static_assert(!Q8 || !GATHER, "int8 caches: no gather mode");
   typedef DecShape<HD> S;
-  TR_DECL;
-  TR(0);                              // entry
-#ifdef PA_TRACE
-  { const void* ka_ = p.k_cache; const uint32_t kb_ = p.base_pos; asm volatile("s_waitcnt lgkmcnt(0)" :: "s"(ka_), "s"(kb_)); }
-  TR(12);                             // kernel arguments read
-#endif
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char* q_lds = smem;                                       // [16*NB][QROW]
   unsigned char* stage_all = smem + 16 * NB * S::QROW;               // [W][STAGE]
@@ -424,7 +399,6 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       qv[j] = *(const f4*)(p.q + (size_t)(c0 + rc / G) * p.q_stride + (size_t)(g * G + rc % G) * HD + 4 * d4);
     }
   }
-  TR(1);                              // q / raw projection loads issued
   // Loads are unconditional: the caches carry TILE rows of padding past max_seq, so a tile that straddles the
   // end of the context reads valid memory; rows at or past t_end are zeroed (V) or masked (scores) below.
   // A wave with no tile of its own (short splits) loads the split's last tile and discards it: the prologue
@@ -476,7 +450,6 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   // the very end of the kernel.  Scored first, that work runs while other waves keep the pipeline full, and what follows
   // the last V load is the V latency, the staging of V and the PV product.  Measured on the 32K decode step: 18.6 -> 18.15 us.
   constexpr bool V_LATE = SR && !GATHER;
-  TR(2);                              // K tile loads issued
   if constexpr (!FUSED && !V_LATE) first_v_loads();
   __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the load issue
   // ---- q -> f16 rows in LDS; waits only for the q loads, which were issued first ----
@@ -536,7 +509,6 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
     }
   }
-  TR(3);                              // pre-step done (fused), q rows staged
   if constexpr (FUSED && !V_LATE) {
     __builtin_amdgcn_sched_barrier(0);
     first_v_loads();
@@ -550,7 +522,6 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
     end_pos[nb] = r < R ? (GATHER ? seq_max : p.base_pos + c0 + r / G + 1 - p.self_row) : 0u;
   }
   __syncthreads();
-  TR(4);                              // barrier 1 passed
   // ---- the column's own row as a partial of its own (slot = number of splits that hold rows): m = its score,
   // l = 1, O = its value row.  The scores run on the VALU over the f16 operands the MFMA path would see, f32 sums in a
   // fixed order; the work hides under the latency of the tile loads.  Decoding a token at a position that is a
@@ -712,10 +683,8 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       const bool has_tile = wave < n_tiles;
       const uint32_t tp = t_begin + min(wave, n_tiles - 1) * TILE;      // the tile this wave holds in registers
       stage_k(tp, false, 0);
-      TR(5);                          // K tile arrived and staged
       f4 s[2][NB];
       qk(s);
-      TR(6);                          // scores done
       const uint32_t row_end = has_tile ? end_pos[0] : 0u;              // a wave without a tile contributes nothing
       float v[8], mx = NEG_INF;
 #pragma unroll
@@ -734,15 +703,11 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
       for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
       ps = rows_sum(ps);
-      TR(7);                          // softmax done
       if constexpr (V_LATE) { __builtin_amdgcn_sched_barrier(0); first_v_loads(); __builtin_amdgcn_sched_barrier(0); }
-      TR(8);                          // V tile loads issued
       stage_v(ILV && ilv ? 0u : tp, false, 0);                          // interleaved splits are whole: no row past the end to zero
       *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pf;
       if (kg == 0) { mex[wave * 16 + ln] = mx; lex[wave * 16 + ln] = ps; }
-      TR(9);                          // V tile arrived and staged, P published
       __syncthreads();
-      TR(10);                         // barrier 2 passed
       {
         // V^T fragments (two transpose reads each) and the tile's P are fetched VD steps ahead of their MFMA
         // (a tile's P is read once, not once per 16-dim block: the tail of the kernel is bound by the LDS port)
@@ -808,8 +773,6 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
           }
           if (wave == 0 && kg == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(M, Lr);
         }
-        TR(11);                       // partial stored
-        TR_FLUSH(W);
       }
     }
     return;

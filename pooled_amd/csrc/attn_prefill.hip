@@ -30,31 +30,16 @@
 //     (m, l, O) go to the same buffers the decode kernel uses and the same merge kernel finishes them.
 #include "pf_common.h"
 
-// Timing-only ablations of the step (python -m pooled_amd.build --prefill-ablation, bench.py --prefill-ablation): PF_ABL is a
-// mask of what is REMOVED from every step -- the results are wrong on purpose.  1: the exponentials (argument passed
-// through), 2: K fragment reads (the first one reused), 4: V^T fragment reads, 8: the whole softmax (scores converted
-// straight to f16), 16: the LDS-direct tile loads after the first.  An ablation build (PF_ABL defined, 0 included) also
-// reports the shader clock: wave 0 of every workgroup writes its shader cycles and 100 MHz ticks to the buffer
-// pa_pf_clk_set names.
-#ifdef PF_ABL
-__device__ unsigned long long* g_pf_clk = nullptr;
-extern "C" int pa_pf_clk_set(void* d_buf) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_pf_clk), &d_buf, sizeof(d_buf)); }
-#define PF_ABLATED(bit) ((PF_ABL) & (bit))
-#else
-#define PF_ABLATED(bit) 0
-#endif
-
 template <int HD, int W> struct PfShape {
   static constexpr int ROWB = HD * 2;             // bytes of one kv head's row
-  static constexpr int TILE = PF_STEP * ROWB;     // bytes of one staged step (K or V)
-  static constexpr int SUBT = PF_TN * ROWB;       // bytes of one 32-position tile of it
+  static constexpr int TILE = PF_TN * ROWB;       // bytes of one staged tile (K or V)
   static constexpr int KS = HD / 16;              // k-steps of QK^T
   static constexpr int DB = HD / 32;              // 32-dim blocks of the output
   static constexpr int QR = HD == 256 ? PF_QR : KS;   // k-steps whose Q fragments stay in registers
   static constexpr int CPR = HD / 8;              // 16-byte chunks per row
   static constexpr int RPB = 64 / CPR;            // rows per 1 KB LDS-direct load
-  static constexpr int NLD = PF_STEP / RPB / W;   // LDS-direct loads per wave, tensor and step
-  static_assert(NLD >= 1 && NLD * W * RPB == PF_STEP, "tile must divide evenly over the waves");
+  static constexpr int NLD = PF_TN / RPB / W;   // LDS-direct loads per wave, tensor and step
+  static_assert(NLD >= 1 && NLD * W * RPB == PF_TN, "tile must divide evenly over the waves");
 };
 
 template <int HD, int QB, int W>
@@ -72,9 +57,6 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   // the same K/V rows.  The grid is one-dimensional; dispatch id i runs on XCD i % 8, and XCD k owns the contiguous
   // item range [k per_xcd, (k + 1) per_xcd): every XCD gets the same number of workgroups whatever the split count,
   // and the workgroups that share a K/V stream share an L2.
-#ifdef PF_ABL
-  const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
-#endif
   const uint32_t total = n_col_blocks * p.n_kv_heads * p.n_splits;
   const uint32_t per_xcd = (total + 7) / 8;
   const uint32_t lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
@@ -92,7 +74,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   const uint32_t t_begin = sp * p.split_len;
   if (t_begin >= seq_max) return;
   const uint32_t t_end = min(t_begin + p.split_len, seq_max);
-  const uint32_t n_steps = (t_end - t_begin + PF_STEP - 1) / PF_STEP;
+  const uint32_t n_steps = (t_end - t_begin + PF_TN - 1) / PF_TN;
   const size_t row_bytes = (size_t)HD * 2;                       // head-major caches: a kv head's rows are contiguous
   const size_t head_rows = (size_t)p.max_seq + PF_TN;            // rows of one kv head's plane, padding included
   const unsigned char* kg_base = (const unsigned char*)(p.k_cache + (size_t)g * head_rows * HD);
@@ -111,7 +93,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   // rows at or past t_end (only in the last tile of the context) come from the zero padding row max_seq
   auto issue_t = [&](const unsigned char* g_base, const uint32_t off, unsigned char* dst, uint32_t tpos) {
     const unsigned char* t0p = g_base + (size_t)tpos * row_bytes;
-    if (tpos + PF_STEP <= t_end) {
+    if (tpos + PF_TN <= t_end) {
 #pragma unroll
       for (int i = 0; i < S::NLD; i++) PF_GLL_S(t0p + i * LD_STRIDE, off, dst + (i * W + wave) * 1024);
     } else {
@@ -199,7 +181,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     h8 ka[KD], qa[QB][KD];
 #pragma unroll
     for (int i = 0; i < KD; i++) {
-      ka[i] = *(const h8*)(kb + (k_rd ^ ((PF_ABLATED(2) ? 0 : i) * 32)));
+      ka[i] = *(const h8*)(kb + (k_rd ^ (i * 32)));
       if (i >= QR) {
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) qa[qb][i] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (i - QR)) * 1024);
@@ -212,7 +194,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 #pragma unroll
       for (int qb = 0; qb < QB; qb++) b[qb] = ks < QR ? qf[qb][ks < QR ? ks : 0] : qa[qb][ks % KD];
       if (ks + KD < S::KS) {
-        if (!PF_ABLATED(2)) ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
+        ka[ks % KD] = *(const h8*)(kb + (k_rd ^ ((ks + KD) * 32)));
         if (ks + KD >= QR) {
 #pragma unroll
           for (int qb = 0; qb < QB; qb++) qa[qb][ks % KD] = *(const h8*)(q_lds + (qb * (S::KS - QR) + (ks + KD - QR)) * 1024);
@@ -227,7 +209,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 #pragma unroll
     for (int ks = 0; ks < S::KS; ks++) {
       __builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
-      if (ks + KD < S::KS) { if (!PF_ABLATED(2)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); if (ks + KD >= QR) __builtin_amdgcn_sched_group_barrier(0x100, QB, 0); }
+      if (ks + KD < S::KS) { __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); if (ks + KD >= QR) __builtin_amdgcn_sched_group_barrier(0x100, QB, 0); }
     }
   };
   // ---- online softmax; lane holds query row ln of each block, positions tp + 8 (i / 4) + 4 hb + i % 4 ----
@@ -235,13 +217,6 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
   // v_dot2 over the f16-rounded probabilities (the values PV really uses), and the mask is a separate pass
   // that only tiles straddling a row end execute.
   auto sm = [&](const uint32_t tp) {
-    if constexpr (PF_ABLATED(8) != 0) {
-#pragma unroll
-      for (int qb = 0; qb < QB; qb++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) pf[qb][i >> 3][i & 7] = (_Float16)s[qb][i];
-      return;
-    }
     if (tp + PF_TN > w_min_end) {
       asm volatile("; causal tile" ::: "memory");   // keeps this a branch: most tiles skip the 3 ops per element
 #pragma unroll
@@ -282,9 +257,8 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
       float ps = l_run[qb];
 #pragma unroll
       for (int i = 0; i < 16; i += 2) {
-        const float a0 = __builtin_fmaf(s[qb][i], c1, nmr), a1 = __builtin_fmaf(s[qb][i + 1], c1, nmr);
-        const float e0 = PF_ABLATED(1) ? a0 : __builtin_amdgcn_exp2f(a0);
-        const float e1 = PF_ABLATED(1) ? a1 : __builtin_amdgcn_exp2f(a1);
+        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i], c1, nmr));
+        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][i + 1], c1, nmr));
         const h2 pp = { (_Float16)e0, (_Float16)e1 };
         ps = __builtin_amdgcn_fdot2(pp, ones, ps, false);
         pf[qb][i >> 3][i & 7] = pp[0]; pf[qb][i >> 3][(i & 7) + 1] = pp[1];
@@ -307,7 +281,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 #pragma unroll
     for (int f = 0; f < NF; f++) {
       const h4 lo = vlo[f % VD], hi = vhi[f % VD];
-      if (f + VD < NF && !PF_ABLATED(4)) {
+      if (f + VD < NF) {
         const int fn = f + VD;
         const unsigned char* vp = vb + (v_rd ^ ((fn % S::DB) * 64)) + (fn / S::DB) * 16 * S::ROWB;
         vlo[f % VD] = lds_read_tr16(vp);
@@ -322,7 +296,7 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
 #pragma unroll
     for (int f = 0; f < NF; f++) {
       __builtin_amdgcn_sched_group_barrier(0x008, QB, 1);
-      if (f + VD < NF && !PF_ABLATED(4)) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+      if (f + VD < NF) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
     }
   };
 
@@ -332,15 +306,11 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     // all waves in phase: QK, softmax, PV of a tile between two barriers (tile i + 1 of both K and V in flight)
     auto step_s = [&](auto PAR, const uint32_t i) {
       constexpr int par = decltype(PAR)::value;
-      const uint32_t tp = t_begin + i * PF_STEP;
-      if (i + 1 < n_steps && !PF_ABLATED(16)) { issue_k(par ? kbuf0 : kbuf1, tp + PF_STEP); issue_v(par ? vbuf0 : vbuf1, tp + PF_STEP); }
-#pragma unroll
-      for (int sub = 0; sub < PF_SUB; sub++) {
-        if (sub > 0 && tp + sub * PF_TN >= t_end) break;               // (the last step of a split: tiles past its end)
-        qk((par ? kbuf1 : kbuf0) + sub * S::SUBT, tp + sub * PF_TN);
-        sm(tp + sub * PF_TN);
-        pv((par ? vbuf1 : vbuf0) + sub * S::SUBT, tp + sub * PF_TN);
-      }
+      const uint32_t tp = t_begin + i * PF_TN;
+      if (i + 1 < n_steps) { issue_k(par ? kbuf0 : kbuf1, tp + PF_TN); issue_v(par ? vbuf0 : vbuf1, tp + PF_TN); }
+      qk(par ? kbuf1 : kbuf0, tp);
+      sm(tp);
+      pv(par ? vbuf1 : vbuf0, tp);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
     };
@@ -351,9 +321,6 @@ __global__ __launch_bounds__(W * 64, W / 4) void pa_prefill_kernel(AttnParams p,
     if (n_steps & 1) step_s(std::integral_constant<int, 0>{}, n_even);
   }
 
-#ifdef PF_ABL
-  if (g_pf_clk && tid == 0) { g_pf_clk[2 * blockIdx.x] = clock64() - clk0; g_pf_clk[2 * blockIdx.x + 1] = wall_clock64() - wall0; }
-#endif
   // ---- epilogue ----
 #pragma unroll
   for (int qb = 0; qb < QB; qb++) {

@@ -13,11 +13,7 @@ typedef __fp16 hh4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 
 #define NEG_INF (-__builtin_inff())
-#define PF_TN 32                 // positions per MFMA tile
-#ifndef PF_SUB
-#define PF_SUB 1                 // tiles per step (between two barriers)
-#endif
-#define PF_STEP (PF_TN * PF_SUB) // positions per step
+#define PF_TN 32                 // positions per step
 #ifndef PF_QR
 #define PF_QR 16                 // head_dim 256: k-steps of Q kept in registers (any others are parked in LDS)
 #endif
