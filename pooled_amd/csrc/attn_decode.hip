@@ -33,6 +33,9 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 #define TILE 32
 
 #define NEG_INF (-__builtin_inff())
+#ifndef PA_V_LATE_MIN_WGS
+#define PA_V_LATE_MIN_WGS 384u   // single-round splits: workgroups from which the V loads wait for the K scores
+#endif
 #define DEC_RESCALE_TH 8.f   // tile loop: a row maximum may pass the reference maximum by this much before O is rescaled
 
 static __device__ inline h4 lds_read_tr16(const unsigned char* p) {
@@ -450,7 +453,10 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   // the very end of the kernel.  Scored first, that work runs while other waves keep the pipeline full, and what follows
   // the last V load is the V latency, the staging of V and the PV product.  Measured on the 32K decode step: 18.6 -> 18.15 us.
   constexpr bool V_LATE = SR && !GATHER;
-  if constexpr (!FUSED && !V_LATE) first_v_loads();
+  // ... when the chip is streaming.  With fewer workgroups than two a CU the memory pipeline is never full, the loads
+  // of a wave are accepted at once, and V behind the scores is one more HBM round trip at the end: then V goes out with K.
+  const bool v_late = V_LATE && gridDim.x * gridDim.y * gridDim.z >= PA_V_LATE_MIN_WGS;
+  if (!FUSED && !v_late) first_v_loads();
   __builtin_amdgcn_sched_barrier(0);   // nothing below may be scheduled above the load issue
   // ---- q -> f16 rows in LDS; waits only for the q loads, which were issued first ----
   if constexpr (FUSED) {
@@ -509,7 +515,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
     }
   }
-  if constexpr (FUSED && !V_LATE) {
+  if (FUSED && !v_late) {
     __builtin_amdgcn_sched_barrier(0);
     first_v_loads();
     __builtin_amdgcn_sched_barrier(0);
@@ -703,7 +709,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
       for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
       ps = rows_sum(ps);
-      if constexpr (V_LATE) { __builtin_amdgcn_sched_barrier(0); first_v_loads(); __builtin_amdgcn_sched_barrier(0); }
+      if (v_late) { __builtin_amdgcn_sched_barrier(0); first_v_loads(); __builtin_amdgcn_sched_barrier(0); }
       stage_v(ILV && ilv ? 0u : tp, false, 0);                          // interleaved splits are whole: no row past the end to zero
       *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pf;
       if (kg == 0) { mex[wave * 16 + ln] = mx; lex[wave * 16 + ln] = ps; }
