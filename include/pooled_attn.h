@@ -268,7 +268,7 @@ int pa_profile_read_each(pa_ctx* ctx, float* ms, uint32_t cap, uint32_t* count);
                          nibble - 8; scales as Q8_0 (base.js:81-118) */
 typedef struct pa_weight pa_weight;
 /* copies a weight matrix to the device.  h_w: the values plane (f32 / int8 / packed nibbles), h_scales: f16 bits
- * (NULL for PA_W_F32).  d_in must be a multiple of 32 and at most 8192 (4096 for PA_W_F32).  A handle belongs to the
+ * (NULL for PA_W_F32).  d_in must be a multiple of 32 and at most 8192.  A handle belongs to the
  * context that made it: use and destroy it through that context only (pa_gemm may attach a derived copy to it, see
  * pa_set_weight_cache, on that context's stream). */
 int pa_weight_create(pa_ctx* ctx, int kind, uint32_t d_out, uint32_t d_in, const void* h_w, const void* h_scales, pa_weight** out);

@@ -654,7 +654,7 @@ extern "C" int pa_weight_create(pa_ctx* ctx, int kind, uint32_t d_out, uint32_t 
   if (kind != PA_W_F32 && kind != PA_W_Q8_0 && kind != PA_W_Q4_0) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": unknown weight kind");
   if (!h_w || (kind != PA_W_F32 && !h_scales)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": null plane");
   if (d_out == 0 || d_in == 0 || (d_in & 31)) return fail(ctx, PA_ERR_INVALID, std::string(who) + ": d_in must be a positive multiple of 32");
-  if (d_in > (kind == PA_W_F32 ? 4096u : 8192u)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": d_in beyond the gfx950 table");
+  if (d_in > 8192u) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": d_in beyond the gfx950 table");
   pa_weight* w = new (std::nothrow) pa_weight();
   if (!w) return fail(ctx, PA_ERR_NOMEM, std::string(who) + ": out of host memory");
   w->kind = kind; w->d_out = d_out; w->d_in = d_in;

@@ -76,8 +76,10 @@ static __device__ inline float dot_block(const BlockRegs<KIND>& r, const float (
   }
 }
 
-// BPL: blocks per lane (d_in <= 2048 * BPL); RW: rows per wave
-template <int KIND, int BPL, int RW, bool NORM>
+// BPL: blocks per lane and pass; PASSES: passes over the input (d_in <= 2048 * BPL * PASSES; two for f32 weights past
+// 4096 inputs, whose 32 registers a block leave no room for four blocks a lane: the second pass's weight rows are
+// requested when the first pass's are consumed); RW: rows per wave
+template <int KIND, int BPL, int RW, bool NORM, int PASSES = 1>
 __global__ __launch_bounds__(256)
 void pa_gemv_kernel(const float* a_x, const float* a_norm_w, const void* a_w, const uint16_t* a_scales, float* a_y, uint32_t a_d_out, uint32_t a_d_in, GemvParams p_in) {
   // The leading arguments repeat fields of p_in: the first twelve dwords of the arguments are preloaded into scalar
@@ -95,7 +97,7 @@ void pa_gemv_kernel(const float* a_x, const float* a_norm_w, const void* a_w, co
   // instead of after it.
   extern __shared__ __attribute__((aligned(16))) float xs[];
   __shared__ float red[4];
-  constexpr int XPT = 2 * BPL;                                         // float4 of x per thread (d_in <= 2048 * BPL)
+  constexpr int XPT = 2 * BPL * PASSES;                                // float4 of x per thread (d_in <= 2048 * BPL * PASSES)
   const uint32_t n4 = p.d_in / 4;
   f4 xv[XPT], wv[NORM ? XPT : 1];
   float ss = 0.f;
@@ -159,10 +161,27 @@ void pa_gemv_kernel(const float* a_x, const float* a_norm_w, const void* a_w, co
     if (e < n4) *(f4*)(xs + (e / 8) * 36 + (e % 8) * 4) = xv[k];
   }
   __syncthreads();
+  float part[RW];
+#pragma unroll
+  for (int r = 0; r < RW; r++) part[r] = 0.f;
+#pragma unroll
+  for (int pass = 0; pass < PASSES; pass++) {
+  if (pass > 0) {                                                      // the next pass's weight rows
+#pragma unroll
+    for (int r = 0; r < RW; r++) {
+      const size_t row = min(row0 + r, (size_t)p.d_out - 1);
+#pragma unroll
+      for (int i = 0; i < BPL; i++) {
+        const uint32_t b = min(lane + 64 * (i + BPL * pass), nb - 1);
+        load_block<KIND>(wr[r][i], wbase, row, nb, b);
+        if constexpr (KIND != PA_W_F32) sc[r][i] = p.scales[row * nb + b];
+      }
+    }
+  }
   float x[BPL][32], sx[BPL];
 #pragma unroll
   for (int i = 0; i < BPL; i++) {
-    const uint32_t b = lane + 64 * i;
+    const uint32_t b = lane + 64 * (i + BPL * pass);
     const bool on = b < nb;
     const f4* src = (const f4*)(xs + min(b, nb - 1) * 36);
 #pragma unroll
@@ -184,10 +203,9 @@ void pa_gemv_kernel(const float* a_x, const float* a_norm_w, const void* a_w, co
 #pragma unroll
     for (int i = 0; i < BPL; i++) sx[i] = 0.f;
   }
-  float part[RW];
 #pragma unroll
   for (int r = 0; r < RW; r++) {
-    float a = 0.f;
+    float a = part[r];
 #pragma unroll
     for (int i = 0; i < BPL; i++) {
       const float d = dot_block<KIND>(wr[r][i], x[i], sx[i]);
@@ -195,6 +213,7 @@ void pa_gemv_kernel(const float* a_x, const float* a_norm_w, const void* a_w, co
       else a = __builtin_fmaf((float)__ushort_as_half(sc[r][i]), d, a);
     }
     part[r] = a;
+  }
   }
 #pragma unroll
   for (int r = 0; r < RW; r++) part[r] = wave_sum_f32(part[r]);
@@ -207,11 +226,11 @@ void pa_gemv_kernel(const float* a_x, const float* a_norm_w, const void* a_w, co
   }
 }
 
-template <int KIND, int BPL, int RW, bool NORM>
+template <int KIND, int BPL, int RW, bool NORM, int PASSES = 1>
 static hipError_t launch_k(const GemvParams& p, hipStream_t s) {
   const uint32_t rows_wg = 4 * RW;
   const size_t lds = (size_t)(p.d_in / 32) * 36 * sizeof(float);
-  hipLaunchKernelGGL((pa_gemv_kernel<KIND, BPL, RW, NORM>), dim3((p.d_out + rows_wg - 1) / rows_wg), dim3(256), lds, s, p.x, p.norm_w, p.w, p.scales, p.y, p.d_out, p.d_in, p);
+  hipLaunchKernelGGL((pa_gemv_kernel<KIND, BPL, RW, NORM, PASSES>), dim3((p.d_out + rows_wg - 1) / rows_wg), dim3(256), lds, s, p.x, p.norm_w, p.w, p.scales, p.y, p.d_out, p.d_in, p);
   return hipGetLastError();
 }
 
@@ -237,6 +256,8 @@ static hipError_t launch_bpl(const GemvParams& p, int n_cu, hipStream_t s) {
   if constexpr (KIND != PA_W_F32) {
     if (nb <= 192) return launch_rw<KIND, 3, NORM>(p, n_cu, s);
     if (nb <= 256) return launch_rw<KIND, 4, NORM>(p, n_cu, s);
+  } else {
+    if (nb <= 256) return launch_k<KIND, 2, 1, NORM, 2>(p, s);        // f32 weights past 4096 inputs: two passes of two blocks a lane
   }
   return hipErrorNotSupported;
 }

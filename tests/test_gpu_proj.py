@@ -31,8 +31,6 @@ def _rel(got, ref):
 @pytest.mark.parametrize("kind", [PA_W_F32, PA_W_Q8_0, PA_W_Q4_0])
 @pytest.mark.parametrize("d_out,d_in", [(9216, 2048), (2048, 4096), (1, 32), (37, 96), (5000, 6144), (130, 8192)])
 def test_gemv_matches_oracle(kind, d_out, d_in):
-    if kind == PA_W_F32 and d_in > 4096:
-        pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
     rng = np.random.default_rng(d_out * 7 + d_in + kind)
     w, sc = _weights(kind, d_out, d_in, rng)
     x = rng.standard_normal(d_in).astype(np.float32)
@@ -125,8 +123,6 @@ def test_attn_layer_decode_matches_oracle(shape, dim, kind, pos):
                                           (100, 384, 65), (64, 128, 33), (4096, 2048, 512),      # the 64 x 64 kernel with an odd stage count, one stage, a C2-sized chunk (as are the first two and the fourth)
                                           (9216, 2048, 8), (2048, 4096, 16), (130, 8192, 3), (70, 64, 1), (2048, 4096, 31), (130, 8192, 17)])   # from (9216, 2048, 8) on: up to 16 columns the skinny-chunk kernel, one or more launches; the last two the 64 x 32 tiles of the mid-size kernel
 def test_gemm_matches_oracle(kind, d_out, d_in, n):
-    if kind == PA_W_F32 and d_in > 4096:
-        pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
     rng = np.random.default_rng(d_out + 3 * d_in + n + kind)
     w, sc = _weights(kind, d_out, d_in, rng)
     x16 = rng.standard_normal((n, d_in)).astype(np.float16)
@@ -155,8 +151,6 @@ def test_gemm_large_chunks(kind, d_out, d_in, n):
     tiled kernel, too few workgroups or d_in not a multiple of 128).  Ragged edges on both axes, padded strides that
     must stay untouched, the accumulating form (the second call on a handle, which finds the kept copy), and a second
     weight."""
-    if kind == PA_W_F32 and d_in > 4096:
-        pytest.skip("f32 weights: d_in <= 4096 on the gfx950 table")
     rng = np.random.default_rng(d_out + d_in + n + kind)
     w, sc = _weights(kind, d_out, d_in, rng)
     x16 = rng.standard_normal((n, d_in)).astype(np.float16)
