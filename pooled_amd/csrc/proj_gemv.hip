@@ -21,6 +21,7 @@
 
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 
 // 32 weights of one block times the lane's 32 activations, scale not applied
 template <int KIND> struct BlockRegs;
@@ -62,16 +63,23 @@ static __device__ inline float dot_block(const BlockRegs<KIND>& r, const float (
       }
     return a;
   } else {
-    // sum (n - 8) x = sum n x - 8 sum x: the nibbles convert with the byte-to-float instructions
+    // sum (n - 8) x = sum n x - 8 sum x.  A nibble n in the low bits of a 16-bit half IS the f16 subnormal n x 2^-24, and
+    // the mixed-precision fma takes an f16 operand as it is: two nibbles of a word are isolated by one shift and one mask
+    // (15 instructions for 8 weights instead of 23 with byte-to-float conversions), the products are the same bits scaled
+    // by a power of two, and the sum is scaled back once.
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-      const uint32_t word = r.w[0][k], lo = word & 0x0F0F0F0Fu, hi = (word >> 4) & 0x0F0F0F0Fu;
+      const uint32_t word = r.w[0][k];
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        a = __builtin_fmaf((float)((lo >> (8 * j)) & 255u), x[4 * k + j], a);
-        a = __builtin_fmaf((float)((hi >> (8 * j)) & 255u), x[16 + 4 * k + j], a);
+      for (int t = 0; t < 4; t++) {
+        const uint32_t pr = (word >> (4 * t)) & 0x000F000Fu;          // nibble t of the word (low half) and nibble t + 4 (high half)
+        h2v v; __builtin_memcpy(&v, &pr, 4);
+        const int e = 4 * k + (t >> 1) + 16 * (t & 1);                 // nibble 2 j of a word is element j of its four bytes, nibble 2 j + 1 element j + 16
+        a = __builtin_fmaf((float)v[0], x[e], a);
+        a = __builtin_fmaf((float)v[1], x[e + 2], a);
       }
     }
+    a *= 16777216.0f;
     return a - 8.0f * sx;
   }
 }
