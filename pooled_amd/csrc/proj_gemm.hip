@@ -216,16 +216,32 @@ __global__ __launch_bounds__(256, XT == 2 ? 2 : 1) void pa_gemm_kernel(GemmParam
 // through LDS (the staging area, free by then): lane t of a wave adds up the 64 partials of its (row, column).
 #define SK_NC 16        // columns a launch serves at most
 template <int KIND, int BPL, int RW>
-__global__ __launch_bounds__(256) void pa_gemm_skinny_kernel(GemmParams p) {
+__global__ __launch_bounds__(256)
+void pa_gemm_skinny_kernel(const uint16_t* a_x, const void* a_w, const uint16_t* a_scales, uint32_t a_x_stride, uint32_t a_d_out, uint32_t a_d_in, uint32_t a_n_cols,
+                           GemmParams p_in) {
   static_assert(KIND == PA_W_Q4_0 || KIND == PA_W_Q8_0, "quantised weights");
-  // (every kernel argument in the first batch of scalar loads instead of a dependent round trip at each first use)
-  asm volatile("" :: "s"(p.w), "s"(p.scales), "s"(p.x), "s"(p.y), "s"(p.x_stride), "s"(p.y_stride), "s"(p.d_out), "s"(p.d_in), "s"(p.n_cols), "s"(p.acc));
+  // (the leading arguments repeat fields of p_in: they are preloaded into scalar registers, so the loads below need no
+  // scalar-load round trip; the other arguments are fetched in one batch behind them)
+  GemmParams p = p_in;
+  p.x = a_x; p.w = a_w; p.scales = a_scales; p.x_stride = a_x_stride; p.d_out = a_d_out; p.d_in = a_d_in; p.n_cols = a_n_cols;
   extern __shared__ __attribute__((aligned(16))) unsigned char sk_lds[];
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t nb = p.d_in / GK, ncol = p.n_cols;
   const uint32_t xcol = nb * GROW;                                    // bytes of a staged column
   const size_t row0 = ((size_t)blockIdx.x * 4 + wave) * RW;
-  // the wave's weights first: they are what the kernel waits for
+  // The first eight 16-byte pieces a thread stages of the chunk's columns (all of them for 8 columns of 2048) are
+  // requested FIRST, the wave's weight rows right behind them: a wave's loads complete in order, the columns come from
+  // L2 in a fraction of the time the weight stream takes from HBM, and their trip into LDS then runs under the latency
+  // of the weights instead of after it.
+  const uint32_t cpc = p.d_in / 8;                                    // 16-byte pieces of a column
+  const uint32_t pieces = ncol * cpc;
+  u4 xv0[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const uint32_t e = min(tid + 256 * j, pieces - 1), c = e / cpc, k8 = e % cpc;
+    xv0[j] = *(const u4*)((const unsigned char*)(p.x + (size_t)c * p.x_stride) + k8 * 16);
+  }
+  __builtin_amdgcn_sched_barrier(0);
   constexpr int WQ = KIND == PA_W_Q4_0 ? 1 : 2;                       // 16-byte words of a packed block
   u4 wq[RW][BPL][WQ];
   uint16_t wsc[RW][BPL];
@@ -241,12 +257,17 @@ __global__ __launch_bounds__(256) void pa_gemm_skinny_kernel(GemmParams p) {
       wsc[r][i] = p.scales[row * nb + b];
     }
   }
-  // the chunk's columns -> LDS, 16 bytes a thread and turn
-  const uint32_t cpc = p.d_in / 8;                                    // 16-byte pieces of a column
-  // (eight loads a thread go out before the first is stored -- unconditional, a turn past the end re-reads the last piece:
-  // one load a loop turn is one round trip a turn, eight of them for 8 columns of 2048)
-  const uint32_t pieces = ncol * cpc;
-  for (uint32_t e0 = tid; e0 < pieces; e0 += 256 * 8) {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("" :: "s"(p.y), "s"(p.y_stride), "s"(p.acc));
+  // the chunk's columns -> LDS, 16 bytes a thread and turn: the pieces requested above, ...
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const uint32_t e = tid + 256 * j, c = e / cpc, k8 = e % cpc;
+    if (e < pieces) *(u4*)(sk_lds + c * xcol + (k8 >> 2) * GROW + (k8 & 3) * 16) = xv0[j];
+  }
+  // ... then any further turns (eight loads a thread go out before the first is stored -- unconditional, a turn past the
+  // end re-reads the last piece: one load a loop turn is one round trip a turn)
+  for (uint32_t e0 = tid + 256 * 8; e0 < pieces; e0 += 256 * 8) {
     u4 v[8];
 #pragma unroll
     for (int j = 0; j < 8; j++) {
@@ -340,7 +361,8 @@ static hipError_t launch_skinny(const GemmParams& p, hipStream_t s) {
     if (e != hipSuccess) return e;
     attr = lds;
   }
-  hipLaunchKernelGGL((pa_gemm_skinny_kernel<KIND, BPL, RW>), dim3((p.d_out + 4 * RW - 1) / (4 * RW)), dim3(256), lds, s, p);
+  hipLaunchKernelGGL((pa_gemm_skinny_kernel<KIND, BPL, RW>), dim3((p.d_out + 4 * RW - 1) / (4 * RW)), dim3(256), lds, s, p.x, p.w, p.scales, p.x_stride, p.d_out, p.d_in,
+                     p.n_cols, p);
   return hipGetLastError();
 }
 template <int KIND>
