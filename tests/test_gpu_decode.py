@@ -85,6 +85,23 @@ def test_decode_split_invariance_and_plan():
         assert np.array_equal(pa.run_attn("decode", 0, q, L - 1), pa.run_attn("decode", 0, q, L - 1))
 
 
+@pytest.mark.parametrize("pos", [63 * 128, 64 * 128, 64 * 128 + 77, 12000])
+def test_decode_either_side_of_the_f16_partials_threshold(pos):
+    """A one-column decode writes f16 O partials from 64 single-round splits on (f32 below): both sides of the threshold,
+    a remainder split, and a longer context against the f64 oracle, with the margin the five configurations are held to."""
+    cfg = SHAPES["qwen36_moe"]
+    rng = np.random.default_rng(pos)
+    k16, v16 = random_cache(cfg, pos + 1, seed=pos + 1)
+    q = rng.standard_normal((1, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    gate = rng.standard_normal(q.shape, dtype=np.float32)
+    ref = C.attention(q, k16, v16, pos, gate=gate)
+    with _ctx_with_cache(cfg, k16, v16, pos + 1) as pa:
+        pl = pa.plan("decode", pos, 1)
+        assert pl["split_len"] == 128 and (pl["n_splits"] >= 64) == (pos >= 64 * 128)
+        for out_dtype in (0, PA_OUT_F16):
+            assert_parity(pa.run_attn("decode", 0, q, pos, gate=gate, out_dtype=out_dtype), ref, "decode at %d, %d splits" % (pos, pl["n_splits"]), tight=True)
+
+
 @pytest.mark.parametrize("shape,n_cols,base", [("qwen36_moe", 4, 996), ("qwen36_moe", 16, 3000), ("qwen38_27b", 8, 2040),
                                                ("qwen3_1p7b", 4, 510), ("qwen38_27b", 16, 17), ("qwen36_moe", 7, 0)])
 def test_verify_equals_sequential_decodes(shape, n_cols, base):

@@ -45,11 +45,12 @@ def test_gather_lists_of_many_lengths(shape):
     assert_parity(one, ref[4:5], "gather single column %s" % shape)
 
 
-@pytest.mark.parametrize("pos", [0, 40, 2050, 6000])
+@pytest.mark.parametrize("pos", [0, 40, 2050, 6000, 9000])
 def test_identity_list_equals_dense_decode(pos):
     """With the list 0 .. pos the gathered kernel computes what the dense kernel computes
     (engine/wgsl/attn_dec.js:35-37).  Not bit for bit: a dense one-column decode folds the column's own row in as a
-    partial of its own (f32 products), the gathered kernel streams every listed row through the f16 MFMA path."""
+    partial of its own (f32 products), the gathered kernel streams every listed row through the f16 MFMA path.  (9000
+    rows are 71 splits: both passes then write f16 partials.)"""
     cfg = SHAPES["qwen36_moe"]
     rng = np.random.default_rng(pos + 1)
     k16, v16 = random_cache(cfg, pos + 1, seed=pos + 2)
