@@ -15,8 +15,7 @@ MAX_ABS, MAX_REL = 2e-3, 1e-2
 
 
 # every parity check of the session: (what, max-abs, relative, max|ref|, effective budget); printed by conftest at the
-# end of the run and appended to the file PA_PARITY_LOG names (default gpurun_out/parity_margins.tsv when that folder
-# exists)
+# end of the run and appended to the file the environment variable PA_PARITY_LOG names, when it is set
 MARGINS = []
 # a "tight" check must stay within this fraction of its effective budget
 TIGHT_FRACTION = 0.25
@@ -25,9 +24,6 @@ TIGHT_FRACTION = 0.25
 def _log_margin(rec):
     MARGINS.append(rec)
     path = os.environ.get("PA_PARITY_LOG")
-    if path is None:
-        d = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
-        path = os.path.join(d, "parity_margins.tsv") if os.path.isdir(d) else ""
     if path:
         try:
             with open(path, "a") as f:
