@@ -250,6 +250,15 @@ static hipError_t launch_rw(const GemvParams& p, int n_cu, hipStream_t s) {
   const uint32_t waves_wanted = 8u * (uint32_t)n_cu;
   uint32_t rw = p.d_out >= 8 * waves_wanted ? 8 : p.d_out >= 4 * waves_wanted ? 4 : p.d_out >= 2 * waves_wanted ? 2 : 1;
   if (rw > (uint32_t)RWMAX) rw = RWMAX;
+  // Once the weights are there the kernel is VALU work, and the SIMD with the most rows sets the time: with four rows a
+  // wave the MoE model's 9216 [q|k|v] rows are 2304 waves, 2.25 a SIMD -- some SIMDs work through three waves (12 rows),
+  // most through two.  Three rows a wave are 3072 waves, three on every SIMD (9 rows).  Taken when it lowers the busiest
+  // SIMD's rows.
+  if constexpr (RWMAX >= 4) {
+    const uint32_t simds = 4u * (uint32_t)n_cu;
+    auto busiest = [&](uint32_t r) { const uint32_t waves = (p.d_out + r - 1) / r; return ((waves + simds - 1) / simds) * r; };
+    if (rw == 4 && busiest(3) < busiest(4)) return launch_k<KIND, BPL, 3, NORM>(p, s);
+  }
   if constexpr (RWMAX >= 8) { if (rw == 8) return launch_k<KIND, BPL, 8, NORM>(p, s); }
   if constexpr (RWMAX >= 4) { if (rw >= 4) return launch_k<KIND, BPL, 4, NORM>(p, s); }
   if constexpr (RWMAX >= 2) { if (rw >= 2) return launch_k<KIND, BPL, 2, NORM>(p, s); }
