@@ -366,8 +366,15 @@ static hipError_t launch_skinny(const GemmParams& p, hipStream_t s) {
   return hipGetLastError();
 }
 template <int KIND>
-static hipError_t launch_skinny_kind(const GemmParams& p, hipStream_t s) {
-  if (p.d_in <= 2048) return launch_skinny<KIND, 1, 4>(p, s);
+static hipError_t launch_skinny_kind(const GemmParams& p, int n_cu, hipStream_t s) {
+  if (p.d_in <= 2048) {
+    // (three rows a wave where that lowers the rows of the busiest SIMD -- 9216 rows: 2304 waves at 2.25 a SIMD, or 3072
+    // at three -- as the one-token GEMV chooses)
+    const uint32_t simds = 4u * (uint32_t)(n_cu > 0 ? n_cu : 256);
+    auto busiest = [&](uint32_t r) { const uint32_t waves = (p.d_out + r - 1) / r; return ((waves + simds - 1) / simds) * r; };
+    if (busiest(3) < busiest(4)) return launch_skinny<KIND, 1, 3>(p, s);
+    return launch_skinny<KIND, 1, 4>(p, s);
+  }
   if (p.d_in <= 4096) return launch_skinny<KIND, 2, 2>(p, s);
   return launch_skinny<KIND, 4, 1>(p, s);
 }
@@ -396,7 +403,7 @@ hipError_t pa_launch_gemm(const GemmParams& p, int n_cu, hipStream_t s) {
         GemmParams q = p;
         q.x = p.x + (size_t)c0 * p.x_stride; q.y = p.y + (size_t)c0 * p.y_stride;
         q.n_cols = p.n_cols - c0 < per ? p.n_cols - c0 : per;
-        const hipError_t e = p.kind == PA_W_Q4_0 ? launch_skinny_kind<PA_W_Q4_0>(q, s) : launch_skinny_kind<PA_W_Q8_0>(q, s);
+        const hipError_t e = p.kind == PA_W_Q4_0 ? launch_skinny_kind<PA_W_Q4_0>(q, n_cu, s) : launch_skinny_kind<PA_W_Q8_0>(q, n_cu, s);
         if (e != hipSuccess) return e;
       }
       return hipSuccess;
