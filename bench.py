@@ -512,7 +512,7 @@ def main():
     kname = pa_decode_kernel_name(plan, args)
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
                     traffic=traffic, traffic_source=traffic_source, kernel=kname, kernel_us=round(k_ms * 1e3, 3), kernel_us_median=round(k_med * 1e3, 3),
-                    kernel_us_min=round(min(kern) * 1e3, 3), reported="mean launch (dispatch-stamped HIP events)",
+                    kernel_us_min=round(min(kern) * 1e3, 3), reported="mean launch (dispatch-stamped HIP events; the step's merge launch is stamped too, as every dispatch is in a kernel trace)",
                     algorithmic_bytes_per_launch=kv_bytes, launches=len(kern), layers_in_rotation=n_rot)
     log("split-K kernel: mean %.2f us/launch (median %.2f) over %d launches -> %.0f GB/s (%.1f%% of 8 TB/s)" % (k_ms * 1e3, k_med * 1e3, len(kern), achieved, 100 * achieved / HBM_PEAK_GBS))
 

@@ -247,7 +247,8 @@ int pa_slot_import(pa_ctx* ctx, uint32_t slot, uint32_t layer, int which, const 
  * pa_timer_start / pa_timer_stop bracket a region; stop blocks and returns milliseconds.
  * pa_profile_enable(1) additionally times every attention call's main kernel (the split-K or prefill kernel, not
  * glue / merge) with an event pair stamped by the dispatch itself (the kernel's own begin / end timestamps, the
- * figure a kernel trace reports); pa_profile_read blocks, returns the sum of those durations and their count
+ * figure a kernel trace reports; the call's merge launch is stamped too, unread, because a kernel between unstamped
+ * neighbours reads about a microsecond longer than in a trace, where every dispatch is stamped); pa_profile_read blocks, returns the sum of those durations and their count
  * since the last read, and resets them.  pa_profile_read_each does the same but hands back every launch's own
  * duration, in launch order (ms[0 .. min(*count, cap))); *count is the number of launches timed since the last read),
  * so that a caller can report a median instead of a mean. */

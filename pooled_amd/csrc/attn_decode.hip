@@ -1281,7 +1281,7 @@ hipError_t pa_launch_decode_gather(const AttnParams& p, uint32_t hd, hipStream_t
   return hipErrorInvalidValue;
 }
 
-hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s) {
+hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t) {
   // many columns, few splits: one thread per (column, head, 4 dims)
   if (p.n_cols >= 16 && p.n_splits <= 32 && (hd == 256 || hd == 128)) {
     const size_t threads = (size_t)p.n_cols * p.n_heads * (hd / 4);
@@ -1292,7 +1292,7 @@ hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s) {
   }
   const uint32_t gx = p.n_heads * (hd / 16), has_sel = p.sel != nullptr;
   if (hd != 256 && hd != 128) return hipErrorInvalidValue;
-#define PA_COMBINE_WAVE(HD_, F16_) hipLaunchKernelGGL((pa_combine_wave_kernel<HD_, 16, F16_>), dim3(gx, p.n_cols), dim3(64), 0, s, (const float*)p.part_o, \
+#define PA_COMBINE_WAVE(HD_, F16_) PA_LAUNCH((pa_combine_wave_kernel<HD_, 16, F16_>), dim3(gx, p.n_cols), dim3(64), 0, s, t, (const float*)p.part_o, \
     (const float*)p.part_ml, p.slots, p.n_heads, p.base_pos, p.self_row, p.split_len, p.n_splits, gx, has_sel, p)
   if (hd == 256) { if (p.part_f16) PA_COMBINE_WAVE(256, true); else PA_COMBINE_WAVE(256, false); }
   else { if (p.part_f16) PA_COMBINE_WAVE(128, true); else PA_COMBINE_WAVE(128, false); }

@@ -84,7 +84,7 @@ hipError_t pa_launch_decode_gather(const AttnParams& p, uint32_t hd, hipStream_t
 // the same with the pre-step of the one column fused in (p.f_* set; one 16-row block, n_cols == 1)
 hipError_t pa_launch_decode_step(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t = nullptr);
 hipError_t pa_prepare_decode_step(uint32_t hd, bool q8);
-hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s);
+hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t = nullptr);
 // MFMA prefill; returns hipErrorNotSupported for shapes it does not cover
 hipError_t pa_launch_prefill(const AttnParams& p, uint32_t hd, uint32_t row_blocks, uint32_t col_groups, hipStream_t s, const PaTiming* t = nullptr);
 
@@ -180,5 +180,7 @@ struct pa_ctx {
   bool profiling = false;
   std::vector<hipEvent_t> prof_events;   // pairs
   size_t prof_used = 0;
+  std::vector<hipEvent_t> prof_aux;      // pairs around the merge launch of a profiled call (stamped, never read; reused in a ring)
+  size_t prof_aux_used = 0;
   std::string err;
 };
