@@ -43,8 +43,10 @@ extern "C" {
                                  (its own splits, its own row block): column c then has the bits of pa_attn_decode(base_pos + c,
                                  n_cols = 1), the invariant the reference states for its pair (engine/wgsl/attn_dec.js:12-16,
                                  tests/test_attn_dec.js:89-97) and its speculative decoding leans on (spec greedy == plain
-                                 greedy).  Cost: the K/V stream is read once per column, as the reference does, instead of
-                                 once per block.  Off by default: see the note at pa_attn_decode. */
+                                 greedy).  Cost: every column streams the K/V rows through its own workgroups; a block whose
+                                 columns share one one-column plan runs as one pass in which a split's columns sit side by
+                                 side on one L2 (about 2.3x the default block's time), a block that straddles a change of
+                                 plan as one pass per column.  Off by default: see the note at pa_attn_decode. */
 
 /* output element types */
 #define PA_OUT_F32 0          /* the engine's attnOut feeding wo (engine/qwen35.js:881) */

@@ -195,7 +195,8 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   // scalar registers by the dispatcher (-amdgpu-kernarg-preload-count), so what the first tile loads' addresses are made
   // of is there when the wave starts instead of a scalar-load round trip later.
   AttnParams p = p_in;
-  p.k_cache = a_k_cache; p.base_pos = a_base_pos; p.max_seq = a_max_seq; p.n_wgs = a_n_wgs; p.n_splits = a_n_splits; p.self_row = a_self_row;
+  p.k_cache = a_k_cache; p.base_pos = a_base_pos; p.max_seq = a_max_seq; p.n_wgs = a_n_wgs; p.n_splits = a_n_splits; p.self_row = a_self_row & 1u;
+  const bool cols_adjacent = (a_self_row & 2u) != 0;                 // (rides in a preloaded argument: see the workgroup mapping below)
   p.f_q_in = a_f_q_in; p.group = a_group; p.f_q_head_stride = a_f_q_head_stride;
   const uint32_t grid_x = a_grid_x;
   static_assert(!SR || NB == 1, "single-round splits: one 16-row block");
@@ -213,16 +214,30 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   // come last in dispatch order (ids past n_wgs x kv heads) whatever the kv head, so that the ones that wait for a
   // free slot are the short remainder splits; they start when the first workgroups retire and end under the tail of
   // the others.
-  uint32_t sp = blockIdx.x, g = blockIdx.y;
+  uint32_t bx = blockIdx.x, by = blockIdx.y, cg = blockIdx.z;
+  if constexpr (SR && !FUSED && !GATHER) {
+    // A column-exact verify block in one launch (every column a column group of its own, all streaming the same rows):
+    // dispatch id i runs on XCD i % 8, and XCD k takes the (split, kv head) items k, k + 8, ... with the columns of an
+    // item on consecutive ids of that XCD, so that they run side by side and share the rows in its L2.  (The items past
+    // the last multiple of eight come last, a column after the other.)
+    if (__builtin_expect(cols_adjacent, 0)) {
+      const uint32_t items = grid_x * gridDim.y, ncols = gridDim.z, items8 = items & ~7u;
+      const uint32_t lin = bx + grid_x * (by + gridDim.y * cg);
+      uint32_t item;
+      if (lin < items8 * ncols) { const uint32_t k = lin % 8, j = lin / 8; item = (j / ncols) * 8 + k; cg = j % ncols; }
+      else { const uint32_t e = lin - items8 * ncols; item = items8 + e / ncols; cg = e % ncols; }
+      bx = item % grid_x; by = item / grid_x;
+    }
+  }
+  uint32_t sp = bx, g = by;
   if constexpr (SR) {
     const uint32_t nf = p.n_wgs ? min(p.n_wgs, grid_x) : grid_x;
     if (__builtin_expect(nf != grid_x, 0)) {                          // (no remainder splits: the grid's own coordinates)
-      const uint32_t lin = blockIdx.x + grid_x * blockIdx.y;
+      const uint32_t lin = bx + grid_x * by;
       if (lin < nf * gridDim.y) { g = lin / nf; sp = lin % nf; }
       else { const uint32_t e = lin - nf * gridDim.y; g = e % gridDim.y; sp = nf + e / gridDim.y; }
     }
   }
-  uint32_t cg = blockIdx.z;
   if constexpr (!SR) {
     // Tile loop: a one-dimensional grid over (kv head, split, column group) items, column group fastest.  Dispatch
     // id i runs on XCD i % 8 and XCD k owns the contiguous item range [k per, (k + 1) per): the column groups of a
@@ -324,7 +339,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   h4 kx = {0, 0, 0, 0}, vx = {0, 0, 0, 0};
   if constexpr (!FUSED && !GATHER && !Q8) {
     if (self_wave) {
-      const size_t ro = (size_t)p.base_pos * row_bytes + min(lane, (uint32_t)HD / 4 - 1) * 8;
+      const size_t ro = (size_t)(p.base_pos + c0) * row_bytes + min(lane, (uint32_t)HD / 4 - 1) * 8;
       kx = *(const h4*)(kbase + ro);
       vx = *(const h4*)(vbase + ro);
     }
@@ -332,7 +347,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   if constexpr (Q8 && !FUSED) {         // int8 row: widened as the tile path widens it (exact integer x f16-rounded scale, one rounding)
     if (self_wave) {
       const uint32_t l4 = min(lane, (uint32_t)HD / 4 - 1);
-      const size_t ro = (size_t)p.base_pos * HD + 4 * l4, so = ((size_t)p.base_pos * S::SPR + l4 / 8) * 4;
+      const size_t ro = (size_t)(p.base_pos + c0) * HD + 4 * l4, so = ((size_t)(p.base_pos + c0) * S::SPR + l4 / 8) * 4;
       const uint32_t kq = *(const uint32_t*)(kbase8 + ro), vq = *(const uint32_t*)(vbase8 + ro);
       const _Float16 ksc = (_Float16)*(const float*)(ksbase + so), vsc = (_Float16)*(const float*)(vsbase + so);
 #pragma unroll
@@ -1202,7 +1217,9 @@ static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipS
   if (e != hipSuccess) return e;
   if (!SR && col_groups != (p.n_cols + p.cols_per_group - 1) / p.cols_per_group) return hipErrorInvalidValue;
   const dim3 grid = SR ? dim3(p.n_splits, p.n_kv_heads, col_groups) : dim3((p.n_splits * p.n_kv_heads * col_groups + 7) / 8 * 8);
-  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), grid, dim3(W * 64), lds, s, t, p.k_cache, p.base_pos, p.max_seq, p.n_wgs, p.n_splits, p.self_row,
+  // (bit 1 of the self_row argument: the columns of a column-exact block on adjacent dispatch ids of an XCD)
+  const uint32_t self_arg = p.self_row | (SR && p.exact_cols ? 2u : 0u);
+  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), grid, dim3(W * 64), lds, s, t, p.k_cache, p.base_pos, p.max_seq, p.n_wgs, p.n_splits, self_arg,
             (uint32_t)grid.x, p.f_q_in, p.group, p.f_q_head_stride, p);
   return hipGetLastError();
 }
@@ -1283,7 +1300,7 @@ hipError_t pa_launch_decode_gather(const AttnParams& p, uint32_t hd, hipStream_t
 
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t) {
   // many columns, few splits: one thread per (column, head, 4 dims)
-  if (p.n_cols >= 16 && p.n_splits <= 32 && (hd == 256 || hd == 128)) {
+  if (p.n_cols >= 16 && p.n_splits <= 32 && (hd == 256 || hd == 128) && !p.exact_cols) {
     const size_t threads = (size_t)p.n_cols * p.n_heads * (hd / 4);
     const dim3 grid((unsigned)((threads + 255) / 256));
     if (hd == 256) hipLaunchKernelGGL(pa_combine_wide_kernel<256>, grid, dim3(256), 0, s, p);

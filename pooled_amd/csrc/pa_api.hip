@@ -525,7 +525,41 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
     return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned with strides a multiple of 4 elements");
   if (kind == 0 && n_cols > 1 && (c.flags & PA_FLAG_VERIFY_EXACT)) {
     // column-exact verify: every column is the one-column decode at its own position (its own splits, its own row
-    // block), so its bits are those of a sequential decode; the K/V stream is read once per column
+    // block), so its bits are those of a sequential decode.
+    // When the first and the last column have the same one-column plan, the block runs as ONE pass: every column a
+    // column group of its own, each workgroup doing exactly what the one-column launch at that column's position does
+    // -- same splits, same row interleave, own row as a partial -- and the wavefront merge over the columns.  The
+    // columns' workgroups of a (split, kv head) run side by side on one XCD and share the rows in its L2, so the cache
+    // is read from HBM about once.
+    {
+      pa_plan p0, p1;
+      uint32_t w0 = 0, w1 = 0;
+      if (plan_decode(ctx, base_pos, 1, &p0, true, &w0) == PA_OK && plan_decode(ctx, base_pos + n_cols - 1, 1, &p1, true, &w1) == PA_OK &&
+          p0.kernel == 0 && p0.row_blocks == 1 && p0.waves == 4 && plan_self_row(p0) && p0.slots <= 8192 &&
+          p1.split_len == p0.split_len && p1.n_splits == p0.n_splits && p1.slots == p0.slots && p1.row_blocks == 1 && p1.waves == 4 && w0 == w1 &&
+          n_cols <= 65535) {
+        if ((rc = ensure_partials(ctx, n_cols, p0.slots))) return rc;
+        AttnParams p; memset(&p, 0, sizeof p);
+        p.q = d_q; p.gate = d_gate; p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+        p.k_scale = ctx->layers[layer].ks; p.v_scale = ctx->layers[layer].vs;
+        p.part_o = ctx->part_o; p.part_ml = ctx->part_ml; p.out = d_out;
+        p.q_stride = q_stride; p.gate_stride = gate_stride; p.out_stride = out_stride;
+        p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
+        p.base_pos = base_pos; p.n_cols = n_cols;
+        p.split_len = p0.split_len; p.n_splits = p0.n_splits; p.slots = p0.slots; p.cols_per_group = 1;
+        p.self_row = 1; p.n_wgs = w0; p.part_f16 = plan_f16_partials(p0, 1); p.exact_cols = 1;
+        p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
+        p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
+        p.gate_head_stride = c.head_dim;
+        PaTiming tm, tm2;
+        if ((rc = prof_pair(ctx, &tm))) return rc;
+        HIPCHK(ctx, pa_launch_decode(p, c.head_dim, 1, 4, n_cols, ctx->stream, &tm));
+        if ((rc = prof_aux_pair(ctx, tm, &tm2))) return rc;
+        HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream, &tm2));
+        return PA_OK;
+      }
+    }
+    // otherwise one pass per column: the K/V stream is read once per column
     const size_t osz = out_dtype == PA_OUT_F16 ? 2 : 4;
     for (uint32_t col = 0; col < n_cols; col++) {
       rc = attn_common(ctx, who, 0, layer, d_q + (size_t)col * q_stride, q_stride, d_gate ? d_gate + (size_t)col * gate_stride : nullptr, gate_stride,

@@ -61,6 +61,8 @@ struct AttnParams {
   // sel_max: the longest list the pass was sized for; a longer length word is read as sel_max (the list cannot run
   // into the next column's), a length of 0 gives a column of zeros
   const uint32_t* sel; uint32_t sel_stride, sel_max;
+  uint32_t exact_cols;                        // 1: a column-exact verify block in one launch: every column is a column group of its
+                                              // own under the plan of a one-column decode (the merge must be the wavefront kernel)
 };
 
 // ---- kernel launchers (defined next to their kernels) ------------------------------------------

@@ -39,8 +39,8 @@ class HipAttention {
     this.pos = 0;
     this.kvQ8 = !!opts.kvQ8;                                       // int8 caches (engine option kvQ8)
     // verifyExact: every column of a verify block is run as the one-column decode at its position, so it has the bits
-    // of a sequential decode (the reference's invariant, engine/wgsl/attn_dec.js:12-16); the K/V stream is then read
-    // once per column.  Off by default: a block's columns then agree with sequential decodes to rounding only.
+    // of a sequential decode (the reference's invariant, engine/wgsl/attn_dec.js:12-16); every column then does a
+    // one-column decode's work (about 2.3x the default block's time).  Off by default: a block's columns then agree with sequential decodes to rounding only.
     this.verifyExact = !!opts.verifyExact;
     const flags = (this.qkNorm ? PA_FLAG_QK_NORM : 0) | (this.gate ? PA_FLAG_GATE : 0) | (this.kvQ8 ? PA_FLAG_KV_Q8 : 0) | (this.verifyExact ? PA_FLAG_VERIFY_EXACT : 0);
     // a readable throw at create, like the engine's KV binding check (engine/qwen35.js:378-383)
@@ -179,7 +179,7 @@ class HipAttention {
   // Unlike the reference's pair (engine/wgsl/attn_dec.js:12-16) a verify column here equals the one-column decode at
   // the same position to rounding only (|difference| <= 1e-3 by test, 3e-4 measured): the block's columns share
   // matrix-core tiles and splits.  Constructing with { verifyExact: true } restores the bit identity at the cost of
-  // one K/V read per column.
+  // a one-column decode's work per column.
   _encAttnCore(p, LB, M, basePos, nCols) {
     const B = this.B, layer = LB.layer;
     addon.kvStore(this.ctx, layer, B.k.ptr, this._strideF(B.k), B.v.ptr, this._strideF(B.v), basePos, nCols);
