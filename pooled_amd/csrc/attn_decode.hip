@@ -69,6 +69,9 @@ static __device__ inline float rows_sum(float v) {
   xrow32(v, a, b); return a + b;
 }
 // lane i's copy of lane (i + N) % 16 of its row of 16 (DPP row rotation)
+#ifndef PA_ABL_NOLOAD
+#define PA_ABL_NOLOAD 0
+#endif
 template <int N>
 static __device__ inline float row_ror(float v) {
   return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x120 + N, 0xf, 0xf, false));
@@ -189,13 +192,13 @@ template <int HD> struct DecShape {
 // and every wave loops over its own tiles.
 template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
 __global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1))
-void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a_max_seq, uint32_t a_n_wgs, uint32_t a_n_splits, uint32_t a_self_row,
+void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a_max_seq, uint32_t a_n_splits, uint32_t a_self_row,
                       uint32_t a_grid_x, const float* a_f_q_in, uint32_t a_group, uint32_t a_f_q_head_stride, AttnParams p_in) {
   // The leading arguments repeat fields of p_in: the first twelve dwords of a kernel's arguments are preloaded into
   // scalar registers by the dispatcher (-amdgpu-kernarg-preload-count), so what the first tile loads' addresses are made
   // of is there when the wave starts instead of a scalar-load round trip later.
   AttnParams p = p_in;
-  p.k_cache = a_k_cache; p.base_pos = a_base_pos; p.max_seq = a_max_seq; p.n_wgs = a_n_wgs; p.n_splits = a_n_splits; p.self_row = a_self_row & 1u;
+  p.k_cache = a_k_cache; p.base_pos = a_base_pos; p.max_seq = a_max_seq; p.n_splits = a_n_splits; p.self_row = a_self_row & 1u;
   const bool cols_adjacent = (a_self_row & 2u) != 0;                 // (rides in a preloaded argument: see the workgroup mapping below)
   p.f_q_in = a_f_q_in; p.group = a_group; p.f_q_head_stride = a_f_q_head_stride;
   const uint32_t grid_x = a_grid_x;
@@ -210,10 +213,6 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   float* mex = (float*)(stage_all + W * S::STAGE);                   // [W][16*NB]
   float* lex = mex + W * 16 * NB;                                    // [W][16*NB]
 
-  // SR: a context a little past the workgroup slots of the chip has a few more splits than slots.  Their workgroups
-  // come last in dispatch order (ids past n_wgs x kv heads) whatever the kv head, so that the ones that wait for a
-  // free slot are the short remainder splits; they start when the first workgroups retire and end under the tail of
-  // the others.
   uint32_t bx = blockIdx.x, by = blockIdx.y, cg = blockIdx.z;
   if constexpr (SR && !FUSED && !GATHER) {
     // A column-exact verify block in one launch (every column a column group of its own, all streaming the same rows):
@@ -229,15 +228,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       bx = item % grid_x; by = item / grid_x;
     }
   }
-  uint32_t sp = bx, g = by;
-  if constexpr (SR) {
-    const uint32_t nf = p.n_wgs ? min(p.n_wgs, grid_x) : grid_x;
-    if (__builtin_expect(nf != grid_x, 0)) {                          // (no remainder splits: the grid's own coordinates)
-      const uint32_t lin = bx + grid_x * by;
-      if (lin < nf * gridDim.y) { g = lin / nf; sp = lin % nf; }
-      else { const uint32_t e = lin - nf * gridDim.y; g = e % gridDim.y; sp = nf + e / gridDim.y; }
-    }
-  }
+  uint32_t sp = bx, g = by;                                          // SR: the grid's own coordinates
   if constexpr (!SR) {
     // Tile loop: a one-dimensional grid over (kv head, split, column group) items, column group fastest.  Dispatch
     // id i runs on XCD i % 8 and XCD k owns the contiguous item range [k per, (k + 1) per): the column groups of a
@@ -260,26 +251,31 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   // self_row (one-column decode): the column's own row base_pos is not streamed with the others -- see below
   const uint32_t seq_max = GATHER ? min(p.sel[c0 * p.sel_stride], p.sel_max) : p.base_pos + c0 + ncl - p.self_row;
   const uint32_t split_len = SR ? (uint32_t)(W * TILE) : p.split_len;   // single-round splits: one tile per wave
-  const uint32_t t_begin = sp * split_len;
+  // TILV (tile loop on a contiguous cache, p.tile_ilv): the tiles of a kv head are dealt round robin to the waves of
+  // all its splits -- wave v of the n_splits x W takes tiles v, v + n_splits W, ... -- so the loads in flight on the chip
+  // sweep one compact window of the cache per kv head instead of n_splits separate streams a split length apart, and
+  // every split has the same number of tiles to within one.  Any partition of the rows is a valid set of splits.
+  const bool tilv = !SR && !GATHER && p.tile_ilv;
+  const uint32_t t_begin = sp * (tilv ? (uint32_t)(W * TILE) : split_len);
   // The workgroup of split 0 turns the column's own row into a partial of its own (wave 0, while the tile loads are
   // in flight), so it runs even when no other row exists (base_pos == 0).
   const bool self_wg = !GATHER && p.self_row && sp == 0;
   if (t_begin >= seq_max && !self_wg) return;
   const bool has_rows = t_begin < seq_max;
-  // the last split is open-ended: the plan may hand it up to one split length of remainder
-  const uint32_t t_end = !SR && sp + 1 == p.n_splits ? seq_max : min(t_begin + split_len, seq_max);
+  // the last split of contiguous splits is open-ended: a splits override or a gather list may leave it a remainder
+  const uint32_t t_end = (!SR && sp + 1 == p.n_splits) || tilv ? seq_max : min(t_begin + split_len, seq_max);
   const size_t head_rows = (size_t)p.max_seq + TILE;              // rows of one kv head's plane, padding included
   // SR: the whole splits of a kv head are interleaved.  With nw = (whole splits) x W waves, wave v of
   // them takes rows [(c nw + v) 8, + 8), c = 0 .. 3, instead of 32 consecutive ones: at any moment the loads in
   // flight on the chip then sweep a compact range of the cache (4 KB pieces, neighbouring waves on neighbouring
   // pieces) instead of 2048 separate 32 KB streams -- the memory controllers see open pages.  Measured on read-only
   // stand-ins of this launch shape: 11.9 -> 11.2 us for 64 MiB.  Any partition of the rows is a valid set of
-  // splits; masks go by position.  A trailing partial split and the remainder splits keep consecutive rows.
+  // splits; masks go by position.  A trailing partial split keeps consecutive rows.
   constexpr bool ILV = SR && !GATHER;
   uint32_t ilv_nw = 0, ilv_wv = 0;
   bool ilv = false;
   if constexpr (ILV) {
-    const uint32_t nfull = min(p.n_wgs ? p.n_wgs : p.n_splits, seq_max / split_len);
+    const uint32_t nfull = min(p.n_splits, seq_max / split_len);
     ilv = sp < nfull;
     ilv_nw = nfull * W;
     ilv_wv = sp * W + (threadIdx.x >> 6);
@@ -305,7 +301,8 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   const unsigned char* vsbase = (const unsigned char*)(p.v_scale + (Q8 ? (size_t)g * head_rows * S::SPR : 0));
   u4 ksr = {0u, 0u, 0u, 0u}, vsr = {0u, 0u, 0u, 0u};
 
-  const uint32_t n_tiles = has_rows ? (t_end - t_begin + TILE - 1) / TILE : 0;
+  const uint32_t n_tiles = has_rows ? (t_end - t_begin + TILE - 1) / TILE : 0;      // (TILV: tiles from the split's first one to the end)
+  const uint32_t tp_step = tilv ? p.n_splits * (uint32_t)(W * TILE) : (uint32_t)(W * TILE);   // from a wave's tile to its next one
   u4 kr[S::NLD], vr[S::NLD];
   const u4 zero4 = {0u, 0u, 0u, 0u};
   uint32_t tile = __builtin_amdgcn_readfirstlane(wave);
@@ -548,7 +545,8 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   // fixed order; the work hides under the latency of the tile loads.  Decoding a token at a position that is a
   // multiple of the split length therefore streams whole tiles only.
   if (self_wave) {
-    const uint32_t self_slot = min((seq_max + split_len - 1) / split_len, p.n_splits);
+    const uint32_t live_len = tilv ? (uint32_t)(W * TILE) : split_len;     // rows from one split's first row to the next one's
+    const uint32_t self_slot = min((seq_max + live_len - 1) / live_len, p.n_splits);
     const bool on = lane < HD / 4;
     const f4 vxf = { (float)vx[0], (float)vx[1], (float)vx[2], (float)vx[3] };
     for (uint32_t r = 0; r < G; r++) {                                 // one column: row r is head g * G + r
@@ -596,7 +594,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::KROW + (lane % S::LPR) * 16) = kr[i];
     }
-    if (!Q8 && more) {
+    if (!Q8 && more && !PA_ABL_NOLOAD) {
       if constexpr (GATHER) {
         gather_offsets(tpn);
 #pragma unroll
@@ -681,7 +679,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
     }
-    if (!Q8 && more) {
+    if (!Q8 && more && !PA_ABL_NOLOAD) {
       if constexpr (GATHER) {                         // goff still holds the next tile's rows (set with the K loads above)
 #pragma unroll
         for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
@@ -807,10 +805,10 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   float m_run[NB], l_run[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) { m_run[nb] = NEG_INF; l_run[nb] = 0.f; }
-  for (; tile < n_tiles; tile += W) {
-    const uint32_t tp = t_begin + tile * TILE;
-    const bool more = tile + W < n_tiles;
-    stage_k(tp, more, tp + W * TILE);
+  const uint32_t tp_lim = t_begin + n_tiles * TILE;
+  for (uint32_t tp = t_begin + tile * TILE; tp < tp_lim; tp += tp_step) {
+    const bool more = tp + tp_step < tp_lim;
+    stage_k(tp, more, tp + tp_step);
     f4 s[2][NB];
     qk(s);
     // ---- online softmax; lane holds row nb*16 + ln, positions tp + pb*16 + 4*kg + i ----
@@ -865,7 +863,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       l_run[nb] += ps;
     }
     // V after the softmax, so that the wait for the V loads comes as late as possible
-    stage_v(tp, more, tp + W * TILE);
+    stage_v(tp, more, tp + tp_step);
     wave_lds_fence();
     // ---- O^T += V^T P^T ----
     {
@@ -1129,7 +1127,8 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
   if (ch >= (size_t)p.n_cols * p.n_heads) return;
   const uint32_t col = (uint32_t)(ch / p.n_heads), h = (uint32_t)(ch % p.n_heads);
   const uint32_t col_end = p.sel ? min(p.sel[col * p.sel_stride], p.sel_max) : p.base_pos + col + 1 - p.self_row;
-  const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
+  const uint32_t live_len = p.tile_ilv ? p.tile_ilv : p.split_len;      // rows from one split's first row to the next one's
+  const uint32_t ns = min((col_end + live_len - 1) / live_len, p.n_splits) + p.self_row;
   const size_t base = ch * p.slots;
   const float* po = p.part_o + base * HD + 4 * d4;
   const float2* pml = (const float2*)p.part_ml + base;
@@ -1219,7 +1218,7 @@ static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipS
   const dim3 grid = SR ? dim3(p.n_splits, p.n_kv_heads, col_groups) : dim3((p.n_splits * p.n_kv_heads * col_groups + 7) / 8 * 8);
   // (bit 1 of the self_row argument: the columns of a column-exact block on adjacent dispatch ids of an XCD)
   const uint32_t self_arg = p.self_row | (SR && p.exact_cols ? 2u : 0u);
-  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), grid, dim3(W * 64), lds, s, t, p.k_cache, p.base_pos, p.max_seq, p.n_wgs, p.n_splits, self_arg,
+  PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), grid, dim3(W * 64), lds, s, t, p.k_cache, p.base_pos, p.max_seq, p.n_splits, self_arg,
             (uint32_t)grid.x, p.f_q_in, p.group, p.f_q_head_stride, p);
   return hipGetLastError();
 }
@@ -1308,9 +1307,11 @@ hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s, co
     return hipGetLastError();
   }
   const uint32_t gx = p.n_heads * (hd / 16), has_sel = p.sel != nullptr;
+  // rows from one split's first row to the next one's (round-robin tiles: a workgroup's first tiles)
+  const uint32_t live_len = p.tile_ilv ? p.tile_ilv : p.split_len;
   if (hd != 256 && hd != 128) return hipErrorInvalidValue;
 #define PA_COMBINE_WAVE(HD_, F16_) PA_LAUNCH((pa_combine_wave_kernel<HD_, 16, F16_>), dim3(gx, p.n_cols), dim3(64), 0, s, t, (const float*)p.part_o, \
-    (const float*)p.part_ml, p.slots, p.n_heads, p.base_pos, p.self_row, p.split_len, p.n_splits, gx, has_sel, p)
+    (const float*)p.part_ml, p.slots, p.n_heads, p.base_pos, p.self_row, live_len, p.n_splits, gx, has_sel, p)
   if (hd == 256) { if (p.part_f16) PA_COMBINE_WAVE(256, true); else PA_COMBINE_WAVE(256, false); }
   else { if (p.part_f16) PA_COMBINE_WAVE(128, true); else PA_COMBINE_WAVE(128, false); }
 #undef PA_COMBINE_WAVE

@@ -111,10 +111,10 @@ extern "C" int pa_create(const pa_config* cfg, pa_ctx** out) {
       && (e = hipStreamSynchronize(ctx->stream)) == hipSuccess;
     if (!ok) { int rc = fail_hip(nullptr, e, "pa_create: rope table"); pa_destroy(ctx); return rc; }
   }
-  // split partials for a one-column decode at any position: at most two workgroup slots a CU, an eighth more for the
-  // remainder splits, the column's own row (wider passes and split overrides grow the buffers on first use)
+  // split partials for a one-column decode at any position: at most two workgroup slots a CU and the column's own row
+  // (wider passes and split overrides grow the buffers on first use)
   {
-    const uint32_t slots = (2u * (uint32_t)ctx->n_cu / c.n_kv_heads + 1) * 9 / 8 + 2;
+    const uint32_t slots = 2u * (uint32_t)ctx->n_cu / c.n_kv_heads + 2;
     int rc = ensure_partials(ctx, 1, slots);
     if (rc) { g_create_err = ctx->err; pa_destroy(ctx); return rc; }
   }
@@ -309,9 +309,10 @@ extern "C" int pa_kv_store(pa_ctx* ctx, uint32_t layer, const float* d_k, uint32
 // ---- the gfx950 plan table ----------------------------------------------------------------------
 // Decode / verify (split-K kernel): a workgroup is 4 wavefronts, each streaming 32-position tiles of one
 // kv head; rows = columns x G stacked into 16-row MFMA blocks (at most 4 per workgroup, more columns go to
-// further column groups).  Splits are sized so that about two workgroups (one when the row blocks need the
-// whole register file) land on each CU, but never shorter than the tiles-per-wave floor that keeps the
-// partial (m, l, O) traffic a few percent of the K/V bytes.
+// further column groups).  One 16-row block over a context that two workgroups a CU hold as one tile per wave runs
+// on the single-round kernel; everything longer or wider on the tile loop, split so that one workgroup lands on each
+// CU, but never with fewer tiles per wave than the floor that keeps the partial (m, l, O) traffic a few percent of the
+// K/V bytes.
 // self_ok: a one-column decode keeps the column's own row out of the streamed rows (the kernel turns it
 // into one more partial: slots = n_splits + 1), so a token at a multiple of the split length streams whole tiles only.
 static bool plan_self_row(const pa_plan& pl) { return pl.kernel == 0 && pl.slots == pl.n_splits + 1; }
@@ -320,16 +321,19 @@ static bool plan_self_row(const pa_plan& pl) { return pl.kernel == 0 && pl.slots
 // (2^-12 of a 128-row average of V) then enters the output with a weight of a sixty-fourth or less, an order of
 // magnitude under what the f16 probabilities of the MFMA path already cost; shorter contexts, where a partial IS most
 // of the output, and every other pass keep f32 partials.
+// round-robin tiles: the tile loop of the split-K kernel (every plan of that kernel but the single-round one) with more
+// than one split; the value is the distance between the first rows of two splits
+static uint32_t plan_tile_ilv(const pa_plan& pl) {
+  return pl.kernel == 0 && pl.split_len != 32 * pl.waves && pl.n_splits > 1 ? 32 * pl.waves : 0;
+}
 #define PA_F16_PARTIALS_MIN_SPLITS 64u
 static bool plan_f16_partials(const pa_plan& pl, uint32_t n_cols) {
   return pl.kernel == 0 && pl.row_blocks == 1 && pl.split_len == 32 * pl.waves && n_cols < 16 && pl.n_splits >= PA_F16_PARTIALS_MIN_SPLITS;
 }
-// wgs (optional): splits per kv head and column group that fit the chip at once; the single-round kernel dispatches
-// the workgroups of further splits (a short remainder) last.
 // rows_cap (optional): at most this many stacked rows per workgroup (16 or 32) instead of the table's choice;
 // one_split: the whole context as one split per workgroup -- with no own-row partial the kernel then writes the
 // output itself (no partials, no merge launch).  Both are what plan_prefill asks for on small chunks.
-static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, bool self_ok = true, uint32_t* wgs = nullptr,
+static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, bool self_ok = true,
                        uint32_t rows_cap = 0, bool one_split = false) {
   const pa_config& c = ctx->cfg;
   const uint32_t G = c.n_heads / c.n_kv_heads;
@@ -356,27 +360,32 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
   const uint32_t seq_max = std::max(base_pos + n_cols - self, 1u);   // streamed rows (position 0 alone: one empty split)
   const uint32_t tiles = ceil_div(seq_max, 32);
   const uint32_t occ = nb == 1 ? 2 : 1;
-  uint32_t target = ctx->decode_splits_override ? ctx->decode_splits_override
-                                                : std::max(1u, (occ * (uint32_t)ctx->n_cu) / (c.n_kv_heads * groups));
-  uint32_t tpw = std::max(ceil_div(tiles, target * W), ctx->decode_splits_override ? 1u : floor_tiles[nb]);
-  if (one_split) tpw = std::max(ceil_div(tiles, W), 1u);
-  uint32_t sl = 32 * W * tpw, ns = ceil_div(seq_max, sl);
-  // A context a little past target x split_len (a 32K context plus the token being decoded) would double the
-  // split length and leave half the workgroup slots empty, or spill a near-empty split into a second round of
-  // workgroups.  The last split takes the remainder instead (the kernels treat split n_splits - 1 as open-ended),
-  // as long as that is less than one more split.
-  if (!ctx->decode_splits_override && !one_split && tpw > floor_tiles[nb]) {
-    const uint32_t tpw_lo = std::max(tiles / (target * W), floor_tiles[nb]), sl_lo = 32 * W * tpw_lo;
-    if ((uint64_t)seq_max < (uint64_t)(target + 1) * sl_lo) { sl = sl_lo; ns = std::max(1u, std::min(target, seq_max / sl_lo)); }
-    // one tile per wave: up to an eighth more splits than slots stay single-round splits (their workgroups start as
-    // the first ones retire and end under the tail of the rest)
-    else if (nb == 1 && tpw_lo == 1 && (uint64_t)seq_max <= (uint64_t)(target + target / 8) * sl_lo) sl = sl_lo;
+  const uint32_t target = ctx->decode_splits_override ? ctx->decode_splits_override
+                                                      : std::max(1u, (occ * (uint32_t)ctx->n_cu) / (c.n_kv_heads * groups));
+  uint32_t sl, ns;
+  if (one_split || ctx->decode_splits_override) {
+    // a given number of splits (a tuning override; its splits are contiguous ranges, the last one open-ended), or one
+    const uint32_t tpw = one_split ? std::max(ceil_div(tiles, W), 1u) : std::max(ceil_div(tiles, target * W), 1u);
+    sl = 32 * W * tpw; ns = ceil_div(seq_max, sl);
+  } else if (nb == 1 && ceil_div(seq_max, 32 * W) <= target) {
+    // One 16-row block and no more one-tile-per-wave splits than two workgroups a CU hold at once: the single-round
+    // kernel, the whole context in flight in one go.  A single split more would run as a second round behind the
+    // first (measured, MoE shape: 32768 rows 16.3 us, 32800 rows 19.7 us, against 18.8 us on the tile loop below).
+    sl = 32 * W; ns = ceil_div(seq_max, sl);
+  } else {
+    // The tile loop, and there ONE workgroup a CU is the target whatever the row blocks: a workgroup keeps 128 KB of
+    // K/V loads in flight, which saturates the memory system from half the CUs on; a second one on the CU only adds
+    // its fixed costs (start-up, the merge of its waves, its partials, a longer merge pass) and, measured on read-only
+    // stand-ins of the loop, lowers the stream's rate (256 MiB: 46 us with one workgroup a CU, 56 - 60 us with two).
+    // Measured, one column: MoE shape at 40000 / 65536 / 131072 rows 24.2 -> 21.0, 32.6 -> 28.9, 56.3 -> 49.7 us; 27B
+    // shape at 65536 rows 57.2 -> 52.6 us.  The loop deals a kv head's tiles round robin to the waves of all its
+    // splits (AttnParams::tile_ilv), so any number of splits is balanced to within a tile and split_len is nominal:
+    // the rows of a split's tiles, rounded up.  Never fewer tiles per wave than the floor that keeps the partial
+    // (m, l, O) traffic a few percent of the K/V bytes.
+    const uint32_t target1 = std::max(1u, (uint32_t)ctx->n_cu / (c.n_kv_heads * groups));
+    ns = std::max(1u, std::min(target1, tiles / (W * floor_tiles[nb])));
+    sl = 32 * W * ceil_div(tiles, ns * W);
   }
-  uint32_t n_wg = ns;
-  // One 16-row block and one tile per wave: the single-round kernel.  Its splits are all whole (no open-ended last
-  // one); a remainder past the workgroup slots is a few more splits.
-  if (nb == 1 && sl == 32 * W) { ns = ceil_div(seq_max, sl); n_wg = std::min(ns, target); }
-  if (wgs) *wgs = n_wg;
   pl->kernel = 0; pl->split_len = sl; pl->n_splits = ns;
   pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = W; pl->row_blocks = nb; pl->slots = pl->n_splits + self;
   return PA_OK;
@@ -386,14 +395,14 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
 // floor(256 / G) columns x G heads.  Chunks wide enough to give every CU a workgroup run unsplit and write the
 // output directly; narrower chunks are also split over the context (partials + merge kernel) until every CU has a
 // workgroup (one is resident per CU; a second round of a few workgroups costs more than longer splits).  Chunks of fewer rows than one wavefront tile go to the split-K decode kernel.
-static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl, uint32_t* wgs = nullptr) {
+static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa_plan* pl) {
   const pa_config& c = ctx->cfg;
   const uint32_t G = c.n_heads / c.n_kv_heads;
   const uint32_t max_rows_sk = c.head_dim == 256 ? 32u : 64u;
-  if (n_cols * G <= max_rows_sk) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
+  if (n_cols * G <= max_rows_sk) return plan_decode(ctx, base_pos, n_cols, pl, true);
   // pa_set_prefill_tile: 2 = never the matrix-core kernel (where the split-K kernel can hold a column's heads),
   // 1 = always (the two table rules below are skipped), 0 = the table
-  if (ctx->prefill_tile_mode == 2 && max_rows_sk >= G) return plan_decode(ctx, base_pos, n_cols, pl, true, wgs);
+  if (ctx->prefill_tile_mode == 2 && max_rows_sk >= G) return plan_decode(ctx, base_pos, n_cols, pl, true);
   const bool table = ctx->prefill_tile_mode == 0;
   // A chunk of a few column groups over a long context (the reference's own prefill passes are 16 columns wide) is
   // bound by the K/V stream, not by the matrix cores: the split-K kernel serves it in column groups, whose workgroups
@@ -401,10 +410,10 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
   // (Q staging, one partial per split and row, the merge) amount to.  Measured crossover on the MoE and 27B shapes
   // at 32K - 64K rows: about 1.4 GB of L2-level K/V traffic; below 4096 rows both kernels take 25 - 40 us.
   if (table && n_cols * G <= 512 && base_pos + n_cols >= 4096 && max_rows_sk >= G) {
-    pa_plan sk; uint32_t sk_wgs = 0;
+    pa_plan sk;
     const uint64_t kv_bytes = 2ull * (base_pos + n_cols) * c.n_kv_heads * c.head_dim * (kv_q8(ctx) ? 1 : 2);
-    if (plan_decode(ctx, base_pos, n_cols, &sk, true, &sk_wgs) == PA_OK && (uint64_t)sk.col_groups * kv_bytes <= 1400000000ull) {
-      *pl = sk; if (wgs) *wgs = sk_wgs;
+    if (plan_decode(ctx, base_pos, n_cols, &sk, true) == PA_OK && (uint64_t)sk.col_groups * kv_bytes <= 1400000000ull) {
+      *pl = sk;
       return PA_OK;
     }
   }
@@ -423,7 +432,7 @@ static int plan_prefill(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, p
       const uint32_t rows = (uint64_t)ceil_div(n_cols, 32 / G) * c.n_kv_heads >= (uint64_t)ctx->n_cu ? 32u : 16u;
       // one split per workgroup only pays when the column groups alone occupy the chip (or the context is a few tiles)
       if ((uint64_t)ceil_div(n_cols, rows / G) * c.n_kv_heads * 2 >= (uint64_t)ctx->n_cu || base_pos + n_cols <= 256)
-        return plan_decode(ctx, base_pos, n_cols, pl, true, wgs, rows, true);
+        return plan_decode(ctx, base_pos, n_cols, pl, true, rows, true);
     }
   }
   const uint32_t rows_wg = 256;
@@ -533,10 +542,11 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
     // is read from HBM about once.
     {
       pa_plan p0, p1;
-      uint32_t w0 = 0, w1 = 0;
-      if (plan_decode(ctx, base_pos, 1, &p0, true, &w0) == PA_OK && plan_decode(ctx, base_pos + n_cols - 1, 1, &p1, true, &w1) == PA_OK &&
+      if (plan_decode(ctx, base_pos, 1, &p0, true) == PA_OK && plan_decode(ctx, base_pos + n_cols - 1, 1, &p1, true) == PA_OK &&
           p0.kernel == 0 && p0.row_blocks == 1 && p0.waves == 4 && plan_self_row(p0) && p0.slots <= 8192 &&
-          p1.split_len == p0.split_len && p1.n_splits == p0.n_splits && p1.slots == p0.slots && p1.row_blocks == 1 && p1.waves == 4 && w0 == w1 &&
+          // (round-robin tiles: the split length is nominal, the splits are the same whenever their number is)
+          (p1.split_len == p0.split_len || (plan_tile_ilv(p0) && plan_tile_ilv(p1))) &&
+          p1.n_splits == p0.n_splits && p1.slots == p0.slots && p1.row_blocks == 1 && p1.waves == 4 &&
           n_cols <= 65535) {
         if ((rc = ensure_partials(ctx, n_cols, p0.slots))) return rc;
         AttnParams p; memset(&p, 0, sizeof p);
@@ -547,7 +557,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
         p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
         p.base_pos = base_pos; p.n_cols = n_cols;
         p.split_len = p0.split_len; p.n_splits = p0.n_splits; p.slots = p0.slots; p.cols_per_group = 1;
-        p.self_row = 1; p.n_wgs = w0; p.part_f16 = plan_f16_partials(p0, 1); p.exact_cols = 1;
+        p.self_row = 1; p.part_f16 = plan_f16_partials(p0, 1); p.exact_cols = 1; p.tile_ilv = plan_tile_ilv(p0);
         p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
         p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
         p.gate_head_stride = c.head_dim;
@@ -569,8 +579,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
     return PA_OK;
   }
   pa_plan pl;
-  uint32_t n_wgs = 0;
-  rc = kind == 0 ? plan_decode(ctx, base_pos, n_cols, &pl, true, &n_wgs) : plan_prefill(ctx, base_pos, n_cols, &pl, &n_wgs);
+  rc = kind == 0 ? plan_decode(ctx, base_pos, n_cols, &pl, true) : plan_prefill(ctx, base_pos, n_cols, &pl);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
   // one split and no own-row partial: the kernel writes the output itself (the prefill kernel, or the split-K kernel's
@@ -607,7 +616,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   p.self_row = plan_self_row(pl) ? 1 : 0;
   p.direct_out = direct && pl.kernel == 0 ? 1 : 0;
   p.part_f16 = !direct && plan_f16_partials(pl, n_cols);
-  p.n_wgs = pl.kernel == 0 ? n_wgs : 0;
+  p.tile_ilv = plan_tile_ilv(pl);
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   p.gate_head_stride = c.head_dim;
@@ -649,8 +658,7 @@ static int decode_step_common(pa_ctx* ctx, const char* who, bool static_scratch,
     return fail(ctx, PA_ERR_INVALID, std::string(who) + ": buffers must be 16-byte aligned");
   if (c.n_heads / c.n_kv_heads > 16) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": more than 16 query heads per kv head");
   pa_plan pl;
-  uint32_t n_wgs = 0;
-  rc = plan_decode(ctx, pos, 1, &pl, true, &n_wgs);
+  rc = plan_decode(ctx, pos, 1, &pl, true);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (pl.slots > 8192) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": too many splits");
   if (pl.row_blocks != 1 || pl.waves != 4 || pl.col_groups != 1 || !plan_self_row(pl)) return fail(ctx, PA_ERR_UNSUPPORTED, std::string(who) + ": plan is not a one-block decode");
@@ -673,7 +681,7 @@ static int decode_step_common(pa_ctx* ctx, const char* who, bool static_scratch,
   p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
   p.base_pos = pos; p.n_cols = 1;
   p.split_len = pl.split_len; p.n_splits = pl.n_splits; p.slots = pl.slots; p.cols_per_group = pl.cols_per_group;
-  p.self_row = 1; p.n_wgs = n_wgs; p.part_f16 = plan_f16_partials(pl, 1);
+  p.self_row = 1; p.part_f16 = plan_f16_partials(pl, 1); p.tile_ilv = plan_tile_ilv(pl);
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   // the pre-step inputs; the gate is read in place from the interleaved [q | gate] heads
@@ -950,14 +958,12 @@ extern "C" int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d
   // splits over list positions: the table's choice for one column of max_rows rows (an identity list then runs
   // exactly the dense decode), thinned when several columns share the chip
   pa_plan pl;
-  uint32_t n_wgs = 0;
-  rc = plan_decode(ctx, max_rows - 1, 1, &pl, false, &n_wgs);
+  rc = plan_decode(ctx, max_rows - 1, 1, &pl, false);
   if (rc) return fail(ctx, rc, std::string(who) + ": shape outside the gfx950 table");
   if (n_cols > 1 && pl.n_splits > 1) {
     const uint32_t want = std::max(1u, pl.n_splits / n_cols);
     pl.split_len = ceil_div(ceil_div(max_rows, want), 128) * 128;
     pl.n_splits = ceil_div(max_rows, pl.split_len);
-    n_wgs = 0;                                  // one workgroup per split
   }
   pl.slots = pl.n_splits;
   if ((rc = ensure_partials(ctx, n_cols, pl.slots))) return rc;
@@ -971,7 +977,7 @@ extern "C" int pa_attn_decode_gather(pa_ctx* ctx, uint32_t layer, const float* d
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   p.gate_head_stride = c.head_dim;
-  p.sel = d_sel; p.sel_stride = sel_stride; p.sel_max = std::min(max_rows, sel_stride - 1); p.n_wgs = n_wgs;
+  p.sel = d_sel; p.sel_stride = sel_stride; p.sel_max = std::min(max_rows, sel_stride - 1);
   p.part_f16 = pl.split_len == 32 * 4 && n_cols < 16 && pl.n_splits >= PA_F16_PARTIALS_MIN_SPLITS;   // (as plan_f16_partials)
   PaTiming tm;
   if ((rc = prof_pair(ctx, &tm))) return rc;

@@ -37,8 +37,6 @@ struct AttnParams {
   uint32_t n_heads, n_kv_heads, group;        // group = nH / nKV
   uint32_t base_pos, n_cols;                  // column c sees rows [0, base_pos + c]
   uint32_t split_len, n_splits, slots;
-  uint32_t n_wgs;                             // single-round decode kernel: splits per kv head whose workgroups are
-                                              // dispatched first (the rest, a remainder past the chip's slots, last); 0 = all
   uint32_t cols_per_group;                    // columns per workgroup (grid z = column groups)
   uint32_t max_seq;
   uint32_t self_row;                          // 1: one-column decode whose own row base_pos is a partial of its own (slot
@@ -63,6 +61,9 @@ struct AttnParams {
   const uint32_t* sel; uint32_t sel_stride, sel_max;
   uint32_t exact_cols;                        // 1: a column-exact verify block in one launch: every column is a column group of its
                                               // own under the plan of a one-column decode (the merge must be the wavefront kernel)
+  uint32_t tile_ilv;                          // tile loop of the split-K kernel on a contiguous cache: rows from one split's first tile
+                                              // to the next split's (32 x waves) when the tiles of a kv head are dealt round robin to the
+                                              // waves of all its splits; 0 = every split a contiguous range of split_len rows
 };
 
 // ---- kernel launchers (defined next to their kernels) ------------------------------------------
