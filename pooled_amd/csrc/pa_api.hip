@@ -384,7 +384,13 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
     // (m, l, O) traffic a few percent of the K/V bytes.
     const uint32_t target1 = std::max(1u, (uint32_t)ctx->n_cu / (c.n_kv_heads * groups));
     ns = std::max(1u, std::min(target1, tiles / (W * floor_tiles[nb])));
-    sl = 32 * W * ceil_div(tiles, ns * W);
+    // ... and the fewest splits with that many tiles per wave: 2049 tiles over 256 waves are nine rounds for one wave
+    // and eight for the rest, the ninth a round trip for 16 KB; over 228 waves they are nine full rounds of fewer bytes
+    // (27B shape, 8 columns at 65536: 59.6 -> 58.5 us; MoE shape, one column at 34000 / 50000 / 100000 rows: 21.3 ->
+    // 19.1, 26.9 -> 24.2, 42.5 -> 40.4 us).
+    const uint32_t tpw = ceil_div(tiles, ns * W);
+    ns = ceil_div(tiles, tpw * W);
+    sl = 32 * W * tpw;
   }
   pl->kernel = 0; pl->split_len = sl; pl->n_splits = ns;
   pl->col_groups = groups; pl->cols_per_group = cw; pl->waves = W; pl->row_blocks = nb; pl->slots = pl->n_splits + self;
@@ -535,27 +541,40 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   if (kind == 0 && n_cols > 1 && (c.flags & PA_FLAG_VERIFY_EXACT)) {
     // column-exact verify: every column is the one-column decode at its own position (its own splits, its own row
     // block), so its bits are those of a sequential decode.
-    // When the first and the last column have the same one-column plan, the block runs as ONE pass: every column a
-    // column group of its own, each workgroup doing exactly what the one-column launch at that column's position does
-    // -- same splits, same row interleave, own row as a partial -- and the wavefront merge over the columns.  The
-    // columns' workgroups of a (split, kv head) run side by side on one XCD and share the rows in its L2, so the cache
-    // is read from HBM about once.
-    {
+    // A run of columns with the same one-column plan is ONE pass: every column a column group of its own, each
+    // workgroup doing exactly what the one-column launch at that column's position does -- same splits, same row
+    // order, own row as a partial -- and the wavefront merge over the columns.  The columns' workgroups of a (split,
+    // kv head) run side by side on one XCD and share the rows in its L2, so the cache is read from HBM about once.
+    // The plan moves at few positions (a split more on the single-round kernel every 128 rows, a tile per wave more
+    // on the tile loop every few thousand), so a block is one run, or two.
+    auto one_col_plan = [&](uint32_t pos, pa_plan* pl) -> bool {
+      return plan_decode(ctx, pos, 1, pl, true) == PA_OK && pl->kernel == 0 && pl->row_blocks == 1 && pl->waves == 4 && plan_self_row(*pl) &&
+             pl->slots <= 8192;
+    };
+    // (round-robin tiles: the split length is nominal, the splits are the same whenever their number is)
+    auto same_plan = [&](const pa_plan& a, const pa_plan& b) -> bool {
+      return (a.split_len == b.split_len || (plan_tile_ilv(a) && plan_tile_ilv(b))) && a.n_splits == b.n_splits && a.slots == b.slots;
+    };
+    const size_t osz = out_dtype == PA_OUT_F16 ? 2 : 4;
+    for (uint32_t col = 0; col < n_cols;) {
       pa_plan p0, p1;
-      if (plan_decode(ctx, base_pos, 1, &p0, true) == PA_OK && plan_decode(ctx, base_pos + n_cols - 1, 1, &p1, true) == PA_OK &&
-          p0.kernel == 0 && p0.row_blocks == 1 && p0.waves == 4 && plan_self_row(p0) && p0.slots <= 8192 &&
-          // (round-robin tiles: the split length is nominal, the splits are the same whenever their number is)
-          (p1.split_len == p0.split_len || (plan_tile_ilv(p0) && plan_tile_ilv(p1))) &&
-          p1.n_splits == p0.n_splits && p1.slots == p0.slots && p1.row_blocks == 1 && p1.waves == 4 &&
-          n_cols <= 65535) {
-        if ((rc = ensure_partials(ctx, n_cols, p0.slots))) return rc;
+      uint32_t run = 1;
+      if (one_col_plan(base_pos + col, &p0))
+        while (col + run < n_cols && run < 65535 && one_col_plan(base_pos + col + run, &p1) && same_plan(p0, p1)) run++;
+      const float* q_c = d_q + (size_t)col * q_stride;
+      const float* gate_c = d_gate ? d_gate + (size_t)col * gate_stride : nullptr;
+      void* out_c = (unsigned char*)d_out + (size_t)col * out_stride * osz;
+      if (run == 1) {                 // a column on its own: the one-column decode itself
+        if ((rc = attn_common(ctx, who, 0, layer, q_c, q_stride, gate_c, gate_stride, base_pos + col, 1, out_c, out_stride, out_dtype))) return rc;
+      } else {
+        if ((rc = ensure_partials(ctx, run, p0.slots))) return rc;
         AttnParams p; memset(&p, 0, sizeof p);
-        p.q = d_q; p.gate = d_gate; p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
+        p.q = q_c; p.gate = gate_c; p.k_cache = ctx->layers[layer].k; p.v_cache = ctx->layers[layer].v;
         p.k_scale = ctx->layers[layer].ks; p.v_scale = ctx->layers[layer].vs;
-        p.part_o = ctx->part_o; p.part_ml = ctx->part_ml; p.out = d_out;
+        p.part_o = ctx->part_o; p.part_ml = ctx->part_ml; p.out = out_c;
         p.q_stride = q_stride; p.gate_stride = gate_stride; p.out_stride = out_stride;
         p.n_heads = c.n_heads; p.n_kv_heads = c.n_kv_heads; p.group = c.n_heads / c.n_kv_heads;
-        p.base_pos = base_pos; p.n_cols = n_cols;
+        p.base_pos = base_pos + col; p.n_cols = run;
         p.split_len = p0.split_len; p.n_splits = p0.n_splits; p.slots = p0.slots; p.cols_per_group = 1;
         p.self_row = 1; p.part_f16 = plan_f16_partials(p0, 1); p.exact_cols = 1; p.tile_ilv = plan_tile_ilv(p0);
         p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
@@ -563,18 +582,11 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
         p.gate_head_stride = c.head_dim;
         PaTiming tm, tm2;
         if ((rc = prof_pair(ctx, &tm))) return rc;
-        HIPCHK(ctx, pa_launch_decode(p, c.head_dim, 1, 4, n_cols, ctx->stream, &tm));
+        HIPCHK(ctx, pa_launch_decode(p, c.head_dim, 1, 4, run, ctx->stream, &tm));
         if ((rc = prof_aux_pair(ctx, tm, &tm2))) return rc;
         HIPCHK(ctx, pa_launch_combine(p, c.head_dim, ctx->stream, &tm2));
-        return PA_OK;
       }
-    }
-    // otherwise one pass per column: the K/V stream is read once per column
-    const size_t osz = out_dtype == PA_OUT_F16 ? 2 : 4;
-    for (uint32_t col = 0; col < n_cols; col++) {
-      rc = attn_common(ctx, who, 0, layer, d_q + (size_t)col * q_stride, q_stride, d_gate ? d_gate + (size_t)col * gate_stride : nullptr, gate_stride,
-                       base_pos + col, 1, (unsigned char*)d_out + (size_t)col * out_stride * osz, out_stride, out_dtype);
-      if (rc) return rc;
+      col += run;
     }
     return PA_OK;
   }

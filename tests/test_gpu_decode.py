@@ -125,14 +125,15 @@ def test_verify_equals_sequential_decodes(shape, n_cols, base):
 
 @pytest.mark.parametrize("shape,n_cols,base", [("qwen36_moe", 4, 996), ("qwen38_27b", 8, 2040), ("qwen3_1p7b", 5, 510), ("qwen36_moe", 3, 32767),
                                                ("qwen36_moe", 8, 9000), ("qwen36_moe", 16, 20000), ("qwen38_27b", 6, 8190), ("qwen3_1p7b", 13, 119),
-                                               ("qwen36_moe", 5, 40000), ("qwen38_27b", 4, 33000)])
+                                               ("qwen36_moe", 5, 40000), ("qwen38_27b", 4, 33000), ("qwen38_27b", 8, 65533)])
 def test_verify_exact_flag_gives_the_sequential_decodes_bits(shape, n_cols, base):
     """PA_FLAG_VERIFY_EXACT: every column of a verify block has the bits of the one-column decode at its position
     (the reference's invariant, engine/wgsl/attn_dec.js:12-16; tests/test_attn_dec.js:89-97 checks it with Object.is);
     the plan a plan query reports is unchanged.  Blocks whose columns share a one-column plan run as one pass (the first
     three cases and the 9000- and 20000-row ones, with f16 partials on the last two; the 40000- and 33000-row ones on the
-    tile loop's longer splits); blocks that straddle a change of plan (32767 .. 32769, 8190 .. 8195, 119 .. 131) fall
-    back to one pass per column."""
+    tile loop's longer splits); blocks that straddle a change of plan (32767 .. 32769, 8190 .. 8195, 119 .. 131, and
+    65536 .. 65543 of the 27B shape, where the tile loop goes from eight to nine tiles a wave) run as one pass per run of
+    columns with the same plan, a lone column as the one-column decode itself."""
     cfg = dict(SHAPES[shape], verify_exact=True)
     rng = np.random.default_rng(base + n_cols)
     L = base + n_cols
