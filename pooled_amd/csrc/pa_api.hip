@@ -311,8 +311,7 @@ extern "C" int pa_kv_store(pa_ctx* ctx, uint32_t layer, const float* d_k, uint32
 // kv head; rows = columns x G stacked into 16-row MFMA blocks (at most 4 per workgroup, more columns go to
 // further column groups).  One 16-row block over a context that two workgroups a CU hold as one tile per wave runs
 // on the single-round kernel; everything longer or wider on the tile loop, split so that one workgroup lands on each
-// CU, but never with fewer tiles per wave than the floor that keeps the partial (m, l, O) traffic a few percent of the
-// K/V bytes.
+// CU (down to one tile per wave on short contexts).
 // self_ok: a one-column decode keeps the column's own row out of the streamed rows (the kernel turns it
 // into one more partial: slots = n_splits + 1), so a token at a multiple of the split length streams whole tiles only.
 static bool plan_self_row(const pa_plan& pl) { return pl.kernel == 0 && pl.slots == pl.n_splits + 1; }
@@ -337,15 +336,14 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
                        uint32_t rows_cap = 0, bool one_split = false) {
   const pa_config& c = ctx->cfg;
   const uint32_t G = c.n_heads / c.n_kv_heads;
-  static const uint32_t floor_tiles[5] = {1, 1, 4, 6, 8};     // tiles per wave, by row blocks
   // rows per workgroup: 16-row blocks whose O^T accumulators fit the register file next to the
   // in-flight K/V tile (hd 256: 2 blocks, 3 in the case below; hd 128: 4 blocks)
   // hd 256: three blocks (48 rows) when that saves a column group and the context is long enough to fill the chip
-  // with splits of the three-block tile floor (27B shape, 8 columns at 64K: one group of 48 rows instead of two)
+  // with splits of six tiles a wave (27B shape, 8 columns at 64K: one group of 48 rows instead of two)
   uint32_t max_rows = c.head_dim == 256 ? 32 : 64;
   if (c.head_dim == 256 && n_cols * G > 32 && 48 / G > 0) {
     const uint32_t g32 = ceil_div(n_cols, 32 / G), g48 = ceil_div(n_cols, 48 / G);
-    const uint32_t splits48 = ceil_div(base_pos + n_cols, 32) / (floor_tiles[3] * 4);
+    const uint32_t splits48 = ceil_div(base_pos + n_cols, 32) / (6 * 4);
     if (g48 < g32 && !ctx->decode_splits_override && (uint64_t)splits48 * c.n_kv_heads * g48 >= (uint64_t)ctx->n_cu) max_rows = 48;
   }
   if (rows_cap) max_rows = rows_cap;
@@ -380,10 +378,13 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
     // Measured, one column: MoE shape at 40000 / 65536 / 131072 rows 24.2 -> 21.0, 32.6 -> 28.9, 56.3 -> 49.7 us; 27B
     // shape at 65536 rows 57.2 -> 52.6 us.  The loop deals a kv head's tiles round robin to the waves of all its
     // splits (AttnParams::tile_ilv), so any number of splits is balanced to within a tile and split_len is nominal:
-    // the rows of a split's tiles, rounded up.  Never fewer tiles per wave than the floor that keeps the partial
-    // (m, l, O) traffic a few percent of the K/V bytes.
+    // the rows of a split's tiles, rounded up.  No floor on the tiles per wave: short and mid-length verify blocks are
+    // bound by the chain of a wave's tiles, not by the bytes of the partials (a former floor of 4 / 6 / 8 tiles a wave
+    // with 2 / 3 / 4 row blocks, meant to keep the partials a few percent of the K/V bytes, left most CUs without a
+    // workgroup: MoE shape, 4 columns at 4096 / 8192 / 16384 rows 20.5 -> 15.9, 20.7 -> 16.3, 21.1 -> 17.7 us; dense
+    // hd-128 shape, 32 columns at 4096 / 8192 rows 26.6 -> 19.0, 26.6 -> 20.4 us).
     const uint32_t target1 = std::max(1u, (uint32_t)ctx->n_cu / (c.n_kv_heads * groups));
-    ns = std::max(1u, std::min(target1, tiles / (W * floor_tiles[nb])));
+    ns = std::max(1u, std::min(target1, tiles / W));
     // ... and the fewest splits with that many tiles per wave: 2049 tiles over 256 waves are nine rounds for one wave
     // and eight for the rest, the ninth a round trip for 16 KB; over 228 waves they are nine full rounds of fewer bytes
     // (27B shape, 8 columns at 65536: 59.6 -> 58.5 us; MoE shape, one column at 34000 / 50000 / 100000 rows: 21.3 ->

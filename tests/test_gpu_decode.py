@@ -261,23 +261,23 @@ def test_c4_verify_64k():
             assert np.abs(single[0] - multi[c]).max() <= 1e-3
 
 
-@pytest.mark.parametrize("shape,n_cols,base,blocks", [("qwen36_moe", 1, 40000, 1), ("qwen36_moe", 4, 6000, 2),
+@pytest.mark.parametrize("shape,n_cols,base,blocks", [("qwen36_moe", 1, 40000, 1), ("qwen36_moe", 4, 40000, 2),
                                                        ("qwen38_27b", 8, 50000, 3)])
 def test_decode_growing_maximum(shape, n_cols, base, blocks):
-    """Scores that jump along the context: K rows alternate between a scale of 0.1 and a scale of 3 every 128 rows,
-    so every wave of the tile loop (tiles w, w + 4, ...) meets a low tile first and then row maxima far beyond the
-    threshold of its lazily updated reference maximum, and has to take the rescale path -- with one, two and three
-    row blocks per workgroup."""
+    """Scores that jump along the context: K rows alternate between a scale of 0.1 and a scale of 4 every eighth of the
+    context, so every wave of the tile loop (its tiles are spread over the whole context, three or more a wave) meets low
+    tiles first and then row maxima far beyond the threshold of its lazily updated reference maximum, and has to take the
+    rescale path -- with one, two and three row blocks per workgroup."""
     cfg = SHAPES[shape]
     rng = np.random.default_rng(base + n_cols)
     rows = base + n_cols
     shp = (rows, cfg["n_kv_heads"], cfg["head_dim"])
-    scale = np.where((np.arange(rows) // 128) % 2 == 0, 0.1, 3.0).astype(np.float32)[:, None, None]
+    scale = np.where((np.arange(rows) // (rows // 8)) % 2 == 0, 0.1, 4.0).astype(np.float32)[:, None, None]
     k16 = (rng.standard_normal(shp, dtype=np.float32) * scale).astype(np.float16).view(np.uint16)
     v16 = rng.standard_normal(shp, dtype=np.float32).astype(np.float16).view(np.uint16)
     q = rng.standard_normal((n_cols, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
     ref = C.attention(q, k16, v16, base)
     with _ctx_with_cache(cfg, k16, v16, rows, max_cols=n_cols) as pa:
         plan = pa.plan("decode", base, n_cols)
-        assert plan["row_blocks"] == blocks and plan["split_len"] > 128, plan     # the tile loop, not single-round splits
+        assert plan["row_blocks"] == blocks and plan["split_len"] >= 3 * 128, plan     # the tile loop, three tiles a wave or more
         assert_parity(pa.run_attn("decode", 0, q, base), ref, "jumping maximum, %d row blocks" % blocks)
