@@ -241,6 +241,23 @@ def test_decode_past_the_single_round_capacity(extra):
     assert_parity(got, ref, "open-ended last split, +%d rows" % extra)
 
 
+def test_decode_one_column_at_128k():
+    """A one-column decode over 131072 cached rows (MoE shape): the tile loop with one workgroup a CU, a kv head's 4096
+    tiles dealt round robin to the 512 waves of its 128 splits, eight a wave; with a gate, f32 and f16 out."""
+    cfg = SHAPES["qwen36_moe"]
+    pos = 131072
+    rng = np.random.default_rng(131)
+    k16, v16 = random_cache(cfg, pos + 1, seed=132)
+    q = rng.standard_normal((1, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    gate = rng.standard_normal(q.shape, dtype=np.float32)
+    ref = C.attention(q, k16, v16, pos, gate=gate)
+    with _ctx_with_cache(cfg, k16, v16, pos + 1, max_cols=1) as pa:
+        pl = pa.plan("decode", pos, 1)
+        assert pl["n_splits"] == 128 and pl["split_len"] == 1024 and pl["slots"] == 129 and pl["row_blocks"] == 1, pl
+        for out_dtype in (0, PA_OUT_F16):
+            assert_parity(pa.run_attn("decode", 0, q, pos, gate=gate, out_dtype=out_dtype), ref, "decode at 128K", tight=True)
+
+
 def test_c4_verify_64k():
     """Config 4: 8-token draft block over a 65536-token cache, Qwen3.8-27B attention shape, gate; equals 8
     sequential decodes (checked on columns 0 and 7) and the oracle."""

@@ -103,7 +103,8 @@ def test_q8_verify_block_prefill_chunk_and_slots():
         assert e.value.code == PA_ERR_UNSUPPORTED
 
 
-@pytest.mark.parametrize("shape,pos", [("qwen36_moe", 0), ("qwen36_moe", 1), ("qwen36_moe", 777), ("qwen36_moe", 4096), ("qwen3_1p7b", 300), ("qwen38_27b", 129)])
+@pytest.mark.parametrize("shape,pos", [("qwen36_moe", 0), ("qwen36_moe", 1), ("qwen36_moe", 777), ("qwen36_moe", 4096), ("qwen3_1p7b", 300), ("qwen38_27b", 129),
+                                       ("qwen3_1p7b", 9001), ("qwen38_27b", 17000)])
 def test_q8_fused_decode_step(shape, pos):
     """pa_attn_decode_step on int8 caches: the row it writes (values and scales) and its output equal pa_glue_kv +
     pa_attn_decode bit for bit, neighbouring rows stay untouched, and the output matches the oracle over the
@@ -114,6 +115,8 @@ def test_q8_fused_decode_step(shape, pos):
     kq, ks, vq, vs, kf, vf = _quantised_cache(cfg, pos + 2, seed=pos + 4)
     with PooledAttn(cfg, pos + 2, n_layers=1, max_cols=1) as pa:
         pa.layer_alloc(0)
+        if pos > 8192:          # past what the single-round kernel holds at these shapes: the tile loop, three tiles a wave or more
+            assert pa.plan("decode", pos, 1)["split_len"] >= 3 * 128
         for w, a in enumerate((kq, vq, ks, vs)):
             pa.kv_write(0, w, 0, a)
         pa.run_glue_kv(0, d["qraw"], d["kraw"][pos:], d["vraw"][pos:], d["qw"], d["kw"], pos)
