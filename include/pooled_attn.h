@@ -74,7 +74,8 @@ typedef struct pa_ctx pa_ctx;
  * formulas: engine/autotune.js:10-68, engine/wgsl/attn_dec.js:40-48, engine/wgsl/attn_tile.js:43-56). */
 typedef struct pa_plan {
   uint32_t kernel;       /* 0 = split-K decode/verify kernel, 1 = MFMA prefill kernel */
-  uint32_t split_len;    /* cache rows per split */
+  uint32_t split_len;    /* cache rows per split (split-K kernel with more than 128 rows a split: the rows of a split's
+                            32-row tiles, which are dealt round robin to the splits of a kv head, not one contiguous range) */
   uint32_t n_splits;     /* splits over the streamed rows; a one-column decode streams rows 0 .. base_pos - 1 */
   uint32_t col_groups;   /* column groups (workgroups = n_splits x kv heads x col_groups) */
   uint32_t cols_per_group;
