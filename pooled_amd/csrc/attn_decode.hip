@@ -191,7 +191,7 @@ template <int HD> struct DecShape {
 // O^T = V^T P^T of a split is divided over the waves by output dims, see the code.  Without SR a split has any length
 // and every wave loops over its own tiles.
 template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
-__global__ __launch_bounds__(W * 64, (NB == 1 && !GATHER && W <= 4 ? 2 : 1))
+__global__ __launch_bounds__(W * 64, ((NB == 1 && !GATHER && W <= 4) || (SR && NB == 2 && HD == 128) ? 2 : 1))
 void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a_max_seq, uint32_t a_n_splits, uint32_t a_self_row,
                       uint32_t a_grid_x, const float* a_f_q_in, uint32_t a_group, uint32_t a_f_q_head_stride, AttnParams p_in) {
   // The leading arguments repeat fields of p_in: the first twelve dwords of a kernel's arguments are preloaded into
@@ -202,7 +202,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   const bool cols_adjacent = (a_self_row & 2u) != 0;                 // (rides in a preloaded argument: see the workgroup mapping below)
   p.f_q_in = a_f_q_in; p.group = a_group; p.f_q_head_stride = a_f_q_head_stride;
   const uint32_t grid_x = a_grid_x;
-  static_assert(!SR || NB == 1, "single-round splits: one 16-row block");
+  static_assert(!SR || NB == 1 || (NB == 2 && W == 4 && !FUSED && !GATHER && !Q8), "single-round splits: one 16-row block, or two on f16 caches");
   static_assert(!FUSED || NB == 1, "the fused pre-step serves one column");
   static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
   static_assert(!Q8 || !GATHER, "int8 caches: no gather mode");
@@ -212,6 +212,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   unsigned char* stage_all = smem + 16 * NB * S::QROW;               // [W][STAGE]
   float* mex = (float*)(stage_all + W * S::STAGE);                   // [W][16*NB]
   float* lex = mex + W * 16 * NB;                                    // [W][16*NB]
+  unsigned char* p_lds = (unsigned char*)(lex + W * 16 * NB);        // [W][NB][64 x 16 B]: the tiles' P, single-round kernel with two row blocks
 
   uint32_t bx = blockIdx.x, by = blockIdx.y, cg = blockIdx.z;
   if constexpr (SR && !FUSED && !GATHER) {
@@ -704,36 +705,50 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       stage_k(tp, false, 0);
       f4 s[2][NB];
       qk(s);
-      const uint32_t row_end = has_tile ? end_pos[0] : 0u;              // a wave without a tile contributes nothing
-      float v[8], mx = NEG_INF;
+      // (a wave without a tile contributes nothing: its rows end at 0)
+      float mxs[NB], pss[NB];
+      h8 pfs[NB];
 #pragma unroll
-      for (int pb = 0; pb < 2; pb++)
+      for (int nb = 0; nb < NB; nb++) {
+        const uint32_t row_end = has_tile ? end_pos[nb] : 0u;
+        float v[8], mx = NEG_INF;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const uint32_t pos = row_pos(tp, pb * 16 + 4 * kg + i);
-          const float x = pos < row_end ? s[pb][0][i] * p.scale : NEG_INF;
-          v[pb * 4 + i] = x;
-          mx = fmaxf(mx, x);
-        }
-      mx = rows_max(mx);
-      const float mw_safe = mx == NEG_INF ? 0.f : mx;
-      float ps = 0.f;
-      h8 pf;
+        for (int pb = 0; pb < 2; pb++)
 #pragma unroll
-      for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
-      ps = rows_sum(ps);
+          for (int i = 0; i < 4; i++) {
+            const uint32_t pos = row_pos(tp, pb * 16 + 4 * kg + i);
+            const float x = pos < row_end ? s[pb][nb][i] * p.scale : NEG_INF;
+            v[pb * 4 + i] = x;
+            mx = fmaxf(mx, x);
+          }
+        mx = rows_max(mx);
+        const float mw_safe = mx == NEG_INF ? 0.f : mx;
+        float ps = 0.f;
+        h8 pf;
+#pragma unroll
+        for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
+        mxs[nb] = mx; pss[nb] = rows_sum(ps); pfs[nb] = pf;
+      }
       if (v_late) { __builtin_amdgcn_sched_barrier(0); first_v_loads(); __builtin_amdgcn_sched_barrier(0); }
       stage_v(ILV && ilv ? 0u : tp, false, 0);                          // interleaved splits are whole: no row past the end to zero
-      *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pf;
-      if (kg == 0) { mex[wave * 16 + ln] = mx; lex[wave * 16 + ln] = ps; }
+      // one row block: P rides in the padding of the staged V rows; two: in a region of its own
+      if constexpr (NB == 1) *(h8*)(stage + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16) = pfs[0];
+      else {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) *(h8*)(p_lds + ((wave * NB + nb) * 64 + lane) * 16) = pfs[nb];
+      }
+      if (kg == 0) {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) { mex[wave * 16 * NB + nb * 16 + ln] = mxs[nb]; lex[wave * 16 * NB + nb * 16 + ln] = pss[nb]; }
+      }
       __syncthreads();
       {
         // V^T fragments (two transpose reads each) and the tile's P are fetched VD steps ahead of their MFMA
         // (a tile's P is read once, not once per 16-dim block: the tail of the kernel is bound by the LDS port)
         constexpr int NS = W * DBW, VD = 4;
         h4 lor[VD], hir[VD];
-        h8 pfr[W];
-        f4 pr[W][DBW];
+        h8 pfr[W][NB];
+        f4 pr[W][DBW][NB];
         auto fetch = [&](int st, int slot) __attribute__((always_inline)) {
           const int w2 = st / DBW, db = wave * DBW + st % DBW;
           const unsigned char* sw = stage_all + w2 * S::STAGE;
@@ -742,7 +757,13 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
           hir[slot] = lds_read_tr16(vp + 16 * S::VROW);
         };
 #pragma unroll
-        for (int w2 = 0; w2 < W; w2++) pfr[w2] = *(const h8*)(stage_all + w2 * S::STAGE + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16);
+        for (int w2 = 0; w2 < W; w2++) {
+          if constexpr (NB == 1) pfr[w2][0] = *(const h8*)(stage_all + w2 * S::STAGE + (lane >> 1) * S::VROW + HD * 2 + (lane & 1) * 16);
+          else {
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) pfr[w2][nb] = *(const h8*)(p_lds + ((w2 * NB + nb) * 64 + lane) * 16);
+          }
+        }
 #pragma unroll
         for (int st = 0; st < VD; st++) fetch(st, st);
 #pragma unroll
@@ -750,47 +771,53 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
           const h4 lo = lor[st % VD], hi = hir[st % VD];
           if (st + VD < NS) fetch(st + VD, st % VD);
           const h8 a = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
-          pr[st / DBW][st % DBW] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pfr[st / DBW], (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+          for (int nb = 0; nb < NB; nb++)
+            pr[st / DBW][st % DBW][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pfr[st / DBW][nb], (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, W, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, W * NB, 1);
 #pragma unroll
         for (int st = 0; st < VD; st++) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
 #pragma unroll
         for (int st = 0; st < NS; st++) {
           if (st + VD < NS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+          __builtin_amdgcn_sched_group_barrier(0x008, NB, 1);
         }
-        // a wave without a tile staged stale rows: its m is -inf, and its products must not reach O even as 0 x NaN
-        float mw[W], lw[W], M = NEG_INF;
 #pragma unroll
-        for (int w2 = 0; w2 < W; w2++) { mw[w2] = mex[w2 * 16 + ln]; lw[w2] = lex[w2 * 16 + ln]; M = fmaxf(M, mw[w2]); }
-        const float m_safe = M == NEG_INF ? 0.f : M;
-        float Lr = 0.f;
-        f4 o[DBW];
+        for (int nb = 0; nb < NB; nb++) {
+          // a wave without a tile staged stale rows: its m is -inf, and its products must not reach O even as 0 x NaN
+          float mw[W], lw[W], M = NEG_INF;
 #pragma unroll
-        for (int j = 0; j < DBW; j++) o[j] = (f4){0.f, 0.f, 0.f, 0.f};
+          for (int w2 = 0; w2 < W; w2++) { mw[w2] = mex[w2 * 16 * NB + nb * 16 + ln]; lw[w2] = lex[w2 * 16 * NB + nb * 16 + ln]; M = fmaxf(M, mw[w2]); }
+          const float m_safe = M == NEG_INF ? 0.f : M;
+          float Lr = 0.f;
+          f4 o[DBW];
 #pragma unroll
-        for (int w2 = 0; w2 < W; w2++) {
-          const bool dead = mw[w2] == NEG_INF;
-          const float c = dead ? 0.f : __expf(mw[w2] - m_safe);
-          Lr += lw[w2] * c;
+          for (int j = 0; j < DBW; j++) o[j] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int j = 0; j < DBW; j++) o[j] += (dead ? (f4){0.f, 0.f, 0.f, 0.f} : pr[w2][j]) * c;
-        }
-        if (ln < R) {
-          const uint32_t col = c0 + ln / G, hq = g * G + ln % G;
-          const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
-          // f16 partials (|O| <= 128 rows x |v|: far inside the range; the merge adds them up in f32): half the bytes this
-          // kernel writes at its very end and half of what the merge kernel waits for
-          if (p.part_f16) {
+          for (int w2 = 0; w2 < W; w2++) {
+            const bool dead = mw[w2] == NEG_INF;
+            const float c = dead ? 0.f : __expf(mw[w2] - m_safe);
+            Lr += lw[w2] * c;
 #pragma unroll
-            for (int j = 0; j < DBW; j++)
-              *(h4*)((_Float16*)p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = (h4){ (_Float16)o[j][0], (_Float16)o[j][1], (_Float16)o[j][2], (_Float16)o[j][3] };
-          } else {
-#pragma unroll
-            for (int j = 0; j < DBW; j++) *(f4*)(p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = o[j];
+            for (int j = 0; j < DBW; j++) o[j] += (dead ? (f4){0.f, 0.f, 0.f, 0.f} : pr[w2][j][nb]) * c;
           }
-          if (wave == 0 && kg == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(M, Lr);
+          const uint32_t r = nb * 16 + ln;
+          if (r < R) {
+            const uint32_t col = c0 + r / G, hq = g * G + r % G;
+            const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
+            // f16 partials (|O| <= 128 rows x |v|: far inside the range; the merge adds them up in f32): half the bytes this
+            // kernel writes at its very end and half of what the merge kernel waits for
+            if (p.part_f16) {
+#pragma unroll
+              for (int j = 0; j < DBW; j++)
+                *(h4*)((_Float16*)p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = (h4){ (_Float16)o[j][0], (_Float16)o[j][1], (_Float16)o[j][2], (_Float16)o[j][3] };
+            } else {
+#pragma unroll
+              for (int j = 0; j < DBW; j++) *(f4*)(p.part_o + slot * HD + (wave * DBW + j) * 16 + 4 * kg) = o[j];
+            }
+            if (wave == 0 && kg == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(M, Lr);
+          }
         }
       }
     }
@@ -1193,7 +1220,7 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
 template <int HD, int NB, int W>
 static constexpr size_t decode_lds_bytes() {
   typedef DecShape<HD> S;
-  return 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float);
+  return 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float) + (NB == 2 && W == 4 ? (size_t)W * NB * 1024 : 0);   // (+ the P region of the single-round kernel with two row blocks)
 }
 // the kernel's dynamic LDS limit, raised once per instantiation (at its first launch, or ahead of it by
 // pa_prepare_decode_step)
@@ -1223,11 +1250,15 @@ static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipS
   return hipGetLastError();
 }
 
-// one 16-row block with splits of one tile per wave: the single-round kernel
+// one 16-row block with splits of one tile per wave: the single-round kernel; two blocks (f16 caches) when the plan asks
+// for it (AttnParams::single_round2: a pass of one split keeps the tile loop, which writes the output itself)
 template <int HD, int NB, int W, bool FUSED, bool GATHER = false, bool Q8 = false>
 static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   if constexpr (NB == 1) {
     if (p.split_len == W * TILE) return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, true>(p, col_groups, s, t);
+  }
+  if constexpr (NB == 2 && W == 4 && !FUSED && !GATHER && !Q8) {
+    if (p.single_round2 && p.split_len == W * TILE) return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, true>(p, col_groups, s, t);
   }
   return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, false>(p, col_groups, s, t);
 }

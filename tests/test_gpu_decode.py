@@ -123,6 +123,35 @@ def test_verify_equals_sequential_decodes(shape, n_cols, base):
             assert np.abs(single[0] - multi[c]).max() <= 1e-3
 
 
+@pytest.mark.parametrize("shape,n_cols,base", [("qwen36_moe", 4, 8000), ("qwen38_27b", 5, 5000), ("qwen3_1p7b", 12, 3000), ("qwen36_moe", 3, 16200),
+                                               ("qwen36_moe", 8, 4090)])
+def test_verify_block_on_the_single_round_kernel_with_two_row_blocks(shape, n_cols, base):
+    """A verify block of 17 .. 32 stacked rows a workgroup over a context that fits one round of one-tile-per-wave splits
+    at one workgroup a CU: the single-round kernel with two row blocks (f16 caches).  Causal ends differ by column, the
+    last split is partial, rows past the context are poisoned; f32 and f16 out, with a gate where the shape has one."""
+    cfg = SHAPES[shape]
+    rng = np.random.default_rng(base + n_cols)
+    L = base + n_cols
+    k16, v16 = random_cache(cfg, L + 40, seed=base)
+    q = rng.standard_normal((n_cols, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+    gate = rng.standard_normal(q.shape, dtype=np.float32) if cfg["gate"] else None
+    ref = C.attention(q, k16, v16, base, gate=gate)
+    with _ctx_with_cache(cfg, k16, v16, L + 40, max_cols=n_cols, poison_from=L) as pa:
+        pl = pa.plan("decode", base, n_cols)
+        assert pl["row_blocks"] == 2 and pl["split_len"] == 128 and pl["n_splits"] == -(-L // 128) and pl["slots"] == pl["n_splits"], pl
+        for out_dtype in (0, PA_OUT_F16):
+            assert_parity(pa.run_attn("decode", 0, q, base, gate=gate, out_dtype=out_dtype), ref, "two row blocks, single round, %d columns at %d" % (n_cols, base), tight=True)
+        pa.set_decode_splits(max(2, pl["n_splits"] // 3))            # the same block on the tile loop's contiguous splits
+        assert pa.plan("decode", base, n_cols)["split_len"] > 128
+        assert np.abs(pa.run_attn("decode", 0, q, base, gate=gate) - pa_first(pa, q, base, gate)).max() <= 2e-4
+
+
+def pa_first(pa, q, base, gate):
+    """The table's plan again (after a splits override)."""
+    pa.set_decode_splits(0)
+    return pa.run_attn("decode", 0, q, base, gate=gate)
+
+
 @pytest.mark.parametrize("shape,n_cols,base", [("qwen36_moe", 4, 996), ("qwen38_27b", 8, 2040), ("qwen3_1p7b", 5, 510), ("qwen36_moe", 3, 32767),
                                                ("qwen36_moe", 8, 9000), ("qwen36_moe", 16, 20000), ("qwen38_27b", 6, 8190), ("qwen3_1p7b", 13, 119),
                                                ("qwen36_moe", 5, 40000), ("qwen38_27b", 4, 33000), ("qwen38_27b", 8, 65533)])
