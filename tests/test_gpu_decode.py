@@ -103,7 +103,8 @@ def test_decode_either_side_of_the_f16_partials_threshold(pos):
 
 
 @pytest.mark.parametrize("shape,n_cols,base", [("qwen36_moe", 4, 996), ("qwen36_moe", 16, 3000), ("qwen38_27b", 8, 2040),
-                                               ("qwen3_1p7b", 4, 510), ("qwen38_27b", 16, 17), ("qwen36_moe", 7, 0)])
+                                               ("qwen3_1p7b", 4, 510), ("qwen38_27b", 16, 17), ("qwen36_moe", 7, 0),
+                                               ("qwen36_moe", 16, 20000), ("qwen38_27b", 12, 30000), ("qwen3_1p7b", 16, 9000)])
 def test_verify_equals_sequential_decodes(shape, n_cols, base):
     """A verify block must equal n sequential single-token decodes (engine/wgsl/attn_dec.js:12-16;
     tests/test_attn_dec.js:89-97) -- here within tolerance -- and the oracle."""
