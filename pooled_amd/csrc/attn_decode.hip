@@ -202,7 +202,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   const bool cols_adjacent = (a_self_row & 2u) != 0;                 // (rides in a preloaded argument: see the workgroup mapping below)
   p.f_q_in = a_f_q_in; p.group = a_group; p.f_q_head_stride = a_f_q_head_stride;
   const uint32_t grid_x = a_grid_x;
-  static_assert(!SR || NB == 1 || (NB == 2 && W == 4 && !FUSED && !GATHER && !Q8), "single-round splits: one 16-row block, or two on f16 caches");
+  static_assert(!SR || NB == 1 || (NB == 2 && W == 4 && !FUSED && !GATHER), "single-round splits: one 16-row block, or two of a verify block");
   static_assert(!FUSED || NB == 1, "the fused pre-step serves one column");
   static_assert(!GATHER || (NB == 1 && !FUSED), "the gather mode serves one column per workgroup");
   static_assert(!Q8 || !GATHER, "int8 caches: no gather mode");
@@ -1250,14 +1250,14 @@ static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipS
   return hipGetLastError();
 }
 
-// one 16-row block with splits of one tile per wave: the single-round kernel; two blocks (f16 caches) when the plan asks
+// one 16-row block with splits of one tile per wave: the single-round kernel; two blocks when the plan asks
 // for it (AttnParams::single_round2: a pass of one split keeps the tile loop, which writes the output itself)
 template <int HD, int NB, int W, bool FUSED, bool GATHER = false, bool Q8 = false>
 static hipError_t launch_decode_t(const AttnParams& p, uint32_t col_groups, hipStream_t s, const PaTiming* t) {
   if constexpr (NB == 1) {
     if (p.split_len == W * TILE) return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, true>(p, col_groups, s, t);
   }
-  if constexpr (NB == 2 && W == 4 && !FUSED && !GATHER && !Q8) {
+  if constexpr (NB == 2 && W == 4 && !FUSED && !GATHER) {
     if (p.single_round2 && p.split_len == W * TILE) return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, true>(p, col_groups, s, t);
   }
   return launch_decode_k<HD, NB, W, FUSED, GATHER, Q8, false>(p, col_groups, s, t);

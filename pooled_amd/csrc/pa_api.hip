@@ -322,7 +322,7 @@ static bool plan_self_row(const pa_plan& pl) { return pl.kernel == 0 && pl.slots
 // of the output, and every other pass keep f32 partials.
 // round-robin tiles: the tile loop of the split-K kernel (every plan of that kernel but the single-round one) with more
 // than one split; the value is the distance between the first rows of two splits
-// two row blocks on the single-round kernel: what plan_decode picks for f16 caches when a verify block's context fits
+// two row blocks on the single-round kernel: what plan_decode picks when a verify block's context fits
 // one round of one-tile-per-wave splits at one workgroup a CU (a pass of a single split stays on the tile loop)
 static bool plan_single_round2(const pa_plan& pl) {
   return pl.kernel == 0 && pl.row_blocks == 2 && pl.waves == 4 && pl.split_len == 32 * pl.waves && pl.n_splits > 1;
@@ -370,7 +370,7 @@ static int plan_decode(const pa_ctx* ctx, uint32_t base_pos, uint32_t n_cols, pa
     // a given number of splits (a tuning override; its splits are contiguous ranges, the last one open-ended), or one
     const uint32_t tpw = one_split ? std::max(ceil_div(tiles, W), 1u) : std::max(ceil_div(tiles, target * W), 1u);
     sl = 32 * W * tpw; ns = ceil_div(seq_max, sl);
-  } else if ((nb == 1 || (nb == 2 && W == 4 && !kv_q8(ctx) && seq_max > 32 * W)) &&
+  } else if ((nb == 1 || (nb == 2 && W == 4 && seq_max > 32 * W)) &&
              ceil_div(seq_max, 32 * W) <= (nb == 2 && c.head_dim == 128 ? 2 * target : target)) {
     // One 16-row block and no more one-tile-per-wave splits than two workgroups a CU hold at once: the single-round
     // kernel, the whole context in flight in one go.  A single split more would run as a second round behind the
@@ -636,7 +636,7 @@ static int attn_common(pa_ctx* ctx, const char* who, int kind, uint32_t layer, c
   p.direct_out = direct && pl.kernel == 0 ? 1 : 0;
   p.part_f16 = !direct && plan_f16_partials(pl, n_cols);
   p.tile_ilv = plan_tile_ilv(pl);
-  p.single_round2 = plan_single_round2(pl) && !kv_q8(ctx);
+  p.single_round2 = plan_single_round2(pl);
   p.max_seq = c.max_seq; p.out_f16 = out_dtype == PA_OUT_F16;
   p.scale = (float)(1.0 / std::sqrt((double)c.head_dim));
   p.gate_head_stride = c.head_dim;

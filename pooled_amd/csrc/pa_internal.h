@@ -61,7 +61,7 @@ struct AttnParams {
   const uint32_t* sel; uint32_t sel_stride, sel_max;
   uint32_t exact_cols;                        // 1: a column-exact verify block in one launch: every column is a column group of its
                                               // own under the plan of a one-column decode (the merge must be the wavefront kernel)
-  uint32_t single_round2;                     // 1: two row blocks on the single-round kernel (splits of one tile per wave, f16 caches)
+  uint32_t single_round2;                     // 1: two row blocks on the single-round kernel (splits of one tile per wave)
   uint32_t tile_ilv;                          // tile loop of the split-K kernel on a contiguous cache: rows from one split's first tile
                                               // to the next split's (32 x waves) when the tiles of a kv head are dealt round robin to the
                                               // waves of all its splits; 0 = every split a contiguous range of split_len rows

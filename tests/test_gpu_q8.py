@@ -82,7 +82,13 @@ def test_q8_verify_block_prefill_chunk_and_slots():
         pa.layer_alloc(0)
         for w, a in enumerate((kq, vq, ks, vs)):
             pa.kv_write(0, w, 0, a)
+        pl = pa.plan("decode", base, 8)      # two column groups of 32 stacked rows: the single-round kernel with two row blocks
+        assert pl["row_blocks"] == 2 and pl["split_len"] == 128 and pl["n_splits"] == -(-(base + 8) // 128) and pl["col_groups"] == 2, pl
         assert_parity(pa.run_attn("decode", 0, q[:8], base, gate=gate[:8]), ref[:8], "q8 verify block")
+        pa.set_decode_splits(4)              # the same block on the tile loop
+        assert pa.plan("decode", base, 8)["split_len"] > 128
+        assert_parity(pa.run_attn("decode", 0, q[:8], base, gate=gate[:8]), ref[:8], "q8 verify block, tile loop")
+        pa.set_decode_splits(0)
         # a narrow chunk runs on the split-K kernel, a wide one on the MFMA prefill kernel over rows widened to f16 (forced:
         # the table would serve a chunk this small on the split-K kernel too)
         pa.set_prefill_tile(1)
