@@ -63,3 +63,33 @@ def test_plans_and_passes_over_random_blocks(shape):
         assert any(s[0] == 1 and s[1] and s[2] for s in seen) and any(s[0] == 2 and s[1] and s[2] for s in seen), seen
         assert any(not s[1] and s[2] for s in seen) and any(not s[2] for s in seen), seen
         assert any(s[3] for s in seen) or cfg["head_dim"] == 128, seen      # (64 rows a workgroup at hd 128: 20 columns of G = 2 are one group)
+
+
+@pytest.mark.parametrize("shape", ["qwen36_moe", "qwen38_27b", "qwen3_1p7b"])
+def test_prefill_plans_and_passes_over_random_chunks(shape):
+    """The same for prefill chunks: narrow chunks on the split-K kernel (column groups over a long context, one launch
+    with direct output over a short one), wider ones on the matrix-core kernel, split over the context or not."""
+    cfg = SHAPES[shape]
+    rng = np.random.default_rng(7 + len(shape))
+    rows, max_cols = 6000, 700
+    k16, v16 = random_cache(cfg, rows + 40, seed=78)
+    cases = [(1, 0), (33, 0), (256, 0), (512, 1536), (700, 5000), (16, 5900), (64, 4096), (100, 4095), (257, 255)]
+    for _ in range(10):
+        n = int(rng.integers(1, max_cols + 1))
+        cases.append((n, int(rng.integers(0, rows - n))))
+    with PooledAttn(cfg, rows + 40, n_layers=1, max_cols=max_cols) as pa:
+        pa.layer_alloc(0)
+        pa.kv_write(0, 0, 0, k16.copy()); pa.kv_write(0, 1, 0, v16.copy())
+        kernels = set()
+        for n_cols, base in cases:
+            pl = pa.plan("prefill", base, n_cols)
+            assert pl["kernel"] in (0, 1) and pl["n_splits"] >= 1 and pl["split_len"] % 32 == 0, pl
+            assert pl["n_splits"] * pl["split_len"] >= base + n_cols, (n_cols, base, pl)
+            assert pl["col_groups"] * pl["cols_per_group"] >= n_cols > (pl["col_groups"] - 1) * pl["cols_per_group"], pl
+            kernels.add((pl["kernel"], pl["n_splits"] > 1))
+            q = rng.standard_normal((n_cols, cfg["n_heads"], cfg["head_dim"]), dtype=np.float32)
+            gate = rng.standard_normal(q.shape, dtype=np.float32) if cfg["gate"] else None
+            ref = C.attention(q, k16, v16, base, gate=gate)
+            assert_parity(pa.run_attn("prefill", 0, q, base, gate=gate), ref, "%s prefill %d columns at %d: %s" % (shape, n_cols, base, pl))
+        # (chunks this narrow leave CUs idle on the matrix-core kernel, so it is always split over the context here)
+        assert (0, False) in kernels and any(k[0] == 1 for k in kernels) and any(k[1] for k in kernels), kernels
