@@ -69,9 +69,6 @@ static __device__ inline float rows_sum(float v) {
   xrow32(v, a, b); return a + b;
 }
 // lane i's copy of lane (i + N) % 16 of its row of 16 (DPP row rotation)
-#ifndef PA_ABL_NOLOAD
-#define PA_ABL_NOLOAD 0
-#endif
 template <int N>
 static __device__ inline float row_ror(float v) {
   return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x120 + N, 0xf, 0xf, false));
@@ -595,7 +592,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::KROW + (lane % S::LPR) * 16) = kr[i];
     }
-    if (!Q8 && more && !PA_ABL_NOLOAD) {
+    if (!Q8 && more) {
       if constexpr (GATHER) {
         gather_offsets(tpn);
 #pragma unroll
@@ -680,7 +677,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
     }
-    if (!Q8 && more && !PA_ABL_NOLOAD) {
+    if (!Q8 && more) {
       if constexpr (GATHER) {                         // goff still holds the next tile's rows (set with the K loads above)
 #pragma unroll
         for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
