@@ -333,34 +333,6 @@ def other_configs():
     return out
 
 
-def tile_loop_ablation_child():
-    """pa_attn_decode on 1 / 4 / 8 columns of the 27B shape (one, two and three row blocks) at 65536 and 131072 rows:
-    microseconds per call (decode kernel + merge kernel), the median of five 100-call windows after a discarded one,
-    three layers' caches in rotation."""
-    from pooled_amd.capi import PooledAttn, PA_OUT_F16
-    cfg = dict(n_heads=24, n_kv_heads=4, head_dim=256, n_rot=64, rope_theta=1e7, eps=1e-6, qk_norm=True, gate=True)
-    qd, layers, out = cfg["n_heads"] * cfg["head_dim"], 3, {}
-    for base in (65536, 131072):
-        pa = PooledAttn(cfg, base + 8, n_layers=layers, max_cols=4096)
-        rs = streams(0x5EED0104, "q", "gate", *["cache%d" % l for l in range(layers)])
-        for l in range(layers):
-            pa.layer_alloc(l)
-            fill_cache(pa, cfg, l, base + 8, rs["cache%d" % l], chunk=4096)
-        dq = pa.to_device(rs["q"].standard_normal((8, qd), dtype=np.float32)); dg = pa.to_device(rs["gate"].standard_normal((8, qd), dtype=np.float32))
-        dout = pa.alloc(8 * qd * 2)
-        for n in (1, 4, 8):
-            wins = []
-            for w in range(6):
-                pa.sync(); pa.timer_start()
-                for i in range(100):
-                    pa.attn("decode", i % layers, dq, qd, dg, qd, base, n, dout, qd, PA_OUT_F16)
-                wins.append(pa.timer_stop() / 100 * 1e3)
-            pl = pa.plan("decode", base, n)
-            out["%d columns at %d (%d splits, %d row blocks)" % (n, base, pl["n_splits"], pl["row_blocks"])] = round(sorted(wins[1:])[2], 2)
-        pa.close()
-    return out
-
-
 def layer_leg(pa, cfg, ctx, steps, warmup, attn_ms, n_rot, rng):
     """The attention half of a layer for one token, projections included (pa_attn_layer_decode: normed [q | k | v]
     GEMV, fused decode step, accumulating output GEMV; Q4_0 weights of the MoE model's shape, a set per layer and
@@ -429,10 +401,6 @@ def main():
     ap.add_argument("--kv-q8", action="store_true", help="run the C3 decode step on int8 caches (one f32 scale per 32 values) instead of f16")
     ap.add_argument("--no-layer", action="store_true", help="skip the whole-layer leg (projections + attention, pa_attn_layer_decode)")
     ap.add_argument("--other-configs", action="store_true", help="only time configurations 1, 2 and 4 (attention call alone, caches in rotation)")
-    ap.add_argument("--tile-loop-ablation", action="store_true",
-                    help="only time 1 / 4 / 8-column blocks of the 27B shape at 65536 and 131072 rows on the split-K kernel's tile loop with parts of it "
-                         "removed (timing-only builds: python -m pooled_amd.build --tile-loop-ablation), each build in a process of its own, two interleaved rounds")
-    ap.add_argument("--tile-loop-ablation-child", type=int, default=-1, help=argparse.SUPPRESS)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 10 device-to-device copies of 256 MiB (the known-size kernel that scales rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--rotation", type=int, default=0, help="time the decode step with this many layers' caches in rotation only (default: sweep %s)" % (ROTATIONS,))
@@ -441,25 +409,6 @@ def main():
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
-    if args.tile_loop_ablation:
-        import subprocess
-        from pooled_amd import build as pa_build
-        rounds = []
-        for rnd in range(2):
-            row = {}
-            for mask, label in pa_build.TILE_LOOP_ABLATIONS:
-                out = subprocess.run([sys.executable, os.path.abspath(__file__), "--tile-loop-ablation-child", str(mask)],
-                                     stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=600, check=True).stdout
-                row[mask] = json.loads(out.strip().splitlines()[-1])
-                log("round %d  removed: %-84s %s" % (rnd + 1, label, row[mask]))
-            rounds.append(row)
-        print(json.dumps({"tile_loop_ablation": [dict(mask=mask, removed=label, us=[r[mask] for r in rounds]) for mask, label in pa_build.TILE_LOOP_ABLATIONS]}))
-        return
-    if args.tile_loop_ablation_child >= 0:
-        from pooled_amd import capi, build as pa_build
-        capi.LIB_PATH = pa_build.ablation_lib(args.tile_loop_ablation_child)
-        print(json.dumps(tile_loop_ablation_child()))
-        return
     from pooled_amd.capi import PooledAttn, PA_OUT_F16, load
     L = load()
     log("library:", L.pa_version().decode())

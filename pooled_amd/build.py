@@ -63,28 +63,6 @@ def build_addon(verbose=False):
     return ADDON
 
 
-# timing-only ablations of the split-K kernel's tile loop (attn_decode.hip, PA_ABL): what is removed
-TILE_LOOP_ABLATIONS = [(0, "nothing"), (1, "the tile loads after a wave's first tile"), (3, "those loads, the merge of the four waves and the partial stores"),
-                       (5, "those loads and the loop (start-up, the waves' merge and the partial stores remain)"),
-                       (7, "all three (launch, start-up and the merge kernel remain)")]
-
-
-def ablation_lib(mask):
-    return os.path.join(LIBDIR, "abl%d" % mask, "libpooled_attn.so")
-
-
-def build_tile_loop_ablations(verbose=False):
-    """One library per ablation mask (results wrong on purpose; bench.py --tile-loop-ablation times them)."""
-    out = []
-    for mask, _ in TILE_LOOP_ABLATIONS:
-        lib = build_lib(verbose, extra=("-DPA_ABL=%d" % mask,), lib=ablation_lib(mask))
-        for f in os.listdir(os.path.dirname(lib)):
-            if f.endswith(".o"):
-                os.remove(os.path.join(os.path.dirname(lib), f))
-        out.append(lib)
-    return out
-
-
 def build_all(verbose=False, extra=()):
     lib = build_lib(verbose, extra=extra)
     addon = build_addon(verbose)
@@ -93,7 +71,4 @@ def build_all(verbose=False, extra=()):
 
 if __name__ == "__main__":
     # -DNAME=VALUE arguments go to hipcc (the prefill kernel's PF_QR / PF_KD / PF_VD constants)
-    if "--tile-loop-ablation" in sys.argv:
-        print(build_tile_loop_ablations(verbose="-v" in sys.argv))
-    else:
-        print(build_all(verbose="-v" in sys.argv, extra=tuple(a for a in sys.argv[1:] if a.startswith("-D"))))
+    print(build_all(verbose="-v" in sys.argv, extra=tuple(a for a in sys.argv[1:] if a.startswith("-D"))))

@@ -69,12 +69,6 @@ static __device__ inline float rows_sum(float v) {
   xrow32(v, a, b); return a + b;
 }
 // lane i's copy of lane (i + N) % 16 of its row of 16 (DPP row rotation)
-// PA_ABL (a development record, not a product option): timing-only builds of the tile loop with parts REMOVED -- the
-// results are wrong on purpose.  1: no tile loads after a wave's first tile (the loop computes on stale registers);
-// 2: the kernel ends after the loop (no merge of the four waves, no partial stores); 4: the loop itself is skipped.
-#ifndef PA_ABL
-#define PA_ABL 0
-#endif
 template <int N>
 static __device__ inline float row_ror(float v) {
   return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x120 + N, 0xf, 0xf, false));
@@ -598,7 +592,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::KROW + (lane % S::LPR) * 16) = kr[i];
     }
-    if (!Q8 && more && !(PA_ABL & 1)) {
+    if (!Q8 && more) {
       if constexpr (GATHER) {
         gather_offsets(tpn);
 #pragma unroll
@@ -683,7 +677,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
     for (int i = 0; i < S::NLD; i++) *(u4*)(stage + (i * S::RPL + lrow) * S::VROW + (lane % S::LPR) * 16) = vr[i];
     }
-    if (!Q8 && more && !(PA_ABL & 1)) {
+    if (!Q8 && more) {
       if constexpr (GATHER) {                         // goff still holds the next tile's rows (set with the K loads above)
 #pragma unroll
         for (int i = 0; i < S::NLD; i++) vr[i] = *(const u4*)(vbase + (size_t)goff[i] * row_bytes + (lane % S::LPR) * 16);
@@ -835,7 +829,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   float m_run[NB], l_run[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) { m_run[nb] = NEG_INF; l_run[nb] = 0.f; }
-  const uint32_t tp_lim = (PA_ABL & 4) ? t_begin : t_begin + n_tiles * TILE;
+  const uint32_t tp_lim = t_begin + n_tiles * TILE;
   for (uint32_t tp = t_begin + tile * TILE; tp < tp_lim; tp += tp_step) {
     const bool more = tp + tp_step < tp_lim;
     stage_k(tp, more, tp + tp_step);
@@ -927,7 +921,6 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   }
 
   // ---- merge the W waves of the workgroup ----
-  if ((PA_ABL & 2) && p.n_cols < 1000000u) return;
   const bool direct = p.direct_out != 0;       // one split and no own-row partial: this workgroup holds the whole result
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
