@@ -184,9 +184,10 @@ template <int HD> struct DecShape {
 // tile -- int8 -> f16 through the 0x6400 | (v + 128) bit pattern (= 1152 + v exactly), a packed subtract and a
 // packed multiply by the f16-rounded scale.  From there on (MFMA, softmax, merge) it is the f16 kernel.
 //
-// SR (single-round splits; one 16-row block): splits are one tile per wave (split_len = W x 32); the product
-// O^T = V^T P^T of a split is divided over the waves by output dims, see the code.  Without SR a split has any length
-// and every wave loops over its own tiles.
+// SR (single-round splits; one 16-row block, or two of a verify block): splits are one tile per wave (split_len = W x
+// 32); the product O^T = V^T P^T of a split is divided over the waves by output dims, see the code.  Without SR every wave
+// loops over its own tiles: contiguous splits of any length, or (AttnParams::tile_ilv) a kv head's tiles dealt round robin
+// to the waves of all its splits.
 template <int HD, int NB, int W, bool FUSED, bool GATHER, bool Q8, bool SR>
 __global__ __launch_bounds__(W * 64, ((NB == 1 && !GATHER && W <= 4) || (SR && NB == 2 && HD == 128) ? 2 : 1))
 void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a_max_seq, uint32_t a_n_splits, uint32_t a_self_row,
