@@ -210,7 +210,10 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   unsigned char* stage_all = smem + 16 * NB * S::QROW;               // [W][STAGE]
   float* mex = (float*)(stage_all + W * S::STAGE);                   // [W][16*NB]
   float* lex = mex + W * 16 * NB;                                    // [W][16*NB]
-  unsigned char* p_lds = (unsigned char*)(lex + W * 16 * NB);        // [W][NB][64 x 16 B]: the tiles' P, single-round kernel with two row blocks
+  float* sct = lex + W * 16 * NB;                                    // [W][16*NB]: the tile loop's merge, a wave's weight exp(m_w - M) per row
+  uint32_t* rowcol = (uint32_t*)(sct + W * 16 * NB);                 // [16*NB]: the column of a stacked row ...
+  uint32_t* rowhq = rowcol + 16 * NB;                                // [16*NB]: ... and its query head (same merge)
+  unsigned char* p_lds = (unsigned char*)(rowhq + 16 * NB);          // [W][NB][64 x 16 B]: the tiles' P, single-round kernel with two row blocks
 
   uint32_t bx = blockIdx.x, by = blockIdx.y, cg = blockIdx.z;
   if constexpr (SR && !FUSED && !GATHER) {
@@ -922,26 +925,30 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   }
 
   // ---- merge the W waves of the workgroup ----
+  // The waves' O rows meet in their staging regions UNSCALED (straight from the accumulators); a wave's weight per row,
+  // exp(m_w - M), comes from a table one thread per (wave, row) fills, and is applied where the rows are summed.  So is the
+  // (column, head) of a stacked row: a table filled once, instead of a division by the group size per element group.
   const bool direct = p.direct_out != 0;       // one split and no own-row partial: this workgroup holds the whole result
+  if (tid < 16 * NB) { rowcol[tid] = c0 + tid / G; rowhq[tid] = g * G + tid % G; }
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     l_run[nb] = rows_sum(l_run[nb]);
     if (kg == 0) { mex[wave * 16 * NB + nb * 16 + ln] = m_run[nb]; lex[wave * 16 * NB + nb * 16 + ln] = l_run[nb]; }
   }
   __syncthreads();
-#pragma unroll
-  for (int nb = 0; nb < NB; nb++) {
+  static_assert(NB <= 4, "one thread per (wave, row) of the weight table");
+  if (tid < W * 16 * NB) {                     // (read after the first barrier below)
+    const uint32_t rw = tid % (16 * NB);
     float M = NEG_INF;
 #pragma unroll
-    for (int w = 0; w < W; w++) M = fmaxf(M, mex[w * 16 * NB + nb * 16 + ln]);
-    const float m_safe = M == NEG_INF ? 0.f : M;
-    const float sc = __expf(m_run[nb] - m_safe);
+    for (int w = 0; w < W; w++) M = fmaxf(M, mex[w * 16 * NB + rw]);
+    sct[tid] = __expf(mex[tid] - (M == NEG_INF ? 0.f : M));
+  }
+#pragma unroll
+  for (int nb = 0; nb < NB; nb++) {
     if (nb * 16 + ln < R) {                                            // padding rows are never read back
 #pragma unroll
-      for (int db = 0; db < S::DB; db++) {
-        const f4 o = acc[db][nb] * sc;
-        *(f4*)(stage + ln * S::OROW + (db * 16 + 4 * kg) * 4) = o;
-      }
+      for (int db = 0; db < S::DB; db++) *(f4*)(stage + ln * S::OROW + (db * 16 + 4 * kg) * 4) = acc[db][nb];
     }
     __syncthreads();
     // rows nb*16 .. nb*16+15, HD/4 float4 each, summed over waves in wave order.  Every thread first issues all
@@ -956,7 +963,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
       for (int j = 0; j < EPT; j++) {
         const uint32_t e = tid + j * W * 64, r = min(nb * 16 + e / (HD / 4), R - 1), d4 = e % (HD / 4);
-        gtv[j] = *(const f4*)(p.gate + (size_t)(c0 + r / G) * p.gate_stride + (size_t)(g * G + r % G) * p.gate_head_stride + 4 * d4);
+        gtv[j] = *(const f4*)(p.gate + (size_t)rowcol[r] * p.gate_stride + (size_t)rowhq[r] * p.gate_head_stride + 4 * d4);
       }
     }
     f4 part[EPT][W];
@@ -981,10 +988,10 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       const uint32_t rr = e / (HD / 4), d4 = e % (HD / 4);
       const uint32_t r = nb * 16 + rr;
       if (r < R) {
-        f4 o = part[j][0];
+        f4 o = part[j][0] * sct[r];
 #pragma unroll
-        for (int w = 1; w < W; w++) o += part[j][w];
-        const uint32_t col = c0 + r / G, hq = g * G + r % G;
+        for (int w = 1; w < W; w++) o += part[j][w] * sct[w * 16 * NB + r];
+        const uint32_t col = rowcol[r], hq = rowhq[r];
         if (direct) {
           // the only split of the pass: normalise, gate, convert and store here -- no partial, no merge launch
           float Mr = NEG_INF, L = 0.f;
@@ -1019,8 +1026,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       float L = 0.f;
 #pragma unroll
       for (int w = 0; w < W; w++) L += lw[w] * __expf(mw[w] - ms);
-      const uint32_t col = c0 + r / G, hq = g * G + r % G;
-      const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
+      const size_t slot = ((size_t)rowcol[r] * nH + rowhq[r]) * p.slots + sp;
       *(float2*)(p.part_ml + slot * 2) = make_float2(Mr, L);
     }
     if (nb + 1 < NB) __syncthreads();                                  // the regions are rewritten by the next row block
@@ -1218,7 +1224,9 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
 template <int HD, int NB, int W>
 static constexpr size_t decode_lds_bytes() {
   typedef DecShape<HD> S;
-  return 16 * NB * S::QROW + (size_t)W * S::STAGE + 2 * W * 16 * NB * sizeof(float) + (NB == 2 && W == 4 ? (size_t)W * NB * 1024 : 0);   // (+ the P region of the single-round kernel with two row blocks)
+  // q rows, the waves' staging regions, the (m, l) exchange and the merge's weight table, its two row tables, and the
+  // P region of the single-round kernel with two row blocks
+  return 16 * NB * S::QROW + (size_t)W * S::STAGE + 3 * W * 16 * NB * sizeof(float) + 2 * 16 * NB * sizeof(uint32_t) + (NB == 2 && W == 4 ? (size_t)W * NB * 1024 : 0);
 }
 // the kernel's dynamic LDS limit, raised once per instantiation (at its first launch, or ahead of it by
 // pa_prepare_decode_step)
