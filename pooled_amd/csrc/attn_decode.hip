@@ -245,6 +245,10 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t ln = lane & 15, kg = lane >> 4;
   const uint32_t G = p.group, nH = p.n_heads;
+  // row r of the stacked tile is (column r / G, head r % G): the quotient as a multiply and a shift (exact for r < 1024 and
+  // G <= 64; a division by a run-time G is some thirty instructions, and the q loads' addresses wait for four of them a row block)
+  const uint32_t g_magic = (65536u + G - 1u) / G;
+  auto div_g = [&](uint32_t r) __attribute__((always_inline)) -> uint32_t { return (r * g_magic) >> 16; };
   const uint32_t c0 = FUSED ? 0u : cg * p.cols_per_group;            // (the fused step serves one column)
   const uint32_t ncl = FUSED ? 1u : min(p.cols_per_group, p.n_cols - c0);
   const uint32_t R = ncl * G;                                        // live rows (<= 16*NB)
@@ -413,7 +417,8 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       const uint32_t e = tid + j * W * 64;
       const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
       const uint32_t rc = min(r, R - 1);                             // padding rows copy the last live row (masked out later)
-      qv[j] = *(const f4*)(p.q + (size_t)(c0 + rc / G) * p.q_stride + (size_t)(g * G + rc % G) * HD + 4 * d4);
+      const uint32_t qc = div_g(rc);
+      qv[j] = *(const f4*)(p.q + (size_t)(c0 + qc) * p.q_stride + (size_t)(g * G + rc - qc * G) * HD + 4 * d4);
     }
   }
   // Loads are unconditional: the caches carry TILE rows of padding past max_seq, so a tile that straddles the
@@ -539,7 +544,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     const uint32_t r = nb * 16 + ln;
-    end_pos[nb] = r < R ? (GATHER ? seq_max : p.base_pos + c0 + r / G + 1 - p.self_row) : 0u;
+    end_pos[nb] = r < R ? (GATHER ? seq_max : p.base_pos + c0 + div_g(r) + 1 - p.self_row) : 0u;
   }
   __syncthreads();
   // ---- the column's own row as a partial of its own (slot = number of splits that hold rows): m = its score,
@@ -805,7 +810,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
           }
           const uint32_t r = nb * 16 + ln;
           if (r < R) {
-            const uint32_t col = c0 + r / G, hq = g * G + r % G;
+            const uint32_t rc = div_g(r), col = c0 + rc, hq = g * G + r - rc * G;
             const size_t slot = ((size_t)col * nH + hq) * p.slots + sp;
             // f16 partials (|O| <= 128 rows x |v|: far inside the range; the merge adds them up in f32): half the bytes this
             // kernel writes at its very end and half of what the merge kernel waits for
@@ -929,7 +934,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   // exp(m_w - M), comes from a table one thread per (wave, row) fills, and is applied where the rows are summed.  So is the
   // (column, head) of a stacked row: a table filled once, instead of a division by the group size per element group.
   const bool direct = p.direct_out != 0;       // one split and no own-row partial: this workgroup holds the whole result
-  if (tid < 16 * NB) { rowcol[tid] = c0 + tid / G; rowhq[tid] = g * G + tid % G; }
+  if (tid < 16 * NB) { const uint32_t rc = div_g(tid); rowcol[tid] = c0 + rc; rowhq[tid] = g * G + tid - rc * G; }
 #pragma unroll
   for (int nb = 0; nb < NB; nb++) {
     l_run[nb] = rows_sum(l_run[nb]);
