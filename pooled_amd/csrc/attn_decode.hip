@@ -236,11 +236,14 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
     // id i runs on XCD i % 8 and XCD k owns the contiguous item range [k per, (k + 1) per): the column groups of a
     // (kv head, split) read the same K/V rows, so they sit on one XCD, side by side, and share the rows in its L2
     // whatever the number of splits.
-    const uint32_t ncg = (p.n_cols + p.cols_per_group - 1) / p.cols_per_group;
+    const uint32_t ncg = p.col_groups;
     const uint32_t total = p.n_splits * p.n_kv_heads * ncg, per = (total + 7) / 8;
     const uint32_t item = (blockIdx.x % 8) * per + blockIdx.x / 8;
     if (item >= total) return;
-    cg = item % ncg; sp = (item / ncg) % p.n_splits; g = item / (ncg * p.n_splits);
+    // floor(n / d) = mulhi(n, ceil(2^32 / d)) while n d < 2^32 (the launcher checks): the first tile's addresses wait for these
+    const uint32_t q1 = p.ncg_magic ? __umulhi(item, p.ncg_magic) : (ncg == 1 ? item : item / ncg);
+    const uint32_t q2 = p.ns_magic ? __umulhi(q1, p.ns_magic) : (p.n_splits == 1 ? q1 : q1 / p.n_splits);
+    cg = item - q1 * ncg; sp = q1 - q2 * p.n_splits; g = q2;
   }
   const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t ln = lane & 15, kg = lane >> 4;
@@ -1254,10 +1257,16 @@ static hipError_t launch_decode_k(const AttnParams& p, uint32_t col_groups, hipS
   if (e != hipSuccess) return e;
   if (!SR && col_groups != (p.n_cols + p.cols_per_group - 1) / p.cols_per_group) return hipErrorInvalidValue;
   const dim3 grid = SR ? dim3(p.n_splits, p.n_kv_heads, col_groups) : dim3((p.n_splits * p.n_kv_heads * col_groups + 7) / 8 * 8);
+  AttnParams pk = p;
+  {
+    const uint64_t total = (uint64_t)p.n_splits * p.n_kv_heads * col_groups;
+    auto magic = [&](uint32_t d) -> uint32_t { return d > 1 && total * d < (1ull << 32) ? (uint32_t)(((1ull << 32) + d - 1) / d) : 0u; };
+    pk.col_groups = col_groups; pk.ncg_magic = magic(col_groups); pk.ns_magic = magic(p.n_splits);
+  }
   // (bit 1 of the self_row argument: the columns of a column-exact block on adjacent dispatch ids of an XCD)
   const uint32_t self_arg = p.self_row | (SR && p.exact_cols ? 2u : 0u);
   PA_LAUNCH((pa_decode_kernel<HD, NB, W, FUSED, GATHER, Q8, SR>), grid, dim3(W * 64), lds, s, t, p.k_cache, p.base_pos, p.max_seq, p.n_splits, self_arg,
-            (uint32_t)grid.x, p.f_q_in, p.group, p.f_q_head_stride, p);
+            (uint32_t)grid.x, p.f_q_in, p.group, p.f_q_head_stride, pk);
   return hipGetLastError();
 }
 

@@ -61,6 +61,9 @@ struct AttnParams {
   const uint32_t* sel; uint32_t sel_stride, sel_max;
   uint32_t exact_cols;                        // 1: a column-exact verify block in one launch: every column is a column group of its
                                               // own under the plan of a one-column decode (the merge must be the wavefront kernel)
+  uint32_t col_groups, ncg_magic, ns_magic;   // tile loop (set by its launcher): the column groups of the pass and ceil(2^32 / d) for d = col_groups
+                                              // and d = n_splits, so that the kernel maps its dispatch id to (column group, split, kv head) with
+                                              // two multiplies instead of four divisions (0: d is 1, or the ids are too large for the identity)
   uint32_t single_round2;                     // 1: two row blocks on the single-round kernel (splits of one tile per wave)
   uint32_t tile_ilv;                          // tile loop of the split-K kernel on a contiguous cache: rows from one split's first tile
                                               // to the next split's (32 x waves) when the tiles of a kv head are dealt round robin to the
