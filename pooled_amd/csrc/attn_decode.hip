@@ -1008,10 +1008,10 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
           const float ms = Mr == NEG_INF ? 0.f : Mr;
 #pragma unroll
           for (int w = 0; w < W; w++) L += lex[w * 16 * NB + r] * __expf(mex[w * 16 * NB + r] - ms);
-          o = o / L;
+          o = o * __builtin_amdgcn_rcpf(L);                              // (v_rcp_f32, 1 ulp, as in the merge kernels)
           if (p.gate) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) o[i] *= 1.f / (1.f + __expf(-gtv[j][i]));
+            for (int i = 0; i < 4; i++) o[i] *= __builtin_amdgcn_rcpf(1.f + __expf(-gtv[j][i]));
           }
           if (p.out_f16) {
             const h4 hv = { (_Float16)o[0], (_Float16)o[1], (_Float16)o[2], (_Float16)o[3] };
@@ -1141,10 +1141,11 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
     }
   }
   if (lane < LPG) {
-    f4 r = ns ? o / L : zero;                      // an empty gather list: a column of zeros
+    // (reciprocals by v_rcp_f32, 1 ulp: eight IEEE divisions were some eighty instructions at the very end of the kernel)
+    f4 r = ns ? o * __builtin_amdgcn_rcpf(L) : zero;   // an empty gather list: a column of zeros
     if (p.gate) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) r[i] *= 1.f / (1.f + __expf(-gt[i]));
+      for (int i = 0; i < 4; i++) r[i] *= __builtin_amdgcn_rcpf(1.f + __expf(-gt[i]));
     }
     if (p.out_f16) {
       const h4 hv = { (_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3] };
@@ -1215,11 +1216,11 @@ __global__ __launch_bounds__(256) void pa_combine_wide_kernel(AttnParams p) {
       }
     }
   }
-  f4 r = ns ? o / L : (f4){0.f, 0.f, 0.f, 0.f};
+  f4 r = ns ? o * __builtin_amdgcn_rcpf(L) : (f4){0.f, 0.f, 0.f, 0.f};
   const uint32_t d = 4 * d4;
   if (p.gate) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) r[i] *= 1.f / (1.f + __expf(-gt[i]));
+    for (int i = 0; i < 4; i++) r[i] *= __builtin_amdgcn_rcpf(1.f + __expf(-gt[i]));
   }
   if (p.out_f16) {
     const h4 hv = { (_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3] };
