@@ -68,6 +68,16 @@ static __device__ inline float rows_sum(float v) {
   xrow16(v, a, b); v = a + b;
   xrow32(v, a, b); return a + b;
 }
+// acc + the sum of eight f16 probabilities, as the numbers the PV product really uses (v_dot2_f32_f16 with ones: products
+// exact, sums in f32): the row total l is then the total of the weights that were applied, so a row's output is a convex
+// combination of value rows whatever the rounding of P did -- one visible row gives that row's bits back, constant
+// values give the constant
+static __device__ inline float sum_f16(const h8 pf, float acc) {
+  const h2 ones = { (_Float16)1.f, (_Float16)1.f };
+#pragma unroll
+  for (int j = 0; j < 8; j += 2) { const h2 pp = { pf[j], pf[j + 1] }; acc = __builtin_amdgcn_fdot2(pp, ones, acc, false); }
+  return acc;
+}
 // lane i's copy of lane (i + N) % 16 of its row of 16 (DPP row rotation)
 template <int N>
 static __device__ inline float row_ror(float v) {
@@ -732,11 +742,10 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
           }
         mx = rows_max(mx);
         const float mw_safe = mx == NEG_INF ? 0.f : mx;
-        float ps = 0.f;
         h8 pf;
 #pragma unroll
-        for (int j = 0; j < 8; j++) { const float e = __expf(v[j] - mw_safe); ps += e; pf[j] = (_Float16)e; }
-        mxs[nb] = mx; pss[nb] = rows_sum(ps); pfs[nb] = pf;
+        for (int j = 0; j < 8; j++) pf[j] = (_Float16)__expf(v[j] - mw_safe);
+        mxs[nb] = mx; pss[nb] = rows_sum(sum_f16(pf, 0.f)); pfs[nb] = pf;
       }
       if (v_late) { __builtin_amdgcn_sched_barrier(0); first_v_loads(); __builtin_amdgcn_sched_barrier(0); }
       stage_v(ILV && ilv ? 0u : tp, false, 0);                          // interleaved splits are whole: no row past the end to zero
@@ -891,12 +900,11 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
       const float m_safe = m_run[nb] == NEG_INF ? 0.f : m_run[nb];
-      float ps = 0.f;
       h8 pf;
 #pragma unroll
-      for (int j = 0; j < 8; j++) { const float e = __expf(v[nb][j] - m_safe); ps += e; pf[j] = (_Float16)e; }
+      for (int j = 0; j < 8; j++) pf[j] = (_Float16)__expf(v[nb][j] - m_safe);
       pfrag[nb] = pf;
-      l_run[nb] += ps;
+      l_run[nb] = sum_f16(pf, l_run[nb]);
     }
     // V after the softmax, so that the wait for the V loads comes as late as possible
     stage_v(tp, more, tp + tp_step);

@@ -61,6 +61,36 @@ def test_decode_closed_forms():
         assert np.abs(pa.run_attn("decode", 0, q, L - 1) - 0.75).max() < 1e-3
 
 
+@pytest.mark.parametrize("shape", ["qwen36_moe", "qwen38_27b", "qwen3_1p7b"])
+def test_outputs_are_convex_combinations_of_value_rows(shape):
+    """Every value row the same vector => the output is that vector, whatever the scores: the row total l is summed
+    from the f16-rounded probabilities the PV product uses, so the weights that are applied add up to exactly the
+    divisor and the rounding of P cancels (with l summed from the unrounded exponentials the outputs were off by up to
+    3e-4 of the value on short contexts).  What is left is f32 accumulation: a few 1e-7.  One-column decodes and verify
+    blocks on the single-round kernel and on the tile loop, chunks on the split-K kernel with direct output and on the
+    matrix-core kernel, with and without a split over the context."""
+    cfg = SHAPES[shape]
+    nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    rng = np.random.default_rng(5)
+    L = 40000
+    k16, _ = random_cache(cfg, L, seed=3, k_scale=2.0)
+    vrow = rng.standard_normal((nKV, hd)).astype(np.float16)
+    v16 = np.broadcast_to(vrow.view(np.uint16), (L, nKV, hd)).copy()
+    want = np.repeat(vrow.astype(np.float64), nH // nKV, axis=0)
+    with _ctx_with_cache(cfg, k16, v16, L, max_cols=400) as pa:
+        kernels = set()
+        for kind, n, lens in (("decode", 1, (1, 2, 3, 17, 40, 129, 1500, 33000, 39999)), ("decode", 5, (6, 40, 1500, 33000)),
+                              ("prefill", 12, (12, 300)), ("prefill", 300, (300, 5000))):
+            for Lc in lens:
+                q = rng.standard_normal((n, nH, hd), dtype=np.float32)
+                pl = pa.plan(kind, Lc - n, n)
+                kernels.add((pl["kernel"], pl["n_splits"] > 1, pl["split_len"] == 128))
+                o = pa.run_attn(kind, 0, q, Lc - n).astype(np.float64)
+                err = np.abs(o - want[None]).max() / np.abs(want).max()
+                assert err < 2e-6, "%s %s %d columns over %d rows: %.2e of the value (%s)" % (shape, kind, n, Lc, err, pl)
+        assert {k[0] for k in kernels} == {0, 1} and any(k[1] and k[2] for k in kernels) and any(k[1] and not k[2] for k in kernels), kernels
+
+
 def test_decode_split_invariance_and_plan():
     cfg = SHAPES["qwen36_moe"]
     rng = np.random.default_rng(11)
