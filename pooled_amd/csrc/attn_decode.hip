@@ -15,7 +15,8 @@
 //     query row, 4+4 positions) is exactly the B-operand layout of the PV product, so probabilities never
 //     leave registers.  All G heads of a kv head and all columns of a verify block are rows of one tile, so
 //     K/V are read once for the whole block.
-//   * Softmax state (m, l) and O are f32; q and P are rounded to f16 for the MFMA operands.
+//   * Softmax state (m, l) and O are f32; q and P are rounded to f16 for the MFMA operands, and l is the sum of the
+//     rounded P (an output is a convex combination of value rows whatever that rounding did).
 //   * Every reduction has a fixed order (lane-group shuffles, wave order, split order): run-to-run deterministic,
 //     no atomics.
 //
@@ -116,11 +117,20 @@ static __device__ inline void dq16(const u4 raw, const float sc, h8& lo, h8& hi)
   hi = (h8){ o[4][0], o[4][1], o[5][0], o[5][1], o[6][0], o[6][1], o[7][0], o[7][1] };
 }
 
+// What the f16 rounding of four q values drops, as f16: q = hi + lo to 2^-22 of q.  With at most eight live query rows
+// in a 16-row block, rows 8 .. 15 of the q tile carry the low halves of rows 0 .. 7: the same MFMAs then also produce
+// K q_lo^T (in the lanes of rows 8 .. 15), one row rotation adds it to K q_hi^T, and the scores see q at f32 precision --
+// the rounding of q to f16 is otherwise the largest error of a decode over a short context.
+static __device__ inline h4 q_lo_row(const f4 v, const h4 hi) {
+  return (h4){ (_Float16)(v[0] - (float)hi[0]), (_Float16)(v[1] - (float)hi[1]), (_Float16)(v[2] - (float)hi[2]), (_Float16)(v[3] - (float)hi[3]) };
+}
+
 // Fused pre-step of N query heads of one wave (heads wave, wave + W, ...): norm + rope side by side, then the heads
 // as f16 rows of the q tile.  xs: wave-private LDS scratch of N x HD floats.
 template <int N, int HD, int W, int QROW>
 static __device__ inline void fused_q_rows(const float (&xq)[16 / W][4], const float (&wq)[4], bool norm, float eps, uint32_t half,
-                                           const float2 (&cs)[2], float* xs, unsigned char* q_lds, uint32_t G, uint32_t wave, uint32_t lane) {
+                                           const float2 (&cs)[2], float* xs, unsigned char* q_lds, uint32_t G, uint32_t wave, uint32_t lane,
+                                           bool qsplit) {
   static_assert(N <= 16 / W, "at most 16 query heads per kv head");
   float x[N][4];
 #pragma unroll
@@ -135,7 +145,11 @@ static __device__ inline void fused_q_rows(const float (&xq)[16 / W][4], const f
       const uint32_t r = wave + W * n;
       if (r < G) {
 #pragma unroll
-        for (int j = 0; j < HD / 64; j++) *(_Float16*)(q_lds + r * QROW + (lane + 64 * j) * 2) = (_Float16)x[n][j];
+        for (int j = 0; j < HD / 64; j++) {
+          const _Float16 hi = (_Float16)x[n][j];
+          *(_Float16*)(q_lds + r * QROW + (lane + 64 * j) * 2) = hi;
+          if (qsplit) *(_Float16*)(q_lds + (r + 8) * QROW + (lane + 64 * j) * 2) = (_Float16)(x[n][j] - (float)hi);     // (see q_lo_row)
+        }
       }
     }
     wave_lds_fence();
@@ -149,10 +163,13 @@ static __device__ inline void fused_q_rows(const float (&xq)[16 / W][4], const f
       const f4 v = *(const f4*)(xs + n * HD + 4 * lane);
       const h4 hv = { (_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3] };
       *(h4*)(q_lds + r * QROW + lane * 8) = hv;
+      if (qsplit) *(h4*)(q_lds + (r + 8) * QROW + lane * 8) = q_lo_row(v, hv);
     }
   }
   wave_lds_fence();
 }
+
+#define PA_QSPLIT_MAX_ROWS 2048u
 
 template <int HD> struct DecShape {
   static constexpr int LPR = HD / 8;            // lanes per f16 row at 16 bytes a lane
@@ -269,6 +286,11 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   // rows visible to the group's last column (gather: the column's list length)
   // self_row (one-column decode): the column's own row base_pos is not streamed with the others -- see below
   const uint32_t seq_max = GATHER ? min(p.sel[c0 * p.sel_stride], p.sel_max) : p.base_pos + c0 + ncl - p.self_row;
+  // rows 8 .. 15 of the q tile hold the low halves of rows 0 .. 7 (q_lo_row): a one-column decode, or a block of at most
+  // eight stacked rows, over a short context -- where a softmax over few rows averages nothing out and the f16 rounding of
+  // q is most of the error (over thousands of rows it is a few percent of the tolerance, and the extra work a few
+  // tenths of a microsecond on a step of sixteen)
+  const bool qsplit = NB == 1 && R <= 8 && seq_max < PA_QSPLIT_MAX_ROWS;
   const uint32_t split_len = SR ? (uint32_t)(W * TILE) : p.split_len;   // single-round splits: one tile per wave
   // TILV (tile loop on a contiguous cache, p.tile_ilv): the tiles of a kv head are dealt round robin to the waves of
   // all its splits -- wave v of the n_splits x W takes tiles v, v + n_splits W, ... -- so the loads in flight on the chip
@@ -429,7 +451,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
     for (int j = 0; j < QPT; j++) {
       const uint32_t e = tid + j * W * 64;
       const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
-      const uint32_t rc = min(r, R - 1);                             // padding rows copy the last live row (masked out later)
+      const uint32_t rc = min(qsplit && r >= 8 ? r - 8 : r, R - 1);  // padding rows copy the last live row (masked out later)
       const uint32_t qc = div_g(rc);
       qv[j] = *(const f4*)(p.q + (size_t)(c0 + qc) * p.q_stride + (size_t)(g * G + rc - qc * G) * HD + 4 * d4);
     }
@@ -495,13 +517,15 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
     float* xs = (float*)stage;       // wave-private scratch (the staging region is not in use yet)
     // this wave's query heads wave, wave + W, ... side by side (ceil(G / W) of them; one past G is computed and dropped)
     switch ((G + W - 1) / W) {
-      case 1: fused_q_rows<1, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
-      case 2: fused_q_rows<2, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
-      case 3: if constexpr (W <= 4) fused_q_rows<3, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
-      default: if constexpr (W <= 4) fused_q_rows<4, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane); break;
+      case 1: fused_q_rows<1, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane, qsplit); break;
+      case 2: fused_q_rows<2, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane, qsplit); break;
+      case 3: if constexpr (W <= 4) fused_q_rows<3, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane, qsplit); break;
+      default: if constexpr (W <= 4) fused_q_rows<4, HD, W, S::QROW>(xq, wq, p.f_qw != nullptr, p.eps, half, cs, xs, q_lds, G, wave, lane, qsplit); break;
     }
-    for (uint32_t e = tid; e < (16 - G) * (HD / 4); e += W * 64)     // padding rows (masked out later)
-      *(h4*)(q_lds + (G + e / (HD / 4)) * S::QROW + (e % (HD / 4)) * 8) = (h4){0, 0, 0, 0};
+    for (uint32_t e = tid; e < (16 - G) * (HD / 4); e += W * 64) {   // padding rows (masked out later)
+      const uint32_t row = G + e / (HD / 4);
+      if (!(qsplit && row - 8 < G)) *(h4*)(q_lds + row * S::QROW + (e % (HD / 4)) * 8) = (h4){0, 0, 0, 0};    // (rows 8 .. 8 + G - 1: the low halves)
+    }
     if (self_wave) {                 // the new key row: normed, roped, rounded; it and the value row go to the cache
       glue_head_wave(xk, wk, p.f_kw != nullptr, p.eps, HD, half, cs, xs, lane);
       if constexpr (Q8) {
@@ -544,7 +568,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       const uint32_t e = tid + j * W * 64;
       const uint32_t r = e / (HD / 4), d4 = e % (HD / 4);
       const h4 hv = { (_Float16)qv[j][0], (_Float16)qv[j][1], (_Float16)qv[j][2], (_Float16)qv[j][3] };
-      *(h4*)(q_lds + r * S::QROW + d4 * 8) = hv;
+      *(h4*)(q_lds + r * S::QROW + d4 * 8) = qsplit && r >= 8 ? q_lo_row(qv[j], hv) : hv;
     }
   }
   if (FUSED && !v_late) {
@@ -571,9 +595,11 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
     const f4 vxf = { (float)vx[0], (float)vx[1], (float)vx[2], (float)vx[3] };
     for (uint32_t r = 0; r < G; r++) {                                 // one column: row r is head g * G + r
       const h4 qv = *(const h4*)(q_lds + r * S::QROW + min(lane, (uint32_t)HD / 4 - 1) * 8);
+      h4 ql = {0, 0, 0, 0};
+      if (qsplit) ql = *(const h4*)(q_lds + (r + 8) * S::QROW + min(lane, (uint32_t)HD / 4 - 1) * 8);
       float d = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; i++) d = __builtin_fmaf((float)qv[i], (float)kx[i], d);
+      for (int i = 0; i < 4; i++) d = __builtin_fmaf((float)qv[i] + (float)ql[i], (float)kx[i], d);
       if (!on) d = 0.f;
       d = wave_sum_f32(d);
       const size_t slot = ((size_t)c0 * nH + g * G + r) * p.slots + self_slot;
@@ -662,6 +688,14 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       for (int ks = 0; ks < S::KS; ks++) {
         if (ks + FD < S::KS) __builtin_amdgcn_sched_group_barrier(0x100, 2 + NB, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
+      }
+    }
+    if constexpr (NB == 1) {
+      if (qsplit) {                      // K q_lo^T sits in the lanes of rows 8 .. 15: rows 0 .. 7 take it from there
+#pragma unroll
+        for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) s[pb][0][i] += row_ror<8>(s[pb][0][i]);
       }
     }
     wave_lds_fence();
@@ -1058,7 +1092,7 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
 // the output partials of its group's splits (group + 16 k) in one round trip, the maximum and the sums over the 16
 // groups are xor-shuffle trees (fixed order), lanes 0 .. 3 finish and store.  The four lanes of a group hold the same
 // (m, l), so each computes its splits' weights itself instead of fetching them from a neighbour.
-template <int HD, int DS, bool PF16>
+template <int HD, int DS, bool PF16, int CH>
 __global__ __launch_bounds__(64)
 void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint32_t a_slots, uint32_t a_n_heads, uint32_t a_base_pos, uint32_t a_self_row,
                             uint32_t a_split_len, uint32_t a_n_splits, uint32_t a_grid_x, uint32_t a_has_sel, AttnParams p_in) {
@@ -1068,7 +1102,9 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
   AttnParams p = p_in;
   p.part_o = const_cast<float*>(a_part_o); p.part_ml = const_cast<float*>(a_part_ml); p.slots = a_slots; p.n_heads = a_n_heads;
   p.base_pos = a_base_pos; p.self_row = a_self_row; p.split_len = a_split_len; p.n_splits = a_n_splits;
-  constexpr int SL = HD / DS, LPG = DS / 4, NG = 64 / LPG, CH = (272 + NG - 1) / NG;     // CH splits per lane and chunk: NG x CH >= 272 (256 + the own-row partial)
+  // CH splits per lane and chunk (a template argument: the launcher takes the smallest of 5 / 9 / 17 whose NG x CH covers the
+  // pass's slots -- 272 = 256 splits and the own-row partial at the most, 129 or 65 on the tile loop's plans; more go round the loop below)
+  constexpr int SL = HD / DS, LPG = DS / 4, NG = 64 / LPG;
   // dispatch id i runs on XCD i % 8: XCD k takes the contiguous slice range [k n / 8, (k + 1) n / 8), so the slices that
   // share the 128-byte lines of a partial row (two 16-dim slices a line) read them through one L2
   uint32_t wg = blockIdx.x;
@@ -1370,10 +1406,15 @@ hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s, co
   // rows from one split's first row to the next one's (round-robin tiles: a workgroup's first tiles)
   const uint32_t live_len = p.tile_ilv ? p.tile_ilv : p.split_len;
   if (hd != 256 && hd != 128) return hipErrorInvalidValue;
-#define PA_COMBINE_WAVE(HD_, F16_) PA_LAUNCH((pa_combine_wave_kernel<HD_, 16, F16_>), dim3(gx, p.n_cols), dim3(64), 0, s, t, (const float*)p.part_o, \
+#define PA_COMBINE_WAVE_(HD_, F16_, CH_) PA_LAUNCH((pa_combine_wave_kernel<HD_, 16, F16_, CH_>), dim3(gx, p.n_cols), dim3(64), 0, s, t, (const float*)p.part_o, \
     (const float*)p.part_ml, p.slots, p.n_heads, p.base_pos, p.self_row, live_len, p.n_splits, gx, has_sel, p)
+  // a lane's unrolled loads are guarded one by one: a pass with few slots takes the instantiation with few of them
+  // (f16 partials come from 64 splits on, so their short form is never needed)
+#define PA_COMBINE_WAVE(HD_, F16_) do { if (F16_ || p.slots > 144) PA_COMBINE_WAVE_(HD_, F16_, 17); \
+    else if (p.slots > 80) PA_COMBINE_WAVE_(HD_, F16_, (F16_ ? 17 : 9)); else PA_COMBINE_WAVE_(HD_, F16_, (F16_ ? 17 : 5)); } while (0)
   if (hd == 256) { if (p.part_f16) PA_COMBINE_WAVE(256, true); else PA_COMBINE_WAVE(256, false); }
   else { if (p.part_f16) PA_COMBINE_WAVE(128, true); else PA_COMBINE_WAVE(128, false); }
 #undef PA_COMBINE_WAVE
+#undef PA_COMBINE_WAVE_
   return hipGetLastError();
 }
