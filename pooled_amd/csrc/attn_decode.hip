@@ -120,7 +120,8 @@ static __device__ inline void dq16(const u4 raw, const float sc, h8& lo, h8& hi)
 // What the f16 rounding of four q values drops, as f16: q = hi + lo to 2^-22 of q.  With at most eight live query rows
 // in a 16-row block, rows 8 .. 15 of the q tile carry the low halves of rows 0 .. 7: the same MFMAs then also produce
 // K q_lo^T (in the lanes of rows 8 .. 15), one row rotation adds it to K q_hi^T, and the scores see q at f32 precision --
-// the rounding of q to f16 is otherwise the largest error of a decode over a short context.
+// the rounding of q to f16 is otherwise the largest error of a decode wherever a few rows share the weight (short
+// contexts, peaked scores).
 static __device__ inline h4 q_lo_row(const f4 v, const h4 hi) {
   return (h4){ (_Float16)(v[0] - (float)hi[0]), (_Float16)(v[1] - (float)hi[1]), (_Float16)(v[2] - (float)hi[2]), (_Float16)(v[3] - (float)hi[3]) };
 }
@@ -168,8 +169,6 @@ static __device__ inline void fused_q_rows(const float (&xq)[16 / W][4], const f
   }
   wave_lds_fence();
 }
-
-#define PA_QSPLIT_MAX_ROWS 2048u
 
 template <int HD> struct DecShape {
   static constexpr int LPR = HD / 8;            // lanes per f16 row at 16 bytes a lane
@@ -286,11 +285,9 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
   // rows visible to the group's last column (gather: the column's list length)
   // self_row (one-column decode): the column's own row base_pos is not streamed with the others -- see below
   const uint32_t seq_max = GATHER ? min(p.sel[c0 * p.sel_stride], p.sel_max) : p.base_pos + c0 + ncl - p.self_row;
-  // rows 8 .. 15 of the q tile hold the low halves of rows 0 .. 7 (q_lo_row): a one-column decode, or a block of at most
-  // eight stacked rows, over a short context -- where a softmax over few rows averages nothing out and the f16 rounding of
-  // q is most of the error (over thousands of rows it is a few percent of the tolerance, and the extra work a few
-  // tenths of a microsecond on a step of sixteen)
-  const bool qsplit = NB == 1 && R <= 8 && seq_max < PA_QSPLIT_MAX_ROWS;
+  // rows 8 .. 15 of the q tile hold the low halves of rows 0 .. 7 (q_lo_row): every one-column decode with G <= 8, and
+  // blocks of at most eight stacked rows
+  const bool qsplit = NB == 1 && R <= 8;
   const uint32_t split_len = SR ? (uint32_t)(W * TILE) : p.split_len;   // single-round splits: one tile per wave
   // TILV (tile loop on a contiguous cache, p.tile_ilv): the tiles of a kv head are dealt round robin to the waves of
   // all its splits -- wave v of the n_splits x W takes tiles v, v + n_splits W, ... -- so the loads in flight on the chip
@@ -593,6 +590,17 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
     const uint32_t self_slot = min((seq_max + live_len - 1) / live_len, p.n_splits);
     const bool on = lane < HD / 4;
     const f4 vxf = { (float)vx[0], (float)vx[1], (float)vx[2], (float)vx[3] };
+    // No store inside the loop: while the chip streams, the memory pipeline accepts a store as slowly as a load, and
+    // with a partial row and an (m, l) pair stored per head this one wave -- the last of the kernel to start on its tile
+    // -- ran microseconds behind the rest and set the end of the kernel.  The G heads of a kv head share the value row, so
+    // it is stored once, under the kv head's first head (the merge reads it there for every head), up front; lane r keeps
+    // head r's score and the G (m, l) pairs leave in one store behind the loop.
+    const size_t slot0 = ((size_t)c0 * nH + g * G) * p.slots + self_slot;
+    if (on) {
+      if (p.part_f16) *(h4*)((_Float16*)p.part_o + slot0 * HD + 4 * lane) = vx;
+      else *(f4*)(p.part_o + slot0 * HD + 4 * lane) = vxf;
+    }
+    float dv = 0.f;
     for (uint32_t r = 0; r < G; r++) {                                 // one column: row r is head g * G + r
       const h4 qv = *(const h4*)(q_lds + r * S::QROW + min(lane, (uint32_t)HD / 4 - 1) * 8);
       h4 ql = {0, 0, 0, 0};
@@ -602,13 +610,9 @@ void pa_decode_kernel(const uint16_t* a_k_cache, uint32_t a_base_pos, uint32_t a
       for (int i = 0; i < 4; i++) d = __builtin_fmaf((float)qv[i] + (float)ql[i], (float)kx[i], d);
       if (!on) d = 0.f;
       d = wave_sum_f32(d);
-      const size_t slot = ((size_t)c0 * nH + g * G + r) * p.slots + self_slot;
-      if (on) {
-        if (p.part_f16) *(h4*)((_Float16*)p.part_o + slot * HD + 4 * lane) = vx;
-        else *(f4*)(p.part_o + slot * HD + 4 * lane) = vxf;
-      }
-      if (lane == 0) *(float2*)(p.part_ml + slot * 2) = make_float2(d * p.scale, 1.f);
+      if (lane == r) dv = d;
     }
+    if (lane < G) *(float2*)(p.part_ml + (slot0 + (size_t)lane * p.slots) * 2) = make_float2(dv * p.scale, 1.f);
   }
   if (!has_rows) return;
 
@@ -1101,9 +1105,10 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
   // arguments are fetched in one batch behind those loads (the compiler would fetch each where it is first used).
   AttnParams p = p_in;
   p.part_o = const_cast<float*>(a_part_o); p.part_ml = const_cast<float*>(a_part_ml); p.slots = a_slots; p.n_heads = a_n_heads;
-  p.base_pos = a_base_pos; p.self_row = a_self_row; p.split_len = a_split_len; p.n_splits = a_n_splits;
-  // CH splits per lane and chunk (a template argument: the launcher takes the smallest of 5 / 9 / 17 whose NG x CH covers the
-  // pass's slots -- 272 = 256 splits and the own-row partial at the most, 129 or 65 on the tile loop's plans; more go round the loop below)
+  // a_self_row: 0, or G | ceil(65536 / G) << 8 for a pass whose columns' own rows are partials of their own
+  p.base_pos = a_base_pos; p.self_row = a_self_row != 0; p.split_len = a_split_len; p.n_splits = a_n_splits;
+  // CH splits per lane and chunk (a template argument: the launcher takes the smallest of 4 / 8 / 16 whose NG x CH covers the
+  // pass's splits -- 256 at the most on the single-round kernel, 128 or 64 on the tile loop's plans; more go round the loop below)
   constexpr int SL = HD / DS, LPG = DS / 4, NG = 64 / LPG;
   // dispatch id i runs on XCD i % 8: XCD k takes the contiguous slice range [k n / 8, (k + 1) n / 8), so the slices that
   // share the 128-byte lines of a partial row (two 16-dim slices a line) read them through one L2
@@ -1111,8 +1116,12 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
   if (a_grid_x % 8 == 0) wg = (blockIdx.x % 8) * (a_grid_x / 8) + blockIdx.x / 8;
   const uint32_t h = wg / SL, dq = wg % SL, col = blockIdx.y, lane = threadIdx.x;
   const uint32_t col_end = a_has_sel ? min(p.sel[col * p.sel_stride], p.sel_max) : p.base_pos + col + 1 - p.self_row;
-  const uint32_t ns = min((col_end + p.split_len - 1) / p.split_len, p.n_splits) + p.self_row;
+  // ns_main splits hold streamed rows; the own row's partial, if there is one, is slot ns_main: its (m, l) under this head,
+  // its O row under the kv head's first head (the G heads share the value row; the decode kernel stores it once)
+  const uint32_t ns_main = min((col_end + p.split_len - 1) / p.split_len, p.n_splits), ns = ns_main + p.self_row;
   const size_t base = ((size_t)col * p.n_heads + h) * p.slots;
+  const uint32_t G_ = a_self_row & 0xffu, h0 = ((h * (a_self_row >> 8)) >> 16) * G_;      // (h / G) G by multiply and shift
+  const size_t own = (((size_t)col * p.n_heads + h0) * p.slots + ns_main) * HD;             // the own row's O, in elements
   const uint32_t grp = lane / LPG, l4 = lane % LPG;
   const float* po = p.part_o + base * HD + dq * DS + 4 * l4;
   const _Float16* po16 = (const _Float16*)p.part_o + base * HD + dq * DS + 4 * l4;       // PF16: f16 partial rows
@@ -1127,13 +1136,18 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
     else return *(const f4*)(po + (size_t)s * HD);
   };
   auto wide = [&](const orow v) __attribute__((always_inline)) -> f4 { return (f4){ (float)v[0], (float)v[1], (float)v[2], (float)v[3] }; };
-  orow ov[CH];
-  float2 mlv[CH];
+  orow ov[CH], ov_own = zrow;
+  float2 mlv[CH], ml_own = make_float2(NEG_INF, 0.f);
+  if (p.self_row) {                             // every group loads the own row (a wave-uniform branch); group 0 counts it
+    ml_own = pml[ns_main];
+    if constexpr (PF16) ov_own = *(const h4*)((const _Float16*)p.part_o + own + dq * DS + 4 * l4);
+    else ov_own = *(const f4*)(p.part_o + own + dq * DS + 4 * l4);
+  }
 #pragma unroll
   for (int k = 0; k < CH; k++) {
     const uint32_t s = grp + NG * k;
-    mlv[k] = s < ns ? pml[s] : make_float2(NEG_INF, 0.f);
-    ov[k] = s < ns ? load_o(s) : zrow;
+    mlv[k] = s < ns_main ? pml[s] : make_float2(NEG_INF, 0.f);
+    ov[k] = s < ns_main ? load_o(s) : zrow;
   }
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("" :: "s"(p.gate), "s"(p.out), "s"(p.gate_stride), "s"(p.out_stride), "s"(p.out_f16), "s"(p.gate_head_stride));
@@ -1143,7 +1157,8 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
   float M = NEG_INF;
 #pragma unroll
   for (int k = 0; k < CH; k++) M = fmaxf(M, mlv[k].x);
-  for (uint32_t s = grp + NG * CH; s < ns; s += NG) M = fmaxf(M, pml[s].x);        // more than 272 splits
+  for (uint32_t s = grp + NG * CH; s < ns_main; s += NG) M = fmaxf(M, pml[s].x);   // more splits than NG x CH
+  M = fmaxf(M, ml_own.x);
   // over the 16 split groups: on the VALU (row rotations + lane swaps) with four lanes a group, else through the LDS crossbar
   if constexpr (LPG == 4 || LPG == 8) M = quads_max<LPG>(M);
   else {
@@ -1158,12 +1173,12 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
     L += mlv[k].y * w;
     o += wide(ov[k]) * w;
   }
-  for (uint32_t s0 = NG * CH; s0 < ns; s0 += NG * CH) {
+  for (uint32_t s0 = NG * CH; s0 < ns_main; s0 += NG * CH) {
 #pragma unroll
     for (int k = 0; k < CH; k++) {
       const uint32_t s = s0 + grp + NG * k;
-      mlv[k] = s < ns ? pml[s] : make_float2(NEG_INF, 0.f);
-      ov[k] = s < ns ? load_o(s) : zrow;
+      mlv[k] = s < ns_main ? pml[s] : make_float2(NEG_INF, 0.f);
+      ov[k] = s < ns_main ? load_o(s) : zrow;
     }
 #pragma unroll
     for (int k = 0; k < CH; k++) {
@@ -1171,6 +1186,11 @@ void pa_combine_wave_kernel(const float* a_part_o, const float* a_part_ml, uint3
       L += mlv[k].y * w;
       o += wide(ov[k]) * w;
     }
+  }
+  {
+    const float w = grp == 0 ? __expf(ml_own.x - M) : 0.f;      // last in group 0's sums, as slot ns_main would be; (-inf, 0) and zeros where there is no own row
+    L += ml_own.y * w;
+    o += wide(ov_own) * w;
   }
   if constexpr (LPG == 4 || LPG == 8) {
     L = quads_sum<LPG>(L);
@@ -1395,7 +1415,7 @@ hipError_t pa_launch_decode_gather(const AttnParams& p, uint32_t hd, hipStream_t
 
 hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s, const PaTiming* t) {
   // many columns, few splits: one thread per (column, head, 4 dims)
-  if (p.n_cols >= 16 && p.n_splits <= 32 && (hd == 256 || hd == 128) && !p.exact_cols) {
+  if (p.n_cols >= 16 && p.n_splits <= 32 && (hd == 256 || hd == 128) && !p.exact_cols && !p.self_row) {
     const size_t threads = (size_t)p.n_cols * p.n_heads * (hd / 4);
     const dim3 grid((unsigned)((threads + 255) / 256));
     if (hd == 256) hipLaunchKernelGGL(pa_combine_wide_kernel<256>, grid, dim3(256), 0, s, p);
@@ -1403,15 +1423,17 @@ hipError_t pa_launch_combine(const AttnParams& p, uint32_t hd, hipStream_t s, co
     return hipGetLastError();
   }
   const uint32_t gx = p.n_heads * (hd / 16), has_sel = p.sel != nullptr;
+  // own rows: the group size and ceil(65536 / G) ride in the self_row argument (the kernel finds a kv head's first head)
+  const uint32_t self_arg = p.self_row ? (p.group | ((65536u + p.group - 1) / p.group) << 8) : 0u;
   // rows from one split's first row to the next one's (round-robin tiles: a workgroup's first tiles)
   const uint32_t live_len = p.tile_ilv ? p.tile_ilv : p.split_len;
   if (hd != 256 && hd != 128) return hipErrorInvalidValue;
 #define PA_COMBINE_WAVE_(HD_, F16_, CH_) PA_LAUNCH((pa_combine_wave_kernel<HD_, 16, F16_, CH_>), dim3(gx, p.n_cols), dim3(64), 0, s, t, (const float*)p.part_o, \
-    (const float*)p.part_ml, p.slots, p.n_heads, p.base_pos, p.self_row, live_len, p.n_splits, gx, has_sel, p)
+    (const float*)p.part_ml, p.slots, p.n_heads, p.base_pos, self_arg, live_len, p.n_splits, gx, has_sel, p)
   // a lane's unrolled loads are guarded one by one: a pass with few slots takes the instantiation with few of them
   // (f16 partials come from 64 splits on, so their short form is never needed)
-#define PA_COMBINE_WAVE(HD_, F16_) do { if (F16_ || p.slots > 144) PA_COMBINE_WAVE_(HD_, F16_, 17); \
-    else if (p.slots > 80) PA_COMBINE_WAVE_(HD_, F16_, (F16_ ? 17 : 9)); else PA_COMBINE_WAVE_(HD_, F16_, (F16_ ? 17 : 5)); } while (0)
+#define PA_COMBINE_WAVE(HD_, F16_) do { if (F16_ || p.n_splits > 128) PA_COMBINE_WAVE_(HD_, F16_, 16); \
+    else if (p.n_splits > 64) PA_COMBINE_WAVE_(HD_, F16_, (F16_ ? 16 : 8)); else PA_COMBINE_WAVE_(HD_, F16_, (F16_ ? 16 : 4)); } while (0)
   if (hd == 256) { if (p.part_f16) PA_COMBINE_WAVE(256, true); else PA_COMBINE_WAVE(256, false); }
   else { if (p.part_f16) PA_COMBINE_WAVE(128, true); else PA_COMBINE_WAVE(128, false); }
 #undef PA_COMBINE_WAVE

@@ -93,19 +93,19 @@ def test_outputs_are_convex_combinations_of_value_rows(shape):
 
 @pytest.mark.parametrize("shape", ["qwen36_moe", "qwen38_27b", "qwen3_1p7b"])
 def test_short_context_decode_sees_q_at_f32_precision(shape):
-    """A block of at most eight stacked rows over fewer than 2048 cache rows carries the f16 rounding error of q in rows
-    8 .. 15 of its q tile, so its scores see q at f32 precision.  Inputs that make the rounding of q visible (q of twice,
-    keys of twice the benchmark's spread: scores of a spread of 4, a few rows share the weight) come out within 6e-4 of
+    """A block of at most eight stacked rows carries the f16 rounding error of q in rows 8 .. 15 of its q tile, so its
+    scores see q at f32 precision.  Inputs that make the rounding of q visible (q of twice, keys of twice the
+    benchmark's spread: scores of a spread of 4, a few rows share the weight whatever the length) come out within 6e-4 of
     the f64 oracle (measured: up to 4.1e-4, what the f16 rounding of P leaves); with q rounded to f16 the same inputs are
     off by 1.6e-3 to 4.7e-3."""
     cfg = SHAPES[shape]
     nH, nKV, hd = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
     rng = np.random.default_rng(11)
-    Lmax = 2100
+    Lmax = 4100
     k16, v16 = random_cache(cfg, Lmax, seed=13, k_scale=2.0)
     with _ctx_with_cache(cfg, k16, v16, Lmax) as pa:
         for n in sorted({1, 8 // (nH // nKV)}):
-            for L in (2, 3, 5, 17, 33, 129, 300, 1000, 2047):
+            for L in (2, 3, 5, 17, 33, 129, 300, 1000, 2047, 2049, 4097):
                 if L <= n:
                     continue
                 for rep in range(3):
