@@ -195,7 +195,8 @@ template <int HD> struct DecShape {
 //
 // self_row (every one-column decode, fused or not, f16 or int8 caches): the column's own row base_pos is not streamed with
 // rows 0 .. base_pos - 1; wave 0 of split 0 holds it in registers (from the pre-step above, or loaded), scores it
-// against the G query rows and writes it as one more split partial, which the merge kernel folds in like any other.
+// against the G query rows and writes it as one more split partial: an (m, l) pair under every head, the O row (the value
+// row, the same for the G heads) once, under the kv head's first head, where the merge kernel reads it for all of them.
 //
 // GATHER (the reference's attn_dec_qsa, engine/wgsl/attn_dec.js:33-38, :105, :170-183): each column attends to a
 // list of cache rows instead of rows 0 .. seqLen - 1.  Column col's list is sel[col * sel_stride] = n, then n row

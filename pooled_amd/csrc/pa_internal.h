@@ -40,7 +40,8 @@ struct AttnParams {
   uint32_t cols_per_group;                    // columns per workgroup (grid z = column groups)
   uint32_t max_seq;
   uint32_t self_row;                          // 1: one-column decode whose own row base_pos is a partial of its own (slot
-                                              // = number of splits that hold rows) instead of a streamed row; else 0
+                                              // = number of splits that hold rows) instead of a streamed row; else 0.
+                                              // Its (m, l) sits under every head, its O row under the kv head's first head only
   int out_f16;
   uint32_t direct_out;                        // tile-loop split-K kernel with one split and no own-row partial: the workgroup
                                               // normalises, gates and stores the output itself (no partials, no merge launch)
