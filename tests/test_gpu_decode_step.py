@@ -113,3 +113,5 @@ def test_group_sizes_one_and_sixteen(cfg):
         refb = C.attention(q, K, V, base, gate=gate)
         assert_parity(pa.run_attn("decode", 0, q[:5], base, gate=None if gate is None else gate[:5]), refb[:5], "verify block")
         assert_parity(pa.run_attn("prefill", 0, q, base, gate=gate), refb, "prefill chunk")
+        # the unfused one-column decode: its own row's O partial sits under the kv head's first head, for G = 1 and 16 too
+        assert_parity(pa.run_attn("decode", 0, q[47:], pos, gate=None if gate is None else gate[47:]), refb[47:], "one-column decode")
